@@ -1,0 +1,260 @@
+/* torpor_amd: C-ABI of the MI355X-native model-swapping inference engine.
+ *
+ * The reference server (FCSLab/torpor) has no C-ABI of its own: its wire layer
+ * calls header-only C++ classes directly.  Each entry point below therefore
+ * names the reference method whose job it does (paths relative to the
+ * reference tree).  A ZMQ front end binds these exactly where the reference
+ * dispatches a SignalRequest (include/server/controller.hpp:128-216) or a
+ * WapperQuery (include/server/cuda_server.hpp:301-455).
+ *
+ * Conventions
+ *   - return value: 0 = ok, negative = engine error (TP_E*), positive = hipError_t.
+ *   - no exceptions or aborts cross this boundary.
+ *   - device addresses handed to callers are opaque 64-bit *virtual* addresses
+ *     that stay valid across swap-out / swap-in (the reference's
+ *     cudaMallocResponse.ptr, proto/cudarpc.proto:303-306).
+ *   - the caller keeps ownership of every host buffer it passes; the engine
+ *     copies in and out.
+ *   - one control thread and one executor thread may call concurrently; there
+ *     is one active function per GPU at a time (cuda_server.hpp:1371,
+ *     controller.hpp:415).
+ *   - asynchronous op failures are sticky and reported by the next
+ *     tp_stream_synchronize / tp_device_synchronize (same wire field as the
+ *     reference's `int32 error`, proto/cudarpc.proto:85-87).
+ */
+#ifndef TORPOR_AMD_H
+#define TORPOR_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tp_server tp_server;
+
+/* ---- error codes (negative) ---- */
+#define TP_OK 0
+#define TP_EINVAL (-22)        /* bad argument / shape */
+#define TP_ENOMEM (-12)        /* pool or host store exhausted */
+#define TP_ENOENT (-2)         /* unknown function / address */
+#define TP_EBUSY (-16)         /* executor busy or function active */
+#define TP_ENODEV (-19)        /* engine created with TP_FLAG_HOST_ONLY: no compute, no device memory */
+#define TP_ESTATE (-71)        /* call not valid in the executor's current mode */
+#define TP_ENOTACTIVE (-72)    /* client id is not the active function */
+#define TP_EUNSUPPORTED (-38)  /* shape / option not implemented */
+#define TP_EFAULT (-14)        /* virtual address does not translate */
+
+/* ---- signal.proto enums (proto/signal.proto:5-30) ---- */
+#define TP_REQ_EXECUTE_AFTER_LOAD 0 /* register model */
+#define TP_REQ_EXECUTE 1            /* invoke */
+#define TP_REQ_LOAD 2               /* swap-in (prefetch) */
+#define TP_REQ_UNLOAD 3             /* swap-out */
+#define TP_REQ_EXECUTE_FOR_RECORD 10
+#define TP_REQ_REPLAY 11
+#define TP_ACK_OK 0
+#define TP_ACK_INAVAIL 1
+
+/* ---- tp_config.flags ---- */
+#define TP_FLAG_HOST_ONLY 1 /* no HIP calls: pool/LRU/state-machine logic only (CPU tests) */
+
+/* ---- activation / epilogue ---- */
+#define TP_ACT_NONE 0
+#define TP_ACT_RELU 1
+#define TP_ACT_GELU 2 /* erf form */
+#define TP_ACT_TANH 3
+
+/* ---- tensor layouts for convolution / pooling / batch-norm ---- */
+#define TP_LAYOUT_NCHW 0
+#define TP_LAYOUT_NHWC 1
+
+/* ---- op ids for tp_launch (takes the place of launching libtorch kernels by
+ *      mangled name, cuda_server.hpp:1226-1310) ----
+ *   ptr / int / float argument lists per op:                                  */
+#define TP_OP_RELU 1         /* p: x,y          i: n */
+#define TP_OP_ADD 2          /* p: a,b,y        i: n, relu */
+#define TP_OP_BIAS_ACT 3     /* p: x,bias,y     i: rows, C, act */
+#define TP_OP_GELU 4         /* p: x,y          i: n */
+#define TP_OP_MAXPOOL 5      /* p: x,y          i: N,H,W,C,k,stride,pad,layout */
+#define TP_OP_AVGPOOL 6      /* p: x,y          i: N,HW,C,layout   (global average) */
+#define TP_OP_LAYERNORM 7    /* p: x,res|0,gamma,beta,y  i: rows,width  f: eps */
+#define TP_OP_SOFTMAX 8      /* p: x,mask|0,y   i: rows,width,rows_per_mask  f: scale */
+#define TP_OP_EMBEDDING 9    /* p: ids,type_ids|0,word,pos|0,type|0,y  i: tokens,seq,width,vocab,n_types */
+#define TP_OP_NCHW_TO_NHWC 10 /* p: x,y         i: N,C,H,W */
+#define TP_OP_NHWC_TO_NCHW 11 /* p: x,y         i: N,C,H,W */
+#define TP_OP_SUM 12         /* p: x,y          i: n */
+#define TP_OP_FILL 13        /* p: y            i: n   f: value */
+
+typedef struct tp_config {
+    uint32_t struct_size;       /* sizeof(tp_config) */
+    int32_t device;             /* HIP device ordinal */
+    uint64_t mem_limit_bytes;   /* LRU budget; 0: env MEM_LIMIT_IN_GB or 24 GiB (controller.hpp:83-93) */
+    uint64_t pool_bytes;        /* HBM arena; 0: mem_limit + pool headroom (memory_manager.hpp:42-44) */
+    uint64_t chunk_bytes;       /* first swap-in gate group; 0: env BUFFER_SIZE or 2 MiB (memory_manager.hpp:22,169-173) */
+    uint64_t chunk_max_bytes;   /* groups double up to this size; 0: 8 MiB; set = chunk_bytes for fixed groups */
+    uint64_t workspace_bytes;   /* split-K scratch; 0: 64 MiB */
+    int32_t flags;              /* TP_FLAG_* */
+    int32_t request_timeout_ms; /* 0: 5000 (cuda_server.hpp:29) */
+} tp_config;
+
+typedef struct tp_epilogue {
+    float alpha;       /* scales the accumulator */
+    float beta;        /* + beta * previous C */
+    uint64_t bias;     /* [N] or 0 */
+    uint64_t bn_scale; /* inference batch-norm gamma [N] or 0; the four bn_* go together */
+    uint64_t bn_bias;
+    uint64_t bn_mean;
+    uint64_t bn_var;
+    float bn_eps;
+    int32_t act;       /* TP_ACT_* */
+    uint64_t residual; /* same shape as C, or 0 */
+    int64_t ldr;       /* row pitch of residual (0: same as C) */
+} tp_epilogue;
+
+/* Row-major GEMM C[r][c] = epilogue(sum_k X(r,k) * Y(c,k)), X(r,k) at x + r*xs_r + k*xs_k
+ * (elements), Y(c,k) at y + c*ys_c + k*ys_k; batch z = b0*nb1 + b1. */
+typedef struct tp_gemm_desc {
+    uint64_t x, y, c;
+    int64_t m, n, k;
+    int64_t xs_r, xs_k, ys_c, ys_k, ldc;
+    int32_t nb0, nb1;
+    int64_t xb0, xb1, yb0, yb1, cb0, cb1;
+    tp_epilogue ep;
+} tp_gemm_desc;
+
+typedef struct tp_conv_desc {
+    uint64_t x, w, y; /* w is [Cout][Cin][KH][KW] */
+    int32_t n, h, w_in, cin, cout, kh, kw;
+    int32_t stride_h, stride_w, pad_h, pad_w, groups;
+    int32_t x_layout, y_layout; /* TP_LAYOUT_* */
+    tp_epilogue ep;
+} tp_conv_desc;
+
+typedef struct tp_pool_stats {
+    uint64_t capacity, used, largest_free;
+    uint64_t live_extents, free_extents;
+    uint64_t lru_budget, lru_used, lru_models;
+    uint64_t evictions, swap_ins;
+} tp_pool_stats;
+
+typedef struct tp_model_info {
+    int32_t registered; /* host store complete */
+    int32_t resident;   /* weights allocated in the pool */
+    int32_t level;
+    int32_t n_params;
+    int32_t n_chunks;
+    int32_t n_ops;       /* recorded program length */
+    uint64_t image_bytes; /* weight image (256 B aligned tensors, first-access order) */
+    uint64_t param_bytes; /* sum of tensor sizes */
+    uint64_t act_bytes;   /* activation arena */
+    uint64_t total_bytes; /* what the LRU charges */
+    uint64_t weight_off;  /* pool offsets when resident */
+    uint64_t act_off;
+} tp_model_info;
+
+typedef struct tp_swap_stats {
+    uint64_t bytes;      /* weight bytes moved by the last swap-in of this model */
+    double copy_ms;      /* first copy issued -> last copy landed, on the copy stream */
+    double alloc_us;     /* host time to (re)acquire pool extents ("CheckMalloc", memory_manager.hpp:499-501) */
+    double evict_us;     /* host time of the last swap-out (memory_manager.hpp:258) */
+    uint32_t chunks;
+    uint32_t gate_waits; /* compute-stream waits issued during the last request */
+} tp_swap_stats;
+
+/* ------------------------------------------------------------------ lifecycle
+ * Controller ctor + CUDAExecutor::start (controller.hpp:54-121, cuda_server.hpp:92-118,
+ * memory_manager.hpp:168-193, block_manager.hpp:264-273). */
+int tp_server_create(const tp_config* cfg, tp_server** out);
+void tp_server_destroy(tp_server* s);
+const char* tp_strerror(int code);
+const char* tp_version(void);
+
+/* ------------------------------------------------------------------ control plane
+ * One SignalRequest -> SignalAck exchange (controller.hpp:131-216).  `function` is the
+ * decimal client id.  When the executor is busy the request is queued
+ * (controller.hpp:156,177) and *deferred is set to 1: its ack appears later through
+ * tp_take_deferred_ack, after the active request completes (controller.hpp:242-262). */
+int tp_signal(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack, int32_t* resp,
+              int32_t* deferred);
+int tp_take_deferred_ack(tp_server* s, int32_t* ack, int32_t* resp); /* 1 = ack produced, 0 = none */
+/* Request-timeout check of the executor loop (cuda_server.hpp:257-264); returns 1 when a
+ * timed-out request was force-completed. */
+int tp_poll(tp_server* s);
+
+/* ------------------------------------------------------------------ data plane: memory
+ * cudaMallocService / cudaFreeService (cuda_server.hpp:965-992, memory_manager.hpp:85-110). */
+int tp_malloc(tp_server* s, int32_t client, uint64_t bytes, uint64_t* vaddr);
+int tp_free(tp_server* s, int32_t client, uint64_t vaddr);
+/* cudaMemcpyService / cudaMemcpyAsyncService H2D (cuda_server.hpp:994-1037); while the
+ * function is being registered the bytes go to the host weight store
+ * (memory_manager.hpp:124-142, model_repo.hpp:151-168). */
+int tp_memcpy_h2d(tp_server* s, int32_t client, uint64_t dst, const void* src, uint64_t bytes);
+/* cudaMemcpyAsyncService D2H (cuda_server.hpp:1038-1045): staged, delivered into `dst` by the
+ * next tp_stream_synchronize, and marks the request finished (send_complete_signal). */
+int tp_memcpy_d2h_async(tp_server* s, int32_t client, void* dst, uint64_t src, uint64_t bytes);
+/* cudaMemcpyService D2H (cuda_server.hpp:1006-1011): synchronous, no completion side effect. */
+int tp_memcpy_d2h(tp_server* s, int32_t client, void* dst, uint64_t src, uint64_t bytes);
+int tp_memcpy_d2d(tp_server* s, int32_t client, uint64_t dst, uint64_t src, uint64_t bytes); /* cuda_server.hpp:1047-1051 */
+int tp_memset_async(tp_server* s, int32_t client, uint64_t dst, int32_t value, uint64_t bytes); /* cuda_server.hpp:1058-1068 */
+/* cudaDeviceSynchronizeService (cuda_server.hpp:951-962): also ends the weight-upload phase of a
+ * registration and starts access tracking. */
+int tp_device_synchronize(tp_server* s, int32_t client);
+/* cudaStreamSynchronizeService (cuda_server.hpp:1132-1149). */
+int tp_stream_synchronize(tp_server* s, int32_t client);
+
+/* ------------------------------------------------------------------ data plane: compute */
+/* cublasSgemmService (cuda_server.hpp:502-522): column-major, op(A) m x k, op(B) k x n.
+ * transa/transb: 0 = N, 1 = T. */
+int tp_sgemm(tp_server* s, int32_t client, int32_t transa, int32_t transb, int32_t m, int32_t n, int32_t k,
+             float alpha, uint64_t a, int32_t lda, uint64_t b, int32_t ldb, float beta, uint64_t c, int32_t ldc);
+/* cublasSgemmStridedBatchedService (cuda_server.hpp:524-550). */
+int tp_sgemm_strided_batched(tp_server* s, int32_t client, int32_t transa, int32_t transb, int32_t m, int32_t n,
+                             int32_t k, float alpha, uint64_t a, int32_t lda, int64_t stride_a, uint64_t b,
+                             int32_t ldb, int64_t stride_b, float beta, uint64_t c, int32_t ldc, int64_t stride_c,
+                             int32_t count);
+/* Row-major GEMM with fused epilogue and two-level batching (the HIP-native form of the two above). */
+int tp_gemm(tp_server* s, int32_t client, const tp_gemm_desc* d);
+/* cudnnConvolutionForwardService (cuda_server.hpp:708-735), shapes inline instead of descriptor
+ * handles (cuda_server.hpp:579-706), optional fused epilogue. */
+int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d);
+/* cudnnBatchNormalizationForwardInferenceService (cuda_server.hpp:737-771). */
+int tp_bn_inference(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
+                    uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
+                    int32_t layout, int32_t relu);
+/* cudaLaunchKernelService (cuda_server.hpp:1226-1310) by op id, pointer slots explicit. */
+int tp_launch(tp_server* s, int32_t client, int32_t op_id, const uint64_t* ptrs, int32_t n_ptrs,
+              const int64_t* ints, int32_t n_ints, const float* floats, int32_t n_floats);
+
+/* ------------------------------------------------------------------ replay
+ * The op stream of the first (tracked) inference is kept per function
+ * (signal.proto ExecuteForRecord / Replay).  tp_replay re-issues it: recorded H2D copies read
+ * consecutive slices of `input`, recorded D2H copies fill consecutive slices of `output`; it
+ * includes the final stream synchronisation and completion signal. */
+int tp_replay(tp_server* s, int32_t client, const void* input, uint64_t input_bytes, void* output,
+              uint64_t output_bytes);
+
+/* ------------------------------------------------------------------ introspection (tests, bench) */
+int tp_model_resident(tp_server* s, int32_t client); /* 1/0, negative on error */
+int tp_get_model_info(tp_server* s, int32_t client, tp_model_info* out);
+int tp_get_pool_stats(tp_server* s, tp_pool_stats* out);
+int tp_get_swap_stats(tp_server* s, int32_t client, tp_swap_stats* out);
+/* Copies the device-resident weight image (waits for an in-flight swap-in). */
+int tp_readback_weights(tp_server* s, int32_t client, void* dst, uint64_t bytes);
+/* The authoritative host copy of the same image, same layout. */
+int tp_host_weights(tp_server* s, int32_t client, const void** ptr, uint64_t* bytes);
+/* Image offset of a weight virtual address (first-access-order layout). */
+int tp_weight_offset(tp_server* s, int32_t client, uint64_t vaddr, uint64_t* image_off);
+/* Name of the kernel variant chosen by the last compute op on the calling thread. */
+const char* tp_last_kernel(void);
+/* Pinned-host -> HBM link probe: one hipMemcpyAsync of `bytes`, median of `iters`; GB/s. */
+int tp_measure_h2d(tp_server* s, uint64_t bytes, int32_t iters, double* gbps);
+/* Runs `iters` timed repetitions of the last compute op recorded for `client` at program index
+ * `op_index` (or -1: last op) and returns the mean duration in microseconds measured with HIP
+ * events on the compute stream. */
+int tp_time_op(tp_server* s, int32_t client, int32_t op_index, int32_t iters, double* mean_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORPOR_AMD_H */

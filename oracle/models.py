@@ -1,0 +1,153 @@
+"""TEST INFRASTRUCTURE ONLY - imported by tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg, never by the product.
+
+Plain `torch.nn` ResNet (v1.5 bottleneck) and BERT encoder, run on the CPU in fp32: the
+"native PyTorch path" the hot path's logits are compared with.  The reference builds its
+served models from torchvision / Hugging Face packages at run time (tests/endpoint.py:16-40),
+which are third-party code absent from the reference tree:
+  - torchvision.models.resnet (v0.10-era, image nvcr.io/nvidia/pytorch:22.01-py3,
+    dockerfiles/base.Dockerfile:18)  - not installed here; its published architecture
+    (He et al. 2015 + stride on the 3x3, BN eps 1e-5, bias-free convs) is restated and pinned
+    by closed-form parameter / MAC counts (tests/test_oracle_models.py).
+  - transformers==4.27.1 BertModel (dockerfiles/client.Dockerfile:4-5) - a newer transformers
+    is installed here; `Bert` below is pinned against it on a small config with shared weights.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+RESNET_LAYERS = {"resnet50": (3, 4, 6, 3), "resnet101": (3, 4, 23, 3), "resnet152": (3, 8, 36, 3)}
+
+
+class Bottleneck(nn.Module):
+    expansion = 4
+
+    def __init__(self, inplanes, planes, stride=1, downsample=None):
+        super().__init__()
+        self.conv1 = nn.Conv2d(inplanes, planes, 1, bias=False)
+        self.bn1 = nn.BatchNorm2d(planes)
+        self.conv2 = nn.Conv2d(planes, planes, 3, stride=stride, padding=1, bias=False)
+        self.bn2 = nn.BatchNorm2d(planes)
+        self.conv3 = nn.Conv2d(planes, planes * 4, 1, bias=False)
+        self.bn3 = nn.BatchNorm2d(planes * 4)
+        self.downsample = downsample
+
+    def forward(self, x):
+        idt = x
+        out = F.relu(self.bn1(self.conv1(x)))
+        out = F.relu(self.bn2(self.conv2(out)))
+        out = self.bn3(self.conv3(out))
+        if self.downsample is not None:
+            idt = self.downsample(x)
+        return F.relu(out + idt)
+
+
+class ResNet(nn.Module):
+    def __init__(self, arch="resnet50", num_classes=1000):
+        super().__init__()
+        self.inplanes = 64
+        self.conv1 = nn.Conv2d(3, 64, 7, stride=2, padding=3, bias=False)
+        self.bn1 = nn.BatchNorm2d(64)
+        blocks = RESNET_LAYERS[arch]
+        self.layer1 = self._make(64, blocks[0], 1)
+        self.layer2 = self._make(128, blocks[1], 2)
+        self.layer3 = self._make(256, blocks[2], 2)
+        self.layer4 = self._make(512, blocks[3], 2)
+        self.fc = nn.Linear(2048, num_classes)
+
+    def _make(self, planes, n, stride):
+        ds = None
+        if stride != 1 or self.inplanes != planes * 4:
+            ds = nn.Sequential(nn.Conv2d(self.inplanes, planes * 4, 1, stride=stride, bias=False),
+                               nn.BatchNorm2d(planes * 4))
+        layers = [Bottleneck(self.inplanes, planes, stride, ds)]
+        self.inplanes = planes * 4
+        for _ in range(1, n):
+            layers.append(Bottleneck(self.inplanes, planes))
+        return nn.Sequential(*layers)
+
+    def forward(self, x):
+        x = F.relu(self.bn1(self.conv1(x)))
+        x = F.max_pool2d(x, 3, 2, 1)
+        x = self.layer4(self.layer3(self.layer2(self.layer1(x))))
+        x = torch.flatten(F.adaptive_avg_pool2d(x, 1), 1)
+        return self.fc(x)
+
+
+class BertLayer(nn.Module):
+    def __init__(self, H, A, Fd, eps):
+        super().__init__()
+        self.A = A
+        att = nn.Module()
+        att.self = nn.Module()
+        att.self.query, att.self.key, att.self.value = nn.Linear(H, H), nn.Linear(H, H), nn.Linear(H, H)
+        att.output = nn.Module()
+        att.output.dense = nn.Linear(H, H)
+        att.output.LayerNorm = nn.LayerNorm(H, eps=eps)
+        self.attention = att
+        self.intermediate = nn.Module()
+        self.intermediate.dense = nn.Linear(H, Fd)
+        self.output = nn.Module()
+        self.output.dense = nn.Linear(Fd, H)
+        self.output.LayerNorm = nn.LayerNorm(H, eps=eps)
+
+    def forward(self, h, mask):
+        B, S, H = h.shape
+        dh = H // self.A
+
+        def heads(t):
+            return t.view(B, S, self.A, dh).permute(0, 2, 1, 3)
+
+        sa = self.attention.self
+        q, k, v = heads(sa.query(h)), heads(sa.key(h)), heads(sa.value(h))
+        scores = q @ k.transpose(-1, -2) / math.sqrt(dh)
+        if mask is not None:
+            scores = scores + mask
+        ctx = (scores.softmax(-1) @ v).permute(0, 2, 1, 3).reshape(B, S, H)
+        h1 = self.attention.output.LayerNorm(self.attention.output.dense(ctx) + h)
+        inter = F.gelu(self.intermediate.dense(h1))
+        return self.output.LayerNorm(self.output.dense(inter) + h1)
+
+
+class Bert(nn.Module):
+    """Parameter names equal those of transformers.BertModel (minus buffers)."""
+
+    def __init__(self, layers=12, hidden=768, heads=12, ffn=3072, vocab=30522, max_pos=512, type_vocab=2,
+                 eps=1e-12):
+        super().__init__()
+        emb = nn.Module()
+        emb.word_embeddings = nn.Embedding(vocab, hidden)
+        emb.position_embeddings = nn.Embedding(max_pos, hidden)
+        emb.token_type_embeddings = nn.Embedding(type_vocab, hidden)
+        emb.LayerNorm = nn.LayerNorm(hidden, eps=eps)
+        self.embeddings = emb
+        self.encoder = nn.Module()
+        self.encoder.layer = nn.ModuleList([BertLayer(hidden, heads, ffn, eps) for _ in range(layers)])
+        self.pooler = nn.Module()
+        self.pooler.dense = nn.Linear(hidden, hidden)
+
+    def forward(self, ids, token_type_ids=None, attention_mask=None):
+        B, S = ids.shape
+        e = self.embeddings
+        tt = token_type_ids if token_type_ids is not None else torch.zeros_like(ids)
+        pos = torch.arange(S).unsqueeze(0).expand(B, S)
+        h = e.LayerNorm(e.word_embeddings(ids) + e.position_embeddings(pos) + e.token_type_embeddings(tt))
+        mask = None
+        if attention_mask is not None:
+            mask = (1.0 - attention_mask[:, None, None, :].float()) * torch.finfo(torch.float32).min
+        for layer in self.encoder.layer:
+            h = layer(h, mask)
+        pooled = torch.tanh(self.pooler.dense(h[:, 0]))
+        return h, pooled
+
+
+def load_numpy_state(module, weights):
+    """Strictly load a {name: np.ndarray} dict (BN `num_batches_tracked` buffers excepted)."""
+    sd = {k: torch.from_numpy(v.copy()) for k, v in weights.items()}
+    missing, unexpected = module.load_state_dict(sd, strict=False)
+    missing = [m for m in missing if not m.endswith("num_batches_tracked")]
+    if missing or unexpected:
+        raise KeyError(f"missing={missing} unexpected={list(unexpected)}")
+    return module.eval()

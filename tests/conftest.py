@@ -1,0 +1,22 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="module")
+def gpu_server():
+    """One engine per test module: 6 GiB pool, 4 GiB LRU budget."""
+    from torpor_amd.server import Server
+
+    s = Server(mem_limit_bytes=4 << 30, pool_bytes=6 << 30)
+    yield s
+    s.close()

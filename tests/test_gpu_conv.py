@@ -1,0 +1,106 @@
+"""Convolution kernels vs the direct-loop fp64 C oracle, through the C-ABI (reference call site
+cudnnConvolutionForward, include/server/cuda_server.hpp:708-735)."""
+import numpy as np
+import pytest
+
+from oracle import ops as ref
+from tests.harness import OpSession, assert_close
+from torpor_amd.server import ACT_NONE, ACT_RELU, NCHW, NHWC
+
+pytestmark = pytest.mark.gpu
+RTOL = 3e-5
+
+
+def _rand(rng, *shape):
+    return rng.standard_normal(shape).astype(np.float32)
+
+
+CASES = [
+    # N, H, W, Cin, Cout, k, stride, pad, x_layout, y_layout, expected kernel
+    (1, 56, 56, 64, 64, 1, 1, 0, NHWC, NHWC, "gemm_fast"),        # 1x1
+    (2, 28, 28, 256, 512, 1, 2, 0, NHWC, NHWC, "gemm_fast"),      # 1x1 stride 2 (downsample)
+    (1, 56, 56, 64, 64, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # 3x3
+    (2, 28, 28, 128, 128, 3, 2, 1, NHWC, NHWC, "conv3x3_fast"),   # 3x3 stride 2
+    (1, 7, 7, 512, 512, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # tiny map, split-K
+    (8, 28, 28, 128, 128, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),   # batch 8
+    (1, 64, 64, 3, 64, 7, 2, 3, NCHW, NHWC, "conv_generic"),      # stem: NCHW in, NHWC out
+    (1, 13, 11, 5, 7, 3, 1, 1, NCHW, NCHW, "conv_generic"),       # odd sizes, NCHW both
+    (1, 9, 9, 12, 20, 5, 2, 2, NHWC, NCHW, "conv_generic"),       # 5x5, mixed layouts
+    (1, 10, 10, 12, 16, 3, 1, 0, NHWC, NHWC, "conv_generic"),     # Cin % 8 != 0
+]
+
+
+@pytest.mark.parametrize("N,H,W,Cin,Cout,k,stride,pad,xl,yl,kern", CASES)
+def test_conv(gpu_server, N, H, W, Cin, Cout, k, stride, pad, xl, yl, kern):
+    rng = np.random.default_rng(N + H * 3 + Cin * 5 + Cout * 7 + k)
+    x_nchw = _rand(rng, N, Cin, H, W)
+    w = _rand(rng, Cout, Cin, k, k) * np.float32(1.0 / np.sqrt(Cin * k * k))
+    x = x_nchw if xl == NCHW else np.ascontiguousarray(x_nchw.transpose(0, 2, 3, 1))
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    with OpSession(gpu_server, [w]) as t:
+        xv = t.act(x)
+        yv = t.empty(N * Ho * Wo * Cout * 4)
+        t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, k, k, stride=stride, pad=pad, x_layout=xl, y_layout=yl)
+        assert t.s.last_kernel().startswith(kern), t.s.last_kernel()
+        got = t.read(yv, (N, Ho, Wo, Cout) if yl == NHWC else (N, Cout, Ho, Wo))
+    want = ref.conv2d(x, w, (stride, stride), (pad, pad), x_nhwc=(xl == NHWC), y_nhwc=(yl == NHWC))
+    assert_close(got, want, RTOL, f"conv {k}x{k} s{stride}")
+
+
+@pytest.mark.parametrize("k,Cin,Cout,HW", [(1, 64, 256, 14), (3, 64, 64, 14), (7, 3, 16, 20)])
+def test_conv_bn_residual_relu(gpu_server, k, Cin, Cout, HW):
+    """The fused epilogue of a bottleneck's last convolution: relu(bn(conv(x)) + identity)."""
+    rng = np.random.default_rng(k)
+    N, pad = 2, k // 2
+    x = _rand(rng, N, HW, HW, Cin)
+    w = _rand(rng, Cout, Cin, k, k) * np.float32(1.0 / np.sqrt(Cin * k * k))
+    g, b, mu = _rand(rng, Cout), _rand(rng, Cout), _rand(rng, Cout)
+    var = rng.uniform(0.5, 2.0, Cout).astype(np.float32)
+    res = _rand(rng, N, HW, HW, Cout)
+    with OpSession(gpu_server, [w, g, b, mu, var]) as t:
+        xv, rv = t.act(x), t.act(res)
+        yv = t.empty(res.nbytes)
+        t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, Cin, Cout, k, k, stride=1, pad=pad, bn=tuple(t.w[1:5]),
+                 bn_eps=1e-5, residual=rv, act=ACT_RELU)
+        got = t.read(yv, res.shape)
+    z = ref.conv2d(x, w, (1, 1), (pad, pad), x_nhwc=True, y_nhwc=True)
+    z = ref.bn(z, g, b, mu, var, 1e-5, Cout, nhwc=True).astype(np.float64) + res
+    assert_close(got, np.maximum(z, 0), 5e-5, "conv+bn+res+relu")
+
+
+def test_conv_identities(gpu_server):
+    """Closed forms: a centred delta kernel is the identity; an all-ones 3x3 kernel on an all-ones
+    image counts the in-bounds taps (4 / 6 / 9 at corner / edge / interior)."""
+    C, HW = 8, 12
+    rng = np.random.default_rng(0)
+    x = _rand(rng, 1, HW, HW, C)
+    delta = np.zeros((C, C, 3, 3), np.float32)
+    for c in range(C):
+        delta[c, c, 1, 1] = 1.0
+    ones_w = np.ones((C, C, 3, 3), np.float32)
+    with OpSession(gpu_server, [delta, ones_w]) as t:
+        xv, ov = t.act(x), t.act(np.ones_like(x))
+        yv = t.empty(x.nbytes)
+        t.s.conv(t.fid, xv, t.w[0], yv, 1, HW, HW, C, C, 3, 3, stride=1, pad=1)
+        got = t.read(yv, x.shape)
+        np.testing.assert_array_equal(got, x)
+        t.s.conv(t.fid, ov, t.w[1], yv, 1, HW, HW, C, C, 3, 3, stride=1, pad=1)
+        cnt = t.read(yv, x.shape)
+    assert cnt[0, 0, 0, 0] == 4 * C and cnt[0, 0, 5, 0] == 6 * C and cnt[0, 5, 5, 0] == 9 * C
+
+
+def test_conv_rejects_bad_shapes(gpu_server):
+    from torpor_amd._lib import TorporError
+    w = np.zeros((8, 8, 3, 3), np.float32)
+    with OpSession(gpu_server, [w]) as t:
+        xv = t.act(np.zeros((1, 6, 6, 8), np.float32))
+        yv = t.empty(1 * 6 * 6 * 8 * 4)
+        with pytest.raises(TorporError):   # claims a larger input than the buffer holds
+            t.s.conv(t.fid, xv, t.w[0], yv, 1, 8, 8, 8, 8, 3, 3, stride=1, pad=1)
+        with pytest.raises(TorporError):   # claims more filters than uploaded
+            t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 16, 3, 3, stride=1, pad=1)
+        with pytest.raises(TorporError):   # grouped convolution is not implemented
+            t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1, groups=2)
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)
+        t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1)

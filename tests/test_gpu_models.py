@@ -1,0 +1,126 @@
+"""Whole-function parity on the GPU: logits against the plain PyTorch CPU forward of the same
+seeded weights and inputs (rel 1e-3, fp32), swapped weights byte-identical to the host copy,
+and warm / cold / replayed requests bit-identical to each other."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import models as om
+from tests.harness import assert_close
+from torpor_amd.functions import bert, resnet
+
+pytestmark = pytest.mark.gpu
+LOGIT_RTOL = 1e-3   # north-star bar: rel 1e-3 (fp32) on logits
+
+
+def _perturb_bn(weights, seed):
+    """Non-trivial batch-norm statistics, so that a wrong BN fold cannot pass."""
+    rng = np.random.default_rng(seed)
+    for k in list(weights):
+        n = weights[k].shape
+        if k.endswith("running_var"):
+            weights[k] = rng.uniform(0.5, 1.5, n).astype(np.float32)
+        elif k.endswith("running_mean"):
+            weights[k] = (rng.standard_normal(n) * 0.1).astype(np.float32)
+        elif ".bn" in k or "downsample.1" in k or k.startswith("bn1"):
+            if k.endswith(".weight"):
+                weights[k] = rng.uniform(0.8, 1.2, n).astype(np.float32)
+            elif k.endswith(".bias"):
+                weights[k] = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    return weights
+
+
+def _check_swap_identity(server, fn, weights):
+    """Every uploaded tensor sits, byte for byte, at its image offset in the host store and in
+    the device copy read back from HBM."""
+    host = server.host_weights(fn.fid)
+    dev = server.readback_weights(fn.fid)
+    assert host.nbytes == dev.nbytes
+    assert np.array_equal(host, dev), "device weight image differs from the host copy"
+    for name, arr in weights.items():
+        if name not in fn.w:
+            continue
+        raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+        off = server.weight_offset(fn.fid, fn.w[name])
+        assert np.array_equal(dev[off:off + raw.size], raw), name
+
+
+def _cycle(server, fn, inputs, first):
+    """warm replay, warm op-by-op, cold replay: all bit-identical to the tracked first run."""
+    warm = fn.invoke(inputs)
+    for a, b in zip(first, warm):
+        assert np.array_equal(a, b), "warm replay differs from the first run"
+    warm2 = fn.invoke(inputs, replay=False)
+    for a, b in zip(first, warm2):
+        assert np.array_equal(a, b), "op-by-op request differs from the first run"
+    ack, resp, _ = fn.unload()
+    assert ack == 0 and resp == -1 and not server.resident(fn.fid)
+    cold = fn.invoke(inputs)
+    assert server.resident(fn.fid)
+    for a, b in zip(first, cold):
+        assert np.array_equal(a, b), "cold (swap-in) request differs from the first run"
+    st = server.swap_stats(fn.fid)
+    assert st["bytes"] == server.model_info(fn.fid)["image_bytes"] and st["copy_ms"] > 0
+    return st
+
+
+@pytest.mark.parametrize("arch,batch", [("resnet50", 1), ("resnet152", 8)])
+def test_resnet(gpu_server, arch, batch):
+    fid = {"resnet50": 1, "resnet152": 3}[arch]
+    weights = _perturb_bn(resnet.init_weights(arch, seed=0), seed=1)
+    x = torch.randn(batch, 3, 224, 224, generator=torch.Generator().manual_seed(0)).numpy()
+    fn = resnet.ResNet(gpu_server, fid, arch, batch=batch, weights=weights)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.ResNet(arch), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    err = assert_close(logits, want, LOGIT_RTOL, f"{arch} logits")
+    print(f"{arch} b{batch}: logits rel err {err:.2e}")
+    info = gpu_server.model_info(fid)
+    n_params = sum(int(np.prod(v.shape)) for k, v in weights.items() if "running" not in k)
+    assert n_params == {"resnet50": 25557032, "resnet152": 60192808}[arch]
+    assert info["param_bytes"] == sum(v.nbytes for v in weights.values())
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    _check_swap_identity(gpu_server, fn, weights)
+    fn.unload()
+
+
+@pytest.mark.parametrize("arch,batch,seq", [("bert-base", 1, 128), ("bert-large", 4, 384)])
+def test_bert(gpu_server, arch, batch, seq):
+    fid = {"bert-base": 2, "bert-large": 4}[arch]
+    weights = bert.init_weights(arch, seed=0)
+    ids = torch.randint(0, 30522, (batch, seq), generator=torch.Generator().manual_seed(0)).numpy()
+    fn = bert.Bert(gpu_server, fid, arch, batch=batch, seq=seq, weights=weights)
+    hidden, pooled = fn.register([ids])
+    model = om.load_numpy_state(om.Bert(**bert.CONFIGS[arch]), weights)
+    with torch.no_grad():
+        want_h, want_p = model(torch.from_numpy(ids))
+    e1 = assert_close(hidden, want_h.numpy(), LOGIT_RTOL, f"{arch} last hidden state")
+    e2 = assert_close(pooled, want_p.numpy(), LOGIT_RTOL, f"{arch} pooled output")
+    print(f"{arch} b{batch} s{seq}: rel err hidden {e1:.2e} pooled {e2:.2e}")
+    n_params = sum(int(np.prod(v.shape)) for v in weights.values())
+    assert n_params == {"bert-base": 109482240, "bert-large": 335141888}[arch]
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [ids], [hidden, pooled])
+    _check_swap_identity(gpu_server, fn, weights)
+    fn.unload()
+
+
+def test_image_is_in_first_access_order(gpu_server):
+    """ResNet uploads `downsample` after `conv3` (state-dict order) but uses it before: after
+    registration the image must hold the tensors in the order the tracked run touched them."""
+    weights = resnet.init_weights("resnet50", seed=3)
+    x = np.zeros((1, 3, 64, 64), np.float32)
+    fn = resnet.ResNet(gpu_server, 9, "resnet50", batch=1, weights=weights, image=64)
+    fn.register([x])
+    off = {k: gpu_server.weight_offset(9, va) for k, va in fn.w.items()}
+    assert off["conv1.weight"] == 0
+    assert off["layer1.0.downsample.0.weight"] < off["layer1.0.conv3.weight"]
+    assert off["layer1.0.conv2.weight"] < off["layer1.0.downsample.0.weight"]
+    assert off["fc.bias"] == max(off.values())
+    ordered = sorted(off.values())
+    sizes = {off[k]: weights[k].nbytes for k in off}
+    for a, b in zip(ordered, ordered[1:]):
+        assert a % 256 == 0 and a + sizes[a] <= b
+    fn.unload()

@@ -1,0 +1,171 @@
+"""HBM-bound operators vs the C oracle, through the C-ABI (reference call sites
+cudnnBatchNormalizationForwardInference, include/server/cuda_server.hpp:737-771, and libtorch
+kernels launched through cudaLaunchKernel, include/server/cuda_server.hpp:1226-1310)."""
+import numpy as np
+import pytest
+
+from oracle import ops as ref
+from tests.harness import OpSession, assert_close
+from torpor_amd.server import (NCHW, NHWC, OP_ADD, OP_AVGPOOL, OP_BIAS_ACT, OP_EMBEDDING, OP_FILL, OP_GELU,
+                               OP_LAYERNORM, OP_MAXPOOL, OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_RELU, OP_SOFTMAX,
+                               OP_SUM, ACT_RELU)
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(rng, *shape):
+    return rng.standard_normal(shape).astype(np.float32)
+
+
+@pytest.mark.parametrize("layout,C,relu", [(NHWC, 64, True), (NHWC, 7, False), (NCHW, 5, True)])
+def test_bn_inference(gpu_server, layout, C, relu):
+    rng = np.random.default_rng(C)
+    N, H, W = 2, 9, 11
+    x = _rand(rng, N, H, W, C) if layout == NHWC else _rand(rng, N, C, H, W)
+    g, b, mu = _rand(rng, C), _rand(rng, C), _rand(rng, C)
+    var = rng.uniform(0.1, 3.0, C).astype(np.float32)
+    with OpSession(gpu_server, [g, b, mu, var]) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        t.s.bn(t.fid, xv, yv, *t.w[:4], 1e-5, N * H * W, C, hw=H * W, layout=layout, relu=relu)
+        got = t.read(yv, x.shape)
+    want = ref.bn(x, g, b, mu, var, 1e-5, C, hw=H * W, nhwc=(layout == NHWC), relu=relu)
+    assert_close(got, want, 1e-6, "bn")
+
+
+def test_bn_identity(gpu_server):
+    """gamma=1, beta=0, mean=0, var=1-eps is the identity map."""
+    rng = np.random.default_rng(1)
+    C = 16
+    x = _rand(rng, 3, 5, 5, C)
+    eps = 1e-5
+    ws = [np.ones(C, np.float32), np.zeros(C, np.float32), np.zeros(C, np.float32),
+          np.full(C, 1.0 - eps, np.float32)]
+    with OpSession(gpu_server, ws) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        t.s.bn(t.fid, xv, yv, *t.w[:4], eps, 75, C)
+        got = t.read(yv, x.shape)
+    assert_close(got, x, 1e-6, "bn identity")
+
+
+@pytest.mark.parametrize("n", [1, 4, 1023, 50000])
+def test_elementwise(gpu_server, n):
+    rng = np.random.default_rng(n)
+    a, b = _rand(rng, n), _rand(rng, n)
+    with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
+        av, bv = t.act(a), t.act(b)
+        yv = t.empty(n * 4)
+        t.s.launch(t.fid, OP_RELU, [av, yv], [n])
+        np.testing.assert_array_equal(t.read(yv, (n,)), np.maximum(a, 0))
+        t.s.launch(t.fid, OP_ADD, [av, bv, yv], [n, 0])
+        np.testing.assert_array_equal(t.read(yv, (n,)), a + b)
+        t.s.launch(t.fid, OP_ADD, [av, bv, yv], [n, 1])
+        np.testing.assert_array_equal(t.read(yv, (n,)), np.maximum(a + b, 0))
+        t.s.launch(t.fid, OP_GELU, [av, yv], [n])
+        assert_close(t.read(yv, (n,)), ref.gelu(a), 2e-6, "gelu")
+        t.s.launch(t.fid, OP_FILL, [yv], [n], [3.25])
+        np.testing.assert_array_equal(t.read(yv, (n,)), np.full(n, 3.25, np.float32))
+        t.s.launch(t.fid, OP_SUM, [av, yv], [n])
+        assert_close(t.read(yv, (1,)), [a.astype(np.float64).sum()], 1e-4 if n > 1 else 1e-6, "sum")
+
+
+def test_bias_act_and_layouts(gpu_server):
+    rng = np.random.default_rng(3)
+    x, bias = _rand(rng, 33, 50), _rand(rng, 50)
+    img = _rand(rng, 2, 5, 37, 41)
+    with OpSession(gpu_server, [bias]) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        t.s.launch(t.fid, OP_BIAS_ACT, [xv, t.w[0], yv], [33, 50, ACT_RELU])
+        np.testing.assert_array_equal(t.read(yv, x.shape), np.maximum(x + bias, 0))
+        iv = t.act(img)
+        ov = t.empty(img.nbytes)
+        t.s.launch(t.fid, OP_NCHW_TO_NHWC, [iv, ov], [2, 5, 37, 41])
+        nhwc = t.read(ov, (2, 37, 41, 5))
+        np.testing.assert_array_equal(nhwc, img.transpose(0, 2, 3, 1))
+        t.s.launch(t.fid, OP_NHWC_TO_NCHW, [ov, iv], [2, 5, 37, 41])
+        np.testing.assert_array_equal(t.read(iv, img.shape), img)
+
+
+@pytest.mark.parametrize("layout", [NHWC, NCHW])
+def test_pooling(gpu_server, layout):
+    rng = np.random.default_rng(9)
+    N, H, W, C = 2, 15, 14, 24
+    x = _rand(rng, N, H, W, C) if layout == NHWC else _rand(rng, N, C, H, W)
+    with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
+        xv = t.act(x)
+        want = ref.maxpool(x, 3, 2, 1, nhwc=(layout == NHWC))
+        yv = t.empty(want.nbytes)
+        t.s.launch(t.fid, OP_MAXPOOL, [xv, yv], [N, H, W, C, 3, 2, 1, layout])
+        np.testing.assert_array_equal(t.read(yv, want.shape), want)
+        av = t.empty(N * C * 4)
+        t.s.launch(t.fid, OP_AVGPOOL, [xv, av], [N, H * W, C, layout])
+        assert_close(t.read(av, (N, C)), ref.avgpool(x, nhwc=(layout == NHWC)), 2e-6, "avgpool")
+
+
+@pytest.mark.parametrize("rows,width", [(128, 768), (5, 1024), (3, 50), (2, 4096), (1, 1)])
+def test_layernorm(gpu_server, rows, width):
+    rng = np.random.default_rng(width)
+    x, r = _rand(rng, rows, width) * 3 + 1, _rand(rng, rows, width)
+    g, b = _rand(rng, width), _rand(rng, width)
+    with OpSession(gpu_server, [g, b]) as t:
+        xv, rv = t.act(x), t.act(r)
+        yv = t.empty(x.nbytes)
+        t.s.launch(t.fid, OP_LAYERNORM, [xv, rv, t.w[0], t.w[1], yv], [rows, width], [1e-12])
+        got = t.read(yv, x.shape)
+        t.s.launch(t.fid, OP_LAYERNORM, [xv, 0, t.w[0], t.w[1], yv], [rows, width], [1e-5])
+        got2 = t.read(yv, x.shape)
+    if width > 1:
+        assert_close(got, ref.layernorm(x, r, g, b, 1e-12), 2e-5, "layernorm+res")
+    assert_close(got2, ref.layernorm(x, None, g, b, 1e-5), 2e-5, "layernorm")
+
+
+def test_layernorm_moments(gpu_server):
+    """gamma=1, beta=0: every output row has mean 0 and variance 1."""
+    rng = np.random.default_rng(0)
+    x = _rand(rng, 16, 768) * 5 + 2
+    with OpSession(gpu_server, [np.ones(768, np.float32), np.zeros(768, np.float32)]) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        t.s.launch(t.fid, OP_LAYERNORM, [xv, 0, t.w[0], t.w[1], yv], [16, 768], [1e-12])
+        y = t.read(yv, x.shape).astype(np.float64)
+    assert np.abs(y.mean(1)).max() < 1e-5 and np.abs(y.var(1) - 1).max() < 1e-4
+
+
+@pytest.mark.parametrize("rows,width,rpm", [(12 * 128, 128, 0), (2 * 4 * 96, 96, 4 * 96), (7, 384, 0), (3, 513, 0)])
+def test_softmax(gpu_server, rows, width, rpm):
+    rng = np.random.default_rng(width)
+    x = _rand(rng, rows, width) * 4
+    mask = None
+    if rpm:
+        mask = np.where(rng.random((rows // rpm, width)) < 0.2, np.float32(-1e30), np.float32(0)).astype(np.float32)
+        mask[:, 0] = 0
+    with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
+        xv = t.act(x)
+        mv = t.act(mask) if mask is not None else 0
+        yv = t.empty(x.nbytes)
+        t.s.launch(t.fid, OP_SOFTMAX, [xv, mv, yv], [rows, width, rpm], [0.125])
+        got = t.read(yv, x.shape)
+    want = ref.softmax(x, mask, 0.125, rpm if rpm else 1)
+    assert_close(got, want, 2e-6, "softmax")
+    assert np.abs(got.astype(np.float64).sum(1) - 1).max() < 1e-5
+    if mask is not None:
+        assert (got[np.repeat(mask, rpm, axis=0) < -1] == 0).all()
+
+
+def test_embedding(gpu_server):
+    rng = np.random.default_rng(2)
+    V, P, T, H, B, S = 100, 40, 2, 96, 3, 17
+    word, pos, typ = _rand(rng, V, H), _rand(rng, P, H), _rand(rng, T, H)
+    ids = rng.integers(0, V, (B, S)).astype(np.int64)
+    tids = rng.integers(0, T, (B, S)).astype(np.int64)
+    with OpSession(gpu_server, [word, pos, typ]) as t:
+        iv, tv = t.act(ids), t.act(tids)
+        yv = t.empty(B * S * H * 4)
+        t.s.launch(t.fid, OP_EMBEDDING, [iv, tv, t.w[0], t.w[1], t.w[2], yv], [B * S, S, H, V, T])
+        got = t.read(yv, (B * S, H))
+        t.s.launch(t.fid, OP_EMBEDDING, [iv, 0, t.w[0], t.w[1], t.w[2], yv], [B * S, S, H, V, T])
+        got0 = t.read(yv, (B * S, H))
+    assert_close(got, ref.embedding(ids, tids, word, pos, typ, S), 1e-6, "embedding")
+    assert_close(got0, ref.embedding(ids, None, word, pos, typ, S), 1e-6, "embedding type 0")

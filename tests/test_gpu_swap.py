@@ -1,0 +1,75 @@
+"""Swap engine, pool and LRU on the device: eviction under a binding budget, repeated
+swap-in / swap-out, prefetch (Load), gate ordering with a poisoned pool."""
+import numpy as np
+import pytest
+
+from torpor_amd.functions import resnet
+from torpor_amd.server import ACK_INAVAIL, ACK_OK, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD, Server
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(server, fid, seed, image=64):
+    fn = resnet.ResNet(server, fid, "resnet50", batch=1, seed=seed, image=image)
+    x = np.random.default_rng(seed).standard_normal((1, 3, image, image)).astype(np.float32)
+    (y,) = fn.register([x])
+    return fn, x, y
+
+
+def test_lru_eviction_and_identity():
+    """Budget fits two ResNet-50s: registering / invoking a third evicts the least recently
+    used one; every model still answers with its own bits after being swapped back in."""
+    with Server(mem_limit_bytes=300 << 20, pool_bytes=512 << 20, chunk_bytes=1 << 20) as s:
+        fns = [_mk(s, i, seed=i) for i in range(3)]
+        info = s.model_info(0)
+        assert 2 * info["total_bytes"] < (300 << 20) <= 3 * info["total_bytes"]
+        assert [s.resident(i) for i in range(3)] == [False, True, True]
+        order = [0, 1, 2, 2, 0, 1, 0, 2, 1, 1, 0]
+        for i in order:
+            fn, x, y = fns[i]
+            (got,) = fn.invoke([x])
+            assert np.array_equal(got, y), f"model {i} changed its answer after swapping"
+            assert s.resident(i)
+            assert sum(s.resident(j) for j in range(3)) <= 2
+            st = s.pool_stats()
+            assert st["lru_used"] < st["lru_budget"] and st["used"] <= st["capacity"]
+        st = s.pool_stats()
+        assert st["evictions"] >= 5 and st["swap_ins"] >= 5
+        for i in range(3):
+            if s.resident(i):
+                assert np.array_equal(s.readback_weights(i), s.host_weights(i))
+
+
+def test_prefetch_then_invoke(gpu_server):
+    fn, x, y = _mk(gpu_server, 20, seed=7)
+    assert fn.unload()[0] == ACK_OK and not gpu_server.resident(20)
+    ack, resp, _ = fn.load()
+    assert ack == ACK_OK and gpu_server.resident(20)
+    assert np.array_equal(gpu_server.readback_weights(20), gpu_server.host_weights(20))
+    (got,) = fn.invoke([x])
+    assert np.array_equal(got, y)
+    fn.unload()
+
+
+def test_unknown_and_active_function(gpu_server):
+    ack, _, _ = gpu_server.signal(REQ_EXECUTE, 3999, "")
+    assert ack == ACK_INAVAIL
+    ack, resp, _ = gpu_server.signal(REQ_UNLOAD, 3999, "")
+    assert ack == ACK_OK and resp == -1
+    assert gpu_server.signal(REQ_LOAD, 3999, "")[0] == ACK_INAVAIL
+
+
+def test_gate_orders_compute_after_copy():
+    """Tiny gate groups (BUFFER_SIZE=1-style ablation): every op waits for exactly its own
+    tensor.  The pool is poisoned between swap-out and swap-in by another model's weights, so
+    an op that ran ahead of its copy would read foreign bytes and change the logits."""
+    with Server(mem_limit_bytes=200 << 20, pool_bytes=384 << 20, chunk_bytes=256, chunk_max_bytes=64 << 10) as s:
+        a, xa, ya = _mk(s, 0, seed=11)
+        b, xb, yb = _mk(s, 1, seed=12)   # evicts model 0 (budget holds one)
+        assert not s.resident(0) and s.resident(1)
+        for _ in range(3):
+            (ga,) = a.invoke([xa])
+            assert np.array_equal(ga, ya)
+            assert s.swap_stats(0)["gate_waits"] > 50
+            (gb,) = b.invoke([xb])
+            assert np.array_equal(gb, yb)

@@ -1,0 +1,153 @@
+"""ctypes binding of libtorpor_amd.so (declared in include/torpor_amd.h).
+
+The library is the product: if it is missing or fails to load this module raises,
+there is no other execution path.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtorpor_amd.so")
+
+
+class TorporError(RuntimeError):
+    def __init__(self, code, what=""):
+        self.code = code
+        msg = lib().tp_strerror(code).decode() if _lib is not None else "error"
+        super().__init__(f"{what}: {msg} ({code})" if what else f"{msg} ({code})")
+
+
+class Config(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("device", C.c_int32),
+        ("mem_limit_bytes", C.c_uint64),
+        ("pool_bytes", C.c_uint64),
+        ("chunk_bytes", C.c_uint64),
+        ("chunk_max_bytes", C.c_uint64),
+        ("workspace_bytes", C.c_uint64),
+        ("flags", C.c_int32),
+        ("request_timeout_ms", C.c_int32),
+    ]
+
+
+class Epilogue(C.Structure):
+    _fields_ = [
+        ("alpha", C.c_float),
+        ("beta", C.c_float),
+        ("bias", C.c_uint64),
+        ("bn_scale", C.c_uint64),
+        ("bn_bias", C.c_uint64),
+        ("bn_mean", C.c_uint64),
+        ("bn_var", C.c_uint64),
+        ("bn_eps", C.c_float),
+        ("act", C.c_int32),
+        ("residual", C.c_uint64),
+        ("ldr", C.c_int64),
+    ]
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [
+        ("x", C.c_uint64), ("y", C.c_uint64), ("c", C.c_uint64),
+        ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64),
+        ("xs_r", C.c_int64), ("xs_k", C.c_int64), ("ys_c", C.c_int64), ("ys_k", C.c_int64), ("ldc", C.c_int64),
+        ("nb0", C.c_int32), ("nb1", C.c_int32),
+        ("xb0", C.c_int64), ("xb1", C.c_int64), ("yb0", C.c_int64), ("yb1", C.c_int64),
+        ("cb0", C.c_int64), ("cb1", C.c_int64),
+        ("ep", Epilogue),
+    ]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [
+        ("x", C.c_uint64), ("w", C.c_uint64), ("y", C.c_uint64),
+        ("n", C.c_int32), ("h", C.c_int32), ("w_in", C.c_int32), ("cin", C.c_int32), ("cout", C.c_int32),
+        ("kh", C.c_int32), ("kw", C.c_int32),
+        ("stride_h", C.c_int32), ("stride_w", C.c_int32), ("pad_h", C.c_int32), ("pad_w", C.c_int32),
+        ("groups", C.c_int32),
+        ("x_layout", C.c_int32), ("y_layout", C.c_int32),
+        ("ep", Epilogue),
+    ]
+
+
+class PoolStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "capacity", "used", "largest_free", "live_extents", "free_extents",
+        "lru_budget", "lru_used", "lru_models", "evictions", "swap_ins")]
+
+
+class ModelInfo(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("registered", "resident", "level", "n_params", "n_chunks", "n_ops")] + \
+               [(n, C.c_uint64) for n in ("image_bytes", "param_bytes", "act_bytes", "total_bytes",
+                                          "weight_off", "act_off")]
+
+
+class SwapStats(C.Structure):
+    _fields_ = [("bytes", C.c_uint64), ("copy_ms", C.c_double), ("alloc_us", C.c_double),
+                ("evict_us", C.c_double), ("chunks", C.c_uint32), ("gate_waits", C.c_uint32)]
+
+
+# every symbol include/torpor_amd.h declares: name -> (restype, argtypes)
+_P = C.c_void_p
+_U64 = C.c_uint64
+_I32 = C.c_int32
+_I64 = C.c_int64
+SYMBOLS = {
+    "tp_server_create": (C.c_int, [C.POINTER(Config), C.POINTER(_P)]),
+    "tp_server_destroy": (None, [_P]),
+    "tp_strerror": (C.c_char_p, [C.c_int]),
+    "tp_version": (C.c_char_p, []),
+    "tp_signal": (C.c_int, [_P, _I32, C.c_char_p, C.c_char_p, C.POINTER(_I32), C.POINTER(_I32), C.POINTER(_I32)]),
+    "tp_take_deferred_ack": (C.c_int, [_P, C.POINTER(_I32), C.POINTER(_I32)]),
+    "tp_poll": (C.c_int, [_P]),
+    "tp_malloc": (C.c_int, [_P, _I32, _U64, C.POINTER(_U64)]),
+    "tp_free": (C.c_int, [_P, _I32, _U64]),
+    "tp_memcpy_h2d": (C.c_int, [_P, _I32, _U64, _P, _U64]),
+    "tp_memcpy_d2h_async": (C.c_int, [_P, _I32, _P, _U64, _U64]),
+    "tp_memcpy_d2h": (C.c_int, [_P, _I32, _P, _U64, _U64]),
+    "tp_memcpy_d2d": (C.c_int, [_P, _I32, _U64, _U64, _U64]),
+    "tp_memset_async": (C.c_int, [_P, _I32, _U64, _I32, _U64]),
+    "tp_device_synchronize": (C.c_int, [_P, _I32]),
+    "tp_stream_synchronize": (C.c_int, [_P, _I32]),
+    "tp_sgemm": (C.c_int, [_P, _I32, _I32, _I32, _I32, _I32, _I32, C.c_float, _U64, _I32, _U64, _I32,
+                           C.c_float, _U64, _I32]),
+    "tp_sgemm_strided_batched": (C.c_int, [_P, _I32, _I32, _I32, _I32, _I32, _I32, C.c_float, _U64, _I32, _I64,
+                                           _U64, _I32, _I64, C.c_float, _U64, _I32, _I64, _I32]),
+    "tp_gemm": (C.c_int, [_P, _I32, C.POINTER(GemmDesc)]),
+    "tp_conv_forward": (C.c_int, [_P, _I32, C.POINTER(ConvDesc)]),
+    "tp_bn_inference": (C.c_int, [_P, _I32, _U64, _U64, _U64, _U64, _U64, _U64, C.c_double, _I64, _I32, _I64,
+                                  _I32, _I32]),
+    "tp_launch": (C.c_int, [_P, _I32, _I32, C.POINTER(_U64), _I32, C.POINTER(_I64), _I32,
+                            C.POINTER(C.c_float), _I32]),
+    "tp_replay": (C.c_int, [_P, _I32, _P, _U64, _P, _U64]),
+    "tp_model_resident": (C.c_int, [_P, _I32]),
+    "tp_get_model_info": (C.c_int, [_P, _I32, C.POINTER(ModelInfo)]),
+    "tp_get_pool_stats": (C.c_int, [_P, C.POINTER(PoolStats)]),
+    "tp_get_swap_stats": (C.c_int, [_P, _I32, C.POINTER(SwapStats)]),
+    "tp_readback_weights": (C.c_int, [_P, _I32, _P, _U64]),
+    "tp_host_weights": (C.c_int, [_P, _I32, C.POINTER(_P), C.POINTER(_U64)]),
+    "tp_weight_offset": (C.c_int, [_P, _I32, _U64, C.POINTER(_U64)]),
+    "tp_last_kernel": (C.c_char_p, []),
+    "tp_measure_h2d": (C.c_int, [_P, _U64, _I32, C.POINTER(C.c_double)]),
+    "tp_time_op": (C.c_int, [_P, _I32, _I32, _I32, C.POINTER(C.c_double)]),
+}
+
+_lib = None
+
+
+def lib():
+    """Load the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `make -C torpor_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback path")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(l, name)  # AttributeError if the library does not export it
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib

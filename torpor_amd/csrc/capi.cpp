@@ -1,0 +1,376 @@
+// extern "C" surface of the engine (include/torpor_amd.h).  Nothing here throws across the
+// boundary: allocation failures and engine errors come back as integer codes.
+#include <cstring>
+#include <new>
+
+#include "engine.hpp"
+#include "kernels/kernels.hpp"
+
+struct tp_server {
+    tp::Engine* engine;
+};
+
+#define TP_GUARD_BEGIN try {
+#define TP_GUARD_END                 \
+    }                                \
+    catch (const std::bad_alloc&) {  \
+        return TP_ENOMEM;            \
+    }                                \
+    catch (...) {                    \
+        return TP_EINVAL;            \
+    }
+
+extern "C" {
+
+const char* tp_version(void) { return "torpor_amd 0.1 (gfx950)"; }
+
+const char* tp_strerror(int code) {
+    switch (code) {
+        case TP_OK: return "ok";
+        case TP_EINVAL: return "invalid argument or shape";
+        case TP_ENOMEM: return "out of pool or host memory";
+        case TP_ENOENT: return "unknown function or address";
+        case TP_EBUSY: return "executor busy";
+        case TP_ENODEV: return "host-only engine: no device";
+        case TP_ESTATE: return "call not valid in the current executor mode";
+        case TP_ENOTACTIVE: return "client is not the active function";
+        case TP_EUNSUPPORTED: return "not supported";
+        case TP_EFAULT: return "virtual address does not translate";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error";
+}
+
+int tp_server_create(const tp_config* cfg, tp_server** out) {
+    TP_GUARD_BEGIN
+    if (!out) return TP_EINVAL;
+    *out = nullptr;
+    tp_config c;
+    std::memset(&c, 0, sizeof(c));
+    if (cfg) {
+        size_t n = cfg->struct_size ? cfg->struct_size : sizeof(tp_config);
+        if (n > sizeof(tp_config)) n = sizeof(tp_config);
+        std::memcpy(&c, cfg, n);
+    }
+    auto* e = new tp::Engine(c);
+    int r = e->init();
+    if (r) {
+        delete e;
+        return r;
+    }
+    *out = new tp_server{e};
+    return 0;
+    TP_GUARD_END
+}
+
+void tp_server_destroy(tp_server* s) {
+    if (!s) return;
+    try {
+        delete s->engine;
+    } catch (...) {
+    }
+    delete s;
+}
+
+#define ENG(s)                  \
+    if (!(s) || !(s)->engine) return TP_EINVAL; \
+    tp::Engine& E = *(s)->engine
+
+int tp_signal(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack, int32_t* resp,
+              int32_t* deferred) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.signal(type, function, payload, ack, resp, deferred);
+    TP_GUARD_END
+}
+int tp_take_deferred_ack(tp_server* s, int32_t* ack, int32_t* resp) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.take_deferred_ack(ack, resp);
+    TP_GUARD_END
+}
+int tp_poll(tp_server* s) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.poll();
+    TP_GUARD_END
+}
+
+int tp_malloc(tp_server* s, int32_t client, uint64_t bytes, uint64_t* vaddr) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_malloc(client, bytes, vaddr);
+    TP_GUARD_END
+}
+int tp_free(tp_server* s, int32_t client, uint64_t vaddr) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_free(client, vaddr);
+    TP_GUARD_END
+}
+int tp_memcpy_h2d(tp_server* s, int32_t client, uint64_t dst, const void* src, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_h2d(client, dst, src, bytes);
+    TP_GUARD_END
+}
+int tp_memcpy_d2h_async(tp_server* s, int32_t client, void* dst, uint64_t src, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_d2h_async(client, dst, src, bytes);
+    TP_GUARD_END
+}
+int tp_memcpy_d2h(tp_server* s, int32_t client, void* dst, uint64_t src, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_d2h(client, dst, src, bytes);
+    TP_GUARD_END
+}
+int tp_memcpy_d2d(tp_server* s, int32_t client, uint64_t dst, uint64_t src, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_d2d(client, dst, src, bytes);
+    TP_GUARD_END
+}
+int tp_memset_async(tp_server* s, int32_t client, uint64_t dst, int32_t value, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_memset(client, dst, value, bytes);
+    TP_GUARD_END
+}
+int tp_device_synchronize(tp_server* s, int32_t client) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_device_sync(client);
+    TP_GUARD_END
+}
+int tp_stream_synchronize(tp_server* s, int32_t client) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.op_stream_sync(client);
+    TP_GUARD_END
+}
+
+static void fill_epilogue(tp::Op& op, const tp_epilogue& e, int pbase, int ibase) {
+    op.p[pbase + 0] = e.bias;
+    op.p[pbase + 1] = e.bn_scale;
+    op.p[pbase + 2] = e.bn_bias;
+    op.p[pbase + 3] = e.bn_mean;
+    op.p[pbase + 4] = e.bn_var;
+    op.p[pbase + 5] = e.residual;
+    op.f[0] = e.alpha;
+    op.f[1] = e.beta;
+    op.f[2] = e.bn_eps;
+    op.nf = 3;
+    op.i[ibase + 0] = e.ldr;
+    op.i[ibase + 1] = e.act;
+}
+
+int tp_gemm(tp_server* s, int32_t client, const tp_gemm_desc* d) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    if (!d) return TP_EINVAL;
+    tp::Op op;
+    op.kind = tp::OPK_GEMM;
+    op.p[0] = d->x;
+    op.p[1] = d->y;
+    op.p[2] = d->c;
+    const int64_t iv[16] = {d->m,   d->n,   d->k,   d->xs_r, d->xs_k, d->ys_c, d->ys_k, d->ldc,
+                            d->nb0, d->nb1, d->xb0, d->xb1,  d->yb0,  d->yb1,  d->cb0,  d->cb1};
+    for (int k = 0; k < 16; ++k) op.i[k] = iv[k];
+    fill_epilogue(op, d->ep, 3, 16);
+    op.np = 9;
+    op.ni = 18;
+    return E.op_compute(client, op);
+    TP_GUARD_END
+}
+
+// Column-major C(m x n) = alpha*op(A)*op(B) + beta*C is the row-major product
+// C'[j][i] = sum_k X(j,k) * Y(i,k) with X(j,k) = op(B)(k,j) and Y(i,k) = op(A)(i,k).
+static int sgemm_common(tp_server* s, int32_t client, int transa, int transb, int m, int n, int k, float alpha,
+                        uint64_t a, int lda, int64_t stride_a, uint64_t b, int ldb, int64_t stride_b, float beta,
+                        uint64_t c, int ldc, int64_t stride_c, int count) {
+    ENG(s);
+    if (m < 0 || n < 0 || k < 0 || count < 1) return TP_EINVAL;
+    if (m == 0 || n == 0) return 0;
+    tp_gemm_desc d;
+    std::memset(&d, 0, sizeof(d));
+    d.x = b;
+    d.y = a;
+    d.c = c;
+    d.m = n;
+    d.n = m;
+    d.k = k;
+    if (transb == 0) {  // B is k x n, element (k,j) at k + j*ldb
+        d.xs_r = ldb;
+        d.xs_k = 1;
+    } else {  // B is n x k, element (j,k) at j + k*ldb
+        d.xs_r = 1;
+        d.xs_k = ldb;
+    }
+    if (transa == 0) {  // A is m x k, element (i,k) at i + k*lda
+        d.ys_c = 1;
+        d.ys_k = lda;
+    } else {  // A is k x m, element (k,i) at k + i*lda
+        d.ys_c = lda;
+        d.ys_k = 1;
+    }
+    d.ldc = ldc;
+    d.nb0 = 1;
+    d.nb1 = count;
+    d.xb1 = stride_b;
+    d.yb1 = stride_a;
+    d.cb1 = stride_c;
+    d.ep.alpha = alpha;
+    d.ep.beta = beta;
+    d.ep.bn_eps = 0.f;
+    return tp_gemm(s, client, &d);
+}
+
+int tp_sgemm(tp_server* s, int32_t client, int32_t transa, int32_t transb, int32_t m, int32_t n, int32_t k,
+             float alpha, uint64_t a, int32_t lda, uint64_t b, int32_t ldb, float beta, uint64_t c, int32_t ldc) {
+    TP_GUARD_BEGIN
+    return sgemm_common(s, client, transa, transb, m, n, k, alpha, a, lda, 0, b, ldb, 0, beta, c, ldc, 0, 1);
+    TP_GUARD_END
+}
+int tp_sgemm_strided_batched(tp_server* s, int32_t client, int32_t transa, int32_t transb, int32_t m, int32_t n,
+                             int32_t k, float alpha, uint64_t a, int32_t lda, int64_t stride_a, uint64_t b,
+                             int32_t ldb, int64_t stride_b, float beta, uint64_t c, int32_t ldc, int64_t stride_c,
+                             int32_t count) {
+    TP_GUARD_BEGIN
+    return sgemm_common(s, client, transa, transb, m, n, k, alpha, a, lda, stride_a, b, ldb, stride_b, beta, c, ldc,
+                        stride_c, count);
+    TP_GUARD_END
+}
+
+int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    if (!d) return TP_EINVAL;
+    if (d->groups != 0 && d->groups != 1) return TP_EUNSUPPORTED;
+    tp::Op op;
+    op.kind = tp::OPK_CONV;
+    op.p[0] = d->x;
+    op.p[1] = d->w;
+    op.p[2] = d->y;
+    const int64_t iv[13] = {d->n,        d->h,     d->w_in,  d->cin,      d->cout,    d->kh, d->kw, d->stride_h,
+                            d->stride_w, d->pad_h, d->pad_w, d->x_layout, d->y_layout};
+    for (int k = 0; k < 13; ++k) op.i[k] = iv[k];
+    fill_epilogue(op, d->ep, 3, 13);
+    op.np = 9;
+    op.ni = 15;
+    return E.op_compute(client, op);
+    TP_GUARD_END
+}
+
+int tp_bn_inference(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
+                    uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
+                    int32_t layout, int32_t relu) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    tp::Op op;
+    op.kind = tp::OPK_BN;
+    op.p[0] = x;
+    op.p[1] = y;
+    op.p[2] = scale;
+    op.p[3] = bias;
+    op.p[4] = mean;
+    op.p[5] = var;
+    op.np = 6;
+    op.i[0] = rows;
+    op.i[1] = channels;
+    op.i[2] = hw;
+    op.i[3] = layout;
+    op.i[4] = relu;
+    op.ni = 5;
+    op.f[0] = (float)eps;
+    op.nf = 1;
+    return E.op_compute(client, op);
+    TP_GUARD_END
+}
+
+int tp_launch(tp_server* s, int32_t client, int32_t op_id, const uint64_t* ptrs, int32_t n_ptrs,
+              const int64_t* ints, int32_t n_ints, const float* floats, int32_t n_floats) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    if (n_ptrs < 0 || n_ptrs > 12 || n_ints < 0 || n_ints > 20 || n_floats < 0 || n_floats > 4) return TP_EINVAL;
+    if ((n_ptrs && !ptrs) || (n_ints && !ints) || (n_floats && !floats)) return TP_EINVAL;
+    tp::Op op;
+    op.kind = tp::OPK_LAUNCH;
+    op.op_id = op_id;
+    op.np = n_ptrs;
+    op.ni = n_ints;
+    op.nf = n_floats;
+    for (int k = 0; k < n_ptrs; ++k) op.p[k] = ptrs[k];
+    for (int k = 0; k < n_ints; ++k) op.i[k] = ints[k];
+    for (int k = 0; k < n_floats; ++k) op.f[k] = floats[k];
+    return E.op_compute(client, op);
+    TP_GUARD_END
+}
+
+int tp_replay(tp_server* s, int32_t client, const void* input, uint64_t input_bytes, void* output,
+              uint64_t output_bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.replay(client, input, input_bytes, output, output_bytes);
+    TP_GUARD_END
+}
+
+int tp_model_resident(tp_server* s, int32_t client) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.model_resident(client);
+    TP_GUARD_END
+}
+int tp_get_model_info(tp_server* s, int32_t client, tp_model_info* out) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.model_info(client, out);
+    TP_GUARD_END
+}
+int tp_get_pool_stats(tp_server* s, tp_pool_stats* out) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.pool_stats(out);
+    TP_GUARD_END
+}
+int tp_get_swap_stats(tp_server* s, int32_t client, tp_swap_stats* out) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.swap_stats(client, out);
+    TP_GUARD_END
+}
+int tp_readback_weights(tp_server* s, int32_t client, void* dst, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.readback_weights(client, dst, bytes);
+    TP_GUARD_END
+}
+int tp_host_weights(tp_server* s, int32_t client, const void** ptr, uint64_t* bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.host_weights(client, ptr, bytes);
+    TP_GUARD_END
+}
+int tp_weight_offset(tp_server* s, int32_t client, uint64_t vaddr, uint64_t* image_off) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.weight_offset(client, vaddr, image_off);
+    TP_GUARD_END
+}
+const char* tp_last_kernel(void) { return tpk::last_kernel_name(); }
+int tp_measure_h2d(tp_server* s, uint64_t bytes, int32_t iters, double* gbps) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.measure_h2d(bytes, iters, gbps);
+    TP_GUARD_END
+}
+int tp_time_op(tp_server* s, int32_t client, int32_t op_index, int32_t iters, double* mean_us) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.time_op(client, op_index, iters, mean_us);
+    TP_GUARD_END
+}
+
+}  // extern "C"

@@ -1,0 +1,1402 @@
+#include "engine.hpp"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "kernels/kernels.hpp"
+
+namespace tp {
+
+using Clock = std::chrono::steady_clock;
+static inline double us_since(Clock::time_point t0) {
+    return std::chrono::duration<double, std::micro>(Clock::now() - t0).count();
+}
+static inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+#define HIPCHK(expr)                         \
+    do {                                     \
+        hipError_t _e = (expr);              \
+        if (_e != hipSuccess) return (int)_e; \
+    } while (0)
+
+static uint64_t env_u64(const char* name, uint64_t dflt) {
+    const char* v = std::getenv(name);
+    if (!v || !*v) return dflt;
+    char* end = nullptr;
+    unsigned long long x = std::strtoull(v, &end, 10);
+    if (end == v) return dflt;
+    return (uint64_t)x;
+}
+
+Engine::Engine(const tp_config& cfg) : cfg_(cfg) {}
+
+int Engine::init() {
+    // controller.hpp:83-93: MEM_LIMIT_IN_GB; the reference caps it below 25 GB for 32 GB parts,
+    // here any positive value up to the device size is accepted.
+    if (cfg_.mem_limit_bytes == 0) cfg_.mem_limit_bytes = env_u64("MEM_LIMIT_IN_GB", 24) << 30;
+    if (cfg_.chunk_bytes == 0) cfg_.chunk_bytes = env_u64("BUFFER_SIZE", 2ull << 20);  // memory_manager.hpp:22
+    if (cfg_.chunk_bytes < kTensorAlign) cfg_.chunk_bytes = kTensorAlign;              // BUFFER_SIZE=1 ablation
+    if (cfg_.chunk_max_bytes == 0) cfg_.chunk_max_bytes = 8ull << 20;
+    if (cfg_.chunk_max_bytes < cfg_.chunk_bytes) cfg_.chunk_max_bytes = cfg_.chunk_bytes;
+    if (cfg_.workspace_bytes == 0) cfg_.workspace_bytes = 64ull << 20;
+    if (cfg_.request_timeout_ms <= 0) cfg_.request_timeout_ms = 5000;  // cuda_server.hpp:29
+    // memory_manager.hpp:42-44 adds 5 GiB of slack above the eviction budget; 1 GiB is enough
+    // here because allocations are whole-model extents, not per-tensor blocks.
+    if (cfg_.pool_bytes == 0) cfg_.pool_bytes = cfg_.mem_limit_bytes + (1ull << 30);
+    lru_.set_budget(cfg_.mem_limit_bytes);
+    pool_.reset(cfg_.pool_bytes);
+
+    if (host_only()) {
+        arena_ = reinterpret_cast<uint8_t*>(0x100000000000ull);
+        return 0;
+    }
+    HIPCHK(hipSetDevice(cfg_.device));
+    tpk::kernels_init(cfg_.device);
+    HIPCHK(hipMalloc(reinterpret_cast<void**>(&arena_), pool_.capacity()));
+    HIPCHK(hipMalloc(reinterpret_cast<void**>(&workspace_), cfg_.workspace_bytes));
+    HIPCHK(hipStreamCreateWithFlags(&compute_, hipStreamNonBlocking));
+    HIPCHK(hipStreamCreateWithFlags(&copy_, hipStreamNonBlocking));
+    HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&h2d_stage_), 16ull << 20, hipHostMallocDefault));
+    h2d_cap_ = 16ull << 20;
+    HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&d2h_stage_), 8ull << 20, hipHostMallocDefault));
+    d2h_cap_ = 8ull << 20;
+    copy_thread_ = std::thread(&Engine::copy_main, this);
+    return 0;
+}
+
+Engine::~Engine() {
+    {
+        std::lock_guard<std::mutex> lk(cmu_);
+        stop_ = true;
+    }
+    ccv_.notify_all();
+    if (copy_thread_.joinable()) copy_thread_.join();
+    if (!host_only()) {
+        (void)hipSetDevice(cfg_.device);
+        (void)hipDeviceSynchronize();
+    }
+    for (auto& kv : models_) {
+        Model& m = *kv.second;
+        host_free(m.host_image);
+        if (!host_only()) {
+            for (auto ev : m.chunk_ev) (void)hipEventDestroy(ev);
+            if (m.t0) (void)hipEventDestroy(m.t0);
+            if (m.t1) (void)hipEventDestroy(m.t1);
+        }
+    }
+    if (!host_only()) {
+        if (h2d_stage_) (void)hipHostFree(h2d_stage_);
+        if (d2h_stage_) (void)hipHostFree(d2h_stage_);
+        if (workspace_) (void)hipFree(workspace_);
+        if (arena_) (void)hipFree(arena_);
+        if (compute_) (void)hipStreamDestroy(compute_);
+        if (copy_) (void)hipStreamDestroy(copy_);
+    }
+}
+
+void* Engine::host_alloc(uint64_t bytes) {
+    if (bytes == 0) bytes = 1;
+    if (host_only()) return std::malloc(bytes);
+    void* p = nullptr;
+    // The host weight store is pinned once, at registration, so a swap-in is a straight DMA.
+    // The reference keeps it pageable (model_repo.hpp:173-177) and stages through pinned
+    // buffers on every swap-in (memory_manager.hpp:311-329,354-370).
+    if (hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess) return nullptr;
+    return p;
+}
+void Engine::host_free(void* p) {
+    if (!p) return;
+    if (host_only())
+        std::free(p);
+    else
+        (void)hipHostFree(p);
+}
+
+Model* Engine::find(int id) {
+    auto it = models_.find(id);
+    return it == models_.end() ? nullptr : it->second.get();
+}
+
+Model* Engine::active_model(int client, int* err) {
+    if (active_ < 0 || mode_ == MODE_NONE) {
+        *err = TP_ESTATE;
+        return nullptr;
+    }
+    if (client != active_) {
+        *err = TP_ENOTACTIVE;
+        return nullptr;
+    }
+    Model* m = find(active_);
+    if (!m) *err = TP_ENOENT;
+    return m;
+}
+
+// ------------------------------------------------------------------ address translation
+// memory_manager.hpp:261-271 (get_cuda_addr), 527-568 (check_param_readiness, get_phy_address):
+// the reference walks several hash maps per pointer; here a weight address is one binary
+// search in the tensor table plus an add, an activation address one map lookup plus an add.
+int Engine::translate(Model& m, uint64_t va, uint64_t span, Xlat* out) {
+    if ((va & kVaTagMask) != kVaTag) return TP_EFAULT;
+    if ((int)((va >> kVaClientShift) & kVaClientMask) != m.id) return TP_EFAULT;
+    const uint64_t off = va & kVaOffMask;
+    if (va & kVaActBit) {
+        auto it = m.ablocks.upper_bound(off);
+        if (it == m.ablocks.begin()) return TP_EFAULT;
+        --it;
+        ABlock& b = it->second;
+        if (!b.live || off >= b.voff + b.size || off + span > b.voff + b.size) return TP_EFAULT;
+        if (m.act_frozen) {
+            if (!m.resident) return TP_EFAULT;
+            out->p = m.a_dev + off;
+        } else {
+            if (b.pool_off == UINT64_MAX) return TP_EFAULT;
+            out->p = arena_ + b.pool_off + (off - b.voff);
+        }
+        out->weight = false;
+        out->param = nullptr;
+        return 0;
+    }
+    // weight region
+    auto it = std::upper_bound(m.params.begin(), m.params.end(), off,
+                               [](uint64_t o, const Param& p) { return o < p.voff; });
+    if (it == m.params.begin()) return TP_EFAULT;
+    --it;
+    if (off >= it->voff + it->size || off + span > it->voff + it->size) return TP_EFAULT;
+    if (m.state == MS_LOADING || !m.resident) return TP_EFAULT;
+    out->p = m.w_dev + it->image_off + (off - it->voff);
+    out->weight = true;
+    out->image_end = it->image_off + it->size;
+    out->param = &*it;
+    return 0;
+}
+
+// memory_manager.hpp:527-533: the reference blocks the executor thread on a host queue until
+// the tensor's transfer group has been host-synchronised.  Here the executor only makes the
+// compute stream wait for the group's event; the host never waits for data.
+int Engine::gate(Model& m, const Xlat& x) {
+    if (!x.weight || m.fully_loaded || host_only()) return 0;
+    if (m.copy_state.load(std::memory_order_acquire) == CS_IDLE) return 0;  // resident from registration
+    auto it = std::lower_bound(m.chunk_end.begin(), m.chunk_end.end(), x.image_end);
+    if (it == m.chunk_end.end()) return TP_EFAULT;
+    const uint32_t idx = (uint32_t)(it - m.chunk_end.begin());
+    if (idx < m.gated_upto) return 0;
+    // the event must have been recorded by the copy thread before the stream may wait on it
+    while (m.issued.load(std::memory_order_acquire) <= idx) {
+        if (m.copy_error.load()) return m.copy_error.load();
+        if (m.copy_state.load(std::memory_order_acquire) != CS_RUNNING && m.issued.load() <= idx) return TP_ESTATE;
+#if defined(__x86_64__)
+        __builtin_ia32_pause();
+#endif
+    }
+    HIPCHK(hipStreamWaitEvent(compute_, m.chunk_ev[idx], 0));
+    m.gated_upto = idx + 1;
+    m.stats.gate_waits++;
+    return 0;
+}
+
+int Engine::resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out) {
+    *out = nullptr;
+    if (va == 0) return optional ? 0 : TP_EFAULT;
+    Xlat x;
+    int r = translate(m, va, span, &x);
+    if (r) return r;
+    if (x.weight) {
+        // memory_manager.hpp:273-284 / model_repo.hpp:102-109: first-access order, tracked run only
+        if (mode_ == MODE_TRACK && x.param->access_rank < 0) x.param->access_rank = m.next_rank++;
+        r = gate(m, x);
+        if (r) return r;
+    }
+    *out = x.p;
+    return 0;
+}
+
+// ------------------------------------------------------------------ memory ops
+int Engine::op_malloc(int client, uint64_t bytes, uint64_t* va) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!va) return TP_EINVAL;
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if (bytes == 0) bytes = 1;
+    const uint64_t base = kVaTag | ((uint64_t)m->id << kVaClientShift);
+    if (mode_ == MODE_LOAD) {  // weight block: cuda_server.hpp:969-970 with load flag set
+        const uint64_t off = m->wbump;
+        if (off + bytes > kVaOffMask) return TP_ENOMEM;
+        m->wbump = align_up(off + bytes, kTensorAlign);
+        m->wblocks.push_back({off, bytes});
+        try {
+            m->staging.resize(m->wbump);
+        } catch (...) {
+            return TP_ENOMEM;
+        }
+        *va = base | off;
+        return 0;
+    }
+    // activation block
+    auto fr = m->afree.find(bytes);
+    if (fr != m->afree.end()) {
+        ABlock& b = m->ablocks[fr->second];
+        m->afree.erase(fr);
+        b.live = true;
+        *va = base | kVaActBit | b.voff;
+        return 0;
+    }
+    if (m->act_frozen) return TP_ENOMEM;  // arena is sized by the first (tracked) inference
+    ABlock b;
+    b.voff = m->abump;
+    b.size = bytes;
+    b.live = true;
+    b.pool_off = pool_.alloc(bytes);
+    if (b.pool_off == UINT64_MAX) return TP_ENOMEM;
+    m->abump = align_up(m->abump + bytes, kTensorAlign);
+    m->ablocks[b.voff] = b;
+    *va = base | kVaActBit | b.voff;
+    return 0;
+}
+
+int Engine::op_free(int client, uint64_t va) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if ((va & kVaTagMask) != kVaTag || (int)((va >> kVaClientShift) & kVaClientMask) != m->id) return TP_EFAULT;
+    if (!(va & kVaActBit)) return TP_EINVAL;  // memory_manager.hpp:99-101: freeing a model block is refused
+    auto it = m->ablocks.find(va & kVaOffMask);
+    if (it == m->ablocks.end() || !it->second.live) return TP_EFAULT;
+    it->second.live = false;
+    m->afree.emplace(it->second.size, it->second.voff);
+    return 0;
+}
+
+int Engine::ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need) {
+    if (need <= *cap) return 0;
+    uint64_t ncap = *cap ? *cap : (1ull << 20);
+    while (ncap < need) ncap *= 2;
+    HIPCHK(hipStreamSynchronize(compute_));
+    uint8_t* nb = nullptr;
+    HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&nb), ncap, hipHostMallocDefault));
+    if (*buf) (void)hipHostFree(*buf);
+    *buf = nb;
+    *cap = ncap;
+    return 0;
+}
+
+int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
+    if (bytes == 0) return 0;
+    if (!src) return TP_EINVAL;
+    if (mode_ == MODE_LOAD) {
+        // memory_manager.hpp:124-142 + model_repo.hpp:151-168: capture into the host weight store
+        if ((dst & kVaTagMask) != kVaTag || (int)((dst >> kVaClientShift) & kVaClientMask) != m.id ||
+            (dst & kVaActBit))
+            return TP_EFAULT;
+        const uint64_t off = dst & kVaOffMask;
+        bool inside = false;
+        for (const WBlock& b : m.wblocks)
+            if (off >= b.voff && off + bytes <= b.voff + b.size) {
+                inside = true;
+                break;
+            }
+        if (!inside) return TP_EFAULT;
+        std::memcpy(m.staging.data() + off, src, bytes);
+        // a tensor is what one upload covers; a repeated upload to the same start replaces it
+        for (Param& p : m.params)
+            if (p.voff == off) {
+                if (p.size != bytes) return TP_EINVAL;
+                return 0;
+            }
+        Param p;
+        p.voff = off;
+        p.size = bytes;
+        m.params.push_back(p);
+        return 0;
+    }
+    if (!(dst & kVaActBit)) return TP_ESTATE;  // the host copy of the weights is authoritative
+    Xlat x;
+    int r = translate(m, dst, bytes, &x);
+    if (r) return r;
+    if (host_only()) return 0;
+    if (h2d_pos_ + bytes > h2d_cap_) {
+        HIPCHK(hipStreamSynchronize(compute_));
+        h2d_pos_ = 0;
+        r = ensure_stage(&h2d_stage_, &h2d_cap_, bytes);
+        if (r) return r;
+    }
+    std::memcpy(h2d_stage_ + h2d_pos_, src, bytes);
+    HIPCHK(hipMemcpyAsync(x.p, h2d_stage_ + h2d_pos_, bytes, hipMemcpyHostToDevice, compute_));
+    h2d_pos_ = align_up(h2d_pos_ + bytes, 256);
+    return 0;
+}
+
+int Engine::op_h2d(int client, uint64_t dst, const void* src, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    int r = do_h2d(*m, dst, src, bytes);
+    if (r == 0 && mode_ == MODE_TRACK) {
+        Op op;
+        op.kind = OPK_H2D;
+        op.p[0] = dst;
+        op.i[0] = (int64_t)bytes;
+        m->program.push_back(op);
+    }
+    if (r && !m->async_error) m->async_error = r;
+    return r;
+}
+
+int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
+    if (!dst && bytes) return TP_EINVAL;
+    void* p = nullptr;
+    int r = resolve(m, src, bytes, false, &p);
+    if (r) return r;
+    if (!host_only() && bytes) {
+        if (d2h_pos_ + bytes > d2h_cap_) {
+            if (!pending_d2h_.empty()) {
+                // pending copies still point into the old buffer: deliver them first
+                HIPCHK(hipStreamSynchronize(compute_));
+                for (auto& pd : pending_d2h_) std::memcpy(pd.dst, d2h_stage_ + pd.stage_off, pd.bytes);
+                pending_d2h_.clear();
+            }
+            d2h_pos_ = 0;
+            r = ensure_stage(&d2h_stage_, &d2h_cap_, bytes);
+            if (r) return r;
+        }
+        HIPCHK(hipMemcpyAsync(d2h_stage_ + d2h_pos_, p, bytes, hipMemcpyDeviceToHost, compute_));
+        pending_d2h_.push_back({dst, d2h_pos_, bytes});
+        d2h_pos_ = align_up(d2h_pos_ + bytes, 256);
+    }
+    d2h_seen_ = true;
+    return 0;
+}
+
+int Engine::op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if (mode_ == MODE_LOAD) return TP_ESTATE;
+    int r = do_d2h_async(*m, dst, src, bytes);
+    if (r) {
+        if (!m->async_error) m->async_error = r;
+        return r;
+    }
+    if (mode_ == MODE_TRACK) {
+        Op op;
+        op.kind = OPK_D2H;
+        op.p[0] = src;
+        op.i[0] = (int64_t)bytes;
+        m->program.push_back(op);
+    }
+    // cuda_server.hpp:1044: the asynchronous D2H copy is the "request finished" marker
+    complete_request();
+    return 0;
+}
+
+int Engine::op_d2h(int client, void* dst, uint64_t src, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if (!dst && bytes) return TP_EINVAL;
+    void* p = nullptr;
+    int r = resolve(*m, src, bytes, false, &p);
+    if (r) return r;
+    if (host_only()) return TP_ENODEV;
+    HIPCHK(hipStreamSynchronize(compute_));
+    HIPCHK(hipMemcpy(dst, p, bytes, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int Engine::op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    Op op;
+    op.kind = OPK_D2D;
+    op.p[0] = dst;
+    op.p[1] = src;
+    op.i[0] = (int64_t)bytes;
+    int r = exec_op(*m, op, nullptr, true);
+    if (r == 0 && mode_ == MODE_TRACK) m->program.push_back(op);
+    if (r && !m->async_error) m->async_error = r;
+    return r;
+}
+
+int Engine::op_memset(int client, uint64_t dst, int value, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    Op op;
+    op.kind = OPK_MEMSET;
+    op.p[0] = dst;
+    op.i[0] = (int64_t)bytes;
+    op.i[1] = value;
+    int r = exec_op(*m, op, nullptr, true);
+    if (r == 0 && mode_ == MODE_TRACK) m->program.push_back(op);
+    if (r && !m->async_error) m->async_error = r;
+    return r;
+}
+
+int Engine::do_stream_sync(Model* m) {
+    int ret = 0;
+    if (!host_only()) {
+        hipError_t e = hipStreamSynchronize(compute_);
+        if (e != hipSuccess) ret = (int)e;
+        for (auto& pd : pending_d2h_)
+            if (!ret) std::memcpy(pd.dst, d2h_stage_ + pd.stage_off, pd.bytes);
+    } else if (d2h_seen_) {
+        ret = TP_ENODEV;  // no device: there is no data to deliver
+    }
+    pending_d2h_.clear();
+    d2h_pos_ = 0;
+    h2d_pos_ = 0;
+    d2h_seen_ = false;
+    if (m) {
+        if (!ret && m->async_error) ret = m->async_error;
+        m->async_error = 0;
+        if (!host_only() && m->resident && !m->fully_loaded && m->copy_state.load() == CS_ISSUED && m->t1 &&
+            hipEventQuery(m->t1) == hipSuccess)
+            m->fully_loaded = true;
+    }
+    return ret;
+}
+
+int Engine::op_stream_sync(int client) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    return do_stream_sync(m);
+}
+
+int Engine::op_device_sync(int client) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    int ret = 0;
+    if (!host_only()) {
+        hipError_t e = hipStreamSynchronize(compute_);
+        if (e != hipSuccess) ret = (int)e;
+    }
+    // cuda_server.hpp:959-961: the first device synchronisation after the uploads ends the
+    // weight-loading phase; what is allocated from now on is not model memory.
+    if (m && client == active_ && mode_ == MODE_LOAD) {
+        int r = finish_loading(*m);
+        if (r) return r;
+        mode_ = MODE_TRACK;
+    }
+    if (m && !ret && m->async_error) {
+        ret = m->async_error;
+        m->async_error = 0;
+    }
+    return ret;
+}
+
+// ------------------------------------------------------------------ image layout
+// The weight image holds every uploaded tensor, 256 B aligned, in first-access order (tensors
+// never touched by the tracked run follow in address order).  The same offsets are used in the
+// pinned host store and in HBM, so a swap-in is a sequential copy and a weight address
+// translates with one add.  (Reference: per-tensor host allocations and a per-tensor
+// virtual->physical map rebuilt on every swap-in, memory_manager.hpp:451-507.)
+int Engine::build_image(Model& m, bool by_access) {
+    std::vector<size_t> order(m.params.size());
+    for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+    if (by_access) {
+        std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) {
+            const int ra = m.params[a].access_rank, rb = m.params[b].access_rank;
+            if ((ra >= 0) != (rb >= 0)) return ra >= 0;
+            if (ra >= 0 && ra != rb) return ra < rb;
+            return m.params[a].voff < m.params[b].voff;
+        });
+    }
+    std::vector<uint64_t> new_off(m.params.size());
+    uint64_t off = 0;
+    bool same = (m.host_image != nullptr);
+    for (size_t k = 0; k < order.size(); ++k) {
+        const Param& p = m.params[order[k]];
+        new_off[order[k]] = off;
+        if (p.image_off != off) same = false;
+        off = align_up(off + p.size, kTensorAlign);
+    }
+    if (same && m.image_bytes == off) return 0;
+    uint8_t* img = static_cast<uint8_t*>(host_alloc(off));
+    if (!img) return TP_ENOMEM;
+    std::memset(img, 0, off ? off : 1);
+    for (size_t i = 0; i < m.params.size(); ++i) {
+        Param& p = m.params[i];
+        const uint8_t* src = m.host_image ? m.host_image + p.image_off : m.staging.data() + p.voff;
+        std::memcpy(img + new_off[i], src, p.size);
+    }
+    for (size_t i = 0; i < m.params.size(); ++i) m.params[i].image_off = new_off[i];
+    host_free(m.host_image);
+    m.host_image = img;
+    m.image_bytes = off;
+    return 1;  // image changed
+}
+
+// Transfer groups: the first is chunk_bytes, each next one doubles up to chunk_max_bytes, so the
+// first layers can start after a short copy while the bulk moves in DMA-efficient pieces.
+// (Reference: fixed >= BUFFER_SIZE groups, memory_manager.hpp:399-409.)
+void Engine::build_chunks(Model& m) {
+    m.chunk_end.clear();
+    uint64_t sz = cfg_.chunk_bytes, pos = 0;
+    while (pos < m.image_bytes) {
+        uint64_t end = pos + align_up(sz, kTensorAlign);
+        if (end > m.image_bytes) end = m.image_bytes;
+        m.chunk_end.push_back(end);
+        pos = end;
+        if (sz < cfg_.chunk_max_bytes) sz = std::min(sz * 2, cfg_.chunk_max_bytes);
+    }
+    if (!host_only()) {
+        while (m.chunk_ev.size() < m.chunk_end.size()) {
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) break;
+            m.chunk_ev.push_back(ev);
+        }
+        if (!m.t0) (void)hipEventCreate(&m.t0);
+        if (!m.t1) (void)hipEventCreate(&m.t1);
+    }
+}
+
+int Engine::finish_loading(Model& m) {
+    std::sort(m.params.begin(), m.params.end(), [](const Param& a, const Param& b) { return a.voff < b.voff; });
+    for (size_t i = 1; i < m.params.size(); ++i)
+        if (m.params[i - 1].voff + m.params[i - 1].size > m.params[i].voff) return TP_EINVAL;  // overlapping uploads
+    m.param_bytes = 0;
+    for (auto& p : m.params) m.param_bytes += p.size;
+    int r = build_image(m, false);
+    if (r < 0) return r;
+    std::vector<uint8_t>().swap(m.staging);
+    // cold start leaves the weights on the device (memory_manager.hpp:141), so the tracked
+    // inference runs with a resident model
+    m.w_pool_off = pool_.alloc(m.image_bytes);
+    if (m.w_pool_off == UINT64_MAX) return TP_ENOMEM;
+    m.w_dev = arena_ + m.w_pool_off;
+    if (!host_only() && m.image_bytes) HIPCHK(hipMemcpy(m.w_dev, m.host_image, m.image_bytes, hipMemcpyHostToDevice));
+    m.resident = true;
+    m.fully_loaded = true;
+    m.state = MS_TRACKING;
+    return 0;
+}
+
+int Engine::finish_tracking(Model& m) {
+    // memory_manager.hpp:73-80 unset_track_model_memory + the layout step described above
+    int r = build_image(m, true);
+    if (r < 0) return r;
+    if (r == 1 && !host_only() && m.image_bytes)
+        HIPCHK(hipMemcpy(m.w_dev, m.host_image, m.image_bytes, hipMemcpyHostToDevice));
+    build_chunks(m);
+    // fold the per-allocation activation extents of the tracked run into one arena
+    if (!host_only()) HIPCHK(hipStreamSynchronize(compute_));
+    for (auto& kv : m.ablocks) {
+        if (kv.second.pool_off != UINT64_MAX) pool_.release(kv.second.pool_off);
+        kv.second.pool_off = UINT64_MAX;
+    }
+    m.act_bytes = m.abump;
+    m.act_frozen = true;
+    m.a_pool_off = pool_.alloc(m.act_bytes);
+    if (m.a_pool_off == UINT64_MAX) return TP_ENOMEM;
+    m.a_dev = arena_ + m.a_pool_off;
+    m.state = MS_READY;
+    return 0;
+}
+
+// ------------------------------------------------------------------ swap engine
+void Engine::copy_main() {
+    (void)hipSetDevice(cfg_.device);
+    for (;;) {
+        Model* m = nullptr;
+        {
+            std::unique_lock<std::mutex> lk(cmu_);
+            ccv_.wait(lk, [&] { return stop_ || !jobs_.empty(); });
+            if (stop_) return;
+            m = jobs_.front();
+            jobs_.pop_front();
+        }
+        // memory_manager.hpp:378-409: walk the tensors in access order, one DMA per group, and
+        // publish each group.  Publishing is an event record, not a host synchronisation.
+        int err = 0;
+        if (!m->cancel.load()) {
+            hipError_t e = hipEventRecord(m->t0, copy_);
+            if (e != hipSuccess) err = (int)e;
+            uint64_t beg = 0;
+            for (size_t i = 0; i < m->chunk_end.size() && !err; ++i) {
+                if (m->cancel.load()) break;
+                const uint64_t end = m->chunk_end[i];
+                e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, copy_);
+                if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], copy_);
+                if (e != hipSuccess) {
+                    err = (int)e;
+                    break;
+                }
+                m->issued.store((uint32_t)i + 1, std::memory_order_release);
+                beg = end;
+            }
+            if (!err) (void)hipEventRecord(m->t1, copy_);
+        }
+        if (err) m->copy_error.store(err);
+        m->copy_state.store(CS_ISSUED, std::memory_order_release);
+    }
+}
+
+void Engine::wait_copy_idle(Model& m) {
+    if (host_only()) return;
+    if (m.copy_state.load(std::memory_order_acquire) == CS_RUNNING) {
+        m.cancel.store(true);
+        while (m.copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
+    }
+    (void)hipStreamSynchronize(copy_);
+}
+
+// memory_manager.hpp:213-227 sig_trans_thread + 451-507 check_and_malloc_model
+int Engine::swap_in(Model& m) {
+    if (m.resident) return 0;
+    const auto t0 = Clock::now();
+    auto try_alloc = [&]() -> bool {
+        m.w_pool_off = pool_.alloc(m.image_bytes);
+        if (m.w_pool_off == UINT64_MAX) return false;
+        m.a_pool_off = pool_.alloc(m.act_bytes);
+        if (m.a_pool_off == UINT64_MAX) {
+            pool_.release(m.w_pool_off);
+            m.w_pool_off = UINT64_MAX;
+            return false;
+        }
+        return true;
+    };
+    while (!try_alloc()) {
+        // The budget test passed but no contiguous extent fits: keep evicting in LRU order.
+        // (The reference exits the process here, block_manager.hpp:345-351.)
+        std::string victim;
+        if (!lru_.peek_victim(std::to_string(m.id), &victim)) return TP_ENOMEM;
+        lru_.force_evict(victim);
+        Model* v = find(std::atoi(victim.c_str()));
+        if (v) evict_model(*v);
+    }
+    m.w_dev = arena_ + m.w_pool_off;
+    m.a_dev = arena_ + m.a_pool_off;
+    m.resident = true;
+    m.fully_loaded = false;
+    m.gated_upto = 0;
+    m.issued.store(0);
+    m.cancel.store(false);
+    m.copy_error.store(0);
+    m.stats.alloc_us = us_since(t0);
+    m.stats.bytes = m.image_bytes;
+    m.stats.chunks = (uint32_t)m.chunk_end.size();
+    ++swap_ins_;
+    if (host_only() || m.image_bytes == 0) {
+        m.fully_loaded = true;
+        return 0;
+    }
+    m.timing_valid = true;
+    m.copy_state.store(CS_RUNNING, std::memory_order_release);
+    {
+        std::lock_guard<std::mutex> lk(cmu_);
+        jobs_.push_back(&m);
+    }
+    ccv_.notify_one();
+    return 0;
+}
+
+// memory_manager.hpp:240-259: metadata only, the host copy stays authoritative.
+void Engine::evict_model(Model& m) {
+    if (!m.resident) return;
+    const auto t0 = Clock::now();
+    wait_copy_idle(m);
+    if (m.w_pool_off != UINT64_MAX) pool_.release(m.w_pool_off);
+    if (m.a_pool_off != UINT64_MAX) pool_.release(m.a_pool_off);
+    m.w_pool_off = m.a_pool_off = UINT64_MAX;
+    m.w_dev = m.a_dev = nullptr;
+    m.resident = false;
+    m.fully_loaded = false;
+    m.copy_state.store(CS_IDLE);
+    m.stats.evict_us = us_since(t0);
+    ++evictions_;
+}
+
+// controller.hpp:392-400
+bool Engine::check_eviction(Model& m) {
+    bool over = false;
+    auto victims = lru_.check_and_add(std::to_string(m.id), m.total_bytes(), &over);
+    for (auto& v : victims) {
+        Model* vm = find(std::atoi(v.c_str()));
+        if (vm) evict_model(*vm);
+    }
+    return !over;
+}
+
+// ------------------------------------------------------------------ controller
+void Engine::start_cold(int id, int level) {
+    // controller.hpp:402-413 + cuda_server.hpp:223-228 (Startup): a re-registration replaces
+    // the previous model of that id
+    Model* old = find(id);
+    if (old) {
+        lru_.force_evict(std::to_string(id));
+        evict_model(*old);
+        wait_copy_idle(*old);
+        host_free(old->host_image);
+        if (!host_only()) {
+            for (auto ev : old->chunk_ev) (void)hipEventDestroy(ev);
+            if (old->t0) (void)hipEventDestroy(old->t0);
+            if (old->t1) (void)hipEventDestroy(old->t1);
+        }
+        models_.erase(id);
+    }
+    auto m = std::make_unique<Model>();
+    m->id = id;
+    m->level = level;
+    models_[id] = std::move(m);
+    active_ = id;
+    mode_ = MODE_LOAD;
+    exec_status_ = ES_COLD;
+}
+
+int Engine::start_execute(int id) {
+    Model* m = find(id);
+    if (!m || m->state != MS_READY) return TP_ENOENT;
+    const bool was_resident = m->resident;
+    // controller.hpp:420-427 send_load_req: eviction check, then the Load signal
+    check_eviction(*m);
+    int r = swap_in(*m);
+    if (r) {
+        lru_.force_evict(std::to_string(id));
+        return r;
+    }
+    // controller.hpp:414-417 + cuda_server.hpp:229-239
+    active_ = id;
+    mode_ = MODE_EXEC;
+    m->stats.gate_waits = 0;
+    req_start_ = Clock::now();
+    if (was_resident)
+        exec_status_ = ES_LOCAL;
+    else
+        exec_status_ = (m->level == 0) ? ES_PCIE_LIGHT : (m->level == 2 ? ES_PCIE_HEAVY : ES_PCIE_MEDIAN);
+    return 0;
+}
+
+// cuda_server.hpp:287-299 send_complete_signal + controller.hpp:218-263
+void Engine::complete_request() {
+    if (active_ < 0) return;
+    Model* m = find(active_);
+    if (m && mode_ == MODE_TRACK) {
+        int r = finish_tracking(*m);
+        if (r && !m->async_error) m->async_error = r;
+    }
+    const int status = exec_status_;
+    active_ = -1;
+    mode_ = MODE_NONE;
+    if (m && m->state == MS_READY) {
+        if (status == ES_COLD) check_eviction(*m);  // controller.hpp:223-227
+    }
+    exec_status_ = ES_AVAIL;
+    if (!req_queue_.empty()) {  // controller.hpp:242-262
+        Queued q = req_queue_.front();
+        req_queue_.pop_front();
+        if (q.cold) {
+            start_cold(q.id, q.level);
+            deferred_acks_.emplace_back(TP_ACK_OK, 0);
+        } else {
+            int r = start_execute(q.id);
+            deferred_acks_.emplace_back(r ? TP_ACK_INAVAIL : TP_ACK_OK, 0);
+        }
+    }
+}
+
+bool Engine::poll_timeout_locked() {
+    // cuda_server.hpp:257-264
+    if (active_ >= 0 && mode_ == MODE_EXEC) {
+        const double ms = us_since(req_start_) / 1000.0;
+        if (ms > (double)cfg_.request_timeout_ms) {
+            if (!host_only()) (void)hipStreamSynchronize(compute_);
+            complete_request();
+            return true;
+        }
+    }
+    return false;
+}
+
+int Engine::poll() {
+    std::lock_guard<std::mutex> lk(mu_);
+    return poll_timeout_locked() ? 1 : 0;
+}
+
+int Engine::take_deferred_ack(int* ack, int* resp) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (deferred_acks_.empty()) return 0;
+    if (ack) *ack = deferred_acks_.front().first;
+    if (resp) *resp = deferred_acks_.front().second;
+    deferred_acks_.pop_front();
+    return 1;
+}
+
+static bool parse_int(const char* s, int* out) {
+    if (!s || !*s) return false;
+    char* end = nullptr;
+    long v = std::strtol(s, &end, 10);
+    if (*end != '\0') return false;
+    *out = (int)v;
+    return true;
+}
+
+int Engine::signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (ack) *ack = TP_ACK_OK;
+    if (resp) *resp = -1;
+    if (deferred) *deferred = 0;
+    int id = -1;
+    if (!parse_int(function, &id) || id < 0 || id > kMaxClient) return TP_EINVAL;  // cuda_server.hpp:221 stoi(func)
+    poll_timeout_locked();
+    const bool busy = exec_status_ != ES_AVAIL;
+    switch (type) {
+        case TP_REQ_EXECUTE_AFTER_LOAD: {  // controller.hpp:141-162
+            int level = 1;
+            int lv = 0;
+            if (payload && *payload && parse_int(payload, &lv) && lv >= 0 && lv <= 2) level = lv;
+            if (busy) {
+                if (active_ == id) {
+                    if (ack) *ack = TP_ACK_INAVAIL;
+                    return 0;
+                }
+                req_queue_.push_back({id, true, level});
+                if (deferred) *deferred = 1;
+                return 0;
+            }
+            start_cold(id, level);
+            if (resp) *resp = 0;
+            return 0;
+        }
+        case TP_REQ_EXECUTE: {  // controller.hpp:163-186
+            if (busy) {
+                req_queue_.push_back({id, false, 1});
+                if (deferred) *deferred = 1;
+                return 0;
+            }
+            int r = start_execute(id);
+            if (r) {
+                if (ack) *ack = TP_ACK_INAVAIL;
+                return 0;
+            }
+            if (resp) *resp = 0;
+            return 0;
+        }
+        case TP_REQ_UNLOAD: {  // controller.hpp:187-207
+            Model* m = find(id);
+            if (active_ == id) {
+                if (ack) *ack = TP_ACK_INAVAIL;
+                return 0;
+            }
+            if (m && m->resident && m->state == MS_READY) {
+                lru_.force_evict(std::to_string(id));
+                evict_model(*m);
+            }
+            return 0;  // ack OK, resp -1
+        }
+        case TP_REQ_LOAD: {  // controller.hpp:208-215
+            Model* m = find(id);
+            if (!m || m->state != MS_READY || active_ == id) {
+                if (ack) *ack = TP_ACK_INAVAIL;
+                return 0;
+            }
+            check_eviction(*m);
+            int r = swap_in(*m);
+            if (r) {
+                lru_.force_evict(std::to_string(id));
+                if (ack) *ack = TP_ACK_INAVAIL;
+            }
+            return 0;
+        }
+        default:  // ExecuteForRecord / Replay are refused like in cuda_server.hpp:188-195
+            if (ack) *ack = TP_ACK_INAVAIL;
+            return 0;
+    }
+}
+
+// ------------------------------------------------------------------ compute ops
+static tpk::EpilogueArgs ep_from(const Op& op, void* const* q, int pbase, int fbase, int ibase) {
+    tpk::EpilogueArgs e;
+    e.alpha = op.f[fbase + 0];
+    e.beta = op.f[fbase + 1];
+    e.bn_eps = op.f[fbase + 2];
+    e.bias = static_cast<const float*>(q[pbase + 0]);
+    e.bn_scale = static_cast<const float*>(q[pbase + 1]);
+    e.bn_bias = static_cast<const float*>(q[pbase + 2]);
+    e.bn_mean = static_cast<const float*>(q[pbase + 3]);
+    e.bn_var = static_cast<const float*>(q[pbase + 4]);
+    e.residual = static_cast<const float*>(q[pbase + 5]);
+    e.ldr = op.i[ibase + 0];
+    e.act = (int)op.i[ibase + 1];
+    return e;
+}
+
+// Layout of Op for the compute kinds (filled by the C-ABI layer):
+//  GEMM  p: x y c bias bns bnb bnm bnv res   i: m n k xs_r xs_k ys_c ys_k ldc nb0 nb1 xb0 xb1 yb0 yb1 cb0 cb1 ldr act
+//        f: alpha beta eps
+//  CONV  p: x w y bias bns bnb bnm bnv res   i: n h w cin cout kh kw sh sw ph pw xl yl ldr act   f: alpha beta eps
+//  BN    p: x y g b mean var                 i: rows C hw layout relu   f: eps
+//  LAUNCH p/i/f per op id (see torpor_amd.h)
+int Engine::exec_compute(Model& m, const Op& op, bool launch) {
+    void* q[12] = {nullptr};
+    const tpk::Workspace ws{workspace_, (size_t)cfg_.workspace_bytes};
+    // Every operand is translated together with the byte span the kernel will touch, so an op
+    // whose shapes do not fit its buffers is refused on the host instead of faulting the GPU.
+    auto R = [&](int idx, bool optional, int64_t elems, int64_t elem_size = 4) -> int {
+        if (elems < 1) elems = 1;
+        return resolve(m, op.p[idx], (uint64_t)elems * (uint64_t)elem_size, optional, &q[idx]);
+    };
+    const int64_t* I = op.i;
+    for (int k = 0; k < op.ni && k < 20; ++k)
+        if (I[k] < 0) return TP_EINVAL;
+    int r = 0;
+    switch (op.kind) {
+        case OPK_GEMM: {
+            const int64_t M = I[0], N = I[1], K = I[2];
+            const int64_t nb0 = I[8], nb1 = I[9];
+            if (M < 1 || N < 1 || nb0 < 1 || nb1 < 1) return TP_EINVAL;
+            const int64_t kx = K > 0 ? K - 1 : 0;
+            const int64_t xs = (M - 1) * I[3] + kx * I[4] + (nb0 - 1) * I[10] + (nb1 - 1) * I[11] + 1;
+            const int64_t ys = (N - 1) * I[5] + kx * I[6] + (nb0 - 1) * I[12] + (nb1 - 1) * I[13] + 1;
+            const int64_t cs = (M - 1) * I[7] + N + (nb0 - 1) * I[14] + (nb1 - 1) * I[15];
+            if (I[7] < N) return TP_EINVAL;
+            const int64_t ldr = I[16] ? I[16] : I[7];
+            if (op.p[8] && (nb0 * nb1 != 1 || ldr < N)) return TP_EUNSUPPORTED;
+            if ((r = R(0, false, xs)) || (r = R(1, false, ys)) || (r = R(2, false, cs))) return r;
+            for (int k = 3; k < 8 && !r; ++k) r = R(k, true, N);
+            if (!r) r = R(8, true, (M - 1) * ldr + N);
+            if (r) return r;
+            if ((q[4] != nullptr) != (q[5] != nullptr) || (q[4] != nullptr) != (q[6] != nullptr) ||
+                (q[4] != nullptr) != (q[7] != nullptr))
+                return TP_EINVAL;
+            tpk::GemmArgs g;
+            g.X = static_cast<const float*>(q[0]);
+            g.Y = static_cast<const float*>(q[1]);
+            g.C = static_cast<float*>(q[2]);
+            g.M = M;
+            g.N = N;
+            g.K = K;
+            g.xs_r = I[3];
+            g.xs_k = I[4];
+            g.ys_c = I[5];
+            g.ys_k = I[6];
+            g.ldc = I[7];
+            g.nb0 = (int)nb0;
+            g.nb1 = (int)nb1;
+            g.xb0 = I[10];
+            g.xb1 = I[11];
+            g.yb0 = I[12];
+            g.yb1 = I[13];
+            g.cb0 = I[14];
+            g.cb1 = I[15];
+            g.ep = ep_from(op, q, 3, 0, 16);
+            g.ep.ldr = ldr;
+            if (!launch) return 0;
+            return tpk::launch_gemm(g, ws, compute_);
+        }
+        case OPK_CONV: {
+            const int64_t N = I[0], H = I[1], W = I[2], Cin = I[3], Cout = I[4], KH = I[5], KW = I[6];
+            const int64_t sh = I[7], sw = I[8], ph = I[9], pw = I[10];
+            if (N < 1 || H < 1 || W < 1 || Cin < 1 || Cout < 1 || KH < 1 || KW < 1 || sh < 1 || sw < 1)
+                return TP_EINVAL;
+            const int64_t Ho = (H + 2 * ph - KH) / sh + 1, Wo = (W + 2 * pw - KW) / sw + 1;
+            if (H + 2 * ph < KH || W + 2 * pw < KW || Ho < 1 || Wo < 1) return TP_EINVAL;
+            const int64_t ys = N * Ho * Wo * Cout;
+            if ((r = R(0, false, N * H * W * Cin)) || (r = R(1, false, Cout * Cin * KH * KW)) || (r = R(2, false, ys)))
+                return r;
+            for (int k = 3; k < 8 && !r; ++k) r = R(k, true, Cout);
+            if (!r) r = R(8, true, ys);
+            if (r) return r;
+            if ((q[4] != nullptr) != (q[5] != nullptr) || (q[4] != nullptr) != (q[6] != nullptr) ||
+                (q[4] != nullptr) != (q[7] != nullptr))
+                return TP_EINVAL;
+            tpk::ConvArgs c;
+            c.x = static_cast<const float*>(q[0]);
+            c.w = static_cast<const float*>(q[1]);
+            c.y = static_cast<float*>(q[2]);
+            c.N = (int)N;
+            c.H = (int)H;
+            c.W = (int)W;
+            c.Cin = (int)Cin;
+            c.Cout = (int)Cout;
+            c.KH = (int)KH;
+            c.KW = (int)KW;
+            c.sh = (int)sh;
+            c.sw = (int)sw;
+            c.ph = (int)ph;
+            c.pw = (int)pw;
+            c.x_nhwc = (int)I[11];
+            c.y_nhwc = (int)I[12];
+            c.ep = ep_from(op, q, 3, 0, 13);
+            c.ep.ldr = 0;  // residual shares the layout and pitch of y
+            if (!launch) return 0;
+            return tpk::launch_conv2d(c, ws, compute_);
+        }
+        case OPK_BN: {
+            const int64_t rows = I[0], C = I[1];
+            if (C < 1) return TP_EINVAL;
+            if ((r = R(0, false, rows * C)) || (r = R(1, false, rows * C))) return r;
+            for (int k = 2; k < 6 && !r; ++k) r = R(k, false, C);
+            if (r) return r;
+            if (!I[3] && I[2] < 1) return TP_EINVAL;
+            if (!launch) return 0;
+            return tpk::launch_bn_inference(static_cast<const float*>(q[0]), static_cast<float*>(q[1]),
+                                            static_cast<const float*>(q[2]), static_cast<const float*>(q[3]),
+                                            static_cast<const float*>(q[4]), static_cast<const float*>(q[5]), op.f[0],
+                                            rows, (int)C, (int)I[3], I[2], (int)I[4], compute_);
+        }
+        case OPK_LAUNCH:
+            break;
+        default:
+            return TP_EINVAL;
+    }
+    // generic launch by op id
+    auto need = [&](int np, int ni, int nf) { return op.np >= np && op.ni >= ni && op.nf >= nf; };
+    auto F = [&](int k) { return static_cast<const float*>(q[k]); };
+    auto Fm = [&](int k) { return static_cast<float*>(q[k]); };
+    switch (op.op_id) {
+        case TP_OP_RELU:
+        case TP_OP_GELU:
+            if (!need(2, 1, 0)) return TP_EINVAL;
+            if ((r = R(0, false, I[0])) || (r = R(1, false, I[0]))) return r;
+            if (!launch) return 0;
+            return op.op_id == TP_OP_RELU ? tpk::launch_relu(F(0), Fm(1), I[0], compute_)
+                                          : tpk::launch_gelu(F(0), Fm(1), I[0], compute_);
+        case TP_OP_ADD:
+            if (!need(3, 2, 0)) return TP_EINVAL;
+            if ((r = R(0, false, I[0])) || (r = R(1, false, I[0])) || (r = R(2, false, I[0]))) return r;
+            if (!launch) return 0;
+            return tpk::launch_add(F(0), F(1), Fm(2), I[0], (int)I[1], compute_);
+        case TP_OP_BIAS_ACT:
+            if (!need(3, 3, 0) || I[1] < 1) return TP_EINVAL;
+            if ((r = R(0, false, I[0] * I[1])) || (r = R(1, false, I[1])) || (r = R(2, false, I[0] * I[1]))) return r;
+            if (!launch) return 0;
+            return tpk::launch_bias_act(F(0), F(1), Fm(2), I[0], (int)I[1], (int)I[2], compute_);
+        case TP_OP_MAXPOOL: {
+            if (!need(2, 8, 0)) return TP_EINVAL;
+            const int64_t N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
+            if (N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || st < 1 || H + 2 * pad < k || W + 2 * pad < k)
+                return TP_EINVAL;
+            const int64_t Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
+            if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, N * Ho * Wo * C))) return r;
+            if (!launch) return 0;
+            return tpk::launch_maxpool2d(F(0), Fm(1), (int)N, (int)H, (int)W, (int)C, (int)k, (int)st, (int)pad,
+                                         (int)I[7], compute_);
+        }
+        case TP_OP_AVGPOOL:
+            if (!need(2, 4, 0)) return TP_EINVAL;
+            if ((r = R(0, false, I[0] * I[1] * I[2])) || (r = R(1, false, I[0] * I[2]))) return r;
+            if (!launch) return 0;
+            return tpk::launch_global_avgpool(F(0), Fm(1), (int)I[0], (int)I[1], (int)I[2], (int)I[3], compute_);
+        case TP_OP_LAYERNORM:
+            if (!need(5, 2, 1)) return TP_EINVAL;
+            if ((r = R(0, false, I[0] * I[1])) || (r = R(1, true, I[0] * I[1])) || (r = R(2, false, I[1])) ||
+                (r = R(3, false, I[1])) || (r = R(4, false, I[0] * I[1])))
+                return r;
+            if (!launch) return 0;
+            return tpk::launch_layernorm(F(0), F(1), F(2), F(3), Fm(4), I[0], (int)I[1], op.f[0], compute_);
+        case TP_OP_SOFTMAX: {
+            if (!need(3, 3, 1)) return TP_EINVAL;
+            const int64_t rpm = I[2] > 0 ? I[2] : 1;
+            if ((r = R(0, false, I[0] * I[1])) || (r = R(1, true, ((I[0] + rpm - 1) / rpm) * I[1])) ||
+                (r = R(2, false, I[0] * I[1])))
+                return r;
+            if (!launch) return 0;
+            return tpk::launch_softmax(F(0), F(1), Fm(2), I[0], (int)I[1], op.f[0], rpm, compute_);
+        }
+        case TP_OP_EMBEDDING:
+            if (!need(6, 5, 0)) return TP_EINVAL;
+            if (I[1] < 1 || I[2] < 1 || I[3] < 1 || I[4] < 1) return TP_EINVAL;
+            if ((r = R(0, false, I[0], 8)) || (r = R(1, true, I[0], 8)) || (r = R(2, false, I[3] * I[2])) ||
+                (r = R(3, true, I[1] * I[2])) || (r = R(4, true, I[4] * I[2])) || (r = R(5, false, I[0] * I[2])))
+                return r;
+            if (!launch) return 0;
+            return tpk::launch_embedding(static_cast<const int64_t*>(q[0]), static_cast<const int64_t*>(q[1]), F(2),
+                                         F(3), F(4), Fm(5), I[0], (int)I[1], (int)I[2], I[3], (int)I[4], compute_);
+        case TP_OP_NCHW_TO_NHWC:
+        case TP_OP_NHWC_TO_NCHW: {
+            if (!need(2, 4, 0)) return TP_EINVAL;
+            const int64_t n = I[0] * I[1] * I[2] * I[3];
+            if ((r = R(0, false, n)) || (r = R(1, false, n))) return r;
+            if (!launch) return 0;
+            return op.op_id == TP_OP_NCHW_TO_NHWC
+                       ? tpk::launch_nchw_to_nhwc(F(0), Fm(1), (int)I[0], (int)I[1], (int)I[2], (int)I[3], compute_)
+                       : tpk::launch_nhwc_to_nchw(F(0), Fm(1), (int)I[0], (int)I[1], (int)I[2], (int)I[3], compute_);
+        }
+        case TP_OP_SUM:
+            if (!need(2, 1, 0)) return TP_EINVAL;
+            if ((r = R(0, false, I[0])) || (r = R(1, false, 1))) return r;
+            if (!launch) return 0;
+            return tpk::launch_sum(F(0), Fm(1), I[0], compute_);
+        case TP_OP_FILL:
+            if (!need(1, 1, 1)) return TP_EINVAL;
+            if ((r = R(0, false, I[0]))) return r;
+            if (!launch) return 0;
+            return tpk::launch_fill(Fm(0), op.f[0], I[0], compute_);
+        default:
+            return TP_EUNSUPPORTED;
+    }
+}
+
+int Engine::exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch) {
+    const bool run = launch && !host_only();
+    switch (op.kind) {
+        case OPK_GEMM:
+        case OPK_CONV:
+        case OPK_BN:
+        case OPK_LAUNCH:
+            return exec_compute(m, op, run);
+        case OPK_H2D: {
+            const uint64_t bytes = (uint64_t)op.i[0];
+            if (!rc) return TP_EINVAL;
+            if (rc->in_pos + bytes > rc->in_bytes) return TP_EINVAL;
+            int r = do_h2d(m, op.p[0], rc->in + rc->in_pos, bytes);
+            rc->in_pos += bytes;
+            return r;
+        }
+        case OPK_D2H: {
+            const uint64_t bytes = (uint64_t)op.i[0];
+            if (!rc) return TP_EINVAL;
+            if (rc->out_pos + bytes > rc->out_bytes) return TP_EINVAL;
+            int r = do_d2h_async(m, rc->out + rc->out_pos, op.p[0], bytes);
+            rc->out_pos += bytes;
+            return r;
+        }
+        case OPK_D2D: {
+            void *d = nullptr, *s = nullptr;
+            const uint64_t bytes = (uint64_t)op.i[0];
+            int r = resolve(m, op.p[0], bytes, false, &d);
+            if (!r) r = resolve(m, op.p[1], bytes, false, &s);
+            if (r) return r;
+            if (!run || bytes == 0) return 0;
+            return tpk::launch_copy(s, d, bytes, compute_);
+        }
+        case OPK_MEMSET: {
+            void* d = nullptr;
+            const uint64_t bytes = (uint64_t)op.i[0];
+            int r = resolve(m, op.p[0], bytes, false, &d);
+            if (r) return r;
+            if (!(op.p[0] & kVaActBit)) return TP_ESTATE;
+            if (!run || bytes == 0) return 0;
+            HIPCHK(hipMemsetAsync(d, (int)op.i[1], bytes, compute_));
+            return 0;
+        }
+        default:
+            return TP_EINVAL;
+    }
+}
+
+int Engine::op_compute(int client, const Op& op) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if (mode_ == MODE_LOAD) return TP_ESTATE;
+    int r = exec_op(*m, op, nullptr, true);
+    if (r) {
+        if (!m->async_error) m->async_error = r;
+        return r;
+    }
+    if (mode_ == MODE_TRACK) m->program.push_back(op);
+    return 0;
+}
+
+int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uint64_t out_bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    int err = 0;
+    Model* m = active_model(client, &err);
+    if (!m) return err;
+    if (mode_ != MODE_EXEC) return TP_ESTATE;
+    if (m->program.empty()) return TP_ENOENT;
+    ReplayCtx rc;
+    rc.in = static_cast<const uint8_t*>(in);
+    rc.in_bytes = in_bytes;
+    rc.out = static_cast<uint8_t*>(out);
+    rc.out_bytes = out_bytes;
+    int ret = 0;
+    bool completed = false;
+    for (const Op& op : m->program) {
+        int r = exec_op(*m, op, &rc, true);
+        if (r && !ret) ret = r;
+        if (r) break;
+        if (op.kind == OPK_D2H) completed = true;
+    }
+    int sr = do_stream_sync(m);
+    if (!ret) ret = sr;
+    (void)completed;
+    complete_request();
+    return ret;
+}
+
+// ------------------------------------------------------------------ introspection
+int Engine::model_resident(int client) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    return m->resident ? 1 : 0;
+}
+
+int Engine::model_info(int client, tp_model_info* out) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!out) return TP_EINVAL;
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    std::memset(out, 0, sizeof(*out));
+    out->registered = m->state == MS_READY;
+    out->resident = m->resident;
+    out->level = m->level;
+    out->n_params = (int)m->params.size();
+    out->n_chunks = (int)m->chunk_end.size();
+    out->n_ops = (int)m->program.size();
+    out->image_bytes = m->image_bytes;
+    out->param_bytes = m->param_bytes;
+    out->act_bytes = m->act_bytes;
+    out->total_bytes = m->total_bytes();
+    out->weight_off = m->w_pool_off;
+    out->act_off = m->a_pool_off;
+    return 0;
+}
+
+int Engine::pool_stats(tp_pool_stats* out) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!out) return TP_EINVAL;
+    out->capacity = pool_.capacity();
+    out->used = pool_.used_bytes();
+    out->largest_free = pool_.largest_free();
+    out->live_extents = pool_.live_extents();
+    out->free_extents = pool_.free_extents();
+    out->lru_budget = lru_.budget();
+    out->lru_used = lru_.cur_size();
+    out->lru_models = lru_.size();
+    out->evictions = evictions_;
+    out->swap_ins = swap_ins_;
+    return 0;
+}
+
+int Engine::swap_stats(int client, tp_swap_stats* out) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!out) return TP_EINVAL;
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (!host_only() && m->timing_valid && m->copy_state.load() == CS_ISSUED && !m->cancel.load()) {
+        if (hipEventSynchronize(m->t1) == hipSuccess) {
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, m->t0, m->t1) == hipSuccess) m->stats.copy_ms = ms;
+        }
+    }
+    *out = m->stats;
+    return 0;
+}
+
+int Engine::readback_weights(int client, void* dst, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (!m->resident) return TP_ESTATE;
+    if (!dst || bytes != m->image_bytes) return TP_EINVAL;
+    if (host_only()) return TP_ENODEV;
+    while (m->copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
+    HIPCHK(hipStreamSynchronize(copy_));
+    HIPCHK(hipStreamSynchronize(compute_));
+    HIPCHK(hipMemcpy(dst, m->w_dev, bytes, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int Engine::host_weights(int client, const void** ptr, uint64_t* bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (!m->host_image) return TP_ESTATE;
+    if (ptr) *ptr = m->host_image;
+    if (bytes) *bytes = m->image_bytes;
+    return 0;
+}
+
+int Engine::weight_offset(int client, uint64_t va, uint64_t* off) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if ((va & kVaTagMask) != kVaTag || (va & kVaActBit)) return TP_EFAULT;
+    const uint64_t o = va & kVaOffMask;
+    for (auto& p : m->params)
+        if (o >= p.voff && o < p.voff + p.size) {
+            if (off) *off = p.image_off + (o - p.voff);
+            return 0;
+        }
+    return TP_EFAULT;
+}
+
+int Engine::measure_h2d(uint64_t bytes, int iters, double* gbps) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (host_only()) return TP_ENODEV;
+    if (!gbps || bytes == 0 || iters <= 0) return TP_EINVAL;
+    if (bytes > pool_.largest_free()) return TP_ENOMEM;
+    const uint64_t off = pool_.alloc(bytes);
+    if (off == UINT64_MAX) return TP_ENOMEM;
+    uint8_t* h = nullptr;
+    int ret = 0;
+    hipEvent_t a = nullptr, b = nullptr;
+    std::vector<float> ms;
+    if (hipHostMalloc(reinterpret_cast<void**>(&h), bytes, hipHostMallocDefault) != hipSuccess) {
+        pool_.release(off);
+        return TP_ENOMEM;
+    }
+    std::memset(h, 0x5a, bytes);
+    (void)hipEventCreate(&a);
+    (void)hipEventCreate(&b);
+    for (int i = 0; i < iters + 1 && !ret; ++i) {
+        hipError_t e = hipEventRecord(a, copy_);
+        if (e == hipSuccess) e = hipMemcpyAsync(arena_ + off, h, bytes, hipMemcpyHostToDevice, copy_);
+        if (e == hipSuccess) e = hipEventRecord(b, copy_);
+        if (e == hipSuccess) e = hipEventSynchronize(b);
+        float t = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&t, a, b);
+        if (e != hipSuccess) ret = (int)e;
+        if (i > 0) ms.push_back(t);  // first one warms the path
+    }
+    if (!ret) {
+        std::sort(ms.begin(), ms.end());
+        const double med = ms[ms.size() / 2];
+        *gbps = (double)bytes / (med * 1e-3) / 1e9;
+    }
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    (void)hipHostFree(h);
+    pool_.release(off);
+    return ret;
+}
+
+int Engine::time_op(int client, int op_index, int iters, double* mean_us) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (host_only()) return TP_ENODEV;
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (!mean_us || iters <= 0) return TP_EINVAL;
+    if (!m->resident || m->state != MS_READY) return TP_ESTATE;
+    if (active_ >= 0) return TP_EBUSY;
+    if (op_index < 0) op_index = (int)m->program.size() - 1;
+    if (op_index < 0 || op_index >= (int)m->program.size()) return TP_EINVAL;
+    const Op& op = m->program[op_index];
+    if (op.kind != OPK_GEMM && op.kind != OPK_CONV && op.kind != OPK_BN && op.kind != OPK_LAUNCH) return TP_EINVAL;
+    while (m->copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
+    HIPCHK(hipStreamSynchronize(copy_));
+    m->fully_loaded = true;
+    hipEvent_t a = nullptr, b = nullptr;
+    HIPCHK(hipEventCreate(&a));
+    HIPCHK(hipEventCreate(&b));
+    int ret = 0;
+    for (int i = 0; i < 3 && !ret; ++i) ret = exec_compute(*m, op, true);  // warm-up
+    if (!ret) {
+        (void)hipEventRecord(a, compute_);
+        for (int i = 0; i < iters && !ret; ++i) ret = exec_compute(*m, op, true);
+        (void)hipEventRecord(b, compute_);
+        hipError_t e = hipEventSynchronize(b);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, a, b);
+        if (e != hipSuccess && !ret) ret = (int)e;
+        *mean_us = (double)ms * 1000.0 / iters;
+    }
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    return ret;
+}
+
+}  // namespace tp

@@ -1,0 +1,235 @@
+// Engine: executor + memory manager + controller of one GPU.
+//
+// Reference counterparts (paths relative to the reference tree):
+//   Controller        include/server/controller.hpp      -> Engine::signal / complete_request
+//   CUDAExecutor      include/server/cuda_server.hpp     -> Engine op entry points / exec_op
+//   MemoryManager     include/server/memory_manager.hpp  -> translate / gate / swap engine
+//   ModelRepo         include/server/model_repo.hpp      -> Model (host weight store, tables)
+// The reference shares these objects between a controller thread, an executor
+// thread and a transfer thread through unsynchronised singletons; here all
+// engine state is owned by one mutex, and the copy thread only touches the
+// per-model atomics and the immutable chunk table of the job it was handed.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <deque>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/torpor_amd.h"
+#include "lru.hpp"
+#include "pool.hpp"
+
+namespace tp {
+
+constexpr uint64_t kTensorAlign = 256;
+constexpr uint64_t kVaTag = 0x7Aull << 56;
+constexpr uint64_t kVaTagMask = 0xFFull << 56;
+constexpr int kVaClientShift = 44;
+constexpr uint64_t kVaClientMask = 0xFFFull;
+constexpr uint64_t kVaActBit = 1ull << 43;
+constexpr uint64_t kVaOffMask = (1ull << 43) - 1;
+constexpr int kMaxClient = 4095;
+
+enum OpKind : int { OPK_GEMM = 1, OPK_CONV, OPK_BN, OPK_LAUNCH, OPK_H2D, OPK_D2H, OPK_D2D, OPK_MEMSET };
+
+// One recorded data-plane call, addresses still virtual.
+struct Op {
+    int kind = 0;
+    int op_id = 0;
+    int np = 0, ni = 0, nf = 0;
+    uint64_t p[12] = {0};
+    int64_t i[20] = {0};
+    float f[4] = {0};
+};
+
+struct Param {  // one uploaded weight tensor (model_repo.hpp:31-36 ModelParamInfo)
+    uint64_t voff = 0;       // offset in the function's weight address region
+    uint64_t size = 0;
+    uint64_t image_off = 0;  // offset in the weight image (host store and device copy alike)
+    int access_rank = -1;    // first-access position in the tracked run, -1 = never touched
+};
+struct WBlock {
+    uint64_t voff, size;
+};
+struct ABlock {  // activation allocation
+    uint64_t voff = 0, size = 0;
+    bool live = false;
+    uint64_t pool_off = UINT64_MAX;  // own extent while tracking, else inside the model's arena
+};
+
+enum ModelState : int { MS_LOADING = 0, MS_TRACKING = 1, MS_READY = 2 };
+enum CopyState : int { CS_IDLE = 0, CS_RUNNING = 1, CS_ISSUED = 2 };
+
+struct Model {
+    int id = -1;
+    int level = 1;
+    int state = MS_LOADING;
+    // weight address region and host store
+    uint64_t wbump = 0;
+    std::vector<WBlock> wblocks;
+    std::vector<Param> params;  // sorted by voff
+    std::vector<uint8_t> staging;
+    uint8_t* host_image = nullptr;
+    uint64_t image_bytes = 0, param_bytes = 0;
+    int next_rank = 0;
+    std::vector<uint64_t> chunk_end;
+    std::vector<hipEvent_t> chunk_ev;
+    // activation region
+    uint64_t abump = 0;
+    std::map<uint64_t, ABlock> ablocks;
+    std::multimap<uint64_t, uint64_t> afree;  // size -> voff
+    uint64_t act_bytes = 0;
+    bool act_frozen = false;
+    // residency
+    bool resident = false;
+    bool fully_loaded = false;
+    uint64_t w_pool_off = UINT64_MAX, a_pool_off = UINT64_MAX;
+    uint8_t* w_dev = nullptr;
+    uint8_t* a_dev = nullptr;
+    std::atomic<uint32_t> issued{0};
+    std::atomic<int> copy_state{CS_IDLE};
+    std::atomic<bool> cancel{false};
+    std::atomic<int> copy_error{0};
+    uint32_t gated_upto = 0;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    bool timing_valid = false;
+    // recorded program
+    std::vector<Op> program;
+    int async_error = 0;
+    tp_swap_stats stats{};
+
+    uint64_t total_bytes() const { return SlabPool::round_up(image_bytes) + SlabPool::round_up(act_bytes); }
+};
+
+struct PendingD2H {
+    void* dst;
+    uint64_t stage_off;
+    uint64_t bytes;
+};
+
+struct ReplayCtx {
+    const uint8_t* in = nullptr;
+    uint64_t in_bytes = 0, in_pos = 0;
+    uint8_t* out = nullptr;
+    uint64_t out_bytes = 0, out_pos = 0;
+};
+
+class Engine {
+public:
+    explicit Engine(const tp_config& cfg);
+    ~Engine();
+    int init();
+
+    int signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred);
+    int take_deferred_ack(int* ack, int* resp);
+    int poll();
+
+    int op_malloc(int client, uint64_t bytes, uint64_t* va);
+    int op_free(int client, uint64_t va);
+    int op_h2d(int client, uint64_t dst, const void* src, uint64_t bytes);
+    int op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes);
+    int op_d2h(int client, void* dst, uint64_t src, uint64_t bytes);
+    int op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes);
+    int op_memset(int client, uint64_t dst, int value, uint64_t bytes);
+    int op_device_sync(int client);
+    int op_stream_sync(int client);
+    int op_compute(int client, const Op& op);  // GEMM / CONV / BN / LAUNCH
+    int replay(int client, const void* in, uint64_t in_bytes, void* out, uint64_t out_bytes);
+
+    int model_resident(int client);
+    int model_info(int client, tp_model_info* out);
+    int pool_stats(tp_pool_stats* out);
+    int swap_stats(int client, tp_swap_stats* out);
+    int readback_weights(int client, void* dst, uint64_t bytes);
+    int host_weights(int client, const void** ptr, uint64_t* bytes);
+    int weight_offset(int client, uint64_t va, uint64_t* off);
+    int measure_h2d(uint64_t bytes, int iters, double* gbps);
+    int time_op(int client, int op_index, int iters, double* mean_us);
+
+private:
+    enum Mode : int { MODE_NONE = 0, MODE_LOAD = 1, MODE_TRACK = 2, MODE_EXEC = 3 };
+    // controller.hpp:17-23
+    enum ExecStatus : int { ES_AVAIL = -1, ES_LOCAL = 0, ES_PCIE_LIGHT = 2, ES_PCIE_MEDIAN = 3, ES_PCIE_HEAVY = 4, ES_COLD = 5 };
+    struct Queued {
+        int id;
+        bool cold;
+        int level;
+    };
+    struct Xlat {
+        uint8_t* p = nullptr;
+        bool weight = false;
+        uint64_t image_end = 0;
+        Param* param = nullptr;
+    };
+
+    bool host_only() const { return (cfg_.flags & TP_FLAG_HOST_ONLY) != 0; }
+    Model* find(int id);
+    Model* active_model(int client, int* err);
+    int translate(Model& m, uint64_t va, uint64_t span, Xlat* out);
+    int gate(Model& m, const Xlat& x);
+    int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out);
+    int exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch);
+    int exec_compute(Model& m, const Op& op, bool launch);
+    int do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes);
+    int do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes);
+    int do_stream_sync(Model* m);
+
+    void start_cold(int id, int level);
+    int start_execute(int id);
+    int swap_in(Model& m);
+    void evict_model(Model& m);
+    bool check_eviction(Model& m);
+    void complete_request();
+    int finish_loading(Model& m);
+    int finish_tracking(Model& m);
+    int build_image(Model& m, bool by_access);
+    void build_chunks(Model& m);
+    void wait_copy_idle(Model& m);
+    void copy_main();
+    int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
+    void* host_alloc(uint64_t bytes);
+    void host_free(void* p);
+    bool poll_timeout_locked();
+
+    tp_config cfg_;
+    std::mutex mu_;
+    SlabPool pool_;
+    LruEvictor lru_;
+    uint8_t* arena_ = nullptr;
+    float* workspace_ = nullptr;
+    hipStream_t compute_ = nullptr, copy_ = nullptr;
+    std::unordered_map<int, std::unique_ptr<Model>> models_;
+
+    int active_ = -1;
+    int mode_ = MODE_NONE;
+    int exec_status_ = ES_AVAIL;
+    std::chrono::steady_clock::time_point req_start_;
+    std::deque<Queued> req_queue_;
+    std::deque<std::pair<int, int>> deferred_acks_;
+    bool d2h_seen_ = false;
+
+    uint8_t* h2d_stage_ = nullptr;
+    uint64_t h2d_cap_ = 0, h2d_pos_ = 0;
+    uint8_t* d2h_stage_ = nullptr;
+    uint64_t d2h_cap_ = 0, d2h_pos_ = 0;
+    std::vector<PendingD2H> pending_d2h_;
+
+    uint64_t evictions_ = 0, swap_ins_ = 0;
+
+    std::thread copy_thread_;
+    std::mutex cmu_;
+    std::condition_variable ccv_;
+    std::deque<Model*> jobs_;
+    bool stop_ = false;
+};
+
+}  // namespace tp

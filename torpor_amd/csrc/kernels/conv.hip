@@ -1,0 +1,340 @@
+// Implicit-GEMM fp32 convolution on MFMA for gfx950.
+//
+// Replaces the cudnnConvolutionForward call site of the reference executor
+// (include/server/cuda_server.hpp:708-735): y = alpha*conv2d(x, w) + beta*y,
+// fp32, groups = 1, weights in the framework's native [Cout][Cin][KH][KW]
+// order (the swapped-in bytes are used as they are; nothing is re-laid-out).
+// The GEMM view is rows = output pixels (n, ho, wo), cols = Cout,
+// K = Cin*KH*KW; the fused epilogue adds bias / inference batch-norm /
+// residual / activation.
+//
+//   1x1, NHWC, Cin%4==0, pad 0      -> the dense GEMM kernel with a row gather
+//   3x3, NHWC, Cin%8==0             -> conv3x3_fast_kernel (K-block = 8 channels x 9 taps)
+//   everything else (7x7 stem, NCHW) -> conv_generic_kernel (scalar gathers)
+#include "kernels.hpp"
+#include "mfma_tile.hpp"
+
+namespace tpk {
+
+void set_last_kernel(const char* n);
+int num_cu();
+Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
+int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, const Epilogue& e, hipStream_t s);
+int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, long* kper_out);
+
+struct ConvDev {
+    const float* x;
+    const float* w;
+    float* y;
+    int N, H, W, Cin, Cout, KH, KW, Ho, Wo, sh, sw, ph, pw;
+    long xs_n, xs_h, xs_w, xs_c;
+    long M;     // N*Ho*Wo
+    long K;     // Cin*KH*KW
+    int splits;
+    long kper;  // K (generic) or channels (3x3 fast) per split
+    float* ws;
+    int tiles_m, tiles_n;
+    Epilogue ep;
+};
+
+__device__ __forceinline__ int remap_xcd_c(int bid, int n) {
+    const int q = n >> 3, rem = n & 7;
+    const int xcd = bid & 7, local = bid >> 3;
+    return xcd * q + (xcd < rem ? xcd : rem) + local;
+}
+
+// K-block = 8 input channels x 9 taps, ordered k_local = tap*8 + c in LDS.
+// Activation side: for (pixel, tap) the 8 channels are 32 contiguous bytes of
+// the NHWC input (two dwordx4 loads by two neighbouring threads).  Weight side:
+// for one output channel the 8x9 block is 72 contiguous floats of the
+// [Cout][Cin][3][3] tensor; each thread loads 36 of them (4 channels x 9 taps)
+// with dwordx4 and transposes in registers to the tap-major LDS order.
+template <class C>
+__global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvDev p) {
+    static_assert(C::BK == 72, "3x3 fast path uses K-blocks of 72");
+    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
+    float* As = lds;
+    float* Bs = lds + C::BM * C::LDK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int t = remap_xcd_c(blockIdx.x, p.tiles_m * p.tiles_n);
+    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
+    const int split = blockIdx.z;
+    const int cbeg = split * (int)p.kper;
+    const int cend = (cbeg + (int)p.kper < p.Cin) ? cbeg + (int)p.kper : p.Cin;
+
+    constexpr int NVA = (C::BM * 18 + C::THREADS - 1) / C::THREADS;
+    long offA[NVA];
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) {
+        const int idx = i * C::THREADS + tid;
+        const int row = idx / 18, t2 = idx - row * 18;
+        const int tap = t2 >> 1, cq = t2 & 1;
+        offA[i] = -1;
+        const long grow = m0 + row;
+        if (idx < C::BM * 18 && grow < p.M) {
+            const int wo = (int)(grow % p.Wo);
+            const long tt = grow / p.Wo;
+            const int ho = (int)(tt % p.Ho);
+            const long n = tt / p.Ho;
+            const int hi = ho * p.sh - p.ph + tap / 3;
+            const int wi = wo * p.sw - p.pw + tap % 3;
+            if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W)
+                offA[i] = n * p.xs_n + (long)hi * p.xs_h + (long)wi * p.xs_w + cq * 4;
+        }
+    }
+    // weight assignment: thread -> (col = tid/2, cq = tid%2)
+    const int wcol = tid >> 1, wcq = tid & 1;
+    const bool wact = (tid < C::BN * 2) && (n0 + wcol < p.Cout);
+    const float* __restrict__ wbase = p.w + ((n0 + wcol) * (long)p.Cin + wcq * 4) * 9;
+
+    f32x16 acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    f32x4 ra[NVA];
+    f32x4 rw[9];
+
+    auto load_regs = [&](int c0) {
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (offA[i] >= 0) v = *reinterpret_cast<const f32x4*>(p.x + offA[i] + c0);
+            ra[i] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < 9; ++j) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (wact) v = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * 9 + j * 4);
+            rw[j] = v;
+        }
+    };
+    auto store_lds = [&]() {
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) {
+            const int idx = i * C::THREADS + tid;
+            const int row = idx / 18, t2 = idx - row * 18;
+            if (idx < C::BM * 18) *reinterpret_cast<f32x4*>(As + row * C::LDK + t2 * 4) = ra[i];
+        }
+        if (tid < C::BN * 2) {
+            // rw holds w[c][tap] for c = 0..3 (this thread's channel quad), flat index c*9 + tap
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+                f32x4 v;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int f = c * 9 + tap;
+                    v[c] = rw[f >> 2][f & 3];
+                }
+                *reinterpret_cast<f32x4*>(Bs + wcol * C::LDK + tap * 8 + wcq * 4) = v;
+            }
+        }
+    };
+
+    load_regs(cbeg);
+    for (int c0 = cbeg; c0 < cend; c0 += 8) {
+        store_lds();
+        __syncthreads();
+        if (c0 + 8 < cend) load_regs(c0 + 8);
+        mma_block<C>(As, Bs, acc, wm, wn, lane);
+        __syncthreads();
+    }
+    float* partial = nullptr;
+    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial);
+}
+
+// Any kernel size / stride / padding / input layout; K ordered (c, kh, kw) as
+// the weights are stored.  One wavefront gathers one k for 64 pixels at a time,
+// so the k -> (c, kh, kw) decode is wavefront-uniform.
+using ConvGenCfg = TileCfg<64, 64, 16, 2, 2>;
+
+__global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(const ConvDev p) {
+    using C = ConvGenCfg;
+    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
+    float* As = lds;
+    float* Bs = lds + C::BM * C::LDK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int t = blockIdx.x;
+    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
+    const int split = blockIdx.z;
+    const long kbeg = (long)split * p.kper;
+    const long kend = (kbeg + p.kper < p.K) ? kbeg + p.kper : p.K;
+
+    // activation gather: thread -> pixel row (tid % 64), k slots wave + 4*i
+    const int arow = tid & 63;
+    const long grow = m0 + arow;
+    const bool rvalid = grow < p.M;
+    int hi0 = 0, wi0 = 0;
+    long nbase = 0;
+    if (rvalid) {
+        const int wo = (int)(grow % p.Wo);
+        const long tt = grow / p.Wo;
+        const int ho = (int)(tt % p.Ho);
+        const long n = tt / p.Ho;
+        hi0 = ho * p.sh - p.ph;
+        wi0 = wo * p.sw - p.pw;
+        nbase = n * p.xs_n;
+    }
+    // weight loads: thread -> (k = tid % 16, col = tid/16 + 16*i)
+    const int wk = tid & 15, wc0 = tid >> 4;
+    const int khw = p.KH * p.KW;
+
+    f32x16 acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    float ra[4], rb[4];
+    auto load_regs = [&](long k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const long k = k0 + wave + 4 * i;
+            float v = 0.f;
+            if (rvalid && k < kend) {
+                const int c = (int)(k / khw);
+                const int rr = (int)(k - (long)c * khw);
+                const int kh = rr / p.KW, kw = rr - kh * p.KW;
+                const int hi = hi0 + kh, wi = wi0 + kw;
+                if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W)
+                    v = p.x[nbase + (long)c * p.xs_c + (long)hi * p.xs_h + (long)wi * p.xs_w];
+            }
+            ra[i] = v;
+            const long col = n0 + wc0 + 16 * i;
+            const long kk = k0 + wk;
+            rb[i] = (col < p.Cout && kk < kend) ? p.w[col * p.K + kk] : 0.f;
+        }
+    };
+    load_regs(kbeg);
+    for (long k0 = kbeg; k0 < kend; k0 += C::BK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            As[arow * C::LDK + wave + 4 * i] = ra[i];
+            Bs[(wc0 + 16 * i) * C::LDK + wk] = rb[i];
+        }
+        __syncthreads();
+        if (k0 + C::BK < kend) load_regs(k0 + C::BK);
+        mma_block<C>(As, Bs, acc, wm, wn, lane);
+        __syncthreads();
+    }
+    float* partial = nullptr;
+    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial);
+}
+
+using Conv3L = TileCfg<128, 128, 72, 2, 2>;
+using Conv3M = TileCfg<64, 64, 72, 2, 2>;
+
+static inline bool aligned16c(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
+    if (!a.x || !a.w || !a.y) return K_EINVAL;
+    if (a.N <= 0 || a.H <= 0 || a.W <= 0 || a.Cin <= 0 || a.Cout <= 0 || a.KH <= 0 || a.KW <= 0) return K_EINVAL;
+    if (a.sh <= 0 || a.sw <= 0 || a.ph < 0 || a.pw < 0) return K_EINVAL;
+    const int Ho = (a.H + 2 * a.ph - a.KH) / a.sh + 1;
+    const int Wo = (a.W + 2 * a.pw - a.KW) / a.sw + 1;
+    if (Ho <= 0 || Wo <= 0) return K_EINVAL;
+    const long M = (long)a.N * Ho * Wo;
+
+    // 1x1 over NHWC is a dense GEMM, with a row gather when strided.
+    if (a.KH == 1 && a.KW == 1 && a.ph == 0 && a.pw == 0 && a.x_nhwc && a.y_nhwc) {
+        GemmArgs g;
+        g.X = a.x;
+        g.Y = a.w;
+        g.C = a.y;
+        g.M = M;
+        g.N = a.Cout;
+        g.K = a.Cin;
+        g.xs_r = a.Cin;
+        g.xs_k = 1;
+        g.ys_c = a.Cin;
+        g.ys_k = 1;
+        g.ldc = a.Cout;
+        if (a.sh != 1 || a.sw != 1) {
+            g.gather = 1;
+            g.Ho = Ho;
+            g.Wo = Wo;
+            g.H = a.H;
+            g.W = a.W;
+            g.sh = a.sh;
+            g.sw = a.sw;
+        }
+        g.ep = a.ep;
+        if (g.ep.residual && g.ep.ldr == 0) g.ep.ldr = a.Cout;
+        return launch_gemm(g, ws, s);
+    }
+
+    ConvDev p;
+    p.x = a.x;
+    p.w = a.w;
+    p.y = a.y;
+    p.N = a.N;
+    p.H = a.H;
+    p.W = a.W;
+    p.Cin = a.Cin;
+    p.Cout = a.Cout;
+    p.KH = a.KH;
+    p.KW = a.KW;
+    p.Ho = Ho;
+    p.Wo = Wo;
+    p.sh = a.sh;
+    p.sw = a.sw;
+    p.ph = a.ph;
+    p.pw = a.pw;
+    if (a.x_nhwc) {
+        p.xs_c = 1;
+        p.xs_w = a.Cin;
+        p.xs_h = (long)a.W * a.Cin;
+        p.xs_n = (long)a.H * a.W * a.Cin;
+    } else {
+        p.xs_w = 1;
+        p.xs_h = a.W;
+        p.xs_c = (long)a.H * a.W;
+        p.xs_n = (long)a.Cin * a.H * a.W;
+    }
+    p.M = M;
+    p.K = (long)a.Cin * a.KH * a.KW;
+    p.ws = ws.ptr;
+    EpilogueArgs ea = a.ep;
+    if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;
+    p.ep = make_epilogue(ea, a.Cout);
+    if (!a.y_nhwc) {
+        p.ep.out_nchw = 1;
+        p.ep.howo = (long)Ho * Wo;
+        p.ep.ncols = a.Cout;
+    }
+
+    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && aligned16c(a.x) && aligned16c(a.w);
+    if (fast3) {
+        const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);
+        const bool big = tl >= 2L * num_cu();
+        const int bm = big ? 128 : 64;
+        p.tiles_m = (int)((M + bm - 1) / bm);
+        p.tiles_n = (a.Cout + bm - 1) / bm;
+        const long tiles = (long)p.tiles_m * p.tiles_n;
+        // split over channel blocks of 8 (one K-block each)
+        long kper_k = 0;
+        p.splits = choose_splits(tiles, p.K, 72, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
+        p.kper = kper_k / 9;  // channels per split (multiple of 8)
+        dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
+        if (big) {
+            hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3L>), grid, dim3(256), 0, s, p);
+            set_last_kernel("conv3x3_fast_128x128");
+        } else {
+            hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3M>), grid, dim3(256), 0, s, p);
+            set_last_kernel("conv3x3_fast_64x64");
+        }
+    } else {
+        p.tiles_m = (int)((M + 63) / 64);
+        p.tiles_n = (a.Cout + 63) / 64;
+        const long tiles = (long)p.tiles_m * p.tiles_n;
+        p.splits = choose_splits(tiles, p.K, 16, M, a.Cout, ws.ptr ? ws.bytes : 0, &p.kper);
+        dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
+        hipLaunchKernelGGL(conv_generic_kernel, grid, dim3(256), 0, s, p);
+        set_last_kernel("conv_generic_64x64");
+    }
+    int err = (int)hipGetLastError();
+    if (err) return err;
+    if (p.splits > 1) return launch_splitk_reduce(ws.ptr, p.splits, M, a.Cout, a.y, p.ep, s);
+    return 0;
+}
+
+}  // namespace tpk

@@ -1,0 +1,89 @@
+// Host-side launch interface of the hand-written gfx950 kernels.  Every
+// launcher validates shapes on the host, enqueues on the given stream and
+// returns a hipError_t-compatible int (0 = ok) or a negative TP_E* code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace tpk {
+
+enum : int { K_OK = 0, K_EINVAL = -22, K_EUNSUPPORTED = -38 };
+
+struct EpilogueArgs {
+    float alpha = 1.f;
+    float beta = 0.f;
+    const float* bias = nullptr;
+    const float* bn_scale = nullptr;
+    const float* bn_bias = nullptr;
+    const float* bn_mean = nullptr;
+    const float* bn_var = nullptr;
+    float bn_eps = 1e-5f;
+    const float* residual = nullptr;
+    long ldr = 0;
+    int act = 0;
+};
+
+// C[r][c] (row pitch ldc) = epilogue( sum_k X(r,k) * Y(c,k) ), X(r,k) at
+// X[r*xs_r + k*xs_k], Y(c,k) at Y[c*ys_c + k*ys_k].  Two-level batching:
+// batch z = b0*nb1 + b1 adds b0*?b0 + b1*?b1 to each base pointer.
+struct GemmArgs {
+    const float* X = nullptr;
+    const float* Y = nullptr;
+    float* C = nullptr;
+    long M = 0, N = 0, K = 0;
+    long xs_r = 0, xs_k = 1, ys_c = 0, ys_k = 1, ldc = 0;
+    int nb0 = 1, nb1 = 1;
+    long xb0 = 0, xb1 = 0, yb0 = 0, yb1 = 0, cb0 = 0, cb1 = 0;
+    // optional row gather (1x1 strided convolution over NHWC): row m =
+    // (n*Ho + ho)*Wo + wo reads X row ((n*H + ho*sh)*W + wo*sw).
+    int gather = 0, Ho = 0, Wo = 0, H = 0, W = 0, sh = 1, sw = 1;
+    EpilogueArgs ep;
+};
+
+struct ConvArgs {
+    const float* x = nullptr;
+    const float* w = nullptr;  // [Cout][Cin][KH][KW]
+    float* y = nullptr;
+    int N = 0, H = 0, W = 0, Cin = 0, Cout = 0, KH = 0, KW = 0;
+    int sh = 1, sw = 1, ph = 0, pw = 0;
+    int x_nhwc = 1, y_nhwc = 1;  // 0 = NCHW
+    EpilogueArgs ep;             // residual shares the layout of y
+};
+
+struct Workspace {
+    float* ptr = nullptr;  // split-K partial sums
+    size_t bytes = 0;
+};
+
+void kernels_init(int device);  // caches CU count
+int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s);
+int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s);
+// introspection for tests/bench: which path the last launch on this thread took
+const char* last_kernel_name();
+
+// ---- HBM-bound operators (elementwise.hip / reduce.hip) ----
+int launch_bn_inference(const float* x, float* y, const float* g, const float* b, const float* mean,
+                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, hipStream_t s);
+int launch_relu(const float* x, float* y, long n, hipStream_t s);
+int launch_add(const float* a, const float* b, float* y, long n, int relu, hipStream_t s);
+int launch_bias_act(const float* x, const float* bias, float* y, long rows, int C, int act, hipStream_t s);
+int launch_gelu(const float* x, float* y, long n, hipStream_t s);
+int launch_nchw_to_nhwc(const float* x, float* y, int N, int C, int H, int W, hipStream_t s);
+int launch_nhwc_to_nchw(const float* x, float* y, int N, int C, int H, int W, hipStream_t s);
+int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, int nhwc,
+                     hipStream_t s);
+int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, hipStream_t s);
+int launch_layernorm(const float* x, const float* residual, const float* gamma, const float* beta, float* y,
+                     long rows, int width, float eps, hipStream_t s);
+// y[row] = softmax(scale * x[row] + mask[(row / rows_per_mask) * width ...]) over `width`
+int launch_softmax(const float* x, const float* mask, float* y, long rows, int width, float scale,
+                   long rows_per_mask, hipStream_t s);
+int launch_embedding(const int64_t* ids, const int64_t* type_ids, const float* word, const float* pos,
+                     const float* type, float* y, long tokens, int seq, int width, long vocab, int n_types,
+                     hipStream_t s);
+int launch_sum(const float* x, float* y, long n, hipStream_t s);  // y[0] = sum(x), two-pass deterministic
+int launch_fill(float* y, float v, long n, hipStream_t s);
+int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t s);
+
+}  // namespace tpk

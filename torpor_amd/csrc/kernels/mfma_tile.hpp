@@ -1,0 +1,162 @@
+// fp32 MFMA block-tile machinery shared by the dense GEMM and implicit-GEMM
+// convolution kernels (gfx950 / CDNA4, 64-wide wavefronts).
+//
+// A workgroup is 256 threads = 4 wavefronts laid out WGM x WGN over a BM x BN
+// output tile.  Each wavefront owns TM x TN accumulators of 32x32, fed by
+// v_mfma_f32_32x32x2_f32.  Both operand tiles live in LDS as [row][k] with a
+// padded row pitch so that one ds_read_b128 per lane fetches four consecutive
+// k values of that lane's row; lane half h (lane/32) takes k = 8g+4h .. 8g+4h+3
+// of every group of eight, and MFMA step s multiplies k = 8g+s (half 0) with
+// k = 8g+4+s (half 1).  The sum over k is order-free, so A and B only have to
+// agree on this permutation, which they do because both use the same lane math.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tpk {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_TANH = 3 };
+
+// out = act( bn( alpha*acc + beta*C_old + bias[n] ) + residual )
+struct Epilogue {
+    float alpha;
+    float beta;
+    const float* bias;      // [N] or nullptr
+    const float* bn_scale;  // gamma[N] or nullptr (all four bn_* set together)
+    const float* bn_bias;   // beta[N]
+    const float* bn_mean;   // running mean[N]
+    const float* bn_var;    // running var[N]
+    float bn_eps;
+    const float* residual;  // [M][ldr] or nullptr (same mapping as C when out_nchw)
+    long ldr;
+    int act;
+    // output mapping: element (row, col) lives at row*ldc + col, or, for an
+    // NCHW convolution output with row = n*howo + p, at (n*ncols + col)*howo + p.
+    long ldc;
+    int out_nchw;
+    long howo;
+    long ncols;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    if (act == ACT_RELU) return v > 0.f ? v : 0.f;
+    if (act == ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    if (act == ACT_TANH) return tanhf(v);
+    return v;
+}
+
+__device__ __forceinline__ long out_index(const Epilogue& e, long row, long col, long pitch) {
+    if (e.out_nchw) {
+        const long n = row / e.howo;
+        const long p = row - n * e.howo;
+        return (n * e.ncols + col) * e.howo + p;
+    }
+    return row * pitch + col;
+}
+
+// Full epilogue for one element given its folded column constants.
+__device__ __forceinline__ void epilogue_store(const Epilogue& e, float* __restrict__ Cout, long row, long col,
+                                               float x, float cs, float ct) {
+    const long ci = out_index(e, row, col, e.ldc);
+    x *= e.alpha;
+    if (e.beta != 0.f) x += e.beta * Cout[ci];
+    x = x * cs + ct;
+    if (e.residual) x += e.residual[out_index(e, row, col, e.ldr)];
+    Cout[ci] = apply_act(x, e.act);
+}
+
+// Per-column constants of the epilogue folded to v*cs + ct.
+__device__ __forceinline__ void epilogue_column(const Epilogue& e, long col, float& cs, float& ct) {
+    float b = e.bias ? e.bias[col] : 0.f;
+    cs = 1.f;
+    ct = b;
+    if (e.bn_scale) {
+        float inv = 1.0f / sqrtf(e.bn_var[col] + e.bn_eps);
+        float g = e.bn_scale[col] * inv;
+        cs = g;
+        ct = (b - e.bn_mean[col]) * g + e.bn_bias[col];
+    }
+}
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+    static constexpr int THREADS = 64 * WGM * WGN;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // per-wavefront tile
+    static constexpr int TM = WTM / 32, TN = WTN / 32;    // 32x32 MFMA tiles per wavefront
+    static constexpr int LDK = BK + 4;                    // LDS row pitch in floats
+    static constexpr int LDS_FLOATS = (BM + BN) * LDK;
+    static_assert(BK % 8 == 0, "BK must be a multiple of 8");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be 32-aligned");
+};
+
+template <class C>
+__device__ __forceinline__ void zero_acc(f32x16 (&acc)[C::TM][C::TN]) {
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+}
+
+// Multiply the LDS-resident BM x BK and BN x BK tiles into the accumulators.
+template <class C>
+__device__ __forceinline__ void mma_block(const float* __restrict__ As, const float* __restrict__ Bs,
+                                          f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane) {
+    const int r = lane & 31;
+    const int h = lane >> 5;
+    const float* ap = As + (wm * C::WTM + r) * C::LDK + 4 * h;
+    const float* bp = Bs + (wn * C::WTN + r) * C::LDK + 4 * h;
+#pragma unroll
+    for (int kk = 0; kk < C::BK; kk += 8) {
+        f32x4 a[C::TM], b[C::TN];
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) a[i] = *reinterpret_cast<const f32x4*>(ap + i * 32 * C::LDK + kk);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) b[j] = *reinterpret_cast<const f32x4*>(bp + j * 32 * C::LDK + kk);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+    }
+}
+
+// Write the accumulators.  `partial` != nullptr: raw sums go to the split-K
+// workspace slice [M][N]; otherwise the epilogue is applied and C is written.
+template <class C>
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
+                                           long M, long N, float* __restrict__ Cout, const Epilogue& e,
+                                           float* __restrict__ partial) {
+    const int r = lane & 31;
+    const int h = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+        const long col = n0 + wn * C::WTN + j * 32 + r;
+        if (col >= N) continue;
+        float cs = 1.f, ct = 0.f;
+        if (!partial) epilogue_column(e, col, cs, ct);
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const long row = m0 + wm * C::WTM + i * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                if (row >= M) continue;
+                float x = acc[i][j][v];
+                if (partial) {
+                    partial[row * N + col] = x;
+                } else {
+                    epilogue_store(e, Cout, row, col, x, cs, ct);
+                }
+            }
+        }
+    }
+}
+
+}  // namespace tpk

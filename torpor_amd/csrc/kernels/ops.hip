@@ -1,0 +1,503 @@
+// HBM-bound operators for gfx950: the kernels the reference runs through
+// cudnnBatchNormalizationForwardInference (include/server/cuda_server.hpp:737-771)
+// and through generic cudaLaunchKernel of libtorch kernels
+// (include/server/cuda_server.hpp:1226-1310): ReLU, residual add, bias add,
+// GELU, max/avg pooling, LayerNorm, softmax, embedding gather, sum.
+//
+// Elementwise kernels move dwordx4 per lane with grid-stride loops; row
+// reductions (LayerNorm, softmax) use one 64-lane wavefront per row and
+// cross-lane shuffles, so a row never touches LDS.
+#include "kernels.hpp"
+#include "mfma_tile.hpp"
+
+namespace tpk {
+
+int num_cu();
+
+static inline int grid_for(long work_items, int block) {
+    long b = (work_items + block - 1) / block;
+    long cap = (long)num_cu() * 16;
+    if (b > cap) b = cap;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+static inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// ---------------------------------------------------------------- batch norm
+// nhwc: channel = i % C ; nchw: channel = (i / hw) % C
+__global__ __launch_bounds__(256) void bn_nhwc_vec_kernel(const f32x4* __restrict__ x, f32x4* __restrict__ y,
+                                                          const float* __restrict__ g, const float* __restrict__ b,
+                                                          const float* __restrict__ mean,
+                                                          const float* __restrict__ var, float eps, long nvec, int C4,
+                                                          int relu) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (long)gridDim.x * blockDim.x) {
+        const int c = (int)(i % C4) * 4;
+        f32x4 v = x[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float sc = g[c + j] * (1.0f / sqrtf(var[c + j] + eps));
+            float o = (v[j] - mean[c + j]) * sc + b[c + j];
+            if (relu) o = o > 0.f ? o : 0.f;
+            v[j] = o;
+        }
+        y[i] = v;
+    }
+}
+__global__ __launch_bounds__(256) void bn_scalar_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                        const float* __restrict__ g, const float* __restrict__ b,
+                                                        const float* __restrict__ mean, const float* __restrict__ var,
+                                                        float eps, long n, int C, long hw, int nhwc, int relu) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int c = nhwc ? (int)(i % C) : (int)((i / hw) % C);
+        const float sc = g[c] * (1.0f / sqrtf(var[c] + eps));
+        float o = (x[i] - mean[c]) * sc + b[c];
+        if (relu) o = o > 0.f ? o : 0.f;
+        y[i] = o;
+    }
+}
+int launch_bn_inference(const float* x, float* y, const float* g, const float* b, const float* mean,
+                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, hipStream_t s) {
+    if (!x || !y || !g || !b || !mean || !var || rows < 0 || C <= 0) return K_EINVAL;
+    const long n = rows * C;  // rows = N*H*W
+    if (n == 0) return 0;
+    if (nhwc && C % 4 == 0 && al16(x) && al16(y)) {
+        hipLaunchKernelGGL(bn_nhwc_vec_kernel, dim3(grid_for(n / 4, 256)), dim3(256), 0, s,
+                           reinterpret_cast<const f32x4*>(x), reinterpret_cast<f32x4*>(y), g, b, mean, var, eps,
+                           n / 4, C / 4, relu);
+    } else {
+        hipLaunchKernelGGL(bn_scalar_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, x, y, g, b, mean, var, eps, n,
+                           C, hw, nhwc, relu);
+    }
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- elementwise
+// mode 0: relu(a); 1: a+b; 2: relu(a+b); 3: gelu(a)
+__global__ __launch_bounds__(256) void ew_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                 float* __restrict__ y, long n, int mode, int vec) {
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, stride = (long)gridDim.x * blockDim.x;
+    if (vec) {
+        const long nv = n >> 2;
+        const f32x4* a4 = reinterpret_cast<const f32x4*>(a);
+        const f32x4* b4 = reinterpret_cast<const f32x4*>(b);
+        f32x4* y4 = reinterpret_cast<f32x4*>(y);
+        for (long i = tid; i < nv; i += stride) {
+            f32x4 v = a4[i];
+            if (mode == 1 || mode == 2) {
+                const f32x4 w = b4[i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] += w[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (mode == 0 || mode == 2) v[j] = v[j] > 0.f ? v[j] : 0.f;
+                if (mode == 3) v[j] = apply_act(v[j], ACT_GELU);
+            }
+            y4[i] = v;
+        }
+        for (long i = (nv << 2) + tid; i < n; i += stride) {
+            float v = a[i];
+            if (mode == 1 || mode == 2) v += b[i];
+            if (mode == 0 || mode == 2) v = v > 0.f ? v : 0.f;
+            if (mode == 3) v = apply_act(v, ACT_GELU);
+            y[i] = v;
+        }
+    } else {
+        for (long i = tid; i < n; i += stride) {
+            float v = a[i];
+            if (mode == 1 || mode == 2) v += b[i];
+            if (mode == 0 || mode == 2) v = v > 0.f ? v : 0.f;
+            if (mode == 3) v = apply_act(v, ACT_GELU);
+            y[i] = v;
+        }
+    }
+}
+static int launch_ew(const float* a, const float* b, float* y, long n, int mode, hipStream_t s) {
+    if (!a || !y || n < 0 || ((mode == 1 || mode == 2) && !b)) return K_EINVAL;
+    if (n == 0) return 0;
+    const int vec = al16(a) && al16(y) && (!b || al16(b));
+    hipLaunchKernelGGL(ew_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n, 256)), dim3(256), 0, s, a, b ? b : a, y, n,
+                       mode, vec);
+    return (int)hipGetLastError();
+}
+int launch_relu(const float* x, float* y, long n, hipStream_t s) { return launch_ew(x, nullptr, y, n, 0, s); }
+int launch_add(const float* a, const float* b, float* y, long n, int relu, hipStream_t s) {
+    return launch_ew(a, b, y, n, relu ? 2 : 1, s);
+}
+int launch_gelu(const float* x, float* y, long n, hipStream_t s) { return launch_ew(x, nullptr, y, n, 3, s); }
+
+__global__ __launch_bounds__(256) void bias_act_kernel(const float* __restrict__ x, const float* __restrict__ bias,
+                                                       float* __restrict__ y, long n, int C, int act) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        y[i] = apply_act(x[i] + bias[i % C], act);
+}
+int launch_bias_act(const float* x, const float* bias, float* y, long rows, int C, int act, hipStream_t s) {
+    if (!x || !bias || !y || rows < 0 || C <= 0) return K_EINVAL;
+    const long n = rows * C;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(bias_act_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, x, bias, y, n, C, act);
+    return (int)hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(float* __restrict__ y, float v, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) y[i] = v;
+}
+int launch_fill(float* y, float v, long n, hipStream_t s) {
+    if (!y || n < 0) return K_EINVAL;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, y, v, n);
+    return (int)hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                   size_t bytes, int vec) {
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    if (vec) {
+        const size_t nv = bytes >> 4;
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(src);
+        f32x4* d4 = reinterpret_cast<f32x4*>(dst);
+        for (size_t i = tid; i < nv; i += stride) d4[i] = s4[i];
+        for (size_t i = (nv << 4) + tid; i < bytes; i += stride) dst[i] = src[i];
+    } else {
+        for (size_t i = tid; i < bytes; i += stride) dst[i] = src[i];
+    }
+}
+int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t s) {
+    if (!src || !dst) return K_EINVAL;
+    if (bytes == 0) return 0;
+    const int vec = al16(src) && al16(dst);
+    hipLaunchKernelGGL(copy_kernel, dim3(grid_for((long)(vec ? (bytes + 15) / 16 : bytes), 256)), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), bytes, vec);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- layout
+// NCHW -> NHWC through a 32x33 LDS tile over (C, HW) per image.
+__global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ x, float* __restrict__ y, int R,
+                                                        int Ccols) {
+    // x: [batch][R][Ccols] -> y: [batch][Ccols][R]
+    __shared__ float tile[32][33];
+    const long base = (long)blockIdx.z * R * Ccols;
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int j = ty; j < 32; j += 8) {
+        const int r = r0 + j, c = c0 + tx;
+        tile[j][tx] = (r < R && c < Ccols) ? x[base + (long)r * Ccols + c] : 0.f;
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        const int c = c0 + j, r = r0 + tx;
+        if (r < R && c < Ccols) y[base + (long)c * R + r] = tile[tx][j];
+    }
+}
+static int launch_transpose(const float* x, float* y, int batch, int R, int Ccols, hipStream_t s) {
+    if (!x || !y || batch <= 0 || R <= 0 || Ccols <= 0) return K_EINVAL;
+    dim3 grid((Ccols + 31) / 32, (R + 31) / 32, batch);
+    if (grid.y > 65535 || grid.z > 65535) return K_EUNSUPPORTED;
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, s, x, y, R, Ccols);
+    return (int)hipGetLastError();
+}
+int launch_nchw_to_nhwc(const float* x, float* y, int N, int C, int H, int W, hipStream_t s) {
+    return launch_transpose(x, y, N, C, H * W, s);
+}
+int launch_nhwc_to_nchw(const float* x, float* y, int N, int C, int H, int W, hipStream_t s) {
+    return launch_transpose(x, y, N, H * W, C, s);
+}
+
+// ---------------------------------------------------------------- pooling
+__global__ __launch_bounds__(256) void maxpool_kernel(const float* __restrict__ x, float* __restrict__ y, int N, int H,
+                                                      int W, int C, int Ho, int Wo, int k, int stride, int pad,
+                                                      int nhwc) {
+    const long total = (long)N * Ho * Wo * C;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        int c, wo, ho;
+        long n;
+        if (nhwc) {
+            c = (int)(i % C);
+            long t = i / C;
+            wo = (int)(t % Wo);
+            t /= Wo;
+            ho = (int)(t % Ho);
+            n = t / Ho;
+        } else {
+            wo = (int)(i % Wo);
+            long t = i / Wo;
+            ho = (int)(t % Ho);
+            t /= Ho;
+            c = (int)(t % C);
+            n = t / C;
+        }
+        float m = -INFINITY;
+        for (int kh = 0; kh < k; ++kh) {
+            const int hi = ho * stride - pad + kh;
+            if (hi < 0 || hi >= H) continue;
+            for (int kw = 0; kw < k; ++kw) {
+                const int wi = wo * stride - pad + kw;
+                if (wi < 0 || wi >= W) continue;
+                const long xi = nhwc ? (((n * H + hi) * W + wi) * C + c) : (((n * C + c) * H + hi) * W + wi);
+                m = fmaxf(m, x[xi]);
+            }
+        }
+        y[i] = m;
+    }
+}
+int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, int nhwc,
+                     hipStream_t s) {
+    if (!x || !y || N <= 0 || H <= 0 || W <= 0 || C <= 0 || k <= 0 || stride <= 0 || pad < 0 || pad * 2 > k)
+        return K_EINVAL;
+    const int Ho = (H + 2 * pad - k) / stride + 1, Wo = (W + 2 * pad - k) / stride + 1;
+    if (Ho <= 0 || Wo <= 0) return K_EINVAL;
+    const long total = (long)N * Ho * Wo * C;
+    hipLaunchKernelGGL(maxpool_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, x, y, N, H, W, C, Ho, Wo, k,
+                       stride, pad, nhwc);
+    return (int)hipGetLastError();
+}
+
+// NHWC: one thread per (n, c), lanes along c (coalesced).  NCHW: one wavefront per (n, c).
+__global__ __launch_bounds__(256) void avgpool_nhwc_kernel(const float* __restrict__ x, float* __restrict__ y, int N,
+                                                           int HW, int C) {
+    const long total = (long)N * C;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long n = i / C;
+        const int c = (int)(i - n * C);
+        const float* p = x + n * HW * C + c;
+        float s = 0.f;
+        for (int j = 0; j < HW; ++j) s += p[(long)j * C];
+        y[i] = s / (float)HW;
+    }
+}
+__global__ __launch_bounds__(256) void avgpool_nchw_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                           long rows, int HW) {
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* p = x + row * HW;
+    float s = 0.f;
+    for (int j = lane; j < HW; j += 64) s += p[j];
+    s = wave_sum(s);
+    if (lane == 0) y[row] = s / (float)HW;
+}
+int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, hipStream_t s) {
+    if (!x || !y || N <= 0 || HW <= 0 || C <= 0) return K_EINVAL;
+    if (nhwc) {
+        hipLaunchKernelGGL(avgpool_nhwc_kernel, dim3(grid_for((long)N * C, 256)), dim3(256), 0, s, x, y, N, HW, C);
+    } else {
+        const long rows = (long)N * C;
+        hipLaunchKernelGGL(avgpool_nchw_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, x, y, rows, HW);
+    }
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- LayerNorm
+// y = (v - mean) / sqrt(var + eps) * gamma + beta with v = x (+ residual);
+// one wavefront per row, two-pass variance, row kept in registers up to 2048 wide.
+template <int MAXV>
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ res,
+                                                        const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta, float* __restrict__ y,
+                                                        long rows, int width, float eps) {
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = x + row * width;
+    const float* rr = res ? res + row * width : nullptr;
+    float* yr = y + row * width;
+    float v[MAXV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        float t = 0.f;
+        if (c < width) {
+            t = xr[c];
+            if (rr) t += rr[c];
+        }
+        v[i] = t;
+        s += t;
+    }
+    const float mean = wave_sum(s) / (float)width;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        const float d = (c < width) ? v[i] - mean : 0.f;
+        q += d * d;
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        if (c < width) yr[c] = (v[i] - mean) * rstd * gamma[c] + beta[c];
+    }
+}
+__global__ __launch_bounds__(256) void layernorm_wide_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ res,
+                                                             const float* __restrict__ gamma,
+                                                             const float* __restrict__ beta, float* __restrict__ y,
+                                                             long rows, int width, float eps) {
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = x + row * width;
+    const float* rr = res ? res + row * width : nullptr;
+    float* yr = y + row * width;
+    float s = 0.f;
+    for (int c = lane; c < width; c += 64) s += xr[c] + (rr ? rr[c] : 0.f);
+    const float mean = wave_sum(s) / (float)width;
+    float q = 0.f;
+    for (int c = lane; c < width; c += 64) {
+        const float d = xr[c] + (rr ? rr[c] : 0.f) - mean;
+        q += d * d;
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
+    // y may alias x or residual element-wise: each lane reads its element before writing it
+    for (int c = lane; c < width; c += 64) {
+        const float t = xr[c] + (rr ? rr[c] : 0.f);
+        yr[c] = (t - mean) * rstd * gamma[c] + beta[c];
+    }
+}
+int launch_layernorm(const float* x, const float* residual, const float* gamma, const float* beta, float* y,
+                     long rows, int width, float eps, hipStream_t s) {
+    if (!x || !gamma || !beta || !y || rows < 0 || width <= 0) return K_EINVAL;
+    if (rows == 0) return 0;
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    if (width <= 64 * 4)
+        hipLaunchKernelGGL(layernorm_kernel<4>, grid, dim3(256), 0, s, x, residual, gamma, beta, y, rows, width, eps);
+    else if (width <= 64 * 16)
+        hipLaunchKernelGGL(layernorm_kernel<16>, grid, dim3(256), 0, s, x, residual, gamma, beta, y, rows, width, eps);
+    else if (width <= 64 * 32)
+        hipLaunchKernelGGL(layernorm_kernel<32>, grid, dim3(256), 0, s, x, residual, gamma, beta, y, rows, width, eps);
+    else
+        hipLaunchKernelGGL(layernorm_wide_kernel, grid, dim3(256), 0, s, x, residual, gamma, beta, y, rows, width,
+                           eps);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- softmax
+template <int MAXV>
+__global__ __launch_bounds__(256) void softmax_kernel(const float* __restrict__ x, const float* __restrict__ mask,
+                                                      float* __restrict__ y, long rows, int width, float scale,
+                                                      long rows_per_mask) {
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = x + row * width;
+    const float* mr = mask ? mask + (row / rows_per_mask) * width : nullptr;
+    float* yr = y + row * width;
+    float v[MAXV];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        float t = -INFINITY;
+        if (c < width) {
+            t = xr[c] * scale;
+            if (mr) t += mr[c];
+        }
+        v[i] = t;
+        m = fmaxf(m, t);
+    }
+    m = wave_max(m);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        const float e = (c < width) ? expf(v[i] - m) : 0.f;
+        v[i] = e;
+        s += e;
+    }
+    const float inv = 1.0f / wave_sum(s);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+        const int c = lane + i * 64;
+        if (c < width) yr[c] = v[i] * inv;
+    }
+}
+int launch_softmax(const float* x, const float* mask, float* y, long rows, int width, float scale,
+                   long rows_per_mask, hipStream_t s) {
+    if (!x || !y || rows < 0 || width <= 0 || (mask && rows_per_mask <= 0)) return K_EINVAL;
+    if (width > 64 * 32) return K_EUNSUPPORTED;
+    if (rows == 0) return 0;
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    if (rows_per_mask <= 0) rows_per_mask = 1;
+    if (width <= 64 * 2)
+        hipLaunchKernelGGL(softmax_kernel<2>, grid, dim3(256), 0, s, x, mask, y, rows, width, scale, rows_per_mask);
+    else if (width <= 64 * 8)
+        hipLaunchKernelGGL(softmax_kernel<8>, grid, dim3(256), 0, s, x, mask, y, rows, width, scale, rows_per_mask);
+    else
+        hipLaunchKernelGGL(softmax_kernel<32>, grid, dim3(256), 0, s, x, mask, y, rows, width, scale, rows_per_mask);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- embedding
+// y[tok] = word[ids[tok]] + pos[tok % seq] + type[type_ids[tok]] ; one wavefront per token
+__global__ __launch_bounds__(256) void embedding_kernel(const int64_t* __restrict__ ids,
+                                                        const int64_t* __restrict__ type_ids,
+                                                        const float* __restrict__ word,
+                                                        const float* __restrict__ pos,
+                                                        const float* __restrict__ type, float* __restrict__ y,
+                                                        long tokens, int seq, int width, long vocab,
+                                                        int n_types) {
+    const int lane = threadIdx.x & 63;
+    const long tok = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tok >= tokens) return;
+    long id = ids[tok];
+    if (id < 0) id = 0;
+    if (id >= vocab) id = vocab - 1;
+    const float* wr = word + id * width;
+    const float* pr = pos ? pos + (tok % seq) * width : nullptr;
+    long ty = type_ids ? type_ids[tok] : 0;
+    if (ty < 0) ty = 0;
+    if (ty >= n_types) ty = n_types - 1;
+    const float* tr = type ? type + ty * width : nullptr;
+    float* yr = y + tok * width;
+    for (int c = lane; c < width; c += 64) {
+        float v = wr[c];
+        if (pr) v += pr[c];
+        if (tr) v += tr[c];
+        yr[c] = v;
+    }
+}
+int launch_embedding(const int64_t* ids, const int64_t* type_ids, const float* word, const float* pos,
+                     const float* type, float* y, long tokens, int seq, int width, long vocab, int n_types,
+                     hipStream_t s) {
+    if (!ids || !word || !y || tokens < 0 || seq <= 0 || width <= 0 || vocab <= 0 || n_types <= 0) return K_EINVAL;
+    if (tokens == 0) return 0;
+    hipLaunchKernelGGL(embedding_kernel, dim3((unsigned)((tokens + 3) / 4)), dim3(256), 0, s, ids, type_ids, word,
+                       pos, type, y, tokens, seq, width, vocab, n_types);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- sum
+// Deterministic: one workgroup, fixed per-thread strides, tree in LDS.
+__global__ __launch_bounds__(1024) void sum_kernel(const float* __restrict__ x, float* __restrict__ y, long n) {
+    __shared__ float part[16];
+    float s = 0.f;
+    for (long i = threadIdx.x; i < n; i += 1024) s += x[i];
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+        for (int i = 0; i < 16; ++i) t += part[i];
+        y[0] = t;
+    }
+}
+int launch_sum(const float* x, float* y, long n, hipStream_t s) {
+    if (!x || !y || n < 0) return K_EINVAL;
+    hipLaunchKernelGGL(sum_kernel, dim3(1), dim3(1024), 0, s, x, y, n);
+    return (int)hipGetLastError();
+}
+
+}  // namespace tpk

@@ -1,0 +1,97 @@
+// Pooled HBM allocator: one arena cut into fixed slabs, extents of whole slabs
+// handed out best-fit with coalescing on release.
+//
+// Takes the place of the reference's BuddyBasedBlockManager / Block
+// (include/server/block_manager.hpp:23-125, 260-418): there, budget/128 MiB
+// physical blocks are cudaMalloc'ed up front and carved into 2 MiB or 16 MiB
+// slots by a first-fit bitmap scan.  Here the arena is one allocation (sized
+// for a 288 GB part), a model occupies two extents (weight image, activation
+// arena), and all bookkeeping is offset arithmetic, so the class is pure host
+// logic and runs without a device.
+#pragma once
+#include <cstdint>
+#include <map>
+
+namespace tp {
+
+class SlabPool {
+public:
+    static constexpr uint64_t kSlab = 2ull << 20;  // 2 MiB, the reference's regular slot (block_manager.hpp:28)
+
+    SlabPool() = default;
+    void reset(uint64_t capacity_bytes) {
+        capacity_ = (capacity_bytes / kSlab) * kSlab;
+        free_.clear();
+        used_.clear();
+        if (capacity_) free_[0] = capacity_;
+        used_bytes_ = 0;
+    }
+    static uint64_t round_up(uint64_t bytes) { return ((bytes + kSlab - 1) / kSlab) * kSlab; }
+
+    // Returns the arena offset of a contiguous extent, or UINT64_MAX.
+    uint64_t alloc(uint64_t bytes) {
+        if (bytes == 0) bytes = 1;
+        const uint64_t need = round_up(bytes);
+        auto best = free_.end();
+        for (auto it = free_.begin(); it != free_.end(); ++it) {
+            if (it->second < need) continue;
+            if (best == free_.end() || it->second < best->second) best = it;
+        }
+        if (best == free_.end()) return UINT64_MAX;
+        const uint64_t off = best->first, len = best->second;
+        free_.erase(best);
+        if (len > need) free_[off + need] = len - need;
+        used_[off] = need;
+        used_bytes_ += need;
+        return off;
+    }
+
+    // Returns false when `off` is not the start of a live extent.
+    bool release(uint64_t off) {
+        auto u = used_.find(off);
+        if (u == used_.end()) return false;
+        uint64_t len = u->second;
+        used_.erase(u);
+        used_bytes_ -= len;
+        auto next = free_.lower_bound(off);
+        if (next != free_.end() && off + len == next->first) {
+            len += next->second;
+            next = free_.erase(next);
+        }
+        if (next != free_.begin()) {
+            auto prev = std::prev(next);
+            if (prev->first + prev->second == off) {
+                prev->second += len;
+                return true;
+            }
+        }
+        free_[off] = len;
+        return true;
+    }
+
+    uint64_t capacity() const { return capacity_; }
+    uint64_t used_bytes() const { return used_bytes_; }
+    uint64_t free_bytes() const { return capacity_ - used_bytes_; }
+    uint64_t largest_free() const {
+        uint64_t m = 0;
+        for (auto& kv : free_)
+            if (kv.second > m) m = kv.second;
+        return m;
+    }
+    size_t live_extents() const { return used_.size(); }
+    size_t free_extents() const { return free_.size(); }
+    uint64_t extent_size(uint64_t off) const {
+        auto u = used_.find(off);
+        return u == used_.end() ? 0 : u->second;
+    }
+    const std::map<uint64_t, uint64_t>& used() const { return used_; }
+    const std::map<uint64_t, uint64_t>& free_map() const { return free_; }
+
+private:
+    uint64_t capacity_ = 0;
+    uint64_t used_bytes_ = 0;
+    std::map<uint64_t, uint64_t> free_;  // offset -> length, address ordered, never adjacent
+    std::map<uint64_t, uint64_t> used_;  // offset -> length
+};
+
+}  // namespace tp
