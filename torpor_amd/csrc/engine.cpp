@@ -146,7 +146,11 @@ int Engine::translate(Model& m, uint64_t va, uint64_t span, Xlat* out) {
         if (it == m.ablocks.begin()) return TP_EFAULT;
         --it;
         ABlock& b = it->second;
-        if (!b.live || off >= b.voff + b.size || off + span > b.voff + b.size) return TP_EFAULT;
+        if (off >= b.voff + b.size || off + span > b.voff + b.size) return TP_EFAULT;
+        // Once the arena is frozen every block keeps its place for good and later requests repeat
+        // the tracked op stream without re-issuing its malloc/free calls, so liveness is only
+        // enforced while the first inference is being tracked.
+        if (!m.act_frozen && !b.live) return TP_EFAULT;
         if (m.act_frozen) {
             if (!m.resident) return TP_EFAULT;
             out->p = m.a_dev + off;
