@@ -254,6 +254,23 @@ int tp_measure_h2d(tp_server* s, uint64_t bytes, int32_t iters, double* gbps);
  * events on the compute stream. */
 int tp_time_op(tp_server* s, int32_t client, int32_t op_index, int32_t iters, double* mean_us);
 
+/* Per-kernel timing of the compute stream, for roofline accounting.  Between begin and end
+ * every compute op is bracketed by two HIP events on the compute stream; end waits for the
+ * stream and aggregates by kernel variant.  tp_profile_read returns TP_ENOENT past the last
+ * entry.  The entry named "__empty_bracket__" is the duration of an empty bracket (event
+ * overhead), measured at end, to be subtracted per launch.  No counterpart in the reference,
+ * which logs host-side timestamps only (memory_manager.hpp:425-431, cuda_server.hpp:294-295). */
+typedef struct tp_kernel_stat {
+    char name[64];
+    uint64_t launches;
+    double total_us; /* sum of bracketed durations */
+    double flops;    /* algorithmic floating-point operations of those launches */
+    double bytes;    /* algorithmic bytes read + written */
+} tp_kernel_stat;
+int tp_profile_begin(tp_server* s);
+int tp_profile_end(tp_server* s);
+int tp_profile_read(tp_server* s, int32_t index, tp_kernel_stat* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,11 @@ class SwapStats(C.Structure):
                 ("evict_us", C.c_double), ("chunks", C.c_uint32), ("gate_waits", C.c_uint32)]
 
 
+class KernelStat(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("launches", C.c_uint64), ("total_us", C.c_double),
+                ("flops", C.c_double), ("bytes", C.c_double)]
+
+
 # every symbol include/torpor_amd.h declares: name -> (restype, argtypes)
 _P = C.c_void_p
 _U64 = C.c_uint64
@@ -131,6 +136,9 @@ SYMBOLS = {
     "tp_last_kernel": (C.c_char_p, []),
     "tp_measure_h2d": (C.c_int, [_P, _U64, _I32, C.POINTER(C.c_double)]),
     "tp_time_op": (C.c_int, [_P, _I32, _I32, _I32, C.POINTER(C.c_double)]),
+    "tp_profile_begin": (C.c_int, [_P]),
+    "tp_profile_end": (C.c_int, [_P]),
+    "tp_profile_read": (C.c_int, [_P, _I32, C.POINTER(KernelStat)]),
 }
 
 _lib = None

@@ -373,4 +373,23 @@ int tp_time_op(tp_server* s, int32_t client, int32_t op_index, int32_t iters, do
     TP_GUARD_END
 }
 
+int tp_profile_begin(tp_server* s) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.profile_begin();
+    TP_GUARD_END
+}
+int tp_profile_end(tp_server* s) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.profile_end();
+    TP_GUARD_END
+}
+int tp_profile_read(tp_server* s, int32_t index, tp_kernel_stat* out) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.profile_read(index, out);
+    TP_GUARD_END
+}
+
 }  // extern "C"

@@ -87,6 +87,7 @@ Engine::~Engine() {
         }
     }
     if (!host_only()) {
+        for (auto e : prof_events_) (void)hipEventDestroy(e);
         if (h2d_stage_) (void)hipHostFree(h2d_stage_);
         if (d2h_stage_) (void)hipHostFree(d2h_stage_);
         if (workspace_) (void)hipFree(workspace_);
@@ -939,7 +940,7 @@ static tpk::EpilogueArgs ep_from(const Op& op, void* const* q, int pbase, int fb
 //  CONV  p: x w y bias bns bnb bnm bnv res   i: n h w cin cout kh kw sh sw ph pw xl yl ldr act   f: alpha beta eps
 //  BN    p: x y g b mean var                 i: rows C hw layout relu   f: eps
 //  LAUNCH p/i/f per op id (see torpor_amd.h)
-int Engine::exec_compute(Model& m, const Op& op, bool launch) {
+int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
     void* q[12] = {nullptr};
     const tpk::Workspace ws{workspace_, (size_t)cfg_.workspace_bytes};
     // Every operand is translated together with the byte span the kernel will touch, so an op
@@ -1138,6 +1139,150 @@ int Engine::exec_compute(Model& m, const Op& op, bool launch) {
         default:
             return TP_EUNSUPPORTED;
     }
+}
+
+// Algorithmic work of one op: floating-point operations and bytes that have to move at least
+// once (each operand read once, each result written once).
+static void op_work(const Op& op, double* flops, double* bytes, const char** name) {
+    const int64_t* I = op.i;
+    *flops = 0;
+    *bytes = 0;
+    *name = "op";
+    switch (op.kind) {
+        case OPK_GEMM: {
+            const double M = (double)I[0], N = (double)I[1], K = (double)I[2], nb = (double)(I[8] * I[9]);
+            *flops = 2.0 * M * N * K * nb;
+            *bytes = 4.0 * (M * K + N * K + M * N) * nb;
+            *name = "gemm";
+            break;
+        }
+        case OPK_CONV: {
+            const double Ho = (double)((I[1] + 2 * I[9] - I[5]) / I[7] + 1), Wo = (double)((I[2] + 2 * I[10] - I[6]) / I[8] + 1);
+            const double M = (double)I[0] * Ho * Wo, kk = (double)(I[3] * I[5] * I[6]);
+            *flops = 2.0 * M * (double)I[4] * kk;
+            *bytes = 4.0 * ((double)(I[0] * I[1] * I[2] * I[3]) + (double)I[4] * kk + M * (double)I[4] * (op.p[8] ? 2.0 : 1.0));
+            *name = "conv";
+            break;
+        }
+        case OPK_BN:
+            *bytes = 8.0 * (double)(I[0] * I[1]);
+            *name = "bn_inference";
+            break;
+        case OPK_LAUNCH:
+            switch (op.op_id) {
+                case TP_OP_RELU: *bytes = 8.0 * (double)I[0]; *name = "relu"; break;
+                case TP_OP_GELU: *bytes = 8.0 * (double)I[0]; *name = "gelu"; break;
+                case TP_OP_ADD: *bytes = 12.0 * (double)I[0]; *name = "add"; break;
+                case TP_OP_BIAS_ACT: *bytes = 8.0 * (double)(I[0] * I[1]); *name = "bias_act"; break;
+                case TP_OP_MAXPOOL: {
+                    const double Ho = (double)((I[1] + 2 * I[6] - I[4]) / I[5] + 1), Wo = (double)((I[2] + 2 * I[6] - I[4]) / I[5] + 1);
+                    *bytes = 4.0 * ((double)(I[0] * I[1] * I[2] * I[3]) + (double)(I[0] * I[3]) * Ho * Wo);
+                    *name = "maxpool";
+                    break;
+                }
+                case TP_OP_AVGPOOL: *bytes = 4.0 * (double)(I[0] * I[1] * I[2] + I[0] * I[2]); *name = "avgpool"; break;
+                case TP_OP_LAYERNORM: *bytes = 4.0 * (double)(I[0] * I[1]) * (op.p[1] ? 3.0 : 2.0); *name = "layernorm"; break;
+                case TP_OP_SOFTMAX: *bytes = 8.0 * (double)(I[0] * I[1]); *name = "softmax"; break;
+                case TP_OP_EMBEDDING: *bytes = 8.0 * (double)(I[0] * I[2]); *name = "embedding"; break;
+                case TP_OP_NCHW_TO_NHWC:
+                case TP_OP_NHWC_TO_NCHW: *bytes = 8.0 * (double)(I[0] * I[1] * I[2] * I[3]); *name = "layout"; break;
+                case TP_OP_SUM: *bytes = 4.0 * (double)I[0]; *name = "sum"; break;
+                case TP_OP_FILL: *bytes = 4.0 * (double)I[0]; *name = "fill"; break;
+                default: break;
+            }
+            break;
+        default:
+            break;
+    }
+}
+
+int Engine::exec_compute(Model& m, const Op& op, bool launch) {
+    if (!profiling_ || !launch || host_only()) return exec_compute_impl(m, op, launch);
+    while (prof_events_.size() < prof_next_ + 2) {
+        hipEvent_t e = nullptr;
+        HIPCHK(hipEventCreate(&e));
+        prof_events_.push_back(e);
+    }
+    hipEvent_t a = prof_events_[prof_next_], b = prof_events_[prof_next_ + 1];
+    prof_next_ += 2;
+    double flops, bytes;
+    const char* name;
+    op_work(op, &flops, &bytes, &name);
+    tpk::set_last_kernel(name);  // the MFMA launchers overwrite this with the variant they pick
+    HIPCHK(hipEventRecord(a, compute_));
+    const int r = exec_compute_impl(m, op, true);
+    HIPCHK(hipEventRecord(b, compute_));
+    prof_records_.push_back({tpk::last_kernel_name(), a, b, flops, bytes});
+    return r;
+}
+
+int Engine::profile_begin() {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (host_only()) return TP_ENODEV;
+    profiling_ = true;
+    prof_next_ = 0;
+    prof_records_.clear();
+    prof_stats_.clear();
+    return 0;
+}
+
+int Engine::profile_end() {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (host_only()) return TP_ENODEV;
+    if (!profiling_) return TP_ESTATE;
+    profiling_ = false;
+    HIPCHK(hipStreamSynchronize(compute_));
+    prof_stats_.clear();
+    for (auto& r : prof_records_) {
+        float ms = 0.f;
+        HIPCHK(hipEventElapsedTime(&ms, r.a, r.b));
+        tp_kernel_stat* st = nullptr;
+        for (auto& s : prof_stats_)
+            if (std::strncmp(s.name, r.name, sizeof(s.name) - 1) == 0) st = &s;
+        if (!st) {
+            tp_kernel_stat ns;
+            std::memset(&ns, 0, sizeof(ns));
+            std::strncpy(ns.name, r.name, sizeof(ns.name) - 1);
+            prof_stats_.push_back(ns);
+            st = &prof_stats_.back();
+        }
+        st->launches++;
+        st->total_us += (double)ms * 1000.0;
+        st->flops += r.flops;
+        st->bytes += r.bytes;
+    }
+    // event overhead: median duration of an empty bracket
+    while (prof_events_.size() < 2) {
+        hipEvent_t e = nullptr;
+        HIPCHK(hipEventCreate(&e));
+        prof_events_.push_back(e);
+    }
+    std::vector<float> empt;
+    for (int i = 0; i < 21; ++i) {
+        HIPCHK(hipEventRecord(prof_events_[0], compute_));
+        HIPCHK(hipEventRecord(prof_events_[1], compute_));
+        HIPCHK(hipEventSynchronize(prof_events_[1]));
+        float ms = 0.f;
+        HIPCHK(hipEventElapsedTime(&ms, prof_events_[0], prof_events_[1]));
+        empt.push_back(ms);
+    }
+    std::sort(empt.begin(), empt.end());
+    tp_kernel_stat es;
+    std::memset(&es, 0, sizeof(es));
+    std::strncpy(es.name, "__empty_bracket__", sizeof(es.name) - 1);
+    es.launches = 1;
+    es.total_us = (double)empt[empt.size() / 2] * 1000.0;
+    prof_stats_.push_back(es);
+    prof_records_.clear();
+    return 0;
+}
+
+int Engine::profile_read(int index, tp_kernel_stat* out) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!out) return TP_EINVAL;
+    if (index < 0 || index >= (int)prof_stats_.size()) return TP_ENOENT;
+    *out = prof_stats_[index];
+    return 0;
 }
 
 int Engine::exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch) {

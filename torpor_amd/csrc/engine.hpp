@@ -154,6 +154,9 @@ public:
     int weight_offset(int client, uint64_t va, uint64_t* off);
     int measure_h2d(uint64_t bytes, int iters, double* gbps);
     int time_op(int client, int op_index, int iters, double* mean_us);
+    int profile_begin();
+    int profile_end();
+    int profile_read(int index, tp_kernel_stat* out);
 
 private:
     enum Mode : int { MODE_NONE = 0, MODE_LOAD = 1, MODE_TRACK = 2, MODE_EXEC = 3 };
@@ -179,6 +182,7 @@ private:
     int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out);
     int exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch);
     int exec_compute(Model& m, const Op& op, bool launch);
+    int exec_compute_impl(Model& m, const Op& op, bool launch);
     int do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes);
     int do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes);
     int do_stream_sync(Model* m);
@@ -224,6 +228,17 @@ private:
     std::vector<PendingD2H> pending_d2h_;
 
     uint64_t evictions_ = 0, swap_ins_ = 0;
+
+    struct ProfRecord {
+        const char* name;
+        hipEvent_t a, b;
+        double flops, bytes;
+    };
+    bool profiling_ = false;
+    std::vector<hipEvent_t> prof_events_;
+    size_t prof_next_ = 0;
+    std::vector<ProfRecord> prof_records_;
+    std::vector<tp_kernel_stat> prof_stats_;
 
     std::thread copy_thread_;
     std::mutex cmu_;

@@ -61,6 +61,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s);
 int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s);
 // introspection for tests/bench: which path the last launch on this thread took
 const char* last_kernel_name();
+void set_last_kernel(const char* name);
 
 // ---- HBM-bound operators (elementwise.hip / reduce.hip) ----
 int launch_bn_inference(const float* x, float* y, const float* g, const float* b, const float* mean,

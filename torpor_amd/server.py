@@ -221,6 +221,26 @@ class Server:
         _chk(self._l.tp_measure_h2d(self._h, nbytes, iters, C.byref(g)), "tp_measure_h2d")
         return g.value
 
+    def profile_begin(self):
+        _chk(self._l.tp_profile_begin(self._h), "tp_profile_begin")
+
+    def profile_end(self):
+        """Returns ({kernel: {launches, total_us, flops, bytes}}, empty_bracket_us)."""
+        _chk(self._l.tp_profile_end(self._h), "tp_profile_end")
+        out, empty, i = {}, 0.0, 0
+        while True:
+            st = _lib.KernelStat()
+            r = self._l.tp_profile_read(self._h, i, C.byref(st))
+            if r != 0:
+                break
+            i += 1
+            name = st.name.decode()
+            if name == "__empty_bracket__":
+                empty = st.total_us
+            else:
+                out[name] = dict(launches=st.launches, total_us=st.total_us, flops=st.flops, bytes=st.bytes)
+        return out, empty
+
     def time_op(self, fid, op_index=-1, iters=20):
         t = C.c_double()
         _chk(self._l.tp_time_op(self._h, fid, op_index, iters, C.byref(t)), "tp_time_op")
