@@ -271,6 +271,31 @@ int tp_profile_begin(tp_server* s);
 int tp_profile_end(tp_server* s);
 int tp_profile_read(tp_server* s, int32_t index, tp_kernel_stat* out);
 
+/* ------------------------------------------------------------------ host-side building blocks
+ * The pool allocator and the eviction policy as stand-alone objects (pure host logic, no device),
+ * so that they can be unit-tested and reused by a front end.
+ * tp_pool: extents of 2 MiB slabs out of one arena, best fit, coalescing; takes the place of
+ *          BuddyBasedBlockManager (block_manager.hpp:260-418).  Offsets are arena-relative;
+ *          UINT64_MAX = no fit.
+ * tp_lru:  LRUEvictor (evictor.hpp:190-264).  check_and_add writes the victims, oldest first and
+ *          newline-separated, into `victims` (truncated to `cap` bytes incl. the terminator). */
+typedef struct tp_pool tp_pool;
+tp_pool* tp_pool_create(uint64_t capacity_bytes);
+void tp_pool_destroy(tp_pool* p);
+uint64_t tp_pool_alloc(tp_pool* p, uint64_t bytes);
+int tp_pool_release(tp_pool* p, uint64_t offset);
+int tp_pool_query(tp_pool* p, uint64_t* capacity, uint64_t* used, uint64_t* largest_free, uint64_t* live_extents,
+                  uint64_t* free_extents);
+typedef struct tp_lru tp_lru;
+tp_lru* tp_lru_create(uint64_t budget_bytes);
+void tp_lru_destroy(tp_lru* l);
+int tp_lru_check_and_add(tp_lru* l, const char* function, uint64_t size, char* victims, uint64_t cap,
+                         int32_t* n_victims, int32_t* over_budget);
+int tp_lru_force_evict(tp_lru* l, const char* function); /* 1 = was tracked, 0 = unknown */
+int tp_lru_lock(tp_lru* l, const char* function);
+int tp_lru_unlock(tp_lru* l, const char* function);
+uint64_t tp_lru_used(tp_lru* l);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,354 @@
+"""Host logic through the C-ABI, no GPU: pool allocator invariants, LRU policy against the
+restatement of the reference's LRUEvictor and against a brute-force model, and the
+controller / executor state machine of a host-only engine (TP_FLAG_HOST_ONLY: no HIP calls, no
+compute - ops are validated, tracked and recorded but not launched)."""
+import ctypes as C
+import random
+
+import numpy as np
+import pytest
+
+from oracle.host_ref import LruRef
+from torpor_amd import _lib
+from torpor_amd._lib import TorporError
+from torpor_amd.functions import resnet
+from torpor_amd.server import (ACK_INAVAIL, ACK_OK, OP_RELU, REQ_EXECUTE, REQ_EXECUTE_AFTER_LOAD, REQ_LOAD,
+                               REQ_UNLOAD, Server)
+
+SLAB = 2 << 20
+NOFIT = (1 << 64) - 1
+
+
+# ---------------------------------------------------------------------------------- pool
+class Pool:
+    def __init__(self, cap):
+        self.l = _lib.lib()
+        self.p = self.l.tp_pool_create(cap)
+
+    def alloc(self, n):
+        return self.l.tp_pool_alloc(self.p, n)
+
+    def release(self, off):
+        return self.l.tp_pool_release(self.p, off)
+
+    def query(self):
+        v = [C.c_uint64() for _ in range(5)]
+        assert self.l.tp_pool_query(self.p, *[C.byref(x) for x in v]) == 0
+        return dict(zip(("capacity", "used", "largest_free", "live", "free_extents"), [x.value for x in v]))
+
+    def __del__(self):
+        self.l.tp_pool_destroy(self.p)
+
+
+def test_pool_basic_and_coalescing():
+    p = Pool(16 * SLAB + 12345)             # capacity rounds down to whole slabs
+    assert p.query()["capacity"] == 16 * SLAB
+    a = p.alloc(1)                          # rounds up to one slab
+    b = p.alloc(3 * SLAB)
+    c = p.alloc(SLAB + 1)                   # two slabs
+    assert (a, b, c) == (0, SLAB, 4 * SLAB)
+    assert p.query()["used"] == 6 * SLAB
+    assert p.release(b) == 0 and p.release(b) != 0          # double free is refused
+    assert p.release(12345) != 0                            # not an extent start
+    d = p.alloc(2 * SLAB)                   # best fit: the 3-slab hole, not the 10-slab tail
+    assert d == SLAB
+    assert p.release(a) == 0 and p.release(d) == 0 and p.release(c) == 0
+    q = p.query()
+    assert q["used"] == 0 and q["free_extents"] == 1 and q["largest_free"] == 16 * SLAB   # fully coalesced
+    assert p.alloc(17 * SLAB) == NOFIT and p.alloc(16 * SLAB) == 0
+
+
+def test_pool_random_invariants():
+    """No overlap, inside the arena, slab aligned, used = sum of live extents, free + used =
+    capacity, no two adjacent free extents (largest_free == capacity once everything is freed)."""
+    rng = random.Random(0)
+    cap = 64 * SLAB
+    p = Pool(cap)
+    live = {}
+    for step in range(3000):
+        if live and (rng.random() < 0.45 or len(live) > 20):
+            off = rng.choice(list(live))
+            assert p.release(off) == 0
+            del live[off]
+        else:
+            n = rng.randint(1, 9 * SLAB)
+            off = p.alloc(n)
+            need = -(-n // SLAB) * SLAB
+            if off == NOFIT:
+                # refusal is only legal when no hole is large enough
+                assert p.query()["largest_free"] < need
+                continue
+            assert off % SLAB == 0 and off + need <= cap
+            for o, s in live.items():
+                assert off + need <= o or o + s <= off, "extents overlap"
+            live[off] = need
+        q = p.query()
+        assert q["used"] == sum(live.values()) and q["live"] == len(live)
+    for off in list(live):
+        assert p.release(off) == 0
+    q = p.query()
+    assert q["used"] == 0 and q["largest_free"] == cap and q["free_extents"] == 1
+
+
+def test_pool_layout_is_deterministic():
+    seq = [(1, 5 * SLAB), (1, SLAB), (0, 0), (1, 2 * SLAB), (1, 7 * SLAB), (0, 1), (1, 3 * SLAB)]
+    outs = []
+    for _ in range(2):
+        p, got, offs = Pool(32 * SLAB), [], []
+        for kind, v in seq:
+            if kind:
+                offs.append(p.alloc(v))
+                got.append(offs[-1])
+            else:
+                p.release(offs[v])
+        outs.append(got)
+    assert outs[0] == outs[1]
+
+
+# ---------------------------------------------------------------------------------- LRU
+class Lru:
+    def __init__(self, budget):
+        self.l = _lib.lib()
+        self.p = self.l.tp_lru_create(budget)
+
+    def check_and_add(self, f, sz):
+        buf = C.create_string_buffer(4096)
+        n, over = C.c_int32(), C.c_int32()
+        assert self.l.tp_lru_check_and_add(self.p, f.encode(), sz, buf, 4096, C.byref(n), C.byref(over)) == 0
+        v = buf.value.decode().split("\n") if buf.value else []
+        assert len(v) == n.value
+        return v, bool(over.value)
+
+    def force_evict(self, f):
+        return self.l.tp_lru_force_evict(self.p, f.encode())
+
+    def lock(self, f):
+        self.l.tp_lru_lock(self.p, f.encode())
+
+    def unlock(self, f):
+        self.l.tp_lru_unlock(self.p, f.encode())
+
+    def used(self):
+        return self.l.tp_lru_used(self.p)
+
+    def __del__(self):
+        self.l.tp_lru_destroy(self.p)
+
+
+def test_lru_textbook_cases():
+    l = Lru(100)
+    assert l.check_and_add("a", 40) == ([], False)
+    assert l.check_and_add("b", 40) == ([], False)
+    assert l.check_and_add("a", 40) == ([], False)            # hit: a becomes most recent
+    assert l.check_and_add("c", 40) == (["b"], False)         # 80 + 40 >= 100 -> evict the oldest = b
+    assert l.used() == 80
+    assert l.check_and_add("d", 20) == (["a"], False)         # '>=': 80 + 20 == budget still evicts
+    l.lock("c")
+    assert l.check_and_add("e", 60) == (["d"], True)          # c is locked: over budget, reported
+    l.unlock("c")
+    assert l.force_evict("zzz") == 0 and l.force_evict("e") == 1
+    assert l.used() == 40
+
+
+def test_lru_matches_reference_restatement_on_random_traces():
+    for seed in range(5):
+        rng = random.Random(seed)
+        budget = 1000
+        mine, ref = Lru(budget), LruRef(budget)
+        brute = []          # brute-force model: list, most recent first
+        sizes = {f"{i}": rng.randint(50, 400) for i in range(12)}
+        for step in range(2000):
+            f = str(rng.randrange(12))
+            r = rng.random()
+            if r < 0.8:
+                got, _ = mine.check_and_add(f, sizes[f])
+                want = ref.check_and_add(f, sizes[f])
+                assert got == want, (seed, step)
+                # brute force (no locks in this trace)
+                if f in brute:
+                    brute.remove(f)
+                    exp = []
+                else:
+                    exp = []
+                    while sum(sizes[x] for x in brute) + sizes[f] >= budget and brute:
+                        exp.append(brute.pop())
+                brute.insert(0, f)
+                assert got == exp
+            else:
+                assert bool(mine.force_evict(f)) == ref.force_evict(f)
+                if f in brute:
+                    brute.remove(f)
+            assert mine.used() == ref.cur == sum(sizes[x] for x in brute)
+            assert mine.used() < budget or len(brute) == 1
+
+
+def test_lru_locked_entries_are_never_evicted():
+    rng = random.Random(7)
+    mine, ref = Lru(500), LruRef(500)
+    locked = set()
+    for step in range(1500):
+        f = str(rng.randrange(8))
+        r = rng.random()
+        if r < 0.6:
+            got, _ = mine.check_and_add(f, 120)
+            assert got == ref.check_and_add(f, 120)
+            assert not (set(got) & locked)
+        elif r < 0.8:
+            mine.lock(f)
+            ref.lock(f)
+            if f in ref.items:
+                locked.add(f)
+        else:
+            mine.unlock(f)
+            ref.unlock(f)
+            locked.discard(f)
+
+
+# ---------------------------------------------------------------------------------- engine state machine
+def _register(s, fid, image=32, seed=0):
+    fn = resnet.ResNet(s, fid, "resnet50", batch=1, seed=seed, image=image)
+    x = np.zeros((1, 3, image, image), np.float32)
+    with pytest.raises(TorporError) as e:        # host-only: the request completes, but there is no data
+        fn.register([x])
+    assert e.value.code == -19
+    return fn
+
+
+@pytest.fixture(scope="module")
+def host_server():
+    s = Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20, request_timeout_ms=200)
+    yield s
+    s.close()
+
+
+def test_register_invoke_unload_flow(host_server):
+    s = host_server
+    fn = _register(s, 0)
+    info = s.model_info(0)
+    assert info["registered"] and info["resident"] and info["n_params"] == 267 and info["n_ops"] == 58
+    assert info["image_bytes"] % 256 == 0 and info["param_bytes"] == sum(v.nbytes for v in fn.weights().values())
+    assert s.pool_stats()["lru_models"] == 1 and s.pool_stats()["live_extents"] == 2
+    # Execute (resident) -> ack OK, gpu 0 ; ops from another client are refused while 0 is active
+    assert s.signal(REQ_EXECUTE, 0, "") == (ACK_OK, 0, False)
+    with pytest.raises(TorporError) as e:
+        s.malloc(5, 64)
+    assert e.value.code == -72
+    # a second request while busy is queued: no ack yet (controller.hpp:177)
+    assert s.signal(REQ_EXECUTE, 0, "")[2] is True
+    assert s.take_deferred_ack() is None
+    # Unload of the active function is refused
+    assert s.signal(REQ_UNLOAD, 0, "")[0] == ACK_INAVAIL
+    # the request ends with its async D2H (here through replay); the queued one is then started
+    packed, outbuf, _ = fn.pack([np.zeros((1, 3, 32, 32), np.float32)])
+    with pytest.raises(TorporError):
+        s.replay(0, packed, outbuf)
+    assert s.take_deferred_ack() == (ACK_OK, 0)
+    with pytest.raises(TorporError):
+        s.replay(0, packed, outbuf)
+    assert s.take_deferred_ack() is None
+    # Unload: ack OK, resp -1, pool back to empty, LRU forgets the model
+    assert s.signal(REQ_UNLOAD, 0, "")[:2] == (ACK_OK, -1)
+    st = s.pool_stats()
+    assert not s.resident(0) and st["used"] == 0 and st["lru_models"] == 0 and st["free_extents"] == 1
+    # Load = prefetch
+    assert s.signal(REQ_LOAD, 0, "")[0] == ACK_OK and s.resident(0)
+    assert s.signal(REQ_UNLOAD, 0, "")[0] == ACK_OK
+
+
+def test_eviction_under_budget_and_deterministic_offsets(host_server):
+    s = host_server
+    fns = [_register(s, i, seed=i) for i in range(1, 5)]
+    total = s.model_info(1)["total_bytes"]
+    assert 3 * total < (330 << 20) <= 4 * total
+    assert [s.resident(i) for i in range(1, 5)] == [False, True, True, True]
+    ref = LruRef(330 << 20)
+    for i in (2, 3, 4):
+        ref.check_and_add(str(i), total)
+    rng = random.Random(1)
+    for step in range(200):
+        i = rng.randint(1, 4)
+        victims = ref.check_and_add(str(i), total)
+        ack, resp, dfr = s.signal(REQ_EXECUTE, i, "")
+        assert (ack, resp, dfr) == (ACK_OK, 0, False)
+        for v in victims:
+            assert not s.resident(int(v))
+        assert s.resident(i)
+        assert sorted(ref.items) == sorted(str(j) for j in range(1, 5) if s.resident(j))
+        st = s.pool_stats()
+        assert st["lru_used"] == ref.cur and st["used"] == len(ref.items) * total
+        # extents of resident models never overlap
+        ext = []
+        for j in range(1, 5):
+            if s.resident(j):
+                mi = s.model_info(j)
+                ext += [(mi["weight_off"], mi["image_bytes"]), (mi["act_off"], mi["act_bytes"])]
+        ext.sort()
+        for (a, n), (b, _) in zip(ext, ext[1:]):
+            assert a + n <= b
+        packed, outbuf, _ = fns[i - 1].pack([np.zeros((1, 3, 32, 32), np.float32)])
+        with pytest.raises(TorporError):
+            s.replay(i, packed, outbuf)
+    for i in range(1, 5):
+        s.signal(REQ_UNLOAD, i, "")
+    assert s.pool_stats()["used"] == 0
+
+
+def test_request_timeout_completes_the_request(host_server):
+    """cuda_server.hpp:257-264: an Execute that sends no ops is force-completed after the timeout
+    (200 ms here) and the executor becomes available again."""
+    import time
+    s = host_server
+    _register(s, 10)
+    assert s.signal(REQ_EXECUTE, 10, "")[0] == ACK_OK
+    assert s.signal(REQ_EXECUTE, 10, "")[2] is True          # busy -> queued
+    assert not s.poll()
+    time.sleep(0.25)
+    assert s.poll()                                          # timed out, completed, queued one started
+    assert s.take_deferred_ack() == (ACK_OK, 0)
+    time.sleep(0.25)
+    assert s.poll()
+    assert s.signal(REQ_UNLOAD, 10, "")[0] == ACK_OK
+
+
+def test_error_paths(host_server):
+    s = host_server
+    assert s.signal(REQ_EXECUTE, 777, "")[0] == ACK_INAVAIL          # never registered
+    assert s.signal(REQ_LOAD, 777, "")[0] == ACK_INAVAIL
+    assert s.signal(REQ_UNLOAD, 777, "")[:2] == (ACK_OK, -1)
+    assert s.signal(10, 1, "")[0] == ACK_INAVAIL                     # ExecuteForRecord is refused
+    assert s.signal(11, 1, "")[0] == ACK_INAVAIL                     # Replay signal is refused
+    with pytest.raises(TorporError):
+        s.signal(REQ_EXECUTE, "abc", "")                             # function must be a decimal id
+    with pytest.raises(TorporError):
+        s.malloc(0, 16)                                              # no active function
+    # registration: ops before the end of the upload phase are refused; uploads outside a block too
+    assert s.signal(REQ_EXECUTE_AFTER_LOAD, 20, "2")[0] == ACK_OK
+    va = s.malloc(20, 1024)
+    s.h2d(20, va, np.arange(256, dtype=np.float32))
+    with pytest.raises(TorporError):
+        s.h2d(20, va + 512, np.zeros(256, np.float32))               # runs past the block
+    with pytest.raises(TorporError):
+        s.launch(20, OP_RELU, [va, va], [4])                         # still uploading
+    with pytest.raises(TorporError):
+        s.device_synchronize(20)       # ends the upload phase, and reports the refused ops above (once)
+    assert s.model_info(20)["level"] == 2
+    act = s.malloc(20, 1024)
+    with pytest.raises(TorporError):
+        s.h2d(20, va, np.zeros(4, np.float32))                       # weights are read-only after registration
+    with pytest.raises(TorporError):
+        s.free(20, va)                                               # freeing a model block is refused
+    s.launch(20, OP_RELU, [va, act], [256])
+    with pytest.raises(TorporError):
+        s.launch(20, OP_RELU, [va, act], [257])                      # longer than the buffers
+    with pytest.raises(TorporError):
+        s.launch(20, OP_RELU, [va, 0x1234], [4])                     # not an address of this server
+    s.free(20, act)
+    with pytest.raises(TorporError):
+        s.launch(20, OP_RELU, [va, act], [4])                        # freed
+    out = np.empty(4, np.float32)
+    act = s.malloc(20, 1024)
+    s.d2h_async(20, out, act)
+    with pytest.raises(TorporError):
+        s.stream_synchronize(20)                                     # sticky op errors + no device
+    assert s.model_info(20)["registered"] == 1
+    assert s.signal(REQ_UNLOAD, 20, "")[0] == ACK_OK

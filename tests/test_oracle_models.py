@@ -1,0 +1,123 @@
+"""Pins the whole-model oracle (oracle/models.py).  ResNet: closed-form parameter and MAC counts
+of the published v1.5 bottleneck architecture (torchvision is not installed).  BERT: the
+installed `transformers` BertModel on a small in-code config with shared weights (third-party
+code, no download).  Product-side weight generators must load strictly into these modules."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import models as om
+from torpor_amd.functions import bert as pbert
+from torpor_amd.functions import resnet as presnet
+
+
+def _macs(model, x):
+    total = [0]
+
+    def hook(mod, inp, out):
+        if isinstance(mod, torch.nn.Conv2d):
+            total[0] += out.numel() * mod.in_channels * mod.kernel_size[0] * mod.kernel_size[1]
+        elif isinstance(mod, torch.nn.Linear):
+            total[0] += out.numel() * mod.in_features
+
+    hs = [m.register_forward_hook(hook) for m in model.modules()]
+    with torch.no_grad():
+        y = model(x)
+    for h in hs:
+        h.remove()
+    return total[0], y
+
+
+def _closed_form_macs(blocks):
+    """MACs of a v1.5 bottleneck ResNet on one 224x224 image, from the architecture table alone."""
+    total = 112 * 112 * 64 * 3 * 49                      # 7x7/2 stem
+    hw, inplanes = 56, 64
+    for stage, n in enumerate(blocks):
+        planes = 64 * 2 ** stage
+        for b in range(n):
+            stride = 2 if (b == 0 and stage > 0) else 1
+            out_hw = hw // stride
+            total += hw * hw * planes * inplanes                     # 1x1 reduce (input resolution)
+            total += out_hw * out_hw * planes * planes * 9           # 3x3, carries the stride
+            total += out_hw * out_hw * planes * 4 * planes           # 1x1 expand
+            if b == 0:
+                total += out_hw * out_hw * planes * 4 * inplanes     # projection shortcut
+            hw, inplanes = out_hw, planes * 4
+    return total + 2048 * 1000
+
+
+@pytest.mark.parametrize("arch,params,gmacs", [("resnet50", 25557032, 4.089), ("resnet152", 60192808, 11.514)])
+def test_resnet_counts(arch, params, gmacs):
+    """25,557,032 / 60,192,808 parameters and 4.089 / 11.514 GMAC per 224x224 image are the
+    published figures for ResNet-50 / -152 (v1.5 moves the stride, not the counts)."""
+    model = om.ResNet(arch).eval()
+    assert sum(p.numel() for p in model.parameters()) == params
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000)
+    assert m == _closed_form_macs(om.RESNET_LAYERS[arch]), m
+    assert round(m / 1e9, 3) == gmacs
+    n_weight_tensors = len(list(model.parameters()))
+    n_bn_buffers = sum(1 for k in model.state_dict() if "running" in k)
+    assert (n_weight_tensors, n_bn_buffers) == {"resnet50": (161, 106), "resnet152": (467, 310)}[arch]
+
+
+def test_resnet_stride_is_on_the_3x3():
+    model = om.ResNet("resnet50")
+    b = model.layer2[0]
+    assert b.conv1.stride == (1, 1) and b.conv2.stride == (2, 2) and b.downsample[0].stride == (2, 2)
+    assert model.bn1.eps == 1e-5 and model.conv1.bias is None
+
+
+@pytest.mark.parametrize("arch", ["resnet50", "resnet152"])
+def test_product_resnet_weights_load_strictly(arch):
+    w = presnet.init_weights(arch, seed=0)
+    om.load_numpy_state(om.ResNet(arch), w)
+    # He-normal, fan_out: std = sqrt(2 / (cout * k * k))
+    c = w["layer1.0.conv2.weight"]
+    assert abs(c.std() - (2.0 / (64 * 9)) ** 0.5) < 2e-3
+    assert np.array_equal(presnet.init_weights(arch, seed=0)["fc.weight"], w["fc.weight"])      # deterministic
+    assert not np.array_equal(presnet.init_weights(arch, seed=1)["fc.weight"], w["fc.weight"])
+
+
+@pytest.mark.parametrize("arch,params", [("bert-base", 109482240), ("bert-large", 335141888)])
+def test_bert_param_counts(arch, params):
+    cfg = pbert.CONFIGS[arch]
+    with torch.device("meta"):
+        model = om.Bert(**cfg)
+    assert sum(p.numel() for p in model.parameters()) == params
+    assert len(list(model.parameters())) == {"bert-base": 199, "bert-large": 391}[arch]
+
+
+def test_bert_matches_transformers():
+    transformers = pytest.importorskip("transformers")
+    cfg = transformers.BertConfig(vocab_size=97, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+                                  intermediate_size=128, max_position_embeddings=40, type_vocab_size=2,
+                                  hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    torch.manual_seed(0)
+    hf = transformers.BertModel(cfg).eval()
+    assert cfg.layer_norm_eps == 1e-12 and cfg.hidden_act == "gelu"
+    mine = om.Bert(layers=2, hidden=64, heads=4, ffn=128, vocab=97, max_pos=40, type_vocab=2)
+    sd = {k: v for k, v in hf.state_dict().items() if k in mine.state_dict()}
+    assert set(sd) == set(mine.state_dict()), set(mine.state_dict()) - set(sd)
+    mine.load_state_dict(sd)
+    mine.eval()
+    ids = torch.randint(0, 97, (3, 17))
+    tt = torch.randint(0, 2, (3, 17))
+    am = torch.ones(3, 17, dtype=torch.long)
+    am[1, 11:] = 0
+    with torch.no_grad():
+        ref = hf(input_ids=ids, token_type_ids=tt, attention_mask=am)
+        h, pooled = mine(ids, tt, am)
+    assert torch.allclose(h, ref.last_hidden_state, atol=2e-5, rtol=1e-4)
+    assert torch.allclose(pooled, ref.pooler_output, atol=2e-5, rtol=1e-4)
+    with torch.no_grad():   # defaults: token types 0, no mask
+        ref0 = hf(input_ids=ids)
+        h0, p0 = mine(ids)
+    assert torch.allclose(h0, ref0.last_hidden_state, atol=2e-5, rtol=1e-4)
+
+
+def test_product_bert_weights_load_strictly():
+    cfg = dict(layers=2, hidden=64, heads=4, ffn=128)
+    w = pbert.init_weights(seed=0, vocab=97, max_pos=40, cfg=cfg)
+    om.load_numpy_state(om.Bert(vocab=97, max_pos=40, **cfg), w)
+    assert abs(w["encoder.layer.0.intermediate.dense.weight"].std() - 0.02) < 2e-3

@@ -139,6 +139,18 @@ SYMBOLS = {
     "tp_profile_begin": (C.c_int, [_P]),
     "tp_profile_end": (C.c_int, [_P]),
     "tp_profile_read": (C.c_int, [_P, _I32, C.POINTER(KernelStat)]),
+    "tp_pool_create": (_P, [_U64]),
+    "tp_pool_destroy": (None, [_P]),
+    "tp_pool_alloc": (_U64, [_P, _U64]),
+    "tp_pool_release": (C.c_int, [_P, _U64]),
+    "tp_pool_query": (C.c_int, [_P] + [C.POINTER(_U64)] * 5),
+    "tp_lru_create": (_P, [_U64]),
+    "tp_lru_destroy": (None, [_P]),
+    "tp_lru_check_and_add": (C.c_int, [_P, C.c_char_p, _U64, C.c_char_p, _U64, C.POINTER(_I32), C.POINTER(_I32)]),
+    "tp_lru_force_evict": (C.c_int, [_P, C.c_char_p]),
+    "tp_lru_lock": (C.c_int, [_P, C.c_char_p]),
+    "tp_lru_unlock": (C.c_int, [_P, C.c_char_p]),
+    "tp_lru_used": (_U64, [_P]),
 }
 
 _lib = None

@@ -392,4 +392,97 @@ int tp_profile_read(tp_server* s, int32_t index, tp_kernel_stat* out) {
     TP_GUARD_END
 }
 
+struct tp_pool {
+    tp::SlabPool pool;
+};
+struct tp_lru {
+    tp::LruEvictor lru;
+};
+
+tp_pool* tp_pool_create(uint64_t capacity_bytes) {
+    try {
+        auto* p = new tp_pool;
+        p->pool.reset(capacity_bytes);
+        return p;
+    } catch (...) {
+        return nullptr;
+    }
+}
+void tp_pool_destroy(tp_pool* p) { delete p; }
+uint64_t tp_pool_alloc(tp_pool* p, uint64_t bytes) {
+    if (!p) return UINT64_MAX;
+    try {
+        return p->pool.alloc(bytes);
+    } catch (...) {
+        return UINT64_MAX;
+    }
+}
+int tp_pool_release(tp_pool* p, uint64_t offset) {
+    TP_GUARD_BEGIN
+    if (!p) return TP_EINVAL;
+    return p->pool.release(offset) ? 0 : TP_ENOENT;
+    TP_GUARD_END
+}
+int tp_pool_query(tp_pool* p, uint64_t* capacity, uint64_t* used, uint64_t* largest_free, uint64_t* live_extents,
+                  uint64_t* free_extents) {
+    if (!p) return TP_EINVAL;
+    if (capacity) *capacity = p->pool.capacity();
+    if (used) *used = p->pool.used_bytes();
+    if (largest_free) *largest_free = p->pool.largest_free();
+    if (live_extents) *live_extents = p->pool.live_extents();
+    if (free_extents) *free_extents = p->pool.free_extents();
+    return 0;
+}
+tp_lru* tp_lru_create(uint64_t budget_bytes) {
+    try {
+        auto* l = new tp_lru;
+        l->lru.set_budget(budget_bytes);
+        return l;
+    } catch (...) {
+        return nullptr;
+    }
+}
+void tp_lru_destroy(tp_lru* l) { delete l; }
+int tp_lru_check_and_add(tp_lru* l, const char* function, uint64_t size, char* victims, uint64_t cap,
+                         int32_t* n_victims, int32_t* over_budget) {
+    TP_GUARD_BEGIN
+    if (!l || !function) return TP_EINVAL;
+    bool over = false;
+    auto v = l->lru.check_and_add(function, size, &over);
+    if (n_victims) *n_victims = (int32_t)v.size();
+    if (over_budget) *over_budget = over ? 1 : 0;
+    if (victims && cap) {
+        std::string joined;
+        for (size_t i = 0; i < v.size(); ++i) {
+            if (i) joined += '\n';
+            joined += v[i];
+        }
+        std::strncpy(victims, joined.c_str(), cap - 1);
+        victims[cap - 1] = '\0';
+    }
+    return 0;
+    TP_GUARD_END
+}
+int tp_lru_force_evict(tp_lru* l, const char* function) {
+    TP_GUARD_BEGIN
+    if (!l || !function) return TP_EINVAL;
+    return l->lru.force_evict(function) ? 1 : 0;
+    TP_GUARD_END
+}
+int tp_lru_lock(tp_lru* l, const char* function) {
+    TP_GUARD_BEGIN
+    if (!l || !function) return TP_EINVAL;
+    l->lru.lock(function);
+    return 0;
+    TP_GUARD_END
+}
+int tp_lru_unlock(tp_lru* l, const char* function) {
+    TP_GUARD_BEGIN
+    if (!l || !function) return TP_EINVAL;
+    l->lru.unlock(function);
+    return 0;
+    TP_GUARD_END
+}
+uint64_t tp_lru_used(tp_lru* l) { return l ? l->lru.cur_size() : 0; }
+
 }  // extern "C"
