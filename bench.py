@@ -94,6 +94,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         cold.append(cold_step())
         st = server.swap_stats(fid)   # waits for the tail of the copy: part of the step
         swap_ms.append(st["copy_ms"])
+        streams = st["copy_streams"]
         swap_gbps.append(st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
     server.stream_synchronize(fid)
     t_total = time.perf_counter() - t_begin
@@ -122,7 +123,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         weight_bytes=info["image_bytes"], act_bytes=info["act_bytes"], ops=info["n_ops"], chunks=info["n_chunks"],
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
-        steps_total_s=t_total,
+        copy_streams=streams, steps_total_s=t_total,
     )
     return res, kstats, empty_us, (fn, inputs, weights, first)
 

@@ -96,6 +96,8 @@ typedef struct tp_config {
     uint64_t workspace_bytes;   /* split-K scratch; 0: 64 MiB */
     int32_t flags;              /* TP_FLAG_* */
     int32_t request_timeout_ms; /* 0: 5000 (cuda_server.hpp:29) */
+    int32_t copy_streams;       /* swap-in copy streams: 0 = chosen per model, 1 or 2 */
+    int32_t reserved0;
 } tp_config;
 
 typedef struct tp_epilogue {
@@ -160,6 +162,8 @@ typedef struct tp_swap_stats {
     double evict_us;     /* host time of the last swap-out (memory_manager.hpp:258) */
     uint32_t chunks;
     uint32_t gate_waits; /* compute-stream waits issued during the last request */
+    uint32_t copy_streams; /* streams the last swap-in alternated over */
+    uint32_t reserved0;
 } tp_swap_stats;
 
 /* ------------------------------------------------------------------ lifecycle

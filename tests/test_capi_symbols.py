@@ -37,7 +37,7 @@ def test_version_and_strerror():
 
 def test_struct_sizes_match_the_header_layout():
     # natural alignment of the fields as declared in include/torpor_amd.h
-    assert ctypes.sizeof(_lib.Config) == 56
+    assert ctypes.sizeof(_lib.Config) == 64
     assert ctypes.sizeof(_lib.Epilogue) == 72
     assert ctypes.sizeof(_lib.GemmDesc) == 3 * 8 + 8 * 8 + 8 + 6 * 8 + 72
     assert ctypes.sizeof(_lib.ConvDesc) == 3 * 8 + 14 * 4 + 72

@@ -100,6 +100,9 @@ struct Model {
     std::atomic<bool> cancel{false};
     std::atomic<int> copy_error{0};
     uint32_t gated_upto = 0;
+    int ncopy = 2;            // copy streams used by the current swap-in plan
+    uint64_t chunk_max = 0;   // largest transfer group of the current plan
+    double warm_us = 0;       // best warm replay so far (host wall clock), 0 = none yet
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing_valid = false;
     // recorded program
@@ -197,6 +200,7 @@ private:
     int finish_tracking(Model& m);
     int build_image(Model& m, bool by_access);
     void build_chunks(Model& m);
+    void choose_copy_plan(Model& m);
     void wait_copy_idle(Model& m);
     void copy_main();
     int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
@@ -210,7 +214,9 @@ private:
     LruEvictor lru_;
     uint8_t* arena_ = nullptr;
     float* workspace_ = nullptr;
-    hipStream_t compute_ = nullptr, copy_ = nullptr;
+    hipStream_t compute_ = nullptr, copy_ = nullptr, copy2_ = nullptr;
+    int copy_streams_cfg_ = 0;
+    bool chunk_max_auto_ = true;
     std::unordered_map<int, std::unique_ptr<Model>> models_;
 
     int active_ = -1;

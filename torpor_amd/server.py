@@ -33,7 +33,7 @@ def _as_bytes_view(a):
 
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
-                 device=0, host_only=False, request_timeout_ms=0):
+                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0):
         self._l = _lib.lib()
         cfg = _lib.Config()
         cfg.struct_size = C.sizeof(_lib.Config)
@@ -45,6 +45,7 @@ class Server:
         cfg.workspace_bytes = workspace_bytes
         cfg.flags = FLAG_HOST_ONLY if host_only else 0
         cfg.request_timeout_ms = request_timeout_ms
+        cfg.copy_streams = copy_streams
         h = C.c_void_p()
         _chk(self._l.tp_server_create(C.byref(cfg), C.byref(h)), "tp_server_create")
         self._h = h
