@@ -1009,7 +1009,9 @@ static tpk::EpilogueArgs ep_from(const Op& op, void* const* q, int pbase, int fb
 //  LAUNCH p/i/f per op id (see torpor_amd.h)
 int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
     void* q[12] = {nullptr};
-    const tpk::Workspace ws{workspace_, (size_t)cfg_.workspace_bytes};
+    // the first 256 bytes of the scratch allocation stay zero for good (padding source of the
+    // 3x3 convolution); split-K partial sums live behind them
+    const tpk::Workspace ws{workspace_ + 64, (size_t)cfg_.workspace_bytes - 256, workspace_};
     // Every operand is translated together with the byte span the kernel will touch, so an op
     // whose shapes do not fit its buffers is refused on the host instead of faulting the GPU.
     auto R = [&](int idx, bool optional, int64_t elems, int64_t elem_size = 4) -> int {

@@ -33,6 +33,7 @@ struct ConvDev {
     int splits;
     long kper;  // K (generic) or channels (3x3 fast) per split
     float* ws;
+    const float* zeros;
     int tiles_m, tiles_n;
     Epilogue ep;
 };
@@ -64,30 +65,35 @@ __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvD
     const int cbeg = split * (int)p.kper;
     const int cend = (cbeg + (int)p.kper < p.Cin) ? cbeg + (int)p.kper : p.Cin;
 
+    // Branch-free operand fetch: rows past the last pixel are clamped to it (computed, then
+    // dropped at the store) and taps that fall into the padding read from a page of zeros with
+    // a zero channel step, so every load in the loop is unconditional.
     constexpr int NVA = (C::BM * 18 + C::THREADS - 1) / C::THREADS;
-    long offA[NVA];
+    const float* pa[NVA];
+    int stepA[NVA];
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
-        const int idx = i * C::THREADS + tid;
+        int idx = i * C::THREADS + tid;
+        if (idx > C::BM * 18 - 1) idx = C::BM * 18 - 1;
         const int row = idx / 18, t2 = idx - row * 18;
         const int tap = t2 >> 1, cq = t2 & 1;
-        offA[i] = -1;
-        const long grow = m0 + row;
-        if (idx < C::BM * 18 && grow < p.M) {
-            const int wo = (int)(grow % p.Wo);
-            const long tt = grow / p.Wo;
-            const int ho = (int)(tt % p.Ho);
-            const long n = tt / p.Ho;
-            const int hi = ho * p.sh - p.ph + tap / 3;
-            const int wi = wo * p.sw - p.pw + tap % 3;
-            if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W)
-                offA[i] = n * p.xs_n + (long)hi * p.xs_h + (long)wi * p.xs_w + cq * 4;
-        }
+        long grow = m0 + row;
+        if (grow > p.M - 1) grow = p.M - 1;
+        const int wo = (int)(grow % p.Wo);
+        const long tt = grow / p.Wo;
+        const int ho = (int)(tt % p.Ho);
+        const long n = tt / p.Ho;
+        const int hi = ho * p.sh - p.ph + tap / 3;
+        const int wi = wo * p.sw - p.pw + tap % 3;
+        const bool inside = hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
+        pa[i] = inside ? p.x + n * p.xs_n + (long)hi * p.xs_h + (long)wi * p.xs_w + cq * 4 : p.zeros;
+        stepA[i] = inside ? 1 : 0;
     }
     // weight assignment: thread -> (col = tid/2, cq = tid%2)
     const int wcol = tid >> 1, wcq = tid & 1;
-    const bool wact = (tid < C::BN * 2) && (n0 + wcol < p.Cout);
-    const float* __restrict__ wbase = p.w + ((n0 + wcol) * (long)p.Cin + wcq * 4) * 9;
+    long wc = n0 + wcol;
+    if (wc > p.Cout - 1) wc = p.Cout - 1;
+    const float* __restrict__ wbase = p.w + (wc * (long)p.Cin + wcq * 4) * 9;
 
     f32x16 acc[C::TM][C::TN];
     zero_acc<C>(acc);
@@ -95,17 +101,12 @@ __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvD
     f32x4 rw[9];
 
     auto load_regs = [&](int c0) {
+        if (c0 > cend - 8) c0 = cend - 8;  // look-ahead past the end re-reads the last block
 #pragma unroll
-        for (int i = 0; i < NVA; ++i) {
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (offA[i] >= 0) v = *reinterpret_cast<const f32x4*>(p.x + offA[i] + c0);
-            ra[i] = v;
-        }
+        for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + c0 * stepA[i]);
+        if (tid < C::BN * 2) {
 #pragma unroll
-        for (int j = 0; j < 9; ++j) {
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (wact) v = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * 9 + j * 4);
-            rw[j] = v;
+            for (int j = 0; j < 9; ++j) rw[j] = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * 9 + j * 4);
         }
     };
     auto store_lds = [&]() {
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvD
     for (int c0 = cbeg; c0 < cend; c0 += 8) {
         store_lds();
         __syncthreads();
-        if (c0 + 8 < cend) load_regs(c0 + 8);
+        load_regs(c0 + 8);
         mma_block<C>(As, Bs, acc, wm, wn, lane);
         __syncthreads();
     }
@@ -293,6 +294,7 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     p.M = M;
     p.K = (long)a.Cin * a.KH * a.KW;
     p.ws = ws.ptr;
+    p.zeros = ws.zeros;
     EpilogueArgs ea = a.ep;
     if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;
     p.ep = make_epilogue(ea, a.Cout);
@@ -302,7 +304,8 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         p.ep.ncols = a.Cout;
     }
 
-    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && aligned16c(a.x) && aligned16c(a.w);
+    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && aligned16c(a.x) &&
+                       aligned16c(a.w) && ws.zeros != nullptr;
     if (fast3) {
         const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);
         const bool big = tl >= 2L * num_cu();

@@ -13,6 +13,8 @@
 #include "kernels.hpp"
 #include "mfma_tile.hpp"
 
+#include <cstdlib>
+
 namespace tpk {
 
 static int g_num_cu = 256;
@@ -61,10 +63,10 @@ __device__ __forceinline__ long gather_row(const GemmDev& p, long grow) {
 }
 
 template <class C, bool YKC>
-__global__ __launch_bounds__(C::THREADS, 2) void gemm_fast_kernel(const GemmDev p) {
-    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
-    float* As = lds;
-    float* Bs = lds + C::BM * C::LDK;
+__global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_fast_kernel(const GemmDev p) {
+    // two LDS stages: while the MFMAs read one, the next K-block is written to the other, so
+    // the loop needs a single barrier per K-block
+    __shared__ __attribute__((aligned(16))) float lds[2 * C::LDS_FLOATS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / C::WGN, wn = wave % C::WGN;
     const int t = remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n);
@@ -114,9 +116,10 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fast_kernel(const GemmDev 
 
     f32x16 acc[C::TM][C::TN];
     zero_acc<C>(acc);
-    f32x4 ra[NVA], rb[NVB];
+    // two register sets: the global loads run two K-blocks ahead of the MFMAs
+    f32x4 ra0[NVA], rb0[NVB], ra1[NVA], rb1[NVB];
 
-    auto load_regs = [&](long k0) {
+    auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0) {
 #pragma unroll
         for (int i = 0; i < NVA; ++i) {
             const int idx = i * C::THREADS + tid;
@@ -149,7 +152,9 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fast_kernel(const GemmDev 
             rb[i] = v;
         }
     };
-    auto store_lds = [&]() {
+    auto store_lds = [&](const f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage) {
+        float* As = lds + stage * C::LDS_FLOATS;
+        float* Bs = As + C::BM * C::LDK;
 #pragma unroll
         for (int i = 0; i < NVA; ++i) {
             const int idx = i * C::THREADS + tid;
@@ -172,13 +177,159 @@ __global__ __launch_bounds__(C::THREADS, 2) void gemm_fast_kernel(const GemmDev 
         }
     };
 
-    load_regs(kbeg);
-    for (long k0 = kbeg; k0 < kend; k0 += C::BK) {
-        store_lds();
+    // K-block i lives in LDS stage i&1 and travels through register set i&1.  While block i is
+    // multiplied, block i+2 is requested from memory and block i+1 (requested one iteration ago)
+    // moves from registers to the other LDS stage; one barrier per K-block.  Loads past the end
+    // of K are predicated off and yield zeros, so the tail needs no special casing.
+    const float* As0 = lds;
+    const float* As1 = lds + C::LDS_FLOATS;
+    load_regs(ra0, rb0, kbeg);
+    load_regs(ra1, rb1, kbeg + C::BK);
+    store_lds(ra0, rb0, 0);
+    __syncthreads();
+    for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
+        load_regs(ra0, rb0, k0 + 2 * C::BK);
+        mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+        store_lds(ra1, rb1, 1);
         __syncthreads();
-        if (k0 + C::BK < kend) load_regs(k0 + C::BK);
-        mma_block<C>(As, Bs, acc, wm, wn, lane);
+        // no early exit between the halves: with an odd number of K-blocks the second half
+        // multiplies a block of zeros, which is cheaper than the accumulator shuffling a
+        // mid-loop exit costs on every iteration
+        load_regs(ra1, rb1, k0 + 3 * C::BK);
+        mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane);
+        store_lds(ra0, rb0, 0);
         __syncthreads();
+    }
+    float* partial = nullptr;
+    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial);
+}
+
+// Branch-free variant of gemm_fast_kernel for the common case: K covered by an even number of
+// whole K-blocks per split.  Rows / columns past the edge are clamped to the last valid one
+// (their products are computed and thrown away at the store) and the look-ahead loads past the
+// end of K are clamped to the last K-block, so the loop body has no predication and no control
+// flow: loads, LDS traffic and MFMAs can be interleaved freely by the scheduler.
+template <class C, bool YKC, int STAGES>
+__global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_clean_kernel(const GemmDev p) {
+    __shared__ __attribute__((aligned(16))) float lds[STAGES * C::LDS_FLOATS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int t = remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n);
+    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
+    int split = 0, batch = blockIdx.z;
+    if (p.splits > 1) {
+        split = blockIdx.z;
+        batch = 0;
+    }
+    const int b0 = batch / p.nb1, b1 = batch - b0 * p.nb1;
+    const float* __restrict__ X = p.X + b0 * p.xb0 + b1 * p.xb1;
+    const float* __restrict__ Y = p.Y + b0 * p.yb0 + b1 * p.yb1;
+    float* __restrict__ Cc = p.C + b0 * p.cb0 + b1 * p.cb1;
+    const long kbeg = (long)split * p.kper;
+    const long kend = (kbeg + p.kper < p.K) ? kbeg + p.kper : p.K;
+    const long klast = kend - C::BK;
+
+    constexpr int KV = C::BK / 4;
+    constexpr int CV = C::BN / 4;
+    constexpr int NVA = C::BM * KV / C::THREADS;
+    constexpr int NVB = (YKC ? C::BN * KV : C::BK * CV) / C::THREADS;
+    static_assert(C::BM * KV % C::THREADS == 0 && C::BN * KV % C::THREADS == 0 && C::BK * CV % C::THREADS == 0,
+                  "tile must split evenly over the workgroup");
+
+    const float* pa[NVA];
+    const float* pb[NVB];
+    int sa[NVA], sb[NVB];  // LDS offsets
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) {
+        const int idx = i * C::THREADS + tid;
+        const int row = idx / KV, kq = idx - row * KV;
+        long grow = m0 + row;
+        if (grow > p.M - 1) grow = p.M - 1;
+        pa[i] = X + gather_row(p, grow) * p.xs_r + kq * 4;
+        sa[i] = row * C::LDK + kq * 4;
+    }
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+        const int idx = i * C::THREADS + tid;
+        if (YKC) {
+            const int col = idx / KV, kq = idx - col * KV;
+            long gcol = n0 + col;
+            if (gcol > p.N - 1) gcol = p.N - 1;
+            pb[i] = Y + gcol * p.ys_c + kq * 4;
+            sb[i] = col * C::LDK + kq * 4;
+        } else {
+            const int kk = idx / CV, cq = idx - kk * CV;
+            long gcol = n0 + cq * 4;
+            if (gcol > p.N - 4) gcol = p.N - 4;
+            pb[i] = Y + kk * p.ys_k + gcol;
+            sb[i] = (cq * 4) * C::LDK + kk;
+        }
+    }
+    const long ystep = YKC ? 1 : p.ys_k;
+
+    f32x16 acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    f32x4 ra0[NVA], rb0[NVB], ra1[NVA], rb1[NVB];
+
+    auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0) {
+        const long k = k0 < klast ? k0 : klast;
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + k);
+#pragma unroll
+        for (int i = 0; i < NVB; ++i) rb[i] = *reinterpret_cast<const f32x4*>(pb[i] + k * ystep);
+    };
+    auto store_lds = [&](const f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage) {
+        float* As = lds + stage * C::LDS_FLOATS;
+        float* Bs = As + C::BM * C::LDK;
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < NVB; ++i) {
+            if (YKC) {
+                *reinterpret_cast<f32x4*>(Bs + sb[i]) = rb[i];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) Bs[sb[i] + j * C::LDK] = rb[i][j];
+            }
+        }
+    };
+
+    const float* As0 = lds;
+    if (STAGES == 2) {
+        const float* As1 = lds + C::LDS_FLOATS;
+        load_regs(ra0, rb0, kbeg);
+        load_regs(ra1, rb1, kbeg + C::BK);
+        store_lds(ra0, rb0, 0);
+        __syncthreads();
+        for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
+            load_regs(ra0, rb0, k0 + 2 * C::BK);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            store_lds(ra1, rb1, 1);
+            __syncthreads();
+            load_regs(ra1, rb1, k0 + 3 * C::BK);
+            mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane);
+            store_lds(ra0, rb0, 0);
+            __syncthreads();
+        }
+    } else {
+        // one LDS stage, two barriers per K-block: half the LDS footprint, so twice as many
+        // workgroups stay resident and hide each other's barrier and memory latency
+        load_regs(ra0, rb0, kbeg);
+        load_regs(ra1, rb1, kbeg + C::BK);
+        for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
+            store_lds(ra0, rb0, 0);
+            __syncthreads();
+            load_regs(ra0, rb0, k0 + 2 * C::BK);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            __syncthreads();
+            store_lds(ra1, rb1, 0);
+            __syncthreads();
+            load_regs(ra1, rb1, k0 + 3 * C::BK);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            __syncthreads();
+        }
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
@@ -303,8 +454,51 @@ int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, 
     return (int)hipGetLastError();
 }
 
-using CfgL = TileCfg<128, 128, 32, 2, 2>;
-using CfgM = TileCfg<64, 64, 32, 2, 2>;
+using CfgL = TileCfg<128, 128, 32, 2, 2>;  // 2x2 accumulators per wavefront
+using CfgW = TileCfg<128, 64, 32, 2, 2>;   // 2x1
+using CfgM = TileCfg<64, 64, 32, 2, 2>;    // 1x1
+
+template <class C>
+static void launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipStream_t s) {
+    // With many tiles per CU a single LDS stage wins (twice the resident workgroups hide each
+    // other's latencies: 99 vs 94 TFLOP/s on 1536x4096x1024); with one or two tiles per CU the
+    // two-stage loop with its single barrier per K-block does (83 vs 79 on 1536x1024x4096).
+    const long tiles = (long)grid.x * grid.z;
+    const bool one_stage = tiles >= 5L * g_num_cu;
+    if (clean && one_stage) {
+        if (y_kc)
+            hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
+        else
+            hipLaunchKernelGGL((gemm_clean_kernel<C, false, 1>), grid, dim3(C::THREADS), 0, s, p);
+    } else if (clean) {
+        if (y_kc)
+            hipLaunchKernelGGL((gemm_clean_kernel<C, true, 2>), grid, dim3(C::THREADS), 0, s, p);
+        else
+            hipLaunchKernelGGL((gemm_clean_kernel<C, false, 2>), grid, dim3(C::THREADS), 0, s, p);
+    } else {
+        if (y_kc)
+            hipLaunchKernelGGL((gemm_fast_kernel<C, true>), grid, dim3(C::THREADS), 0, s, p);
+        else
+            hipLaunchKernelGGL((gemm_fast_kernel<C, false>), grid, dim3(C::THREADS), 0, s, p);
+    }
+}
+
+// Tile shape.  Measured on MI355X over the served shapes (BERT-large 1536 x {1024,4096} x
+// {1024,4096}, ResNet 1x1 convolutions from 25088x256x64 to 392x2048x512), the 64x64 tile is
+// the fastest everywhere: it keeps the most workgroups resident per CU, and for fp32 MFMA
+// (2 k per instruction) occupancy hides more latency than larger register tiles save in LDS
+// traffic.  The 128x128 / 128x64 variants are kept for very large grids and for experiments
+// (TORPOR_GEMM_CFG=0/1/2 forces one).
+static int choose_tile(long M, long N, int batch) {
+    static const int forced = [] {
+        const char* e = getenv("TORPOR_GEMM_CFG");
+        return e ? atoi(e) : -1;
+    }();
+    if (forced >= 0 && forced <= 2) return forced;
+    const long tiles_w = ((M + 127) / 128) * ((N + 63) / 64) * batch;
+    if (tiles_w >= 64L * g_num_cu) return 1;  // enough 128x64 tiles to keep every CU full for long
+    return 2;
+}
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -322,6 +516,7 @@ int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, l
         if (want > 1) splits = (int)want;
     }
     long per_blocks = (kblocks + splits - 1) / splits;
+    if (splits > 1 && (per_blocks & 1)) ++per_blocks;  // whole pairs of K-blocks per split
     splits = (int)((kblocks + per_blocks - 1) / per_blocks);
     *kper_out = per_blocks * bk;
     return splits;
@@ -369,32 +564,27 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     const bool y_fast = (y_kc || y_cc) && aligned16(a.Y) && (a.yb0 % 4 == 0) && (a.yb1 % 4 == 0);
 
     if (x_fast && y_fast) {
-        const long tl = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
-        const bool big = tl >= 2L * g_num_cu;
-        const int bm = big ? 128 : 64;
+        const int cfg = choose_tile(a.M, a.N, batch);
+        const int bm = cfg == 2 ? 64 : 128, bn = cfg == 0 ? 128 : 64;
         p.tiles_m = (int)((a.M + bm - 1) / bm);
-        p.tiles_n = (int)((a.N + bm - 1) / bm);
+        p.tiles_n = (int)((a.N + bn - 1) / bn);
         const long tiles = (long)p.tiles_m * p.tiles_n * batch;
         p.splits = 1;
         p.kper = ((a.K + 31) / 32) * 32;
         if (batch == 1) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits > 1 ? p.splits : batch);
-        if (big) {
-            if (y_kc) {
-                hipLaunchKernelGGL((gemm_fast_kernel<CfgL, true>), grid, dim3(256), 0, s, p);
-                g_last_kernel = "gemm_fast_128x128_kc";
-            } else {
-                hipLaunchKernelGGL((gemm_fast_kernel<CfgL, false>), grid, dim3(256), 0, s, p);
-                g_last_kernel = "gemm_fast_128x128_cc";
-            }
+        static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
+        const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
+                           (y_kc || (a.N % 4 == 0 && a.N >= 4));
+        if (cfg == 0) {
+            launch_fast<CfgL>(p, y_kc, clean, grid, s);
+            g_last_kernel = y_kc ? "gemm_fast_128x128_kc" : "gemm_fast_128x128_cc";
+        } else if (cfg == 1) {
+            launch_fast<CfgW>(p, y_kc, clean, grid, s);
+            g_last_kernel = y_kc ? "gemm_fast_128x64_kc" : "gemm_fast_128x64_cc";
         } else {
-            if (y_kc) {
-                hipLaunchKernelGGL((gemm_fast_kernel<CfgM, true>), grid, dim3(256), 0, s, p);
-                g_last_kernel = "gemm_fast_64x64_kc";
-            } else {
-                hipLaunchKernelGGL((gemm_fast_kernel<CfgM, false>), grid, dim3(256), 0, s, p);
-                g_last_kernel = "gemm_fast_64x64_cc";
-            }
+            launch_fast<CfgM>(p, y_kc, clean, grid, s);
+            g_last_kernel = y_kc ? "gemm_fast_64x64_kc" : "gemm_fast_64x64_cc";
         }
     } else {
         p.tiles_m = (int)((a.M + 63) / 64);

@@ -54,6 +54,7 @@ struct ConvArgs {
 struct Workspace {
     float* ptr = nullptr;  // split-K partial sums
     size_t bytes = 0;
+    const float* zeros = nullptr;  // >= 64 zero bytes, 16 B aligned: source for padded convolution taps
 };
 
 void kernels_init(int device);  // caches CU count

@@ -103,7 +103,9 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[C::TM][C::TN]) {
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 }
 
-// Multiply the LDS-resident BM x BK and BN x BK tiles into the accumulators.
+// Multiply the LDS-resident BM x BK and BN x BK tiles into the accumulators.  The operand
+// fragments of k-group g+1 are fetched from LDS before the MFMAs of group g are issued, so the
+// LDS latency hides behind matrix work instead of stalling every eighth MFMA.
 template <class C>
 __device__ __forceinline__ void mma_block(const float* __restrict__ As, const float* __restrict__ Bs,
                                           f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane) {
@@ -111,20 +113,30 @@ __device__ __forceinline__ void mma_block(const float* __restrict__ As, const fl
     const int h = lane >> 5;
     const float* ap = As + (wm * C::WTM + r) * C::LDK + 4 * h;
     const float* bp = Bs + (wn * C::WTN + r) * C::LDK + 4 * h;
+    constexpr int G = C::BK / 8;
+    f32x4 a[2][C::TM], b[2][C::TN];
 #pragma unroll
-    for (int kk = 0; kk < C::BK; kk += 8) {
-        f32x4 a[C::TM], b[C::TN];
+    for (int i = 0; i < C::TM; ++i) a[0][i] = *reinterpret_cast<const f32x4*>(ap + i * 32 * C::LDK);
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) a[i] = *reinterpret_cast<const f32x4*>(ap + i * 32 * C::LDK + kk);
+    for (int j = 0; j < C::TN; ++j) b[0][j] = *reinterpret_cast<const f32x4*>(bp + j * 32 * C::LDK);
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) b[j] = *reinterpret_cast<const f32x4*>(bp + j * 32 * C::LDK + kk);
+    for (int g = 0; g < G; ++g) {
+        const int cur = g & 1, nxt = cur ^ 1;
+        if (g + 1 < G) {
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+                a[nxt][i] = *reinterpret_cast<const f32x4*>(ap + i * 32 * C::LDK + (g + 1) * 8);
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j)
+                b[nxt][j] = *reinterpret_cast<const f32x4*>(bp + j * 32 * C::LDK + (g + 1) * 8);
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
             for (int i = 0; i < C::TM; ++i)
 #pragma unroll
                 for (int j = 0; j < C::TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][s], b[cur][j][s], acc[i][j], 0, 0, 0);
     }
 }
 
