@@ -140,3 +140,37 @@ def test_gemm_rejects_out_of_bounds(gpu_server):
         with pytest.raises(TorporError):
             t.s.stream_synchronize(t.fid)   # the refused ops are also reported (once) at the next sync
         t.s.gemm(t.fid, x, t.w[0], c, 4, 8, 8, xs_r=8, ys_c=8, ldc=8)
+
+
+@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "128x64"), (2, "64x64")])
+def test_forced_tile_configs(cfg, name):
+    """Every tile shape of the fast kernel (TORPOR_GEMM_CFG forces one; read once per process,
+    hence the subprocess): ragged and exact shapes, predicated and branch-free variants."""
+    import os
+    import subprocess
+    import sys
+    code = r'''
+import numpy as np, sys
+from torpor_amd.server import Server
+from tests.harness import OpSession, assert_close
+rng = np.random.default_rng(0)
+with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
+    for (M, N, K) in [(200, 136, 128), (257, 130, 100), (64, 64, 64), (300, 520, 192)]:
+        X = rng.standard_normal((M, K)).astype(np.float32)
+        W = rng.standard_normal((N, K)).astype(np.float32)
+        V = rng.standard_normal((K, N)).astype(np.float32)
+        with OpSession(s, [W]) as t:
+            x, v = t.act(X), t.act(V)
+            c = t.empty(M * N * 4)
+            s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N)
+            assert sys.argv[1] in s.last_kernel(), s.last_kernel()
+            assert_close(t.read(c, (M, N)), X.astype(np.float64) @ W.astype(np.float64).T, 2e-5, "kc")
+            s.gemm(t.fid, x, v, c, M, N, K, xs_r=K, ys_c=1, ys_k=N, ldc=N)
+            assert_close(t.read(c, (M, N)), X.astype(np.float64) @ V.astype(np.float64), 2e-5, "cc")
+print("ok")
+'''
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, TORPOR_GEMM_CFG=str(cfg), PYTHONPATH=root)
+    r = subprocess.run([sys.executable, "-c", code, name], env=env, cwd=root, capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr

@@ -42,6 +42,7 @@ struct GemmDev {
     long kper;
     float* ws;
     int tiles_m, tiles_n;
+    int xr, xc;  // the 8 XCDs form an xr x xc grid over the tile grid (xr*xc == 8), 0 = linear mapping
     Epilogue ep;
 };
 
@@ -51,6 +52,32 @@ __device__ __forceinline__ int remap_xcd(int bid, int n) {
     const int q = n >> 3, rem = n & 7;
     const int xcd = bid & 7, local = bid >> 3;
     return xcd * q + (xcd < rem ? xcd : rem) + local;
+}
+
+// Workgroup -> tile with a 2-D partition over the XCDs.  XCD x = bid % 8 owns the rectangle
+// (x / xc, x % xc) of an xr x xc split of the tile grid, so that its private L2 sees only
+// 1/xr of the X rows and 1/xc of the Y rows.  The grid is padded to 8 * (largest rectangle);
+// workgroups beyond their XCD's rectangle return false and exit.
+__device__ __forceinline__ bool tile_of(const GemmDev& p, int bid, int* tm, int* tn, int* t) {
+    if (p.xr == 0) {
+        const int n = p.tiles_m * p.tiles_n;
+        if (bid >= n) return false;
+        *t = remap_xcd(bid, n);
+        *tm = *t / p.tiles_n;
+        *tn = *t - *tm * p.tiles_n;
+        return true;
+    }
+    const int xcd = bid & 7, local = bid >> 3;
+    const int br = xcd / p.xc, bc = xcd - br * p.xc;
+    const int r0 = (int)((long)p.tiles_m * br / p.xr), r1 = (int)((long)p.tiles_m * (br + 1) / p.xr);
+    const int c0 = (int)((long)p.tiles_n * bc / p.xc), c1 = (int)((long)p.tiles_n * (bc + 1) / p.xc);
+    const int w = c1 - c0, h = r1 - r0;
+    if (local >= w * h) return false;
+    const int lr = local / w;
+    *tm = r0 + lr;
+    *tn = c0 + (local - lr * w);
+    *t = *tm * p.tiles_n + *tn;
+    return true;
 }
 
 __device__ __forceinline__ long gather_row(const GemmDev& p, long grow) {
@@ -69,8 +96,8 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
     __shared__ __attribute__((aligned(16))) float lds[2 * C::LDS_FLOATS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / C::WGN, wn = wave % C::WGN;
-    const int t = remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n);
-    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    int tm, tn, t;
+    if (!tile_of(p, blockIdx.x, &tm, &tn, &t)) return;
     const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
 
     int split = 0, batch = blockIdx.z;
@@ -215,8 +242,8 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
     __shared__ __attribute__((aligned(16))) float lds[STAGES * C::LDS_FLOATS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / C::WGN, wn = wave % C::WGN;
-    const int t = remap_xcd(blockIdx.x, p.tiles_m * p.tiles_n);
-    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    int tm, tn, t;
+    if (!tile_of(p, blockIdx.x, &tm, &tn, &t)) return;
     const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
     int split = 0, batch = blockIdx.z;
     if (p.splits > 1) {
@@ -454,6 +481,33 @@ int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, 
     return (int)hipGetLastError();
 }
 
+// XCD partition of the tile grid: X is re-fetched once per column group and Y once per row
+// group, so pick the split of 8 that moves the fewest bytes; returns the padded grid.x.
+static int plan_xcd_grid(GemmDev& p, long M, long N) {
+    const int cand[4][2] = {{1, 8}, {2, 4}, {4, 2}, {8, 1}};
+    double best = 1e300;
+    p.xr = 0;
+    p.xc = 0;
+    for (auto& c : cand) {
+        if (c[0] > p.tiles_m || c[1] > p.tiles_n) continue;
+        const double cost = (double)M * c[1] + (double)N * c[0];
+        if (cost < best) {
+            best = cost;
+            p.xr = c[0];
+            p.xc = c[1];
+        }
+    }
+    if (p.xr == 0) return p.tiles_m * p.tiles_n;  // fewer tiles than a split needs: linear mapping
+    int biggest = 0;
+    for (int br = 0; br < p.xr; ++br)
+        for (int bc = 0; bc < p.xc; ++bc) {
+            const int h = (int)((long)p.tiles_m * (br + 1) / p.xr) - (int)((long)p.tiles_m * br / p.xr);
+            const int w = (int)((long)p.tiles_n * (bc + 1) / p.xc) - (int)((long)p.tiles_n * bc / p.xc);
+            if (h * w > biggest) biggest = h * w;
+        }
+    return 8 * biggest;
+}
+
 using CfgL = TileCfg<128, 128, 32, 2, 2>;  // 2x2 accumulators per wavefront
 using CfgW = TileCfg<128, 64, 32, 2, 2>;   // 2x1
 using CfgM = TileCfg<64, 64, 32, 2, 2>;    // 1x1
@@ -463,7 +517,7 @@ static void launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipS
     // With many tiles per CU a single LDS stage wins (twice the resident workgroups hide each
     // other's latencies: 99 vs 94 TFLOP/s on 1536x4096x1024); with one or two tiles per CU the
     // two-stage loop with its single barrier per K-block does (83 vs 79 on 1536x1024x4096).
-    const long tiles = (long)grid.x * grid.z;
+    const long tiles = (long)p.tiles_m * p.tiles_n * grid.z;
     const bool one_stage = tiles >= 5L * g_num_cu;
     if (clean && one_stage) {
         if (y_kc)
@@ -572,7 +626,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         p.splits = 1;
         p.kper = ((a.K + 31) / 32) * 32;
         if (batch == 1) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
-        dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits > 1 ? p.splits : batch);
+        dim3 grid(plan_xcd_grid(p, a.M, a.N), 1, p.splits > 1 ? p.splits : batch);
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
@@ -593,6 +647,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         p.splits = 1;
         p.kper = ((a.K + 15) / 16) * 16;
         if (batch == 1) p.splits = choose_splits(tiles, a.K, 16, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
+        p.xr = p.xc = 0;
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits > 1 ? p.splits : batch);
         hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, s, p);
         g_last_kernel = "gemm_generic_64x64";
