@@ -18,6 +18,7 @@ seeded model timed on this box's host cores (oracle/models.py, a reported baseli
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -128,23 +129,37 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
     return res, kstats, empty_us, (fn, inputs, weights, first)
 
 
-def roofline_from(kstats, empty_us):
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` in `workload`, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE runs of this same script, scaled by the copy-kernel calibration
+    stated in that file); None when no summary covers this workload / kernel."""
+    path = os.path.join(ROOT, "profiles", workload.replace("-", "_") + "_pmc_traffic.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"^traffic_bytes_per_launch\[" + re.escape(kernel) + r"\]:\s*(\d+)", text, re.M)
+    return int(m.group(1)) if m else None
+
+
+def roofline_from(kstats, empty_us, workload):
     """Dominant kernel = largest summed duration; achieved = algorithmic work / time."""
     if not kstats:
         return None
     name, st = max(kstats.items(), key=lambda kv: kv[1]["total_us"])
+    traffic = measured_traffic(workload, name)
     n = st["launches"]
     t_us = max(st["total_us"] - n * empty_us, 1e-3)
     avg_us = t_us / n
     if st["flops"] > 0:
         ach = st["flops"] / (t_us * 1e-6) / 1e12
         return dict(kernel=name, bound="mfma", achieved=ach, peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s",
-                    frac=ach / PEAK_FP32_MFMA_TFLOPS, traffic=None, launches=n, avg_launch_us=avg_us,
-                    event_overhead_us=empty_us, flop_per_launch=st["flops"] / n,
+                    frac=ach / PEAK_FP32_MFMA_TFLOPS, traffic=traffic, launches=n, avg_launch_us=avg_us,
+                    event_overhead_us=empty_us, flop_per_launch=st["flops"] / n, bytes_per_launch=st["bytes"] / n,
                     hbm_gbps=st["bytes"] / (t_us * 1e-6) / 1e9)
     ach = st["bytes"] / (t_us * 1e-6) / 1e9
     return dict(kernel=name, bound="hbm", achieved=ach, peak=PEAK_HBM_GBPS, unit="GB/s", frac=ach / PEAK_HBM_GBPS,
-                traffic=None, launches=n, avg_launch_us=avg_us, event_overhead_us=empty_us,
+                traffic=traffic, launches=n, avg_launch_us=avg_us, event_overhead_us=empty_us,
                 bytes_per_launch=st["bytes"] / n)
 
 
@@ -211,7 +226,7 @@ def main():
     for fid, name in enumerate(names):
         res, kstats, empty_us, ctx = run_workload(server, fid, name, args.steps, args.warmup, link)
         results[name] = res
-        roof[name] = roofline_from(kstats, empty_us)
+        roof[name] = roofline_from(kstats, empty_us, name)
         res["kernels"] = {k: dict(launches=v["launches"], avg_us=max(v["total_us"] / v["launches"] - empty_us, 0.0),
                                   tflops=(v["flops"] / max(v["total_us"] - v["launches"] * empty_us, 1e-3) / 1e6),
                                   gbps=(v["bytes"] / max(v["total_us"] - v["launches"] * empty_us, 1e-3) / 1e3))

@@ -34,7 +34,7 @@ def test_gemm_tn(gpu_server, M, N, K, kernel):
         c = t.empty(M * N * 4)
         t.s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=max(K, 1), ys_c=max(K, 1), ldc=N, bias=t.w[1])
         if kernel:
-            assert t.s.last_kernel() == kernel
+            assert t.s.last_kernel().startswith(kernel), t.s.last_kernel()
         got = t.read(c, (M, N))
     if M * N * K > 5e7:   # too slow for the triple loop: fp64 BLAS matmul instead
         want = X.astype(np.float64) @ W.astype(np.float64).T + b
@@ -99,7 +99,7 @@ def test_attention_gemms(gpu_server, B, A, S, dh):
         k2 = t.s.last_kernel()
         got_ctx = t.read(ctx, (B, S, A, dh))
     if dh % 4 == 0 and S % 4 == 0:
-        assert k1.endswith("_kc") and k2.endswith("_cc"), (k1, k2)
+        assert "_kc" in k1 and "_cc" in k2, (k1, k2)
     Qh = Q.reshape(B, S, A, dh).transpose(0, 2, 1, 3).astype(np.float64)
     Kh = Kx.reshape(B, S, A, dh).transpose(0, 2, 1, 3).astype(np.float64)
     Vh = V.reshape(B, S, A, dh).transpose(0, 2, 1, 3).astype(np.float64)

@@ -512,8 +512,9 @@ using CfgL = TileCfg<128, 128, 32, 2, 2>;  // 2x2 accumulators per wavefront
 using CfgW = TileCfg<128, 64, 32, 2, 2>;   // 2x1
 using CfgM = TileCfg<64, 64, 32, 2, 2>;    // 1x1
 
+// Returns 0 = predicated kernel, 1 = branch-free with one LDS stage, 2 = branch-free with two.
 template <class C>
-static void launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipStream_t s) {
+static int launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipStream_t s) {
     // With many tiles per CU a single LDS stage wins (twice the resident workgroups hide each
     // other's latencies: 99 vs 94 TFLOP/s on 1536x4096x1024); with one or two tiles per CU the
     // two-stage loop with its single barrier per K-block does (83 vs 79 on 1536x1024x4096).
@@ -524,17 +525,20 @@ static void launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipS
             hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
         else
             hipLaunchKernelGGL((gemm_clean_kernel<C, false, 1>), grid, dim3(C::THREADS), 0, s, p);
+        return 1;
     } else if (clean) {
         if (y_kc)
             hipLaunchKernelGGL((gemm_clean_kernel<C, true, 2>), grid, dim3(C::THREADS), 0, s, p);
         else
             hipLaunchKernelGGL((gemm_clean_kernel<C, false, 2>), grid, dim3(C::THREADS), 0, s, p);
+        return 2;
     } else {
         if (y_kc)
             hipLaunchKernelGGL((gemm_fast_kernel<C, true>), grid, dim3(C::THREADS), 0, s, p);
         else
             hipLaunchKernelGGL((gemm_fast_kernel<C, false>), grid, dim3(C::THREADS), 0, s, p);
     }
+    return 0;
 }
 
 // Tile shape.  Measured on MI355X over the served shapes (BERT-large 1536 x {1024,4096} x
@@ -630,16 +634,23 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
-        if (cfg == 0) {
-            launch_fast<CfgL>(p, y_kc, clean, grid, s);
-            g_last_kernel = y_kc ? "gemm_fast_128x128_kc" : "gemm_fast_128x128_cc";
-        } else if (cfg == 1) {
-            launch_fast<CfgW>(p, y_kc, clean, grid, s);
-            g_last_kernel = y_kc ? "gemm_fast_128x64_kc" : "gemm_fast_128x64_cc";
-        } else {
-            launch_fast<CfgM>(p, y_kc, clean, grid, s);
-            g_last_kernel = y_kc ? "gemm_fast_64x64_kc" : "gemm_fast_64x64_cc";
-        }
+        // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
+        // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
+        static const char* const names[3][2][3] = {
+            {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2"},
+             {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2"}},
+            {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2"},
+             {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2"}},
+            {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2"},
+             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}}};
+        int variant;
+        if (cfg == 0)
+            variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
+        else if (cfg == 1)
+            variant = launch_fast<CfgW>(p, y_kc, clean, grid, s);
+        else
+            variant = launch_fast<CfgM>(p, y_kc, clean, grid, s);
+        g_last_kernel = names[cfg][y_kc ? 1 : 0][variant];
     } else {
         p.tiles_m = (int)((a.M + 63) / 64);
         p.tiles_n = (int)((a.N + 63) / 64);
