@@ -18,7 +18,8 @@ def _rand(rng, *shape):
 @pytest.mark.parametrize("M,N,K,kernel", [
     (128, 768, 768, "gemm_fast_64x64_kc"),      # BERT-base projection
     (128, 3072, 768, "gemm_fast_64x64_kc"),
-    (1536, 1024, 1024, None),                   # BERT-large projection
+    (1536, 1024, 1024, "gemm_fast_64x32_kc"),   # BERT-large projection: 384 64x64 tiles = 1.5 per CU -> 64x32
+    (1536, 1024, 4096, "gemm_fast_64x32_kc"),   # BERT-large FFN down-projection
     (4096, 2048, 160, "gemm_fast_64x64_kc"),    # K % 64 != 0: predicated kernel
     (1, 1000, 2048, "gemm_fast_64x64_kc"),      # ResNet classifier, batch 1 (split-K)
     (49, 512, 2048, "gemm_fast_64x64_kc"),      # ragged M
@@ -142,7 +143,7 @@ def test_gemm_rejects_out_of_bounds(gpu_server):
         t.s.gemm(t.fid, x, t.w[0], c, 4, 8, 8, xs_r=8, ys_c=8, ldc=8)
 
 
-@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "128x64"), (2, "64x64")])
+@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "128x64"), (2, "64x64"), (3, "64x32")])
 def test_forced_tile_configs(cfg, name):
     """Every tile shape of the fast kernel (TORPOR_GEMM_CFG forces one; read once per process,
     hence the subprocess): ragged and exact shapes, predicated and branch-free variants."""
@@ -155,7 +156,7 @@ from torpor_amd.server import Server
 from tests.harness import OpSession, assert_close
 rng = np.random.default_rng(0)
 with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
-    for (M, N, K) in [(200, 136, 128), (257, 130, 100), (64, 64, 64), (300, 520, 192)]:
+    for (M, N, K) in [(200, 136, 128), (257, 130, 100), (64, 64, 64), (300, 520, 192), (257, 130, 256), (300, 100, 384)]:
         X = rng.standard_normal((M, K)).astype(np.float32)
         W = rng.standard_normal((N, K)).astype(np.float32)
         V = rng.standard_normal((K, N)).astype(np.float32)
@@ -163,7 +164,9 @@ with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
             x, v = t.act(X), t.act(V)
             c = t.empty(M * N * 4)
             s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N)
-            assert sys.argv[1] in s.last_kernel(), s.last_kernel()
+            # the 64x32 tile (K split over wavefront pairs) exists for K % 128 == 0 only
+            want = sys.argv[1] if (sys.argv[1] != "64x32" or K % 128 == 0) else "64x64"
+            assert want in s.last_kernel(), s.last_kernel()
             assert_close(t.read(c, (M, N)), X.astype(np.float64) @ W.astype(np.float64).T, 2e-5, "kc")
             s.gemm(t.fid, x, v, c, M, N, K, xs_r=K, ys_c=1, ys_k=N, ldc=N)
             assert_close(t.read(c, (M, N)), X.astype(np.float64) @ V.astype(np.float64), 2e-5, "cc")

@@ -101,9 +101,14 @@ def test_bert(gpu_server, arch, batch, seq):
     print(f"{arch} b{batch} s{seq}: rel err hidden {e1:.2e} pooled {e2:.2e}")
     n_params = sum(int(np.prod(v.shape)) for v in weights.values())
     assert n_params == {"bert-base": 109482240, "bert-large": 335141888}[arch]
-    _check_swap_identity(gpu_server, fn, weights)
+    uploaded = fn.weights()   # query / key / value stacked per layer, everything else as in `weights`
+    assert sum(v.size for v in uploaded.values()) == n_params
+    qkv = uploaded["encoder.layer.0.attention.self.qkv.weight"]
+    hdim = bert.CONFIGS[arch]["hidden"]
+    assert np.array_equal(qkv[hdim:2 * hdim], weights["encoder.layer.0.attention.self.key.weight"])
+    _check_swap_identity(gpu_server, fn, uploaded)
     _cycle(gpu_server, fn, [ids], [hidden, pooled])
-    _check_swap_identity(gpu_server, fn, weights)
+    _check_swap_identity(gpu_server, fn, uploaded)
     fn.unload()
 
 

@@ -104,7 +104,7 @@ def test_pooling(gpu_server, layout):
         assert_close(t.read(av, (N, C)), ref.avgpool(x, nhwc=(layout == NHWC)), 2e-6, "avgpool")
 
 
-@pytest.mark.parametrize("rows,width", [(128, 768), (5, 1024), (3, 50), (2, 4096), (1, 1)])
+@pytest.mark.parametrize("rows,width", [(128, 768), (5, 1024), (3, 50), (2, 4096), (1, 1), (7, 1540), (4, 2050), (3, 260), (2, 3000)])
 def test_layernorm(gpu_server, rows, width):
     rng = np.random.default_rng(width)
     x, r = _rand(rng, rows, width) * 3 + 1, _rand(rng, rows, width)

@@ -59,10 +59,10 @@ __device__ __forceinline__ int remap_xcd(int bid, int n) {
 // 1/xr of the X rows and 1/xc of the Y rows.  The grid is padded to 8 * (largest rectangle);
 // workgroups beyond their XCD's rectangle return false and exit.
 __device__ __forceinline__ bool tile_of(const GemmDev& p, int bid, int* tm, int* tn, int* t) {
-    if (p.xr == 0) {
+    if (p.xr <= 0) {
         const int n = p.tiles_m * p.tiles_n;
         if (bid >= n) return false;
-        *t = remap_xcd(bid, n);
+        *t = p.xr == 0 ? remap_xcd(bid, n) : bid;
         *tm = *t / p.tiles_n;
         *tn = *t - *tm * p.tiles_n;
         return true;
@@ -241,7 +241,8 @@ template <class C, bool YKC, int STAGES>
 __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_clean_kernel(const GemmDev p) {
     __shared__ __attribute__((aligned(16))) float lds[STAGES * C::LDS_FLOATS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
+    const int wm = wsp / C::WGN, wn = wsp % C::WGN;
     int tm, tn, t;
     if (!tile_of(p, blockIdx.x, &tm, &tn, &t)) return;
     const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
@@ -332,11 +333,11 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
         __syncthreads();
         for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
             load_regs(ra0, rb0, k0 + 2 * C::BK);
-            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             store_lds(ra1, rb1, 1);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane);
+            mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             store_lds(ra0, rb0, 0);
             __syncthreads();
         }
@@ -349,13 +350,40 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
             store_lds(ra0, rb0, 0);
             __syncthreads();
             load_regs(ra0, rb0, k0 + 2 * C::BK);
-            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
             store_lds(ra1, rb1, 0);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane);
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
+        }
+    }
+    if (C::WGK > 1) {
+        // the wavefronts of K slices 1.. hand their sums to slice 0 through LDS (every
+        // wavefront has passed the loop's last barrier, so the operand stages are free)
+        constexpr int PER_WAVE = C::TM * C::TN * 16 * 64;
+        static_assert((C::WGK - 1) * C::WGM * C::WGN * PER_WAVE <= STAGES * C::LDS_FLOATS, "reduction must fit the stages");
+        if (wk > 0) {
+            float* dst = lds + ((wk - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) dst[((i * C::TN + j) * 16 + v) * 64] = acc[i][j][v];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int z = 1; z < C::WGK; ++z) {
+            const float* src = lds + ((z - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
+#pragma unroll
+            for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[i][j][v] += src[((i * C::TN + j) * 16 + v) * 64];
         }
     }
     float* partial = nullptr;
@@ -488,6 +516,11 @@ static int plan_xcd_grid(GemmDev& p, long M, long N) {
     double best = 1e300;
     p.xr = 0;
     p.xc = 0;
+    static const int dbg_xcd = getenv("TORPOR_GEMM_XCD") ? atoi(getenv("TORPOR_GEMM_XCD")) : 1;
+    if (dbg_xcd <= 0) {
+        p.xr = dbg_xcd;  // 0: linear + remap, -1: identity
+        return p.tiles_m * p.tiles_n;
+    }
     for (auto& c : cand) {
         if (c[0] > p.tiles_m || c[1] > p.tiles_n) continue;
         const double cost = (double)M * c[1] + (double)N * c[0];
@@ -511,6 +544,7 @@ static int plan_xcd_grid(GemmDev& p, long M, long N) {
 using CfgL = TileCfg<128, 128, 32, 2, 2>;  // 2x2 accumulators per wavefront
 using CfgW = TileCfg<128, 64, 32, 2, 2>;   // 2x1
 using CfgM = TileCfg<64, 64, 32, 2, 2>;    // 1x1
+using CfgS = TileCfg<64, 32, 64, 2, 1, 2>; // 1x1, two wavefronts per output tile split each K-block
 
 // Returns 0 = predicated kernel, 1 = branch-free with one LDS stage, 2 = branch-free with two.
 template <class C>
@@ -519,7 +553,8 @@ static int launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipSt
     // other's latencies: 99 vs 94 TFLOP/s on 1536x4096x1024); with one or two tiles per CU the
     // two-stage loop with its single barrier per K-block does (83 vs 79 on 1536x1024x4096).
     const long tiles = (long)p.tiles_m * p.tiles_n * grid.z;
-    const bool one_stage = tiles >= 5L * g_num_cu;
+    static const int dbg_st = getenv("TORPOR_GEMM_STAGES") ? atoi(getenv("TORPOR_GEMM_STAGES")) : 0;
+    const bool one_stage = dbg_st ? dbg_st == 1 : tiles >= 5L * g_num_cu;
     if (clean && one_stage) {
         if (y_kc)
             hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
@@ -541,20 +576,50 @@ static int launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipSt
     return 0;
 }
 
+// Tiles that exist only as the branch-free kernel (the caller has checked its preconditions).
+template <class C>
+static int launch_clean_only(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t s) {
+    static const int dbg_st = getenv("TORPOR_GEMM_STAGES") ? atoi(getenv("TORPOR_GEMM_STAGES")) : 0;
+    if (dbg_st == 1) {
+        if (y_kc)
+            hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
+        else
+            hipLaunchKernelGGL((gemm_clean_kernel<C, false, 1>), grid, dim3(C::THREADS), 0, s, p);
+        return 1;
+    }
+    if (y_kc)
+        hipLaunchKernelGGL((gemm_clean_kernel<C, true, 2>), grid, dim3(C::THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((gemm_clean_kernel<C, false, 2>), grid, dim3(C::THREADS), 0, s, p);
+    return 2;
+}
+
 // Tile shape.  Measured on MI355X over the served shapes (BERT-large 1536 x {1024,4096} x
 // {1024,4096}, ResNet 1x1 convolutions from 25088x256x64 to 392x2048x512), the 64x64 tile is
 // the fastest everywhere: it keeps the most workgroups resident per CU, and for fp32 MFMA
 // (2 k per instruction) occupancy hides more latency than larger register tiles save in LDS
 // traffic.  The 128x128 / 128x64 variants are kept for very large grids and for experiments
 // (TORPOR_GEMM_CFG=0/1/2 forces one).
-static int choose_tile(long M, long N, int batch) {
+static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
     static const int forced = [] {
         const char* e = getenv("TORPOR_GEMM_CFG");
         return e ? atoi(e) : -1;
     }();
-    if (forced >= 0 && forced <= 2) return forced;
+    if (forced >= 0 && forced <= 3) return forced;
     const long tiles_w = ((M + 127) / 128) * ((N + 63) / 64) * batch;
     if (tiles_w >= 64L * g_num_cu) return 1;  // enough 128x64 tiles to keep every CU full for long
+    // Tile quantisation: with t tiles on n CUs the slowest CU works ceil(t/n) tiles.  When
+    // halving the tile (64x32, K split over wavefront pairs) evens that out, take it: 384 tiles
+    // of 64x64 on 256 CUs are two rounds, 768 of 64x32 are three rounds of half the work
+    // (1536x1024x4096: 140 -> 114 us).  Only for long K and few rounds, where it was measured
+    // to win; the [K][N] weight layout and short K lose with it.
+    const long t64 = ((M + 63) / 64) * ((N + 63) / 64) * batch;
+    const long t32 = ((M + 63) / 64) * ((N + 31) / 32) * batch;
+    if (y_kc && K >= 512 && K % 128 == 0 && t64 >= g_num_cu && t64 < 3L * g_num_cu) {
+        const double r64 = (double)((t64 + g_num_cu - 1) / g_num_cu);
+        const double r32 = 0.5 * (double)((t32 + g_num_cu - 1) / g_num_cu);
+        if (r32 <= 0.8 * r64) return 3;
+    }
     return 2;
 }
 
@@ -622,32 +687,37 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     const bool y_fast = (y_kc || y_cc) && aligned16(a.Y) && (a.yb0 % 4 == 0) && (a.yb1 % 4 == 0);
 
     if (x_fast && y_fast) {
-        const int cfg = choose_tile(a.M, a.N, batch);
-        const int bm = cfg == 2 ? 64 : 128, bn = cfg == 0 ? 128 : 64;
+        int cfg = choose_tile(a.M, a.N, a.K, batch, y_kc);
+        if (cfg == 3 && !(a.K >= 128 && a.K % 128 == 0 && (y_kc || a.N % 4 == 0))) cfg = 2;  // 64x32 is branch-free only
+        const int bm = cfg >= 2 ? 64 : 128, bn = cfg == 0 ? 128 : cfg == 3 ? 32 : 64;
         p.tiles_m = (int)((a.M + bm - 1) / bm);
         p.tiles_n = (int)((a.N + bn - 1) / bn);
         const long tiles = (long)p.tiles_m * p.tiles_n * batch;
         p.splits = 1;
         p.kper = ((a.K + 31) / 32) * 32;
-        if (batch == 1) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
+        if (batch == 1 && cfg != 3) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
         dim3 grid(plan_xcd_grid(p, a.M, a.N), 1, p.splits > 1 ? p.splits : batch);
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
-        static const char* const names[3][2][3] = {
+        static const char* const names[4][2][3] = {
             {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2"},
              {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2"}},
             {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2"},
              {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2"}},
             {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2"},
-             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}}};
+             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}},
+            {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2"},
+             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}}};
         int variant;
         if (cfg == 0)
             variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
         else if (cfg == 1)
             variant = launch_fast<CfgW>(p, y_kc, clean, grid, s);
+        else if (cfg == 3)
+            variant = launch_clean_only<CfgS>(p, y_kc, grid, s);
         else
             variant = launch_fast<CfgM>(p, y_kc, clean, grid, s);
         g_last_kernel = names[cfg][y_kc ? 1 : 0][variant];

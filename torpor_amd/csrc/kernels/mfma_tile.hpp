@@ -81,15 +81,18 @@ __device__ __forceinline__ void epilogue_column(const Epilogue& e, long col, flo
     }
 }
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+// WGM x WGN wavefronts tile the BM x BN output; WGK > 1 adds wavefronts that share an output
+// tile and each multiply a 1/WGK slice of every K-block (their sums are combined through LDS
+// when the K loop ends), which keeps four wavefronts busy on tiles as small as 64x32.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int WGK_ = 1>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
-    static constexpr int THREADS = 64 * WGM * WGN;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, WGK = WGK_;
+    static constexpr int THREADS = 64 * WGM * WGN * WGK;
     static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // per-wavefront tile
     static constexpr int TM = WTM / 32, TN = WTN / 32;    // 32x32 MFMA tiles per wavefront
     static constexpr int LDK = BK + 4;                    // LDS row pitch in floats
     static constexpr int LDS_FLOATS = (BM + BN) * LDK;
-    static_assert(BK % 8 == 0, "BK must be a multiple of 8");
+    static_assert(BK % (8 * WGK) == 0, "each K slice must be a multiple of 8");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be 32-aligned");
 };
 
@@ -108,12 +111,12 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[C::TM][C::TN]) {
 // LDS latency hides behind matrix work instead of stalling every eighth MFMA.
 template <class C>
 __device__ __forceinline__ void mma_block(const float* __restrict__ As, const float* __restrict__ Bs,
-                                          f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane) {
+                                          f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, int wk = 0) {
     const int r = lane & 31;
     const int h = lane >> 5;
-    const float* ap = As + (wm * C::WTM + r) * C::LDK + 4 * h;
-    const float* bp = Bs + (wn * C::WTN + r) * C::LDK + 4 * h;
-    constexpr int G = C::BK / 8;
+    constexpr int G = C::BK / 8 / C::WGK;  // k-groups of 8 in this wavefront's slice
+    const float* ap = As + (wm * C::WTM + r) * C::LDK + 4 * h + wk * (G * 8);
+    const float* bp = Bs + (wn * C::WTN + r) * C::LDK + 4 * h + wk * (G * 8);
     f32x4 a[2][C::TM], b[2][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) a[0][i] = *reinterpret_cast<const f32x4*>(ap + i * 32 * C::LDK);

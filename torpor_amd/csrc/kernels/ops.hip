@@ -341,6 +341,73 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
         if (c < width) yr[c] = (v[i] - mean) * rstd * gamma[c] + beta[c];
     }
 }
+// One 256-thread workgroup per row, 128-bit accesses (width % 4 == 0, width <= 1024 * MAXQ, 16 B
+// aligned rows): four times the wavefronts of the wave-per-row kernel are in flight, which is
+// what hides the memory latency when there are only a few thousand rows.
+template <int MAXQ>
+__global__ __launch_bounds__(256) void layernorm_block_kernel(const float* __restrict__ x, const float* __restrict__ res,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta, float* __restrict__ y,
+                                                              int width, float eps) {
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const long row = blockIdx.x;
+    const float4* xr = reinterpret_cast<const float4*>(x + row * width);
+    const float4* rr = res ? reinterpret_cast<const float4*>(res + row * width) : nullptr;
+    const float4* gr = reinterpret_cast<const float4*>(gamma);
+    const float4* br = reinterpret_cast<const float4*>(beta);
+    float4* yr = reinterpret_cast<float4*>(y + row * width);
+    const int nq = width >> 2;
+    float4 v[MAXQ], g[MAXQ], b[MAXQ];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXQ; ++i) {
+        const int c = tid + i * 256;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < nq) {
+            v[i] = xr[c];
+            if (rr) {
+                const float4 t = rr[c];
+                v[i].x += t.x;
+                v[i].y += t.y;
+                v[i].z += t.z;
+                v[i].w += t.w;
+            }
+            g[i] = gr[c];  // issued now, needed only after both reductions
+            b[i] = br[c];
+        }
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    s = wave_sum(s);
+    if (lane == 0) red[0][wave] = s;
+    __syncthreads();
+    const float mean = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)width;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXQ; ++i) {
+        const int c = tid + i * 256;
+        if (c < nq) {
+            const float dx = v[i].x - mean, dy = v[i].y - mean, dz = v[i].z - mean, dw = v[i].w - mean;
+            q += (dx * dx + dy * dy) + (dz * dz + dw * dw);
+        }
+    }
+    q = wave_sum(q);
+    if (lane == 0) red[1][wave] = q;
+    __syncthreads();
+    const float rstd = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (float)width + eps);
+#pragma unroll
+    for (int i = 0; i < MAXQ; ++i) {
+        const int c = tid + i * 256;
+        if (c < nq) {
+            float4 o;
+            o.x = (v[i].x - mean) * rstd * g[i].x + b[i].x;
+            o.y = (v[i].y - mean) * rstd * g[i].y + b[i].y;
+            o.z = (v[i].z - mean) * rstd * g[i].z + b[i].z;
+            o.w = (v[i].w - mean) * rstd * g[i].w + b[i].w;
+            yr[c] = o;
+        }
+    }
+}
 __global__ __launch_bounds__(256) void layernorm_wide_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ res,
                                                              const float* __restrict__ gamma,
@@ -371,6 +438,18 @@ int launch_layernorm(const float* x, const float* residual, const float* gamma, 
                      long rows, int width, float eps, hipStream_t s) {
     if (!x || !gamma || !beta || !y || rows < 0 || width <= 0) return K_EINVAL;
     if (rows == 0) return 0;
+    const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (width % 4 == 0 && width > 256 && width <= 4096 && rows <= 0x7fffffffL && al16(x) && al16(y) && al16(gamma) &&
+        al16(beta) && (!residual || al16(residual))) {
+        const dim3 g1((unsigned)rows);
+        if (width <= 1024)
+            hipLaunchKernelGGL(layernorm_block_kernel<1>, g1, dim3(256), 0, s, x, residual, gamma, beta, y, width, eps);
+        else if (width <= 2048)
+            hipLaunchKernelGGL(layernorm_block_kernel<2>, g1, dim3(256), 0, s, x, residual, gamma, beta, y, width, eps);
+        else
+            hipLaunchKernelGGL(layernorm_block_kernel<4>, g1, dim3(256), 0, s, x, residual, gamma, beta, y, width, eps);
+        return (int)hipGetLastError();
+    }
     const dim3 grid((unsigned)((rows + 3) / 4));
     if (width <= 64 * 4)
         hipLaunchKernelGGL(layernorm_kernel<4>, grid, dim3(256), 0, s, x, residual, gamma, beta, y, rows, width, eps);
