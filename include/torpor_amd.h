@@ -85,6 +85,12 @@ typedef struct tp_server tp_server;
 #define TP_OP_NHWC_TO_NCHW 11 /* p: x,y         i: N,C,H,W */
 #define TP_OP_SUM 12         /* p: x,y          i: n */
 #define TP_OP_FILL 13        /* p: y            i: n   f: value */
+/* Fused attention, out[b,q,a,:] = softmax_k(scale * Q[b,q,a,:].K[b,k,a,:] + mask[b,k]) . V[b,k,a,:].  Row (b*S + t)
+ * of q / k / v / out starts at pointer + (b*S + t)*ld floats, head a at column a*dh; mask is [B][S] additive or 0.
+ * Stands in for the reference's cublasSgemmStridedBatched + softmax launch + cublasSgemmStridedBatched sequence
+ * (include/server/cuda_server.hpp:524-550,1226-1310).  dh must be 64, strides multiples of 4 floats, pointers 16 B
+ * aligned (TP_EUNSUPPORTED otherwise: issue the three separate calls instead). */
+#define TP_OP_ATTENTION 14   /* p: q,k,v,mask|0,out  i: B,A,S,dh,ldq,ldk,ldv,ldo  f: scale */
 
 typedef struct tp_config {
     uint32_t struct_size;       /* sizeof(tp_config) */

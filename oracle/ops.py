@@ -95,6 +95,21 @@ def softmax(x, mask=None, scale=1.0, rows_per_mask=1):
     return y
 
 
+def attention(q, k, v, mask=None, scale=1.0):
+    """q, k, v: [B, S, A, dh]; mask: [B, S] additive or None.  Returns [B, S, A, dh] float32:
+    softmax over keys of scale * q.k + mask, times v, all in float64 (the sequence the reference
+    forwards as cublasSgemmStridedBatched, softmax, cublasSgemmStridedBatched,
+    include/server/cuda_server.hpp:524-550)."""
+    q, k, v = (np.asarray(t, dtype=np.float64) for t in (q, k, v))
+    s = np.einsum("bqad,bkad->baqk", q, k) * scale
+    if mask is not None:
+        s = s + np.asarray(mask, dtype=np.float64)[:, None, None, :]
+    s = s - s.max(-1, keepdims=True)
+    e = np.exp(s)
+    pr = e / e.sum(-1, keepdims=True)
+    return np.einsum("baqk,bkad->bqad", pr, v).astype(np.float32)
+
+
 def gelu(x):
     x = _f32(x)
     y = np.empty_like(x)

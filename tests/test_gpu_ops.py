@@ -6,9 +6,9 @@ import pytest
 
 from oracle import ops as ref
 from tests.harness import OpSession, assert_close
-from torpor_amd.server import (NCHW, NHWC, OP_ADD, OP_AVGPOOL, OP_BIAS_ACT, OP_EMBEDDING, OP_FILL, OP_GELU,
+from torpor_amd.server import (NCHW, NHWC, OP_ADD, OP_ATTENTION, OP_AVGPOOL, OP_BIAS_ACT, OP_EMBEDDING, OP_FILL, OP_GELU,
                                OP_LAYERNORM, OP_MAXPOOL, OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_RELU, OP_SOFTMAX,
-                               OP_SUM, ACT_RELU)
+                               OP_SUM, ACT_RELU, TorporError)
 
 pytestmark = pytest.mark.gpu
 
@@ -152,6 +152,47 @@ def test_softmax(gpu_server, rows, width, rpm):
     assert np.abs(got.astype(np.float64).sum(1) - 1).max() < 1e-5
     if mask is not None:
         assert (got[np.repeat(mask, rpm, axis=0) < -1] == 0).all()
+
+
+@pytest.mark.parametrize("B,A,S,packed,masked", [
+    (1, 12, 128, True, False),    # BERT-base shape, heads read from a [tokens, 3H] projection
+    (2, 16, 384, True, False),    # BERT-large shape (batch 2), 96 heads-times-blocks per XCD
+    (2, 3, 100, False, True),     # ragged sequence (padded keys and queries), key mask, no XCD remap
+    (1, 8, 32, False, True),      # a single key block: three of the four wavefronts idle
+    (3, 1, 7, False, False),      # shorter than one block
+])
+def test_attention(gpu_server, B, A, S, packed, masked):
+    rng = np.random.default_rng(S + A)
+    dh, H = 64, A * 64
+    scale = 0.125
+    if packed:
+        qkv = _rand(rng, B * S, 3 * H)
+        q, k, v = (qkv[:, i * H:(i + 1) * H].reshape(B, S, A, dh) for i in range(3))
+    else:
+        q, k, v = (_rand(rng, B, S, A, dh) * 2 for _ in range(3))
+    mask = None
+    if masked:
+        mask = np.where(rng.random((B, S)) < 0.25, np.float32(-1e4), np.float32(0)).astype(np.float32)
+        mask[:, 0] = 0
+    with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
+        if packed:
+            base = t.act(qkv)
+            ptrs, ld = [base, base + H * 4, base + 2 * H * 4], 3 * H
+        else:
+            ptrs, ld = [t.act(np.ascontiguousarray(x)) for x in (q, k, v)], H
+        mv = t.act(mask) if mask is not None else 0
+        ov = t.empty(B * S * H * 4)
+        t.s.launch(t.fid, OP_ATTENTION, ptrs + [mv, ov], [B, A, S, dh, ld, ld, ld, H], [scale])
+        assert t.s.last_kernel() == "attention_32q_dh64"
+        got = t.read(ov, (B, S, A, dh))
+        # unsupported head width and out-of-span operands are refused, not launched
+        with pytest.raises(TorporError):
+            t.s.launch(t.fid, OP_ATTENTION, ptrs + [mv, ov], [B, A * 2, S, 32, ld, ld, ld, H], [scale])
+        with pytest.raises(TorporError):
+            t.s.launch(t.fid, OP_ATTENTION, ptrs + [mv, ov], [B, A, S + 1, dh, ld, ld, ld, H], [scale])
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)   # refused ops are reported once more at the next sync
+    assert_close(got, ref.attention(q, k, v, mask, scale), 2e-5, "attention")
 
 
 def test_embedding(gpu_server):

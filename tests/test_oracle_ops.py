@@ -104,6 +104,24 @@ def test_layernorm_softmax_gelu_vs_torch():
     assert ref.gelu(np.zeros(1, np.float32))[0] == 0
 
 
+def test_attention_vs_torch():
+    """The fused-attention oracle against torch's scaled_dot_product_attention (float64), with
+    and without an additive key mask, and against the closed form for identical keys (uniform
+    probabilities -> the mean of V)."""
+    rng = np.random.default_rng(9)
+    B, S, A, dh = 2, 37, 3, 16
+    q, k, v = _rand(rng, B, S, A, dh), _rand(rng, B, S, A, dh), _rand(rng, B, S, A, dh)
+    mask = np.where(rng.random((B, S)) < 0.3, -1e4, 0).astype(np.float32)
+    mask[:, 0] = 0
+    tq, tk, tv = (torch.from_numpy(t).double().permute(0, 2, 1, 3) for t in (q, k, v))
+    for m in (None, mask):
+        am = None if m is None else torch.from_numpy(m).double()[:, None, None, :]
+        want = F.scaled_dot_product_attention(tq, tk, tv, attn_mask=am, scale=0.25).permute(0, 2, 1, 3).numpy()
+        _close(ref.attention(q, k, v, m, 0.25), want, 1e-6)
+    same_k = np.broadcast_to(k[:, :1], k.shape)
+    _close(ref.attention(q, same_k, v, None, 0.7), np.broadcast_to(v.mean(1, keepdims=True), v.shape), 1e-6)
+
+
 @pytest.mark.parametrize("nhwc", [True, False])
 def test_pool_vs_torch(nhwc):
     rng = np.random.default_rng(5)

@@ -1200,6 +1200,21 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             if ((r = R(0, false, I[0])) || (r = R(1, false, 1))) return r;
             if (!launch) return 0;
             return tpk::launch_sum(F(0), Fm(1), I[0], compute_);
+        case TP_OP_ATTENTION: {
+            if (!need(5, 8, 1)) return TP_EINVAL;
+            const int64_t B = I[0], A = I[1], S = I[2], dh = I[3];
+            if (B < 1 || A < 1 || S < 1 || dh < 1 || B * S > 0x7fffffff || A * dh > 0x7fffffff) return TP_EINVAL;
+            for (int k = 4; k < 8; ++k)
+                if (I[k] < A * dh) return TP_EINVAL;
+            // span of a strided [B*S][A*dh] view: last row start + one row
+            auto span = [&](int64_t ld) { return (B * S - 1) * ld + A * dh; };
+            if ((r = R(0, false, span(I[4]))) || (r = R(1, false, span(I[5]))) || (r = R(2, false, span(I[6]))) ||
+                (r = R(3, true, B * S)) || (r = R(4, false, span(I[7]))))
+                return r;
+            if (!launch) return 0;
+            return tpk::launch_attention(F(0), F(1), F(2), F(3), Fm(4), (int)B, (int)A, (int)S, (int)dh, I[4], I[5],
+                                         I[6], I[7], op.f[0], compute_);
+        }
         case TP_OP_FILL:
             if (!need(1, 1, 1)) return TP_EINVAL;
             if ((r = R(0, false, I[0]))) return r;
@@ -1257,6 +1272,11 @@ static void op_work(const Op& op, double* flops, double* bytes, const char** nam
                 case TP_OP_NHWC_TO_NCHW: *bytes = 8.0 * (double)(I[0] * I[1] * I[2] * I[3]); *name = "layout"; break;
                 case TP_OP_SUM: *bytes = 4.0 * (double)I[0]; *name = "sum"; break;
                 case TP_OP_FILL: *bytes = 4.0 * (double)I[0]; *name = "fill"; break;
+                case TP_OP_ATTENTION:
+                    *flops = 4.0 * (double)(I[0] * I[1]) * (double)(I[2] * I[2]) * (double)I[3];
+                    *bytes = 16.0 * (double)(I[0] * I[2]) * (double)(I[1] * I[3]);
+                    *name = "attention";
+                    break;
                 default: break;
             }
             break;

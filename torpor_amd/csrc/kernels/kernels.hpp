@@ -81,6 +81,10 @@ int launch_layernorm(const float* x, const float* residual, const float* gamma, 
 // y[row] = softmax(scale * x[row] + mask[(row / rows_per_mask) * width ...]) over `width`
 int launch_softmax(const float* x, const float* mask, float* y, long rows, int width, float scale,
                    long rows_per_mask, hipStream_t s);
+// out[b,q,a,:] = softmax_k(scale * Q[b,q,a,:].K[b,k,a,:] + mask[b,k]) . V[b,k,a,:]; row (b*S + t) of each
+// operand is at pointer + (b*S + t)*ld, head a at column a*dh.  dh must be 64.
+int launch_attention(const float* q, const float* k, const float* v, const float* mask, float* out, int B, int A, int S,
+                     int dh, long ldq, long ldk, long ldv, long ldo, float scale, hipStream_t s);
 int launch_embedding(const int64_t* ids, const int64_t* type_ids, const float* word, const float* pos,
                      const float* type, float* y, long tokens, int seq, int width, long vocab, int n_types,
                      hipStream_t s);

@@ -5,8 +5,9 @@ reach the server as cublasSgemm, the attention products as cublasSgemmStridedBat
 everything else as libtorch kernel launches.  Here: dense GEMMs with bias (+GELU / tanh) fused in
 the epilogue, the query / key / value projections as one GEMM over the stacked [3H, H] weight
 (stacked once, at upload; 4.5 tiles per CU instead of three launches of 1.5), head-strided
-batched GEMMs straight on that [tokens, 3H] projection (no permute/contiguous copies),
-one-wavefront-per-row softmax and residual LayerNorm.  Weight names
+the attention core as one fused kernel reading the heads in place from that [tokens, 3H]
+projection (head width 64; other widths fall back to two head-strided batched GEMMs around a
+softmax launch), and residual LayerNorm.  Weight names
 and conventions follow `transformers.BertModel` (LayerNorm eps 1e-12, erf GELU, additive mask,
 absolute position + token-type embeddings, tanh pooler on the first token).
 """
@@ -14,7 +15,7 @@ from collections import OrderedDict
 
 import numpy as np
 
-from ..server import ACT_GELU, ACT_NONE, ACT_TANH, OP_EMBEDDING, OP_LAYERNORM, OP_SOFTMAX
+from ..server import ACT_GELU, ACT_NONE, ACT_TANH, OP_ATTENTION, OP_EMBEDDING, OP_LAYERNORM, OP_SOFTMAX
 from .base import Function
 
 CONFIGS = {
@@ -127,18 +128,23 @@ class Bert(Function):
             qkv = self._linear(h, tok, H, 3 * H, p + ".attention.self.qkv")
             H3 = 3 * H
             q_va, k_va, v_va = qkv.va, qkv.va + H * 4, qkv.va + 2 * H * 4
-            scores = self.alloc(B * A * S * S * 4)
-            # scores[b,a] = Q[b,:,a,:] . K[b,:,a,:]^T, read in place from the [tok, 3H] projection
-            self.s.gemm(self.fid, q_va, k_va, scores.va, S, S, dh, xs_r=H3, ys_c=H3, ldc=S, nb0=B, nb1=A,
-                        xb0=S * H3, xb1=dh, yb0=S * H3, yb1=dh, cb0=A * S * S, cb1=S * S)
-            probs = self.alloc(B * A * S * S * 4)
-            self.s.launch(self.fid, OP_SOFTMAX, [scores.va, 0, probs.va], [B * A * S, S, A * S], [scale])
-            self.release(scores)
             ctx = self.alloc(tok * H * 4)
-            # ctx[b,:,a,:] = P[b,a] . V[b,:,a,:]
-            self.s.gemm(self.fid, probs.va, v_va, ctx.va, S, dh, S, xs_r=S, ys_c=1, ys_k=H3, ldc=H, nb0=B, nb1=A,
-                        xb0=A * S * S, xb1=S * S, yb0=S * H3, yb1=dh, cb0=S * H, cb1=dh)
-            self.release(probs)
+            if dh == 64:
+                # fused softmax(Q.K^T / sqrt(dh)) . V, heads read in place from the [tok, 3H] projection
+                self.s.launch(self.fid, OP_ATTENTION, [q_va, k_va, v_va, 0, ctx.va],
+                              [B, A, S, dh, H3, H3, H3, H], [scale])
+            else:
+                scores = self.alloc(B * A * S * S * 4)
+                # scores[b,a] = Q[b,:,a,:] . K[b,:,a,:]^T
+                self.s.gemm(self.fid, q_va, k_va, scores.va, S, S, dh, xs_r=H3, ys_c=H3, ldc=S, nb0=B, nb1=A,
+                            xb0=S * H3, xb1=dh, yb0=S * H3, yb1=dh, cb0=A * S * S, cb1=S * S)
+                probs = self.alloc(B * A * S * S * 4)
+                self.s.launch(self.fid, OP_SOFTMAX, [scores.va, 0, probs.va], [B * A * S, S, A * S], [scale])
+                self.release(scores)
+                # ctx[b,:,a,:] = P[b,a] . V[b,:,a,:]
+                self.s.gemm(self.fid, probs.va, v_va, ctx.va, S, dh, S, xs_r=S, ys_c=1, ys_k=H3, ldc=H, nb0=B, nb1=A,
+                            xb0=A * S * S, xb1=S * S, yb0=S * H3, yb1=dh, cb0=S * H, cb1=dh)
+                self.release(probs)
             self.release(qkv)
             ao = self._linear(ctx, tok, H, H, p + ".attention.output.dense")
             self.release(ctx)

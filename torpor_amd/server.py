@@ -17,7 +17,7 @@ ACK_OK, ACK_INAVAIL = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
 NCHW, NHWC = 0, 1
 (OP_RELU, OP_ADD, OP_BIAS_ACT, OP_GELU, OP_MAXPOOL, OP_AVGPOOL, OP_LAYERNORM, OP_SOFTMAX, OP_EMBEDDING,
- OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL) = range(1, 14)
+ OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION) = range(1, 15)
 FLAG_HOST_ONLY = 1
 
 
