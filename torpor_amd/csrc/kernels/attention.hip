@@ -48,14 +48,6 @@ struct AttnDev {
     int xcd_remap;
 };
 
-// LDS traffic inside one wavefront needs no hardware barrier (the LDS serves a wavefront's
-// instructions in order); this only stops the compiler from moving accesses across it.
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 __global__ __launch_bounds__(256, 3) void attention_kernel(const AttnDev p) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;

@@ -53,7 +53,7 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
 template <class C>
 __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvDev p) {
     static_assert(C::BK == 72, "3x3 fast path uses K-blocks of 72");
-    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvD
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
 // Any kernel size / stride / padding / input layout; K ordered (c, kh, kw) as
@@ -151,7 +151,7 @@ using ConvGenCfg = TileCfg<64, 64, 16, 2, 2>;
 
 __global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(const ConvDev p) {
     using C = ConvGenCfg;
-    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(co
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
 using Conv3L = TileCfg<128, 128, 72, 2, 2>;

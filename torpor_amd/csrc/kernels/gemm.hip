@@ -93,7 +93,7 @@ template <class C, bool YKC>
 __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_fast_kernel(const GemmDev p) {
     // two LDS stages: while the MFMAs read one, the next K-block is written to the other, so
     // the loop needs a single barrier per K-block
-    __shared__ __attribute__((aligned(16))) float lds[2 * C::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, stage_floats<C>())];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / C::WGN, wn = wave % C::WGN;
     int tm, tn, t;
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
 // Branch-free variant of gemm_fast_kernel for the common case: K covered by an even number of
@@ -238,8 +238,12 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
 // end of K are clamped to the last K-block, so the loop body has no predication and no control
 // flow: loads, LDS traffic and MFMAs can be interleaved freely by the scheduler.
 template <class C, bool YKC, int STAGES>
-__global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_clean_kernel(const GemmDev p) {
-    __shared__ __attribute__((aligned(16))) float lds[STAGES * C::LDS_FLOATS];
+#ifndef TP_CLEAN_OCC
+#define TP_CLEAN_OCC (C::TM * C::TN >= 4 ? 1 : 2)
+#endif
+__global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(const GemmDev p) {
+    constexpr int RED_FLOATS = (C::WGK - 1) * C::WGM * C::WGN * C::TM * C::TN * 16 * 64;  // K-slice reduction
+    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>())];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
     const int wm = wsp / C::WGN, wn = wsp % C::WGN;
@@ -363,7 +367,7 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
         // the wavefronts of K slices 1.. hand their sums to slice 0 through LDS (every
         // wavefront has passed the loop's last barrier, so the operand stages are free)
         constexpr int PER_WAVE = C::TM * C::TN * 16 * 64;
-        static_assert((C::WGK - 1) * C::WGM * C::WGN * PER_WAVE <= STAGES * C::LDS_FLOATS, "reduction must fit the stages");
+        static_assert((C::WGK - 1) * C::WGM * C::WGN * PER_WAVE == RED_FLOATS, "reduction area size");
         if (wk > 0) {
             float* dst = lds + ((wk - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
 #pragma unroll
@@ -388,7 +392,7 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK);
 }
 
 // Any strides, any alignment.  64x64x16 tile, scalar loads.
@@ -396,7 +400,7 @@ using GenCfg = TileCfg<64, 64, 16, 2, 2>;
 
 __global__ __launch_bounds__(GenCfg::THREADS, 2) void gemm_generic_kernel(const GemmDev p) {
     using C = GenCfg;
-    __shared__ __attribute__((aligned(16))) float lds[C::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -465,7 +469,7 @@ __global__ __launch_bounds__(GenCfg::THREADS, 2) void gemm_generic_kernel(const 
     }
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, long M, long N,

@@ -143,33 +143,60 @@ __device__ __forceinline__ void mma_block(const float* __restrict__ As, const fl
     }
 }
 
-// Write the accumulators.  `partial` != nullptr: raw sums go to the split-K
-// workspace slice [M][N]; otherwise the epilogue is applied and C is written.
+// LDS traffic inside one wavefront needs no hardware barrier (the LDS serves a wavefront's
+// instructions in order); this only keeps the compiler from moving accesses across it.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// LDS floats store_tile needs: one 32x32 staging block per wavefront.
+constexpr int STAGE_BLOCK = 32 * 32;
+template <class C>
+constexpr int stage_floats() {
+    return (C::THREADS / 64) * STAGE_BLOCK;
+}
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+// Write the accumulators.  `partial` != nullptr: raw sums go to the split-K workspace slice
+// [M][N]; otherwise the epilogue is applied and C is written.
+//
+// Each 32x32 accumulator block first goes to `stage` (1024 floats of LDS private to this
+// wavefront; the caller guarantees that every wavefront has finished reading the operand
+// tiles), then a rolled 16-step loop writes two rows per step.  The rolled loop keeps one copy
+// of the epilogue in the program instead of one per accumulator register: the unrolled form
+// was tens of thousands of instructions, whose fetch alone cost up to a third of a GEMM.
 template <class C>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
                                            long M, long N, float* __restrict__ Cout, const Epilogue& e,
-                                           float* __restrict__ partial) {
+                                           float* __restrict__ partial, float* __restrict__ stage) {
     const int r = lane & 31;
     const int h = lane >> 5;
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const long col = n0 + wn * C::WTN + j * 32 + r;
-        if (col >= N) continue;
+        const bool col_ok = col < N;
         float cs = 1.f, ct = 0.f;
-        if (!partial) epilogue_column(e, col, cs, ct);
+        if (!partial && col_ok) epilogue_column(e, col, cs, ct);
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const long row = m0 + wm * C::WTM + i * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
-                if (row >= M) continue;
-                float x = acc[i][j][v];
-                if (partial) {
-                    partial[row * N + col] = x;
-                } else {
-                    epilogue_store(e, Cout, row, col, x, cs, ct);
+            for (int v = 0; v < 16; ++v) stage[((v >> 2) * 8 + h * 4 + (v & 3)) * 32 + r] = acc[i][j][v];
+            wave_lds_sync();
+            const long row0 = m0 + wm * C::WTM + i * 32 + h;
+#pragma unroll 1
+            for (int it = 0; it < 16; ++it) {
+                const long row = row0 + 2 * it;
+                const float x = stage[(2 * it + h) * 32 + r];
+                if (row < M && col_ok) {
+                    if (partial)
+                        partial[row * N + col] = x;
+                    else
+                        epilogue_store(e, Cout, row, col, x, cs, ct);
                 }
             }
+            wave_lds_sync();
         }
     }
 }
