@@ -16,12 +16,13 @@ def _rand(rng, *shape):
 
 
 @pytest.mark.parametrize("M,N,K,kernel", [
-    (128, 768, 768, "gemm_fast_64x64_kc"),      # BERT-base projection
-    (128, 3072, 768, "gemm_fast_64x64_kc"),
+    (128, 768, 768, "gemm_fast_32x32_kc"),      # BERT-base projection: 24 64x64 tiles -> 96 32x32 tiles
+    (128, 3072, 768, "gemm_fast_32x32_kc"),     # 96 64x64 tiles -> 384 32x32 tiles, K split in the workgroup
     (1536, 1024, 1024, "gemm_fast_64x32_kc"),   # BERT-large projection: 384 64x64 tiles = 1.5 per CU -> 64x32
     (1536, 1024, 4096, "gemm_fast_64x32_kc"),   # BERT-large FFN down-projection
     (4096, 2048, 160, "gemm_fast_64x64_kc"),    # K % 64 != 0: predicated kernel
     (1, 1000, 2048, "gemm_fast_64x64_kc"),      # ResNet classifier, batch 1 (split-K)
+    (1568, 256, 1024, "gemm_fast_32x32_kc"),    # ResNet-152 batch 8 layer3 1x1: 100 64x64 tiles -> 32x32, K split in the workgroup
     (49, 512, 2048, "gemm_fast_64x64_kc"),      # ragged M
     (100, 37, 52, "gemm_fast_64x64_kc"),        # ragged N, K % 32 != 0
     (33, 65, 7, "gemm_generic_64x64"),          # K % 4 != 0 -> scalar path
@@ -143,7 +144,7 @@ def test_gemm_rejects_out_of_bounds(gpu_server):
         t.s.gemm(t.fid, x, t.w[0], c, 4, 8, 8, xs_r=8, ys_c=8, ldc=8)
 
 
-@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "128x64"), (2, "64x64"), (3, "64x32")])
+@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "128x64"), (2, "64x64"), (3, "64x32"), (4, "32x32")])
 def test_forced_tile_configs(cfg, name):
     """Every tile shape of the fast kernel (TORPOR_GEMM_CFG forces one; read once per process,
     hence the subprocess): ragged and exact shapes, predicated and branch-free variants."""
@@ -164,8 +165,8 @@ with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
             x, v = t.act(X), t.act(V)
             c = t.empty(M * N * 4)
             s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N)
-            # the 64x32 tile (K split over wavefront pairs) exists for K % 128 == 0 only
-            want = sys.argv[1] if (sys.argv[1] != "64x32" or K % 128 == 0) else "64x64"
+            # the tiles that split K over wavefronts (64x32, 32x32) exist for K % 128 == 0 only
+            want = sys.argv[1] if (sys.argv[1] not in ("64x32", "32x32") or K % 128 == 0) else "64x64"
             assert want in s.last_kernel(), s.last_kernel()
             assert_close(t.read(c, (M, N)), X.astype(np.float64) @ W.astype(np.float64).T, 2e-5, "kc")
             s.gemm(t.fid, x, v, c, M, N, K, xs_r=K, ys_c=1, ys_k=N, ldc=N)

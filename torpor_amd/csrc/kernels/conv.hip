@@ -50,14 +50,20 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
 // for one output channel the 8x9 block is 72 contiguous floats of the
 // [Cout][Cin][3][3] tensor; each thread loads 36 of them (4 channels x 9 taps)
 // with dwordx4 and transposes in registers to the tap-major LDS order.
+//
+// WGK > 1 (3 or 9: the nine k-groups of a K-block split evenly) lets extra wavefronts share one
+// output tile; with few output tiles this replaces a split over workgroups, whose partial sums
+// go through memory and a reduction launch.
 template <class C>
-__global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvDev p) {
+__global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x3_fast_kernel(const ConvDev p) {
     static_assert(C::BK == 72, "3x3 fast path uses K-blocks of 72");
-    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
+    static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, red_floats<C>() + stage_floats<C>())];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
+    const int wm = wsp / C::WGN, wn = wsp % C::WGN;
     const int t = remap_xcd_c(blockIdx.x, p.tiles_m * p.tiles_n);
     const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
     const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
@@ -136,12 +142,14 @@ __global__ __launch_bounds__(C::THREADS, 2) void conv3x3_fast_kernel(const ConvD
         store_lds();
         __syncthreads();
         load_regs(c0 + 8);
-        mma_block<C>(As, Bs, acc, wm, wn, lane);
+        mma_block<C>(As, Bs, acc, wm, wn, lane, wk);
         __syncthreads();
     }
+    if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial, lds + wave * STAGE_BLOCK);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial,
+                  lds + red_floats<C>() + wsp * STAGE_BLOCK);
 }
 
 // Any kernel size / stride / padding / input layout; K ordered (c, kh, kw) as
@@ -223,6 +231,9 @@ __global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(co
 
 using Conv3L = TileCfg<128, 128, 72, 2, 2>;
 using Conv3M = TileCfg<64, 64, 72, 2, 2>;
+using Conv3S = TileCfg<64, 64, 72, 2, 2, 3>;  // 12 wavefronts: 2x2 over the tile, 3 K slices
+using Conv3T = TileCfg<32, 32, 72, 1, 1, 9>;  // 9 wavefronts, one k-group each
+using Conv3U = TileCfg<32, 32, 72, 1, 1, 3>;  // 3 wavefronts
 
 static inline bool aligned16c(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -308,22 +319,50 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
                        aligned16c(a.w) && ws.zeros != nullptr;
     if (fast3) {
         const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);
-        const bool big = tl >= 2L * num_cu();
-        const int bm = big ? 128 : 64;
+        const long t64 = ((M + 63) / 64) * ((a.Cout + 63) / 64);
+        static const int forced = getenv("TORPOR_CONV3_CFG") ? atoi(getenv("TORPOR_CONV3_CFG")) : -1;
+        // 0: 128x128, 1: 64x64, 2: 64x64 with 3 K slices, 3: 32x32 with 9 K slices, 4: 32x32 with 3
+        // Measured on MI355X (ResNet shapes, 1.85 GFLOP each): with between half a tile and one
+        // tile per CU, three K slices per 64x64 tile beat a 2-3 way split over workgroups
+        // (8x28x28x128: 38.8 -> 32.9 us); a short K with many pixels runs best as 32x32 tiles
+        // with nine K slices (1x56x56x64: 13.5 -> 9.0 us); elsewhere 64x64 tiles, split over
+        // workgroups when there are fewer tiles than CUs.
+        const long t32 = ((M + 31) / 32) * ((a.Cout + 31) / 32);
+        int cfg = tl >= 2L * num_cu() ? 0 : 1;
+        if (cfg == 1 && t64 >= num_cu() / 2 && t64 < num_cu()) cfg = 2;
+        if (cfg == 1 && t64 < num_cu() / 4 && t32 >= num_cu() / 2 && a.Cin <= 128) cfg = 3;
+        if (forced >= 0 && forced <= 4) cfg = forced;
+        const int bm = cfg == 0 ? 128 : cfg <= 2 ? 64 : 32;
         p.tiles_m = (int)((M + bm - 1) / bm);
         p.tiles_n = (a.Cout + bm - 1) / bm;
         const long tiles = (long)p.tiles_m * p.tiles_n;
         // split over channel blocks of 8 (one K-block each)
-        long kper_k = 0;
-        p.splits = choose_splits(tiles, p.K, 72, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
+        long kper_k = p.K;
+        p.splits = 1;
+        if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
-        if (big) {
-            hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3L>), grid, dim3(256), 0, s, p);
-            set_last_kernel("conv3x3_fast_128x128");
-        } else {
-            hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3M>), grid, dim3(256), 0, s, p);
-            set_last_kernel("conv3x3_fast_64x64");
+        switch (cfg) {
+            case 0:
+                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3L>), grid, dim3(Conv3L::THREADS), 0, s, p);
+                set_last_kernel("conv3x3_fast_128x128");
+                break;
+            case 1:
+                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3M>), grid, dim3(Conv3M::THREADS), 0, s, p);
+                set_last_kernel("conv3x3_fast_64x64");
+                break;
+            case 2:
+                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3S>), grid, dim3(Conv3S::THREADS), 0, s, p);
+                set_last_kernel("conv3x3_fast_64x64_k3");
+                break;
+            case 3:
+                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3T>), grid, dim3(Conv3T::THREADS), 0, s, p);
+                set_last_kernel("conv3x3_fast_32x32_k9");
+                break;
+            default:
+                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3U>), grid, dim3(Conv3U::THREADS), 0, s, p);
+                set_last_kernel("conv3x3_fast_32x32_k3");
+                break;
         }
     } else {
         p.tiles_m = (int)((M + 63) / 64);

@@ -242,7 +242,7 @@ template <class C, bool YKC, int STAGES>
 #define TP_CLEAN_OCC (C::TM * C::TN >= 4 ? 1 : 2)
 #endif
 __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(const GemmDev p) {
-    constexpr int RED_FLOATS = (C::WGK - 1) * C::WGM * C::WGN * C::TM * C::TN * 16 * 64;  // K-slice reduction
+    constexpr int RED_FLOATS = red_floats<C>();  // K-slice reduction area, then the epilogue staging blocks
     __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>())];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
@@ -363,33 +363,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             __syncthreads();
         }
     }
-    if (C::WGK > 1) {
-        // the wavefronts of K slices 1.. hand their sums to slice 0 through LDS (every
-        // wavefront has passed the loop's last barrier, so the operand stages are free)
-        constexpr int PER_WAVE = C::TM * C::TN * 16 * 64;
-        static_assert((C::WGK - 1) * C::WGM * C::WGN * PER_WAVE == RED_FLOATS, "reduction area size");
-        if (wk > 0) {
-            float* dst = lds + ((wk - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
-#pragma unroll
-            for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) dst[((i * C::TN + j) * 16 + v) * 64] = acc[i][j][v];
-        }
-        __syncthreads();
-        if (wk > 0) return;
-#pragma unroll
-        for (int z = 1; z < C::WGK; ++z) {
-            const float* src = lds + ((z - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
-#pragma unroll
-            for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-                for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[i][j][v] += src[((i * C::TN + j) * 16 + v) * 64];
-        }
-    }
+    if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
     if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK);
@@ -549,6 +523,7 @@ using CfgL = TileCfg<128, 128, 32, 2, 2>;  // 2x2 accumulators per wavefront
 using CfgW = TileCfg<128, 64, 32, 2, 2>;   // 2x1
 using CfgM = TileCfg<64, 64, 32, 2, 2>;    // 1x1
 using CfgS = TileCfg<64, 32, 64, 2, 1, 2>; // 1x1, two wavefronts per output tile split each K-block
+using CfgT = TileCfg<32, 32, 64, 1, 1, 4>; // one 32x32 tile, its four wavefronts split each K-block
 
 // Returns 0 = predicated kernel, 1 = branch-free with one LDS stage, 2 = branch-free with two.
 template <class C>
@@ -609,7 +584,7 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
         const char* e = getenv("TORPOR_GEMM_CFG");
         return e ? atoi(e) : -1;
     }();
-    if (forced >= 0 && forced <= 3) return forced;
+    if (forced >= 0 && forced <= 4) return forced;
     const long tiles_w = ((M + 127) / 128) * ((N + 63) / 64) * batch;
     if (tiles_w >= 64L * g_num_cu) return 1;  // enough 128x64 tiles to keep every CU full for long
     // Tile quantisation: with t tiles on n CUs the slowest CU works ceil(t/n) tiles.  When
@@ -624,6 +599,10 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
         const double r32 = 0.5 * (double)((t32 + g_num_cu - 1) / g_num_cu);
         if (r32 <= 0.8 * r64) return 3;
     }
+    // Fewer 64x64 tiles than CUs: rather than splitting K across workgroups (partial sums through
+    // memory plus a reduction launch), quarter the tile and split K inside the workgroup.
+    const long t3232 = ((M + 31) / 32) * ((N + 31) / 32) * batch;
+    if (batch == 1 && K >= 256 && K % 128 == 0 && t64 < g_num_cu && t3232 >= 3 * g_num_cu / 8) return 4;
     return 2;
 }
 
@@ -692,21 +671,21 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
 
     if (x_fast && y_fast) {
         int cfg = choose_tile(a.M, a.N, a.K, batch, y_kc);
-        if (cfg == 3 && !(a.K >= 128 && a.K % 128 == 0 && (y_kc || a.N % 4 == 0))) cfg = 2;  // 64x32 is branch-free only
-        const int bm = cfg >= 2 ? 64 : 128, bn = cfg == 0 ? 128 : cfg == 3 ? 32 : 64;
+        if (cfg >= 3 && !(a.K >= 128 && a.K % 128 == 0 && (y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
+        const int bm = cfg == 4 ? 32 : cfg >= 2 ? 64 : 128, bn = cfg == 0 ? 128 : cfg >= 3 ? 32 : 64;
         p.tiles_m = (int)((a.M + bm - 1) / bm);
         p.tiles_n = (int)((a.N + bn - 1) / bn);
         const long tiles = (long)p.tiles_m * p.tiles_n * batch;
         p.splits = 1;
         p.kper = ((a.K + 31) / 32) * 32;
-        if (batch == 1 && cfg != 3) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
+        if (batch == 1 && cfg < 3) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
         dim3 grid(plan_xcd_grid(p, a.M, a.N), 1, p.splits > 1 ? p.splits : batch);
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
-        static const char* const names[4][2][3] = {
+        static const char* const names[5][2][3] = {
             {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2"},
              {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2"}},
             {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2"},
@@ -714,7 +693,9 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
             {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2"},
              {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}},
             {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2"},
-             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}}};
+             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}},
+            {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2"},
+             {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2"}}};
         int variant;
         if (cfg == 0)
             variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
@@ -722,6 +703,8 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
             variant = launch_fast<CfgW>(p, y_kc, clean, grid, s);
         else if (cfg == 3)
             variant = launch_clean_only<CfgS>(p, y_kc, grid, s);
+        else if (cfg == 4)
+            variant = launch_clean_only<CfgT>(p, y_kc, grid, s);
         else
             variant = launch_fast<CfgM>(p, y_kc, clean, grid, s);
         g_last_kernel = names[cfg][y_kc ? 1 : 0][variant];

@@ -155,9 +155,49 @@ __device__ __forceinline__ void wave_lds_sync() {
 constexpr int STAGE_BLOCK = 32 * 32;
 template <class C>
 constexpr int stage_floats() {
-    return (C::THREADS / 64) * STAGE_BLOCK;
+    return C::WGM * C::WGN * STAGE_BLOCK;
 }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+// LDS floats reduce_k_slices needs.
+template <class C>
+constexpr int red_floats() {
+    return (C::WGK - 1) * C::WGM * C::WGN * C::TM * C::TN * 16 * 64;
+}
+
+// WGK > 1: the wavefronts of K slices 1.. hand their sums to slice 0 through `red`
+// (red_floats<C>() floats of LDS that no wavefront still reads operands from: call it after the
+// K loop's last barrier).  Returns false for the wavefronts that are done (slices 1..); the
+// slice-0 wavefronts return true with the complete sums in acc.  wsp = wavefront index within
+// its slice (wm * WGN + wn).
+template <class C>
+__device__ __forceinline__ bool reduce_k_slices(f32x16 (&acc)[C::TM][C::TN], float* __restrict__ red, int wk, int wsp,
+                                                int lane) {
+    if (C::WGK == 1) return true;
+    constexpr int PER_WAVE = C::TM * C::TN * 16 * 64;
+    if (wk > 0) {
+        float* dst = red + ((wk - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dst[((i * C::TN + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (wk > 0) return false;
+#pragma unroll 1
+    for (int z = 1; z < C::WGK; ++z) {
+        const float* src = red + ((z - 1) * C::WGM * C::WGN + wsp) * PER_WAVE + lane;
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] += src[((i * C::TN + j) * 16 + v) * 64];
+    }
+    return true;
+}
 
 // Write the accumulators.  `partial` != nullptr: raw sums go to the split-K workspace slice
 // [M][N]; otherwise the epilogue is applied and C is written.
