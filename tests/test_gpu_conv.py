@@ -106,7 +106,8 @@ def test_conv_rejects_bad_shapes(gpu_server):
         t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1)
 
 
-@pytest.mark.parametrize("cfg,name", [(0, "128x128"), (1, "64x64"), (2, "64x64_k3"), (3, "32x32_k9"), (4, "32x32_k3")])
+@pytest.mark.parametrize("cfg,name", [(0, "fast_128x128"), (1, "fast_64x64"), (2, "fast_64x64_k3"), (3, "fast_32x32_k9"),
+                                      (4, "fast_32x32_k3")])
 def test_forced_conv3x3_configs(cfg, name):
     """Every tile shape of the 3x3 kernel, including those whose wavefronts split the K-block
     (TORPOR_CONV3_CFG forces one; read once per process, hence the subprocess): ragged pixel
@@ -121,7 +122,8 @@ from torpor_amd.server import Server
 from tests.harness import OpSession, assert_close
 rng = np.random.default_rng(1)
 with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
-    for (N, H, W, Cin, Cout, stride) in [(1, 14, 14, 64, 64, 1), (2, 9, 7, 8, 40, 1), (1, 15, 15, 48, 72, 2), (3, 7, 7, 256, 96, 1)]:
+    for (N, H, W, Cin, Cout, stride) in [(1, 14, 14, 64, 64, 1), (2, 9, 7, 8, 40, 1), (1, 15, 15, 48, 72, 2), (3, 7, 7, 256, 96, 1),
+                                         (2, 16, 16, 64, 32, 2), (1, 56, 56, 32, 64, 1), (5, 5, 3, 96, 70, 1)]:
         x = rng.standard_normal((N, H, W, Cin)).astype(np.float32)
         w = (rng.standard_normal((Cout, Cin, 3, 3)) / np.sqrt(Cin * 9)).astype(np.float32)
         Ho, Wo = (H + 2 - 3) // stride + 1, (W + 2 - 3) // stride + 1
@@ -129,7 +131,7 @@ with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
             xv = t.act(x)
             yv = t.empty(N * Ho * Wo * Cout * 4)
             s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, 3, 3, stride=stride, pad=1)
-            assert s.last_kernel() == "conv3x3_fast_" + sys.argv[1], s.last_kernel()
+            assert s.last_kernel() == "conv3x3_" + sys.argv[1], s.last_kernel()
             got = t.read(yv, (N, Ho, Wo, Cout))
         want = ref.conv2d(x, w, (stride, stride), (1, 1), x_nhwc=True, y_nhwc=True)
         assert_close(got, want, 3e-5, "conv3x3 " + sys.argv[1])
