@@ -115,7 +115,7 @@ class Bert(nn.Module):
     """Parameter names equal those of transformers.BertModel (minus buffers)."""
 
     def __init__(self, layers=12, hidden=768, heads=12, ffn=3072, vocab=30522, max_pos=512, type_vocab=2,
-                 eps=1e-12):
+                 eps=1e-12, qa_head=False):
         super().__init__()
         emb = nn.Module()
         emb.word_embeddings = nn.Embedding(vocab, hidden)
@@ -127,6 +127,8 @@ class Bert(nn.Module):
         self.encoder.layer = nn.ModuleList([BertLayer(hidden, heads, ffn, eps) for _ in range(layers)])
         self.pooler = nn.Module()
         self.pooler.dense = nn.Linear(hidden, hidden)
+        # transformers.BertForQuestionAnswering: span start / end logits from the last hidden state
+        self.qa_outputs = nn.Linear(hidden, 2) if qa_head else None
 
     def forward(self, ids, token_type_ids=None, attention_mask=None):
         B, S = ids.shape
@@ -139,6 +141,9 @@ class Bert(nn.Module):
             mask = (1.0 - attention_mask[:, None, None, :].float()) * torch.finfo(torch.float32).min
         for layer in self.encoder.layer:
             h = layer(h, mask)
+        if self.qa_outputs is not None:
+            logits = self.qa_outputs(h)
+            return logits[..., 0], logits[..., 1]
         pooled = torch.tanh(self.pooler.dense(h[:, 0]))
         return h, pooled
 

@@ -112,6 +112,47 @@ def test_bert(gpu_server, arch, batch, seq):
     fn.unload()
 
 
+@pytest.mark.parametrize("heads", [2, 4])
+def test_bert_qa_with_token_types_and_mask(gpu_server, heads):
+    """The question-answering head with token type ids and a padding mask (the call the
+    reference's endpoint makes, tests/endpoint.py:52-57), head width 64 (fused attention) and
+    32 (batched GEMMs + softmax), against the PyTorch oracle."""
+    cfg = dict(layers=2, hidden=128, heads=heads, ffn=256)
+    B, S = 3, 40
+    weights = bert.init_weights(seed=5, vocab=300, max_pos=64, cfg=cfg, qa_head=True)
+    g = torch.Generator().manual_seed(7)
+    ids = torch.randint(0, 300, (B, S), generator=g).numpy()
+    tt = torch.randint(0, 2, (B, S), generator=g).numpy()
+    am = np.ones((B, S), np.int64)
+    am[0, 29:] = 0
+    am[2, 8:] = 0
+    fn = bert.Bert(gpu_server, 11, batch=B, seq=S, weights=weights, cfg=cfg, token_types=True, masked=True)
+    inputs = [ids, tt, bert.Bert.additive_mask(am)]
+    start, end = fn.register(inputs)
+    model = om.load_numpy_state(om.Bert(vocab=300, max_pos=64, qa_head=True, **cfg), weights)
+    with torch.no_grad():
+        want_s, want_e = model(torch.from_numpy(ids), torch.from_numpy(tt), torch.from_numpy(am))
+    assert start.shape == (B, S)
+    assert_close(start, want_s.numpy(), LOGIT_RTOL, "start logits")
+    assert_close(end, want_e.numpy(), LOGIT_RTOL, "end logits")
+    _cycle(gpu_server, fn, inputs, [start, end])
+    fn.unload()
+
+
+def test_resnet101(gpu_server):
+    """ResNet-101 (served by the reference next to -50 and -152, tests/endpoint.py:16-29)."""
+    weights = _perturb_bn(resnet.init_weights("resnet101", seed=2), seed=3)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(4)).numpy()
+    fn = resnet.ResNet(gpu_server, 12, "resnet101", batch=1, weights=weights)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.ResNet("resnet101"), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    assert_close(logits, want, LOGIT_RTOL, "resnet101 logits")
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
 def test_image_is_in_first_access_order(gpu_server):
     """ResNet uploads `downsample` after `conv3` (state-dict order) but uses it before: after
     registration the image must hold the tensors in the order the tracked run touched them."""

@@ -46,10 +46,11 @@ def _closed_form_macs(blocks):
     return total + 2048 * 1000
 
 
-@pytest.mark.parametrize("arch,params,gmacs", [("resnet50", 25557032, 4.089), ("resnet152", 60192808, 11.514)])
+@pytest.mark.parametrize("arch,params,gmacs", [("resnet50", 25557032, 4.089), ("resnet101", 44549160, 7.801),
+                                               ("resnet152", 60192808, 11.514)])
 def test_resnet_counts(arch, params, gmacs):
-    """25,557,032 / 60,192,808 parameters and 4.089 / 11.514 GMAC per 224x224 image are the
-    published figures for ResNet-50 / -152 (v1.5 moves the stride, not the counts)."""
+    """25,557,032 / 44,549,160 / 60,192,808 parameters and 4.089 / 7.801 / 11.514 GMAC per 224x224
+    image are the published figures for ResNet-50 / -101 / -152 (v1.5 moves the stride, not the counts)."""
     model = om.ResNet(arch).eval()
     assert sum(p.numel() for p in model.parameters()) == params
     m, y = _macs(model, torch.zeros(1, 3, 224, 224))
@@ -58,7 +59,7 @@ def test_resnet_counts(arch, params, gmacs):
     assert round(m / 1e9, 3) == gmacs
     n_weight_tensors = len(list(model.parameters()))
     n_bn_buffers = sum(1 for k in model.state_dict() if "running" in k)
-    assert (n_weight_tensors, n_bn_buffers) == {"resnet50": (161, 106), "resnet152": (467, 310)}[arch]
+    assert (n_weight_tensors, n_bn_buffers) == {"resnet50": (161, 106), "resnet101": (314, 208), "resnet152": (467, 310)}[arch]
 
 
 def test_resnet_stride_is_on_the_3x3():
@@ -121,3 +122,36 @@ def test_product_bert_weights_load_strictly():
     w = pbert.init_weights(seed=0, vocab=97, max_pos=40, cfg=cfg)
     om.load_numpy_state(om.Bert(vocab=97, max_pos=40, **cfg), w)
     assert abs(w["encoder.layer.0.intermediate.dense.weight"].std() - 0.02) < 2e-3
+
+
+def test_bert_qa_head_matches_transformers():
+    """The question-answering variant the reference serves (tests/endpoint.py:36-40,
+    BertForQuestionAnswering called with input ids and token type ids): span logits of the oracle
+    against the installed transformers implementation with shared weights."""
+    transformers = pytest.importorskip("transformers")
+    cfg = transformers.BertConfig(vocab_size=97, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+                                  intermediate_size=128, max_position_embeddings=40, type_vocab_size=2,
+                                  hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    torch.manual_seed(1)
+    hf = transformers.BertForQuestionAnswering(cfg).eval()
+    mine = om.Bert(layers=2, hidden=64, heads=4, ffn=128, vocab=97, max_pos=40, type_vocab=2, qa_head=True)
+    want = {k[len("bert."):] if k.startswith("bert.") else k: v for k, v in hf.state_dict().items()}
+    sd = {k: v for k, v in want.items() if k in mine.state_dict()}
+    # the transformers model has no pooler; the oracle's stays at its initial value and is unused
+    assert set(mine.state_dict()) - set(sd) == {"pooler.dense.weight", "pooler.dense.bias"}
+    mine.load_state_dict(sd, strict=False)
+    mine.eval()
+    ids = torch.randint(0, 97, (2, 19))
+    tt = torch.randint(0, 2, (2, 19))
+    am = torch.ones(2, 19, dtype=torch.long)
+    am[0, 13:] = 0
+    with torch.no_grad():
+        ref = hf(input_ids=ids, token_type_ids=tt, attention_mask=am)
+        start, end = mine(ids, tt, am)
+    assert torch.allclose(start, ref.start_logits, atol=2e-5, rtol=1e-4)
+    assert torch.allclose(end, ref.end_logits, atol=2e-5, rtol=1e-4)
+    # product-side weight generator loads strictly, and its mask helper equals the oracle's convention
+    w = pbert.init_weights(cfg=dict(layers=2, hidden=64, heads=4, ffn=128), vocab=97, max_pos=40, qa_head=True)
+    om.load_numpy_state(om.Bert(layers=2, hidden=64, heads=4, ffn=128, vocab=97, max_pos=40, qa_head=True), w)
+    add = pbert.Bert.additive_mask(am.numpy())
+    assert add.dtype == np.float32 and (add[0, :13] == 0).all() and (add[0, 13:] == np.finfo(np.float32).min).all()

@@ -25,7 +25,7 @@ CONFIGS = {
 LN_EPS = 1e-12
 
 
-def init_weights(arch="bert-base", seed=0, vocab=30522, max_pos=512, type_vocab=2, cfg=None):
+def init_weights(arch="bert-base", seed=0, vocab=30522, max_pos=512, type_vocab=2, cfg=None, qa_head=False):
     """Random-init weights: N(0, 0.02) matrices, embeddings and biases, LayerNorm gamma
     N(1, 0.02) / beta N(0, 0.02).  (Hugging Face zero-initialises biases and uses gamma=1,
     beta=0; small random values are used instead so that every tensor influences the output.)"""
@@ -62,19 +62,29 @@ def init_weights(arch="bert-base", seed=0, vocab=30522, max_pos=512, type_vocab=
         linear(p + ".output.dense", H, F)
         ln(p + ".output.LayerNorm")
     linear("pooler.dense", H, H)
+    if qa_head:
+        # BertForQuestionAnswering (what the reference serves, tests/endpoint.py:36-40): span start / end logits
+        linear("qa_outputs", 2, H)
     return w
 
 
 class Bert(Function):
+    """inputs: ids [B, S] int64, then token type ids [B, S] int64 if `token_types`, then the
+    attention mask [B, S] (1 = attend, 0 = padding) if `masked`.  Outputs: last hidden state and
+    pooled output, or, with a `qa_outputs` head in the weights, the span start and end logits
+    [B, S] each (transformers.BertForQuestionAnswering)."""
+
     def __init__(self, server, fid, arch="bert-base", batch=1, seq=128, weights=None, seed=0, level=1, cfg=None,
-                 vocab=30522):
+                 vocab=30522, token_types=False, masked=False):
         super().__init__(server, fid, level)
+        self.token_types, self.masked = token_types, masked
         self.cfg = dict(CONFIGS[arch]) if cfg is None else dict(cfg)
         self.batch, self.seq = batch, seq
         self._weights = weights if weights is not None else init_weights(arch, seed, vocab=vocab, cfg=self.cfg)
         self.vocab = self._weights["embeddings.word_embeddings.weight"].shape[0]
         self.max_pos = self._weights["embeddings.position_embeddings.weight"].shape[0]
         self.type_vocab = self._weights["embeddings.token_type_embeddings.weight"].shape[0]
+        self.qa_head = "qa_outputs.weight" in self._weights
 
     def weights(self):
         """Tensors as uploaded: the Hugging Face state dict, except that each layer's query, key
@@ -91,7 +101,19 @@ class Bert(Function):
         return out
 
     def input_specs(self):
-        return [((self.batch, self.seq), np.int64)]
+        specs = [((self.batch, self.seq), np.int64)]
+        if self.token_types:
+            specs.append(((self.batch, self.seq), np.int64))
+        if self.masked:
+            specs.append(((self.batch, self.seq), np.float32))   # additive form, see additive_mask()
+        return specs
+
+    @staticmethod
+    def additive_mask(attention_mask):
+        """1 / 0 attention mask -> the additive float mask the model adds to the scores
+        (0 where attended, the most negative float32 where not: transformers' convention)."""
+        m = np.asarray(attention_mask, dtype=np.float32)
+        return ((1.0 - m) * np.finfo(np.float32).min).astype(np.float32)
 
     def _linear(self, x, tok, inp, out, name, act=ACT_NONE, xs_r=None):
         y = self.alloc(tok * out * 4)
@@ -108,14 +130,16 @@ class Bert(Function):
         return y
 
     def forward(self, inputs):
-        (ids,) = inputs
+        ids = inputs[0]
+        tt_va = inputs[1].va if self.token_types else 0
+        mask_va = inputs[-1].va if self.masked else 0
         B, S = self.batch, self.seq
         H, A, F, L = self.cfg["hidden"], self.cfg["heads"], self.cfg["ffn"], self.cfg["layers"]
         dh = H // A
         tok = B * S
         emb = self.alloc(tok * H * 4)
         self.s.launch(self.fid, OP_EMBEDDING,
-                      [ids.va, 0, self.w["embeddings.word_embeddings.weight"],
+                      [ids.va, tt_va, self.w["embeddings.word_embeddings.weight"],
                        self.w["embeddings.position_embeddings.weight"],
                        self.w["embeddings.token_type_embeddings.weight"], emb.va],
                       [tok, S, H, self.vocab, self.type_vocab])
@@ -131,7 +155,7 @@ class Bert(Function):
             ctx = self.alloc(tok * H * 4)
             if dh == 64:
                 # fused softmax(Q.K^T / sqrt(dh)) . V, heads read in place from the [tok, 3H] projection
-                self.s.launch(self.fid, OP_ATTENTION, [q_va, k_va, v_va, 0, ctx.va],
+                self.s.launch(self.fid, OP_ATTENTION, [q_va, k_va, v_va, mask_va, ctx.va],
                               [B, A, S, dh, H3, H3, H3, H], [scale])
             else:
                 scores = self.alloc(B * A * S * S * 4)
@@ -139,7 +163,7 @@ class Bert(Function):
                 self.s.gemm(self.fid, q_va, k_va, scores.va, S, S, dh, xs_r=H3, ys_c=H3, ldc=S, nb0=B, nb1=A,
                             xb0=S * H3, xb1=dh, yb0=S * H3, yb1=dh, cb0=A * S * S, cb1=S * S)
                 probs = self.alloc(B * A * S * S * 4)
-                self.s.launch(self.fid, OP_SOFTMAX, [scores.va, 0, probs.va], [B * A * S, S, A * S], [scale])
+                self.s.launch(self.fid, OP_SOFTMAX, [scores.va, mask_va, probs.va], [B * A * S, S, A * S], [scale])
                 self.release(scores)
                 # ctx[b,:,a,:] = P[b,a] . V[b,:,a,:]
                 self.s.gemm(self.fid, probs.va, v_va, ctx.va, S, dh, S, xs_r=S, ys_c=1, ys_k=H3, ldc=H, nb0=B, nb1=A,
@@ -157,6 +181,11 @@ class Bert(Function):
             h = self._ln(out, h1, tok, p + ".output.LayerNorm")
             self.release(out)
             self.release(h1)
+        if self.qa_head:
+            # span logits [tok, 2]; de-interleaved into start / end on the host
+            out = self._linear(h, tok, H, 2, "qa_outputs")
+            self.release(h)
+            return [(out, (tok * 2,), np.float32)]
         # One result buffer = [last hidden state | pooled], because the first D2H copy of a request
         # is its completion marker (reference cuda_server.hpp:1044).
         out = self.alloc((tok * H + B * H) * 4)
@@ -170,4 +199,7 @@ class Bert(Function):
     def postprocess(self, host):
         (flat,) = host
         B, S, H = self.batch, self.seq, self.cfg["hidden"]
+        if self.qa_head:
+            logits = flat.reshape(B, S, 2)
+            return [np.ascontiguousarray(logits[..., 0]), np.ascontiguousarray(logits[..., 1])]
         return [flat[:B * S * H].reshape(B, S, H), flat[B * S * H:].reshape(B, H)]
