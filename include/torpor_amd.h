@@ -64,6 +64,9 @@ typedef struct tp_server tp_server;
 #define TP_ACT_RELU 1
 #define TP_ACT_GELU 2 /* erf form */
 #define TP_ACT_TANH 3
+#define TP_ACT_RELU6 4
+#define TP_ACT_SILU 5
+#define TP_ACT_SIGMOID 6
 
 /* ---- tensor layouts for convolution / pooling / batch-norm ---- */
 #define TP_LAYOUT_NCHW 0
@@ -91,6 +94,8 @@ typedef struct tp_server tp_server;
  * (include/server/cuda_server.hpp:524-550,1226-1310).  dh must be 64, strides multiples of 4 floats, pointers 16 B
  * aligned (TP_EUNSUPPORTED otherwise: issue the three separate calls instead). */
 #define TP_OP_ATTENTION 14   /* p: q,k,v,mask|0,out  i: B,A,S,dh,ldq,ldk,ldv,ldo  f: scale */
+#define TP_OP_AVGPOOL2D 15   /* p: x,y   i: N,H,W,C,k,stride,pad,y_pitch|0   NHWC window average, padding counted */
+#define TP_OP_COPY2D 16      /* p: src,dst   i: rows,width,src_pitch,dst_pitch   (elements) */
 
 typedef struct tp_config {
     uint32_t struct_size;       /* sizeof(tp_config) */
@@ -136,6 +141,10 @@ typedef struct tp_conv_desc {
     int32_t n, h, w_in, cin, cout, kh, kw;
     int32_t stride_h, stride_w, pad_h, pad_w, groups;
     int32_t x_layout, y_layout; /* TP_LAYOUT_* */
+    /* NHWC only: elements between consecutive pixels of x / y, 0 = cin / cout.  A larger pitch reads the first
+     * cin channels of a wider tensor, or writes a channel slice of one (concatenation without a copy).
+     * groups: 0 / 1, or cin == cout == groups (depthwise, NHWC, w is [C][1][KH][KW]). */
+    int64_t x_pitch, y_pitch;
     tp_epilogue ep;
 } tp_conv_desc;
 
@@ -232,6 +241,11 @@ int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d);
 int tp_bn_inference(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
                     uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
                     int32_t layout, int32_t relu);
+/* The same with rows of x `x_pitch` elements apart (NHWC; 0 = channels): normalises the first `channels`
+ * channels of a wider tensor into a dense y. */
+int tp_bn_inference_pitched(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
+                            uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
+                            int32_t layout, int32_t relu, int64_t x_pitch);
 /* cudaLaunchKernelService (cuda_server.hpp:1226-1310) by op id, pointer slots explicit. */
 int tp_launch(tp_server* s, int32_t client, int32_t op_id, const uint64_t* ptrs, int32_t n_ptrs,
               const int64_t* ints, int32_t n_ints, const float* floats, int32_t n_floats);

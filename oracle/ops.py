@@ -110,6 +110,49 @@ def attention(q, k, v, mask=None, scale=1.0):
     return np.einsum("baqk,bkad->bqad", pr, v).astype(np.float32)
 
 
+def depthwise_conv2d(x, w, stride=(1, 1), pad=(0, 0)):
+    """x: [N,H,W,C] (NHWC), w: [C,1,KH,KW]; groups == C.  float64 accumulation, float32 result
+    (cudnnConvolutionForward with a group count equal to the channel count)."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    N, H, W, Cc = x.shape
+    KH, KW = w.shape[2], w.shape[3]
+    Ho, Wo = (H + 2 * pad[0] - KH) // stride[0] + 1, (W + 2 * pad[1] - KW) // stride[1] + 1
+    xp = np.zeros((N, H + 2 * pad[0], W + 2 * pad[1], Cc))
+    xp[:, pad[0]:pad[0] + H, pad[1]:pad[1] + W] = x
+    y = np.zeros((N, Ho, Wo, Cc))
+    for kh in range(KH):
+        for kw in range(KW):
+            y += xp[:, kh:kh + (Ho - 1) * stride[0] + 1:stride[0], kw:kw + (Wo - 1) * stride[1] + 1:stride[1]] * w[:, 0, kh, kw]
+    return y.astype(np.float32)
+
+
+def avgpool2d(x, k, stride, pad=0):
+    """x: [N,H,W,C]; k x k window average with the zero padding counted in the divisor."""
+    x = np.asarray(x, dtype=np.float64)
+    N, H, W, Cc = x.shape
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    xp = np.zeros((N, H + 2 * pad, W + 2 * pad, Cc))
+    xp[:, pad:pad + H, pad:pad + W] = x
+    y = np.zeros((N, Ho, Wo, Cc))
+    for kh in range(k):
+        for kw in range(k):
+            y += xp[:, kh:kh + (Ho - 1) * stride + 1:stride, kw:kw + (Wo - 1) * stride + 1:stride]
+    return (y / (k * k)).astype(np.float32)
+
+
+def activation(x, name):
+    """relu6 / silu / sigmoid in float64 (the activations of the MobileNet / EfficientNet families)."""
+    x = np.asarray(x, dtype=np.float64)
+    if name == "relu6":
+        return np.clip(x, 0.0, 6.0).astype(np.float32)
+    if name == "silu":
+        return (x / (1.0 + np.exp(-x))).astype(np.float32)
+    if name == "sigmoid":
+        return (1.0 / (1.0 + np.exp(-x))).astype(np.float32)
+    raise ValueError(name)
+
+
 def gelu(x):
     x = _f32(x)
     y = np.empty_like(x)

@@ -40,5 +40,5 @@ def test_struct_sizes_match_the_header_layout():
     assert ctypes.sizeof(_lib.Config) == 64
     assert ctypes.sizeof(_lib.Epilogue) == 72
     assert ctypes.sizeof(_lib.GemmDesc) == 3 * 8 + 8 * 8 + 8 + 6 * 8 + 72
-    assert ctypes.sizeof(_lib.ConvDesc) == 3 * 8 + 14 * 4 + 72
+    assert ctypes.sizeof(_lib.ConvDesc) == 3 * 8 + 14 * 4 + 2 * 8 + 72
     assert ctypes.sizeof(_lib.KernelStat) == 64 + 8 + 3 * 8

@@ -5,7 +5,7 @@ import pytest
 
 from oracle import ops as ref
 from tests.harness import OpSession, assert_close
-from torpor_amd.server import ACT_NONE, ACT_RELU, NCHW, NHWC
+from torpor_amd.server import ACT_NONE, ACT_RELU, NCHW, NHWC, TorporError
 
 pytestmark = pytest.mark.gpu
 RTOL = 3e-5
@@ -104,6 +104,60 @@ def test_conv_rejects_bad_shapes(gpu_server):
         with pytest.raises(TorporError):
             t.s.stream_synchronize(t.fid)
         t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1)
+
+
+@pytest.mark.parametrize("C,k,stride,HW", [(32, 3, 1, 14), (24, 3, 2, 15), (16, 5, 2, 9), (8, 3, 1, 5)])
+def test_depthwise(gpu_server, C, k, stride, HW):
+    """groups == channels (MobileNet-style), with the fused batch-norm + relu6 epilogue."""
+    from torpor_amd.server import ACT_RELU6
+    rng = np.random.default_rng(C + k)
+    N, pad = 2, k // 2
+    x = _rand(rng, N, HW, HW, C) * 2
+    w = _rand(rng, C, 1, k, k)
+    g, b, mu = _rand(rng, C), _rand(rng, C), _rand(rng, C)
+    var = rng.uniform(0.5, 2.0, C).astype(np.float32)
+    Ho = (HW + 2 * pad - k) // stride + 1
+    with OpSession(gpu_server, [w, g, b, mu, var]) as t:
+        xv = t.act(x)
+        yv = t.empty(N * Ho * Ho * C * 4)
+        t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=C)
+        assert t.s.last_kernel() == "depthwise_nhwc"
+        plain = t.read(yv, (N, Ho, Ho, C))
+        t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=C,
+                 bn=tuple(t.w[1:5]), bn_eps=1e-5, act=ACT_RELU6)
+        fused = t.read(yv, (N, Ho, Ho, C))
+        with pytest.raises(TorporError):   # grouped but not depthwise
+            t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=2)
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)
+    want = ref.depthwise_conv2d(x, w, (stride, stride), (pad, pad))
+    assert_close(plain, want, RTOL, "depthwise")
+    z = ref.bn(want, g, b, mu, var, 1e-5, C, nhwc=True)
+    assert_close(fused, ref.activation(z, "relu6"), 5e-5, "depthwise+bn+relu6")
+
+
+@pytest.mark.parametrize("k", [1, 3])
+def test_conv_channel_slices(gpu_server, k):
+    """DenseNet-style concatenation without copies: read the first Cin channels of a wider
+    tensor (x_pitch) and write Cout channels into a slice of another (y_pitch, pointer offset)."""
+    rng = np.random.default_rng(k)
+    N, HW, Cin, Cout, XP, YP, off = 2, 12, 32, 16, 48, 40, 8
+    xw = _rand(rng, N, HW, HW, XP)
+    w = _rand(rng, Cout, Cin, k, k) * np.float32(1.0 / np.sqrt(Cin * k * k))
+    ywide = np.full((N, HW, HW, YP), 3.0, np.float32)
+    with OpSession(gpu_server, [w]) as t:
+        xv, yv = t.act(xw), t.act(ywide)
+        t.s.conv(t.fid, xv, t.w[0], yv + off * 4, N, HW, HW, Cin, Cout, k, k, stride=1, pad=k // 2, x_pitch=XP,
+                 y_pitch=YP)
+        got = t.read(yv, ywide.shape)
+        with pytest.raises(TorporError):   # slice would run past the end of y
+            t.s.conv(t.fid, xv, t.w[0], yv + (YP - Cout + 1) * 4, N, HW, HW, Cin, Cout, k, k, stride=1, pad=k // 2,
+                     x_pitch=XP, y_pitch=YP)
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)
+    want = ref.conv2d(np.ascontiguousarray(xw[..., :Cin]), w, (1, 1), (k // 2, k // 2), x_nhwc=True, y_nhwc=True)
+    assert_close(got[..., off:off + Cout], want, RTOL, "conv into a channel slice")
+    assert (got[..., :off] == 3).all() and (got[..., off + Cout:] == 3).all()
 
 
 @pytest.mark.parametrize("cfg,name", [(0, "fast_128x128"), (1, "fast_64x64"), (2, "fast_64x64_k3"), (3, "fast_32x32_k9"),

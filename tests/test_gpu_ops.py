@@ -8,7 +8,7 @@ from oracle import ops as ref
 from tests.harness import OpSession, assert_close
 from torpor_amd.server import (NCHW, NHWC, OP_ADD, OP_ATTENTION, OP_AVGPOOL, OP_BIAS_ACT, OP_EMBEDDING, OP_FILL, OP_GELU,
                                OP_LAYERNORM, OP_MAXPOOL, OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_RELU, OP_SOFTMAX,
-                               OP_SUM, ACT_RELU, TorporError)
+                               OP_SUM, OP_AVGPOOL2D, OP_COPY2D, ACT_RELU, ACT_RELU6, ACT_SILU, ACT_SIGMOID, TorporError)
 
 pytestmark = pytest.mark.gpu
 
@@ -86,6 +86,54 @@ def test_bias_act_and_layouts(gpu_server):
         np.testing.assert_array_equal(nhwc, img.transpose(0, 2, 3, 1))
         t.s.launch(t.fid, OP_NHWC_TO_NCHW, [ov, iv], [2, 5, 37, 41])
         np.testing.assert_array_equal(t.read(iv, img.shape), img)
+
+
+def test_new_activations_window_average_and_strided_views(gpu_server):
+    """relu6 / silu / sigmoid, k x k average pooling (also into a channel slice of a wider tensor),
+    2-D strided copy, and batch-norm over the first channels of a wider tensor."""
+    rng = np.random.default_rng(21)
+    x, bias = _rand(rng, 17, 24) * 4, _rand(rng, 24)
+    img = _rand(rng, 2, 9, 8, 12)
+    g, b, mu = _rand(rng, 8), _rand(rng, 8), _rand(rng, 8)
+    var = rng.uniform(0.2, 2.0, 8).astype(np.float32)
+    with OpSession(gpu_server, [bias, g, b, mu, var]) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        for act, name in ((ACT_RELU6, "relu6"), (ACT_SILU, "silu"), (ACT_SIGMOID, "sigmoid")):
+            t.s.launch(t.fid, OP_BIAS_ACT, [xv, t.w[0], yv], [17, 24, act])
+            assert_close(t.read(yv, x.shape), ref.activation(x + bias, name), 2e-6, name)
+        iv = t.act(img)
+        for k, st, pad in ((2, 2, 0), (3, 1, 1), (3, 2, 1)):
+            want = ref.avgpool2d(img, k, st, pad)
+            ov = t.empty(want.nbytes)
+            t.s.launch(t.fid, OP_AVGPOOL2D, [iv, ov], [2, 9, 8, 12, k, st, pad, 0])
+            assert_close(t.read(ov, want.shape), want, 2e-6, f"avgpool2d {k}/{st}/{pad}")
+        # ... into channels 4..15 of a 20-channel tensor that holds a marker value elsewhere
+        want = ref.avgpool2d(img, 2, 2, 0)
+        wide = np.full(want.shape[:3] + (20,), 7.0, np.float32)
+        wv = t.act(wide)
+        t.s.launch(t.fid, OP_AVGPOOL2D, [iv, wv + 4 * 4], [2, 9, 8, 12, 2, 2, 0, 20])
+        got = t.read(wv, wide.shape)
+        assert_close(got[..., 4:16], want, 2e-6, "avgpool2d into a slice")
+        assert (got[..., :4] == 7).all() and (got[..., 16:] == 7).all()
+        # strided copy: columns 3..10 of x into columns 1..8 of a 12-wide matrix
+        dst = np.zeros((17, 12), np.float32)
+        dv = t.act(dst)
+        t.s.launch(t.fid, OP_COPY2D, [xv + 3 * 4, dv + 1 * 4], [17, 8, 24, 12])
+        got = t.read(dv, dst.shape)
+        np.testing.assert_array_equal(got[:, 1:9], x[:, 3:11])
+        assert (got[:, 0] == 0).all() and (got[:, 9:] == 0).all()
+        # batch-norm + relu over the first 8 of 12 channels
+        bv = t.empty(2 * 9 * 8 * 8 * 4)
+        t.s.bn(t.fid, iv, bv, t.w[1], t.w[2], t.w[3], t.w[4], 1e-5, 2 * 9 * 8, 8, relu=True, x_pitch=12)
+        want = ref.bn(np.ascontiguousarray(img[..., :8]), g, b, mu, var, 1e-5, 8, nhwc=True, relu=True)
+        assert_close(t.read(bv, want.shape), want, 2e-6, "bn over a channel prefix")
+        with pytest.raises(TorporError):   # pitch smaller than the channel count
+            t.s.bn(t.fid, iv, bv, t.w[1], t.w[2], t.w[3], t.w[4], 1e-5, 2 * 9 * 8, 8, relu=True, x_pitch=4)
+        with pytest.raises(TorporError):   # the view would run past the end of the source
+            t.s.launch(t.fid, OP_COPY2D, [xv + 3 * 4, dv], [17, 8, 25, 12])
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)
 
 
 @pytest.mark.parametrize("layout", [NHWC, NCHW])

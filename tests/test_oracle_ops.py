@@ -104,6 +104,26 @@ def test_layernorm_softmax_gelu_vs_torch():
     assert ref.gelu(np.zeros(1, np.float32))[0] == 0
 
 
+def test_depthwise_avgpool2d_activations_vs_torch():
+    rng = np.random.default_rng(11)
+    x, w = _rand(rng, 2, 9, 7, 8), _rand(rng, 8, 1, 3, 3)
+    for stride, pad in ((1, 1), (2, 1), (1, 0)):
+        want = F.conv2d(torch.from_numpy(x).double().permute(0, 3, 1, 2), torch.from_numpy(w).double(), stride=stride,
+                        padding=pad, groups=8).permute(0, 2, 3, 1).numpy()
+        _close(ref.depthwise_conv2d(x, w, (stride, stride), (pad, pad)), want, 1e-6)
+    w5 = _rand(rng, 8, 1, 5, 5)
+    want = F.conv2d(torch.from_numpy(x).double().permute(0, 3, 1, 2), torch.from_numpy(w5).double(), stride=2, padding=2,
+                    groups=8).permute(0, 2, 3, 1).numpy()
+    _close(ref.depthwise_conv2d(x, w5, (2, 2), (2, 2)), want, 1e-6)
+    for k, stride, pad in ((2, 2, 0), (3, 1, 1), (3, 2, 1)):
+        want = F.avg_pool2d(torch.from_numpy(x).double().permute(0, 3, 1, 2), k, stride, pad).permute(0, 2, 3, 1).numpy()
+        _close(ref.avgpool2d(x, k, stride, pad), want, 1e-6)
+    t = torch.from_numpy(x).double() * 4
+    _close(ref.activation(x * 4, "relu6"), F.relu6(t).numpy(), 1e-7)
+    _close(ref.activation(x * 4, "silu"), F.silu(t).numpy(), 1e-6)
+    _close(ref.activation(x * 4, "sigmoid"), torch.sigmoid(t).numpy(), 1e-6)
+
+
 def test_attention_vs_torch():
     """The fused-attention oracle against torch's scaled_dot_product_attention (float64), with
     and without an additive key mask, and against the closed form for identical keys (uniform

@@ -69,6 +69,7 @@ class ConvDesc(C.Structure):
         ("stride_h", C.c_int32), ("stride_w", C.c_int32), ("pad_h", C.c_int32), ("pad_w", C.c_int32),
         ("groups", C.c_int32),
         ("x_layout", C.c_int32), ("y_layout", C.c_int32),
+        ("x_pitch", C.c_int64), ("y_pitch", C.c_int64),
         ("ep", Epilogue),
     ]
 
@@ -126,6 +127,8 @@ SYMBOLS = {
     "tp_conv_forward": (C.c_int, [_P, _I32, C.POINTER(ConvDesc)]),
     "tp_bn_inference": (C.c_int, [_P, _I32, _U64, _U64, _U64, _U64, _U64, _U64, C.c_double, _I64, _I32, _I64,
                                   _I32, _I32]),
+    "tp_bn_inference_pitched": (C.c_int, [_P, _I32, _U64, _U64, _U64, _U64, _U64, _U64, C.c_double, _I64, _I32,
+                                          _I64, _I32, _I32, _I64]),
     "tp_launch": (C.c_int, [_P, _I32, _I32, C.POINTER(_U64), _I32, C.POINTER(_I64), _I32,
                             C.POINTER(C.c_float), _I32]),
     "tp_replay": (C.c_int, [_P, _I32, _P, _U64, _P, _U64]),

@@ -421,17 +421,18 @@ class RemoteServer:
         self._async(Q_SGEMM_BATCHED, body.bytes())
 
     def conv(self, fid, x, w, y, n, h, w_in, cin, cout, kh, kw, stride=1, pad=0, x_layout=NHWC, y_layout=NHWC,
-             groups=1, **ep):
+             groups=1, x_pitch=0, y_pitch=0, **ep):
         sh, sw = (stride, stride) if isinstance(stride, int) else stride
         ph, pw = (pad, pad) if isinstance(pad, int) else pad
         b = Msg().u(4, x).u(6, w).u(13, y).u(20, n).u(21, h).u(22, w_in).u(23, cin).u(24, cout).u(25, kh).u(26, kw)
         b.u(27, sh).u(28, sw).u(29, ph).u(30, pw).u(31, groups).u(32, x_layout).u(33, y_layout)
-        b.sub(34, self._ep(**ep))
+        b.sub(34, self._ep(**ep)).u(35, x_pitch).u(36, y_pitch)
         self._async(Q_CONV, b.bytes())
 
-    def bn(self, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw=1, layout=NHWC, relu=False):
+    def bn(self, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw=1, layout=NHWC, relu=False, x_pitch=0):
         b = Msg().u(6, x).u(8, y).u(10, scale).u(11, bias).u(12, mean).u(13, var).f64(14, eps)
-        self._async(Q_BN, b.u(20, rows).u(21, channels).u(22, hw).u(23, layout).u(24, int(relu)).bytes())
+        b.u(20, rows).u(21, channels).u(22, hw).u(23, layout).u(24, int(relu)).u(25, x_pitch)
+        self._async(Q_BN, b.bytes())
 
     def launch(self, fid, op_id, ptrs, ints=(), floats=()):
         # packed repeated fields keep zero elements (a null pointer slot must stay in place)

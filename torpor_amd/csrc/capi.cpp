@@ -248,7 +248,7 @@ int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d) {
     TP_GUARD_BEGIN
     ENG(s);
     if (!d) return TP_EINVAL;
-    if (d->groups != 0 && d->groups != 1) return TP_EUNSUPPORTED;
+    if (d->groups < 0) return TP_EINVAL;
     tp::Op op;
     op.kind = tp::OPK_CONV;
     op.p[0] = d->x;
@@ -258,8 +258,11 @@ int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d) {
                             d->stride_w, d->pad_h, d->pad_w, d->x_layout, d->y_layout};
     for (int k = 0; k < 13; ++k) op.i[k] = iv[k];
     fill_epilogue(op, d->ep, 3, 13);
+    op.i[15] = d->x_pitch;
+    op.i[16] = d->y_pitch;
+    op.i[17] = d->groups > 0 ? d->groups : 1;
     op.np = 9;
-    op.ni = 15;
+    op.ni = 18;
     return E.op_compute(client, op);
     TP_GUARD_END
 }
@@ -284,6 +287,33 @@ int tp_bn_inference(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64
     op.i[3] = layout;
     op.i[4] = relu;
     op.ni = 5;
+    op.f[0] = (float)eps;
+    op.nf = 1;
+    return E.op_compute(client, op);
+    TP_GUARD_END
+}
+
+int tp_bn_inference_pitched(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
+                    uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
+                    int32_t layout, int32_t relu, int64_t x_pitch) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    tp::Op op;
+    op.kind = tp::OPK_BN;
+    op.p[0] = x;
+    op.p[1] = y;
+    op.p[2] = scale;
+    op.p[3] = bias;
+    op.p[4] = mean;
+    op.p[5] = var;
+    op.np = 6;
+    op.i[0] = rows;
+    op.i[1] = channels;
+    op.i[2] = hw;
+    op.i[3] = layout;
+    op.i[4] = relu;
+    op.i[5] = x_pitch;
+    op.ni = 6;
     op.f[0] = (float)eps;
     op.nf = 1;
     return E.op_compute(client, op);

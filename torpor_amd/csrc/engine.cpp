@@ -1073,11 +1073,17 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
                 return TP_EINVAL;
             const int64_t Ho = (H + 2 * ph - KH) / sh + 1, Wo = (W + 2 * pw - KW) / sw + 1;
             if (H + 2 * ph < KH || W + 2 * pw < KW || Ho < 1 || Wo < 1) return TP_EINVAL;
-            const int64_t ys = N * Ho * Wo * Cout;
-            if ((r = R(0, false, N * H * W * Cin)) || (r = R(1, false, Cout * Cin * KH * KW)) || (r = R(2, false, ys)))
+            const int64_t xpitch = op.ni > 15 ? I[15] : 0, ypitch = op.ni > 16 ? I[16] : 0;
+            const int64_t groups = (op.ni > 17 && I[17] > 0) ? I[17] : 1;
+            const bool x_nhwc = I[11] != 0, y_nhwc = I[12] != 0;
+            if ((xpitch && (!x_nhwc || xpitch < Cin)) || (ypitch && (!y_nhwc || ypitch < Cout))) return TP_EINVAL;
+            if (groups != 1 && (groups != Cin || Cin != Cout)) return TP_EUNSUPPORTED;
+            const int64_t ys = ypitch ? (N * Ho * Wo - 1) * ypitch + Cout : N * Ho * Wo * Cout;
+            const int64_t xs = xpitch ? (N * H * W - 1) * xpitch + Cin : N * H * W * Cin;
+            if ((r = R(0, false, xs)) || (r = R(1, false, Cout * (Cin / groups) * KH * KW)) || (r = R(2, false, ys)))
                 return r;
             for (int k = 3; k < 8 && !r; ++k) r = R(k, true, Cout);
-            if (!r) r = R(8, true, ys);
+            if (!r) r = R(8, true, N * Ho * Wo * Cout);  // residual: dense unless ldr says otherwise
             if (r) return r;
             if ((q[4] != nullptr) != (q[5] != nullptr) || (q[4] != nullptr) != (q[6] != nullptr) ||
                 (q[4] != nullptr) != (q[7] != nullptr))
@@ -1099,6 +1105,9 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             c.pw = (int)pw;
             c.x_nhwc = (int)I[11];
             c.y_nhwc = (int)I[12];
+            c.x_pitch = xpitch;
+            c.y_pitch = ypitch;
+            c.groups = (int)groups;
             c.ep = ep_from(op, q, 3, 0, 13);
             c.ep.ldr = 0;  // residual shares the layout and pitch of y
             if (!launch) return 0;
@@ -1106,8 +1115,10 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         }
         case OPK_BN: {
             const int64_t rows = I[0], C = I[1];
-            if (C < 1) return TP_EINVAL;
-            if ((r = R(0, false, rows * C)) || (r = R(1, false, rows * C))) return r;
+            const int64_t xpitch = op.ni > 5 ? I[5] : 0;
+            if (C < 1 || (xpitch && xpitch < C)) return TP_EINVAL;
+            const int64_t xspan = (xpitch && rows > 0) ? (rows - 1) * xpitch + C : rows * C;
+            if ((r = R(0, false, xspan)) || (r = R(1, false, rows * C))) return r;
             for (int k = 2; k < 6 && !r; ++k) r = R(k, false, C);
             if (r) return r;
             if (!I[3] && I[2] < 1) return TP_EINVAL;
@@ -1115,7 +1126,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             return tpk::launch_bn_inference(static_cast<const float*>(q[0]), static_cast<float*>(q[1]),
                                             static_cast<const float*>(q[2]), static_cast<const float*>(q[3]),
                                             static_cast<const float*>(q[4]), static_cast<const float*>(q[5]), op.f[0],
-                                            rows, (int)C, (int)I[3], I[2], (int)I[4], compute_);
+                                            rows, (int)C, (int)I[3], I[2], (int)I[4], xpitch, compute_);
         }
         case OPK_LAUNCH:
             break;
@@ -1200,6 +1211,27 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             if ((r = R(0, false, I[0])) || (r = R(1, false, 1))) return r;
             if (!launch) return 0;
             return tpk::launch_sum(F(0), Fm(1), I[0], compute_);
+        case TP_OP_AVGPOOL2D: {
+            if (!need(2, 8, 0)) return TP_EINVAL;
+            const int64_t N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
+            if (N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || st < 1 || H + 2 * pad < k || W + 2 * pad < k)
+                return TP_EINVAL;
+            const int64_t yp = I[7] ? I[7] : C;
+            if (yp < C) return TP_EINVAL;
+            const int64_t Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
+            if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, (N * Ho * Wo - 1) * yp + C))) return r;
+            if (!launch) return 0;
+            return tpk::launch_avgpool2d(F(0), Fm(1), (int)N, (int)H, (int)W, (int)C, (int)k, (int)st, (int)pad, yp,
+                                         compute_);
+        }
+        case TP_OP_COPY2D: {
+            if (!need(2, 4, 0)) return TP_EINVAL;
+            const int64_t rows = I[0], width = I[1], sp = I[2], dp = I[3];
+            if (rows < 1 || width < 1 || sp < width || dp < width) return TP_EINVAL;
+            if ((r = R(0, false, (rows - 1) * sp + width)) || (r = R(1, false, (rows - 1) * dp + width))) return r;
+            if (!launch) return 0;
+            return tpk::launch_copy2d(F(0), Fm(1), rows, (int)width, sp, dp, compute_);
+        }
         case TP_OP_ATTENTION: {
             if (!need(5, 8, 1)) return TP_EINVAL;
             const int64_t B = I[0], A = I[1], S = I[2], dh = I[3];
@@ -1272,6 +1304,8 @@ static void op_work(const Op& op, double* flops, double* bytes, const char** nam
                 case TP_OP_NHWC_TO_NCHW: *bytes = 8.0 * (double)(I[0] * I[1] * I[2] * I[3]); *name = "layout"; break;
                 case TP_OP_SUM: *bytes = 4.0 * (double)I[0]; *name = "sum"; break;
                 case TP_OP_FILL: *bytes = 4.0 * (double)I[0]; *name = "fill"; break;
+                case TP_OP_AVGPOOL2D: *bytes = 4.0 * (double)(I[0] * I[1] * I[2] * I[3]) * 1.25; *name = "avgpool2d"; break;
+                case TP_OP_COPY2D: *bytes = 8.0 * (double)(I[0] * I[1]); *name = "copy2d"; break;
                 case TP_OP_ATTENTION:
                     *flops = 4.0 * (double)(I[0] * I[1]) * (double)(I[2] * I[2]) * (double)I[3];
                     *bytes = 16.0 * (double)(I[0] * I[2]) * (double)(I[1] * I[3]);

@@ -235,6 +235,85 @@ using Conv3S = TileCfg<64, 64, 72, 2, 2, 3>;  // 12 wavefronts: 2x2 over the til
 using Conv3T = TileCfg<32, 32, 72, 1, 1, 9>;  // 9 wavefronts, one k-group each
 using Conv3U = TileCfg<32, 32, 72, 1, 1, 3>;  // 3 wavefronts
 
+// Depthwise convolution (groups == Cin == Cout), NHWC, weights [C][1][KH][KW]: HBM-bound, one
+// thread per output pixel and channel quad, taps accumulated in registers, same fused epilogue
+// as the MFMA kernels (folded batch-norm / bias, residual, activation).
+struct DwDev {
+    const float* x;
+    const float* w;
+    float* y;
+    int H, W, C, KH, KW, Ho, Wo, sh, sw, ph, pw;
+    long xp, yp;
+    long total;  // N*Ho*Wo*(C/4)
+    Epilogue ep;
+};
+__global__ __launch_bounds__(256) void depthwise_kernel(const DwDev p) {
+    const long st = (long)gridDim.x * blockDim.x;
+    const int C4 = p.C >> 2;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total; i += st) {
+        const int c = (int)(i % C4) * 4;
+        long t = i / C4;
+        const long row = t;  // output pixel index (n, ho, wo)
+        const int wo = (int)(t % p.Wo);
+        t /= p.Wo;
+        const int ho = (int)(t % p.Ho);
+        const long n = t / p.Ho;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const float* wc = p.w + (long)c * p.KH * p.KW;
+        const int kk = p.KH * p.KW;
+        for (int kh = 0; kh < p.KH; ++kh) {
+            const int hi = ho * p.sh - p.ph + kh;
+            if (hi < 0 || hi >= p.H) continue;
+            for (int kw = 0; kw < p.KW; ++kw) {
+                const int wi = wo * p.sw - p.pw + kw;
+                if (wi < 0 || wi >= p.W) continue;
+                const f32x4 xv = *reinterpret_cast<const f32x4*>(p.x + ((n * p.H + hi) * p.W + wi) * p.xp + c);
+                const int tap = kh * p.KW + kw;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] += xv[j] * wc[j * kk + tap];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float cs, ct;
+            epilogue_column(p.ep, c + j, cs, ct);
+            epilogue_store(p.ep, p.y, row, c + j, acc[j], cs, ct);
+        }
+    }
+}
+
+static int launch_depthwise(const ConvArgs& a, int Ho, int Wo, long xp, long yp, hipStream_t s) {
+    if (a.groups != a.Cin || a.Cin != a.Cout) return K_EUNSUPPORTED;  // only groups == channels
+    if (!a.x_nhwc || !a.y_nhwc || a.Cin % 4 != 0 || xp % 4 != 0) return K_EUNSUPPORTED;
+    if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0) return K_EUNSUPPORTED;
+    DwDev p;
+    p.x = a.x;
+    p.w = a.w;
+    p.y = a.y;
+    p.H = a.H;
+    p.W = a.W;
+    p.C = a.Cin;
+    p.KH = a.KH;
+    p.KW = a.KW;
+    p.Ho = Ho;
+    p.Wo = Wo;
+    p.sh = a.sh;
+    p.sw = a.sw;
+    p.ph = a.ph;
+    p.pw = a.pw;
+    p.xp = xp;
+    p.yp = yp;
+    p.total = (long)a.N * Ho * Wo * (a.Cin / 4);
+    EpilogueArgs ea = a.ep;
+    if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;
+    p.ep = make_epilogue(ea, yp);
+    long blocks = (p.total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(depthwise_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p);
+    set_last_kernel("depthwise_nhwc");
+    return (int)hipGetLastError();
+}
+
 static inline bool aligned16c(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
@@ -246,6 +325,12 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     if (Ho <= 0 || Wo <= 0) return K_EINVAL;
     const long M = (long)a.N * Ho * Wo;
 
+    if ((a.x_pitch && (!a.x_nhwc || a.x_pitch < a.Cin)) || (a.y_pitch && (!a.y_nhwc || a.y_pitch < a.Cout)))
+        return K_EINVAL;
+    const long xp = a.x_pitch ? a.x_pitch : a.Cin;   // floats between pixels (NHWC)
+    const long yp = a.y_pitch ? a.y_pitch : a.Cout;
+    if (a.groups != 1) return launch_depthwise(a, Ho, Wo, xp, yp, s);
+
     // 1x1 over NHWC is a dense GEMM, with a row gather when strided.
     if (a.KH == 1 && a.KW == 1 && a.ph == 0 && a.pw == 0 && a.x_nhwc && a.y_nhwc) {
         GemmArgs g;
@@ -255,11 +340,11 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         g.M = M;
         g.N = a.Cout;
         g.K = a.Cin;
-        g.xs_r = a.Cin;
+        g.xs_r = xp;
         g.xs_k = 1;
         g.ys_c = a.Cin;
         g.ys_k = 1;
-        g.ldc = a.Cout;
+        g.ldc = yp;
         if (a.sh != 1 || a.sw != 1) {
             g.gather = 1;
             g.Ho = Ho;
@@ -293,9 +378,9 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     p.pw = a.pw;
     if (a.x_nhwc) {
         p.xs_c = 1;
-        p.xs_w = a.Cin;
-        p.xs_h = (long)a.W * a.Cin;
-        p.xs_n = (long)a.H * a.W * a.Cin;
+        p.xs_w = xp;
+        p.xs_h = (long)a.W * xp;
+        p.xs_n = (long)a.H * a.W * xp;
     } else {
         p.xs_w = 1;
         p.xs_h = a.W;
@@ -308,14 +393,14 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     p.zeros = ws.zeros;
     EpilogueArgs ea = a.ep;
     if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;
-    p.ep = make_epilogue(ea, a.Cout);
+    p.ep = make_epilogue(ea, yp);
     if (!a.y_nhwc) {
         p.ep.out_nchw = 1;
         p.ep.howo = (long)Ho * Wo;
         p.ep.ncols = a.Cout;
     }
 
-    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && aligned16c(a.x) &&
+    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && (xp % 4 == 0) && aligned16c(a.x) &&
                        aligned16c(a.w) && ws.zeros != nullptr;
     if (fast3) {
         const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);

@@ -48,6 +48,11 @@ struct ConvArgs {
     int N = 0, H = 0, W = 0, Cin = 0, Cout = 0, KH = 0, KW = 0;
     int sh = 1, sw = 1, ph = 0, pw = 0;
     int x_nhwc = 1, y_nhwc = 1;  // 0 = NCHW
+    // NHWC only: floats between consecutive pixels of x / y (0 = Cin / Cout).  A larger pitch
+    // reads the first Cin channels of a wider tensor or writes a channel slice of one (how
+    // DenseNet-style concatenation is served without a copy).
+    long x_pitch = 0, y_pitch = 0;
+    int groups = 1;              // 1, or Cin == Cout == groups (depthwise, NHWC, w is [C][1][KH][KW])
     EpilogueArgs ep;             // residual shares the layout of y
 };
 
@@ -65,8 +70,16 @@ const char* last_kernel_name();
 void set_last_kernel(const char* name);
 
 // ---- HBM-bound operators (elementwise.hip / reduce.hip) ----
+// x_pitch: NHWC only, floats between consecutive rows of x (0 = C); y is always dense.
 int launch_bn_inference(const float* x, float* y, const float* g, const float* b, const float* mean,
-                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, hipStream_t s);
+                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, long x_pitch,
+                        hipStream_t s);
+// NHWC average pooling, window k x k, zero padding counted in the divisor (torch's
+// count_include_pad=True); y_pitch = floats between output pixels (0 = C).
+int launch_avgpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, long y_pitch,
+                     hipStream_t s);
+// dst[r*dst_pitch + c] = src[r*src_pitch + c], r < rows, c < width
+int launch_copy2d(const float* src, float* dst, long rows, int width, long src_pitch, long dst_pitch, hipStream_t s);
 int launch_relu(const float* x, float* y, long n, hipStream_t s);
 int launch_add(const float* a, const float* b, float* y, long n, int relu, hipStream_t s);
 int launch_bias_act(const float* x, const float* bias, float* y, long rows, int C, int act, hipStream_t s);

@@ -18,7 +18,7 @@ namespace tpk {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_TANH = 3 };
+enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_TANH = 3, ACT_RELU6 = 4, ACT_SILU = 5, ACT_SIGMOID = 6 };
 
 // out = act( bn( alpha*acc + beta*C_old + bias[n] ) + residual )
 struct Epilogue {
@@ -45,6 +45,9 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == ACT_RELU) return v > 0.f ? v : 0.f;
     if (act == ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
     if (act == ACT_TANH) return tanhf(v);
+    if (act == ACT_RELU6) return fminf(fmaxf(v, 0.f), 6.f);
+    if (act == ACT_SILU) return v / (1.0f + expf(-v));
+    if (act == ACT_SIGMOID) return 1.0f / (1.0f + expf(-v));
     return v;
 }
 

@@ -66,11 +66,40 @@ __global__ __launch_bounds__(256) void bn_scalar_kernel(const float* __restrict_
         y[i] = o;
     }
 }
+// rows of C floats at x + row*x_pitch -> dense y
+__global__ __launch_bounds__(256) void bn_nhwc_pitch_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                            const float* __restrict__ g, const float* __restrict__ b,
+                                                            const float* __restrict__ mean,
+                                                            const float* __restrict__ var, float eps, long n4, int C4,
+                                                            long x_pitch, int relu) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        const long row = i / C4;
+        const int c = (int)(i - row * C4) * 4;
+        f32x4 v = *reinterpret_cast<const f32x4*>(x + row * x_pitch + c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float sc = g[c + j] / sqrtf(var[c + j] + eps);
+            float t = (v[j] - mean[c + j]) * sc + b[c + j];
+            if (relu) t = t > 0.f ? t : 0.f;
+            v[j] = t;
+        }
+        reinterpret_cast<f32x4*>(y)[i] = v;
+    }
+}
 int launch_bn_inference(const float* x, float* y, const float* g, const float* b, const float* mean,
-                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, hipStream_t s) {
+                        const float* var, float eps, long rows, int C, int nhwc, long hw, int relu, long x_pitch,
+                        hipStream_t s) {
     if (!x || !y || !g || !b || !mean || !var || rows < 0 || C <= 0) return K_EINVAL;
     const long n = rows * C;  // rows = N*H*W
     if (n == 0) return 0;
+    if (x_pitch != 0 && x_pitch != C) {
+        if (!nhwc || x_pitch < C) return K_EINVAL;
+        if (C % 4 != 0 || x_pitch % 4 != 0 || !al16(x) || !al16(y)) return K_EUNSUPPORTED;
+        hipLaunchKernelGGL(bn_nhwc_pitch_kernel, dim3(grid_for(n / 4, 256)), dim3(256), 0, s, x, y, g, b, mean, var,
+                           eps, n / 4, C / 4, x_pitch, relu);
+        return (int)hipGetLastError();
+    }
     if (nhwc && C % 4 == 0 && al16(x) && al16(y)) {
         hipLaunchKernelGGL(bn_nhwc_vec_kernel, dim3(grid_for(n / 4, 256)), dim3(256), 0, s,
                            reinterpret_cast<const f32x4*>(x), reinterpret_cast<f32x4*>(y), g, b, mean, var, eps,
@@ -79,6 +108,64 @@ int launch_bn_inference(const float* x, float* y, const float* g, const float* b
         hipLaunchKernelGGL(bn_scalar_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, x, y, g, b, mean, var, eps, n,
                            C, hw, nhwc, relu);
     }
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- pooling window / strided copy
+__global__ __launch_bounds__(256) void avgpool2d_kernel(const float* __restrict__ x, float* __restrict__ y, int H,
+                                                        int W, int C, int Ho, int Wo, int k, int stride, int pad,
+                                                        long y_pitch, long total) {
+    const long st = (long)gridDim.x * blockDim.x;
+    const float inv = 1.0f / (float)(k * k);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += st) {
+        const int c = (int)(i % C);
+        long t = i / C;
+        const int wo = (int)(t % Wo);
+        t /= Wo;
+        const int ho = (int)(t % Ho);
+        const long n = t / Ho;
+        float acc = 0.f;
+        for (int kh = 0; kh < k; ++kh) {
+            const int hi = ho * stride - pad + kh;
+            if (hi < 0 || hi >= H) continue;
+            for (int kw = 0; kw < k; ++kw) {
+                const int wi = wo * stride - pad + kw;
+                if (wi < 0 || wi >= W) continue;
+                acc += x[((n * H + hi) * W + wi) * C + c];
+            }
+        }
+        y[((n * Ho + ho) * Wo + wo) * y_pitch + c] = acc * inv;
+    }
+}
+int launch_avgpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, long y_pitch,
+                     hipStream_t s) {
+    if (!x || !y || N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || stride < 1 || pad < 0 || H + 2 * pad < k ||
+        W + 2 * pad < k)
+        return K_EINVAL;
+    if (y_pitch == 0) y_pitch = C;
+    if (y_pitch < C) return K_EINVAL;
+    const int Ho = (H + 2 * pad - k) / stride + 1, Wo = (W + 2 * pad - k) / stride + 1;
+    const long total = (long)N * Ho * Wo * C;
+    hipLaunchKernelGGL(avgpool2d_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, x, y, H, W, C, Ho, Wo, k,
+                       stride, pad, y_pitch, total);
+    return (int)hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void copy2d_kernel(const float* __restrict__ src, float* __restrict__ dst, long total,
+                                                     int width, long src_pitch, long dst_pitch) {
+    const long st = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += st) {
+        const long r = i / width;
+        const int c = (int)(i - r * width);
+        dst[r * dst_pitch + c] = src[r * src_pitch + c];
+    }
+}
+int launch_copy2d(const float* src, float* dst, long rows, int width, long src_pitch, long dst_pitch, hipStream_t s) {
+    if (!src || !dst || rows < 0 || width < 1 || src_pitch < width || dst_pitch < width) return K_EINVAL;
+    const long total = rows * width;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(copy2d_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, src, dst, total, width, src_pitch,
+                       dst_pitch);
     return (int)hipGetLastError();
 }
 

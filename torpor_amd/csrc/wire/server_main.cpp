@@ -283,6 +283,8 @@ bool handle_query(Server& S, int type, const pb::View& q, int client, std::strin
                     case 31: d.groups = (int32_t)u; break;
                     case 32: d.x_layout = (int32_t)u; break;
                     case 33: d.y_layout = (int32_t)u; break;
+                    case 35: d.x_pitch = (int64_t)u; break;
+                    case 36: d.y_pitch = (int64_t)u; break;
                     default: break;
                 }
             }
@@ -294,7 +296,7 @@ bool handle_query(Server& S, int type, const pb::View& q, int client, std::strin
         case Q_BN: {
             uint64_t x = 0, y = 0, g = 0, b = 0, mu = 0, var = 0;
             double eps = 0.0;
-            int64_t rows = 0, hw = 1;
+            int64_t rows = 0, hw = 1, x_pitch = 0;
             int channels = 0, layout = 0, relu = 0;
             while (r.next(&f, &wt)) {
                 if (f == 14 && wt == pb::WT_FIXED64) { eps = r.f64(); continue; }
@@ -311,10 +313,12 @@ bool handle_query(Server& S, int type, const pb::View& q, int client, std::strin
                     case 22: hw = (int64_t)u; break;
                     case 23: layout = (int)u; break;
                     case 24: relu = (int)u; break;
+                    case 25: x_pitch = (int64_t)u; break;
                     default: break;
                 }
             }
-            (void)tp_bn_inference(S.eng, client, x, y, g, b, mu, var, eps, rows, channels, hw, layout, relu);
+            (void)tp_bn_inference_pitched(S.eng, client, x, y, g, b, mu, var, eps, rows, channels, hw, layout, relu,
+                                          x_pitch);
             return false;
         }
         case Q_LAUNCH: {

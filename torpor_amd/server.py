@@ -14,10 +14,10 @@ from ._lib import TorporError
 
 REQ_EXECUTE_AFTER_LOAD, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD = 0, 1, 2, 3
 ACK_OK, ACK_INAVAIL = 0, 1
-ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH, ACT_RELU6, ACT_SILU, ACT_SIGMOID = 0, 1, 2, 3, 4, 5, 6
 NCHW, NHWC = 0, 1
 (OP_RELU, OP_ADD, OP_BIAS_ACT, OP_GELU, OP_MAXPOOL, OP_AVGPOOL, OP_LAYERNORM, OP_SOFTMAX, OP_EMBEDDING,
- OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION) = range(1, 15)
+ OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION, OP_AVGPOOL2D, OP_COPY2D) = range(1, 17)
 FLAG_HOST_ONLY = 1
 
 
@@ -148,7 +148,7 @@ class Server:
                                               beta, c, ldc, sc, count), "tp_sgemm_strided_batched")
 
     def conv(self, fid, x, w, y, n, h, w_in, cin, cout, kh, kw, stride=1, pad=0, x_layout=NHWC, y_layout=NHWC,
-             groups=1, **ep):
+             groups=1, x_pitch=0, y_pitch=0, **ep):
         d = _lib.ConvDesc()
         d.x, d.w, d.y = x, w, y
         d.n, d.h, d.w_in, d.cin, d.cout, d.kh, d.kw = n, h, w_in, cin, cout, kh, kw
@@ -156,12 +156,13 @@ class Server:
         ph, pw = (pad, pad) if isinstance(pad, int) else pad
         d.stride_h, d.stride_w, d.pad_h, d.pad_w, d.groups = sh, sw, ph, pw, groups
         d.x_layout, d.y_layout = x_layout, y_layout
+        d.x_pitch, d.y_pitch = x_pitch, y_pitch
         self._epilogue(d.ep, **ep)
         _chk(self._l.tp_conv_forward(self._h, fid, C.byref(d)), "tp_conv_forward")
 
-    def bn(self, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw=1, layout=NHWC, relu=False):
-        _chk(self._l.tp_bn_inference(self._h, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw, layout,
-                                     int(relu)), "tp_bn_inference")
+    def bn(self, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw=1, layout=NHWC, relu=False, x_pitch=0):
+        _chk(self._l.tp_bn_inference_pitched(self._h, fid, x, y, scale, bias, mean, var, eps, rows, channels, hw,
+                                             layout, int(relu), x_pitch), "tp_bn_inference")
 
     def launch(self, fid, op_id, ptrs, ints=(), floats=()):
         P = (C.c_uint64 * max(1, len(ptrs)))(*ptrs)
