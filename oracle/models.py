@@ -148,6 +148,115 @@ class Bert(nn.Module):
         return h, pooled
 
 
+DENSENET_BLOCKS = {"densenet121": (6, 12, 24, 16), "densenet169": (6, 12, 32, 32), "densenet201": (6, 12, 48, 32)}
+
+
+class _DenseLayer(nn.Module):
+    def __init__(self, cin, growth=32, bn_size=4):
+        super().__init__()
+        self.norm1 = nn.BatchNorm2d(cin)
+        self.conv1 = nn.Conv2d(cin, bn_size * growth, 1, bias=False)
+        self.norm2 = nn.BatchNorm2d(bn_size * growth)
+        self.conv2 = nn.Conv2d(bn_size * growth, growth, 3, padding=1, bias=False)
+
+    def forward(self, x):
+        return self.conv2(F.relu(self.norm2(self.conv1(F.relu(self.norm1(x))))))
+
+
+class DenseNet(nn.Module):
+    """Densely connected network (Huang et al. 2017) with torchvision's layer names: growth 32,
+    bottleneck width 4 x growth, 64 stem channels, transitions halve channels and resolution."""
+
+    def __init__(self, arch="densenet169", num_classes=1000, growth=32):
+        super().__init__()
+        f = nn.Sequential()
+        f.add_module("conv0", nn.Conv2d(3, 64, 7, stride=2, padding=3, bias=False))
+        f.add_module("norm0", nn.BatchNorm2d(64))
+        c = 64
+        blocks = DENSENET_BLOCKS[arch]
+        for bi, n in enumerate(blocks):
+            blk = nn.Module()
+            for li in range(n):
+                blk.add_module(f"denselayer{li + 1}", _DenseLayer(c + li * growth, growth))
+            f.add_module(f"denseblock{bi + 1}", blk)
+            c += n * growth
+            if bi != len(blocks) - 1:
+                tr = nn.Module()
+                tr.norm = nn.BatchNorm2d(c)
+                tr.conv = nn.Conv2d(c, c // 2, 1, bias=False)
+                f.add_module(f"transition{bi + 1}", tr)
+                c //= 2
+        f.add_module("norm5", nn.BatchNorm2d(c))
+        self.features = f
+        self.blocks = blocks
+        self.classifier = nn.Linear(c, num_classes)
+
+    def forward(self, x):
+        f = self.features
+        x = F.max_pool2d(F.relu(f.norm0(f.conv0(x))), 3, 2, 1)
+        for bi, n in enumerate(self.blocks):
+            blk = getattr(f, f"denseblock{bi + 1}")
+            for li in range(n):
+                x = torch.cat([x, getattr(blk, f"denselayer{li + 1}")(x)], 1)
+            if bi != len(self.blocks) - 1:
+                tr = getattr(f, f"transition{bi + 1}")
+                x = F.avg_pool2d(tr.conv(F.relu(tr.norm(x))), 2, 2)
+        x = F.relu(f.norm5(x))
+        return self.classifier(x.mean((2, 3)))
+
+
+MOBILENET_V2 = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1))
+
+
+class _ConvBN(nn.Sequential):
+    def __init__(self, cin, cout, k, stride=1, groups=1):
+        super().__init__(nn.Conv2d(cin, cout, k, stride, k // 2, groups=groups, bias=False), nn.BatchNorm2d(cout))
+
+
+class _InvertedResidual(nn.Module):
+    def __init__(self, cin, cout, stride, expand):
+        super().__init__()
+        hidden = cin * expand
+        layers = []
+        if expand != 1:
+            layers.append(_ConvBN(cin, hidden, 1))          # + relu6
+        layers.append(_ConvBN(hidden, hidden, 3, stride, groups=hidden))  # depthwise, + relu6
+        layers.append(_ConvBN(hidden, cout, 1))             # linear projection
+        self.conv = nn.Sequential(*layers)
+        self.residual = stride == 1 and cin == cout
+
+    def forward(self, x):
+        y = x
+        for i, m in enumerate(self.conv):
+            y = m(y)
+            if i != len(self.conv) - 1:
+                y = F.relu6(y)
+        return x + y if self.residual else y
+
+
+class MobileNetV2(nn.Module):
+    """MobileNetV2 (Sandler et al. 2018), width 1.0: inverted residuals with linear bottlenecks."""
+
+    def __init__(self, num_classes=1000):
+        super().__init__()
+        feats = [_ConvBN(3, 32, 3, 2)]
+        c = 32
+        for t, cout, n, s in MOBILENET_V2:
+            for i in range(n):
+                feats.append(_InvertedResidual(c, cout, s if i == 0 else 1, t))
+                c = cout
+        feats.append(_ConvBN(c, 1280, 1))
+        self.features = nn.Sequential(*feats)
+        self.classifier = nn.Linear(1280, num_classes)
+
+    def forward(self, x):
+        x = F.relu6(self.features[0](x))
+        for m in list(self.features)[1:-1]:
+            x = m(x)
+        x = F.relu6(self.features[-1](x))
+        return self.classifier(x.mean((2, 3)))
+
+
 def load_numpy_state(module, weights):
     """Strictly load a {name: np.ndarray} dict (BN `num_batches_tracked` buffers excepted)."""
     sd = {k: torch.from_numpy(v.copy()) for k, v in weights.items()}

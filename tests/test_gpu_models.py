@@ -7,7 +7,7 @@ import torch
 
 from oracle import models as om
 from tests.harness import assert_close
-from torpor_amd.functions import bert, resnet
+from torpor_amd.functions import bert, densenet, mobilenet, resnet
 
 pytestmark = pytest.mark.gpu
 LOGIT_RTOL = 1e-3   # north-star bar: rel 1e-3 (fp32) on logits
@@ -22,7 +22,7 @@ def _perturb_bn(weights, seed):
             weights[k] = rng.uniform(0.5, 1.5, n).astype(np.float32)
         elif k.endswith("running_mean"):
             weights[k] = (rng.standard_normal(n) * 0.1).astype(np.float32)
-        elif ".bn" in k or "downsample.1" in k or k.startswith("bn1"):
+        elif len(n) == 1 and (k[:-len(".weight")] + ".running_var" in weights or k[:-len(".bias")] + ".running_var" in weights):
             if k.endswith(".weight"):
                 weights[k] = rng.uniform(0.8, 1.2, n).astype(np.float32)
             elif k.endswith(".bias"):
@@ -149,6 +149,41 @@ def test_resnet101(gpu_server):
     with torch.no_grad():
         want = model(torch.from_numpy(x)).numpy()
     assert_close(logits, want, LOGIT_RTOL, "resnet101 logits")
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+@pytest.mark.parametrize("arch,image,batch", [("densenet121", 64, 2), ("densenet169", 224, 1)])
+def test_densenet(gpu_server, arch, image, batch):
+    """DenseNet (served by the reference, tests/endpoint.py:20-23): dense blocks built in place in one
+    wide buffer (pitched batch-norm input, convolution output into a channel slice)."""
+    weights = _perturb_bn(densenet.init_weights(arch, seed=6), seed=7)
+    x = torch.randn(batch, 3, image, image, generator=torch.Generator().manual_seed(8)).numpy()
+    fn = densenet.DenseNet(gpu_server, 13, arch, batch=batch, weights=weights, image=image)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.DenseNet(arch), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, f"{arch} logits")
+    print(f"{arch} b{batch} {image}px: rel err {e:.2e}")
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+@pytest.mark.parametrize("image,batch", [(96, 2), (224, 1)])
+def test_mobilenet_v2(gpu_server, image, batch):
+    """MobileNetV2 (tests/endpoint.py:30-31): depthwise convolutions, relu6, linear bottlenecks."""
+    weights = _perturb_bn(mobilenet.init_weights(seed=9), seed=10)
+    x = torch.randn(batch, 3, image, image, generator=torch.Generator().manual_seed(11)).numpy()
+    fn = mobilenet.MobileNetV2(gpu_server, 14, batch=batch, weights=weights, image=image)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.MobileNetV2(), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, "mobilenet_v2 logits")
+    print(f"mobilenet_v2 b{batch} {image}px: rel err {e:.2e}")
+    _check_swap_identity(gpu_server, fn, weights)
     _cycle(gpu_server, fn, [x], [logits])
     fn.unload()
 

@@ -5,6 +5,7 @@ code, no download).  Product-side weight generators must load strictly into thes
 import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import models as om
 from torpor_amd.functions import bert as pbert
@@ -16,7 +17,7 @@ def _macs(model, x):
 
     def hook(mod, inp, out):
         if isinstance(mod, torch.nn.Conv2d):
-            total[0] += out.numel() * mod.in_channels * mod.kernel_size[0] * mod.kernel_size[1]
+            total[0] += out.numel() * (mod.in_channels // mod.groups) * mod.kernel_size[0] * mod.kernel_size[1]
         elif isinstance(mod, torch.nn.Linear):
             total[0] += out.numel() * mod.in_features
 
@@ -155,3 +156,59 @@ def test_bert_qa_head_matches_transformers():
     om.load_numpy_state(om.Bert(layers=2, hidden=64, heads=4, ffn=128, vocab=97, max_pos=40, qa_head=True), w)
     add = pbert.Bert.additive_mask(am.numpy())
     assert add.dtype == np.float32 and (add[0, :13] == 0).all() and (add[0, 13:] == np.finfo(np.float32).min).all()
+
+
+@pytest.mark.parametrize("arch,params,gmacs", [("densenet121", 7978856, 2.834), ("densenet169", 14149480, 3.360),
+                                               ("densenet201", 20013928, 4.291)])
+def test_densenet_counts(arch, params, gmacs):
+    """Published parameter counts (7,978,856 / 14,149,480 / 20,013,928) and multiply-accumulates per
+    224x224 image (2.83 / 3.36 / 4.29 G) of DenseNet-121 / -169 / -201, and the channel bookkeeping
+    of the dense blocks (each layer sees 32 more channels; transitions halve them)."""
+    model = om.DenseNet(arch).eval()
+    assert sum(p.numel() for p in model.parameters()) == params
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000)
+    assert round(m / 1e9, 3) == gmacs
+    c = 64
+    for bi, n in enumerate(om.DENSENET_BLOCKS[arch]):
+        blk = getattr(model.features, f"denseblock{bi + 1}")
+        for li in range(n):
+            assert getattr(blk, f"denselayer{li + 1}").conv1.in_channels == c + 32 * li
+        c += 32 * n
+        if bi != 3:
+            assert getattr(model.features, f"transition{bi + 1}").conv.out_channels == c // 2
+            c //= 2
+    assert model.classifier.in_features == c == {"densenet121": 1024, "densenet169": 1664, "densenet201": 1920}[arch]
+
+
+def test_densenet_layer_matches_functional_definition():
+    """One dense layer is conv3x3(relu(bn(conv1x1(relu(bn(x)))))) concatenated to its input."""
+    torch.manual_seed(3)
+    model = om.DenseNet("densenet121").eval()
+    layer = model.features.denseblock1.denselayer1
+    for bn in (layer.norm1, layer.norm2):
+        bn.running_mean.normal_()
+        bn.running_var.uniform_(0.5, 2.0)
+    x = torch.randn(2, 64, 9, 9)
+    with torch.no_grad():
+        t = F.batch_norm(x, layer.norm1.running_mean, layer.norm1.running_var, layer.norm1.weight, layer.norm1.bias,
+                         False, 0.0, 1e-5).relu()
+        t = F.conv2d(t, layer.conv1.weight)
+        t = F.batch_norm(t, layer.norm2.running_mean, layer.norm2.running_var, layer.norm2.weight, layer.norm2.bias,
+                         False, 0.0, 1e-5).relu()
+        want = F.conv2d(t, layer.conv2.weight, padding=1)
+        assert torch.allclose(layer(x), want, atol=1e-6)
+
+
+def test_mobilenet_v2_counts():
+    """3,504,872 parameters and 300.8 M multiply-accumulates per 224x224 image (published), 17
+    inverted-residual blocks of which 10 have an identity shortcut."""
+    model = om.MobileNetV2().eval()
+    assert sum(p.numel() for p in model.parameters()) == 3504872
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000)
+    assert round(m / 1e6, 1) == 300.8
+    blocks = [b for b in model.features if isinstance(b, om._InvertedResidual)]
+    assert len(blocks) == 17 and sum(b.residual for b in blocks) == 10
+    dw = [c for b in blocks for c in b.modules() if isinstance(c, torch.nn.Conv2d) and c.groups > 1]
+    assert len(dw) == 17 and all(c.groups == c.in_channels == c.out_channels for c in dw)
