@@ -41,15 +41,36 @@ WORKLOADS = {
     "bert-large-b4-s384": ("bert", "bert-large", 4, 384),
 }
 PRIMARY = "bert-large-b4-s384"
+# further served models (not part of the default run; `--workload <name>` measures one)
+EXTRA_WORKLOADS = {
+    "resnet101-b1": ("resnet", "resnet101", 1, None),
+    "densenet169-b1": ("densenet", "densenet169", 1, None),
+    "densenet201-b1": ("densenet", "densenet201", 1, None),
+    "mobilenetv2-b1": ("mobilenet", "mobilenet_v2", 1, None),
+    "bert-large-qa-b1-s512": ("bert-qa", "bert-large", 1, 512),   # the reference endpoint's own call
+}
 
 
 def make_function(server, fid, name, seed=0):
     import torch
-    from torpor_amd.functions import bert, resnet
+    from torpor_amd.functions import bert, densenet, mobilenet, resnet
 
-    family, arch, batch, seq = WORKLOADS[name]
+    family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     g = torch.Generator().manual_seed(0)
-    if family == "resnet":
+    if family == "densenet":
+        weights = densenet.init_weights(arch, seed=seed)
+        fn = densenet.DenseNet(server, fid, arch, batch=batch, weights=weights)
+        inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
+    elif family == "mobilenet":
+        weights = mobilenet.init_weights(seed=seed)
+        fn = mobilenet.MobileNetV2(server, fid, batch=batch, weights=weights)
+        inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
+    elif family == "bert-qa":
+        weights = bert.init_weights(arch, seed=seed, qa_head=True)
+        fn = bert.Bert(server, fid, arch, batch=batch, seq=seq, weights=weights, token_types=True)
+        inputs = [torch.randint(0, 30522, (batch, seq), generator=g).numpy(),
+                  torch.randint(0, 2, (batch, seq), generator=g).numpy()]
+    elif family == "resnet":
         weights = resnet.init_weights(arch, seed=seed)
         fn = resnet.ResNet(server, fid, arch, batch=batch, weights=weights)
         inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
@@ -169,13 +190,19 @@ def cpu_baseline(name, weights, inputs, first):
     from oracle import models as om
     from torpor_amd.functions import bert
 
-    family, arch, batch, seq = WORKLOADS[name]
+    family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     cores = int(os.environ.get("OMP_NUM_THREADS") or torch.get_num_threads())
     torch.set_num_threads(cores)
-    if family == "resnet":
-        model = om.load_numpy_state(om.ResNet(arch), weights)
+    if family in ("resnet", "densenet", "mobilenet"):
+        net = {"resnet": lambda: om.ResNet(arch), "densenet": lambda: om.DenseNet(arch),
+               "mobilenet": lambda: om.MobileNetV2()}[family]()
+        model = om.load_numpy_state(net, weights)
         x = torch.from_numpy(inputs[0])
         fwd = lambda: (model(x),)
+    elif family == "bert-qa":
+        model = om.load_numpy_state(om.Bert(qa_head=True, **bert.CONFIGS[arch]), weights)
+        x, tt = torch.from_numpy(inputs[0]), torch.from_numpy(inputs[1])
+        fwd = lambda: model(x, tt)
     else:
         model = om.load_numpy_state(om.Bert(**bert.CONFIGS[arch]), weights)
         x = torch.from_numpy(inputs[0])
@@ -202,7 +229,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", help="all | " + " | ".join(WORKLOADS))
+    ap.add_argument("--workload", default="all", help="all | " + " | ".join(list(WORKLOADS) + list(EXTRA_WORKLOADS)))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--chunk-max-bytes", type=int, default=0)

@@ -1274,7 +1274,8 @@ static void op_work(const Op& op, double* flops, double* bytes, const char** nam
         }
         case OPK_CONV: {
             const double Ho = (double)((I[1] + 2 * I[9] - I[5]) / I[7] + 1), Wo = (double)((I[2] + 2 * I[10] - I[6]) / I[8] + 1);
-            const double M = (double)I[0] * Ho * Wo, kk = (double)(I[3] * I[5] * I[6]);
+            const double groups = (op.ni > 17 && I[17] > 0) ? (double)I[17] : 1.0;
+            const double M = (double)I[0] * Ho * Wo, kk = (double)(I[3] * I[5] * I[6]) / groups;
             *flops = 2.0 * M * (double)I[4] * kk;
             *bytes = 4.0 * ((double)(I[0] * I[1] * I[2] * I[3]) + (double)I[4] * kk + M * (double)I[4] * (op.p[8] ? 2.0 : 1.0));
             *name = "conv";
