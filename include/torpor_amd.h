@@ -96,6 +96,7 @@ typedef struct tp_server tp_server;
 #define TP_OP_ATTENTION 14   /* p: q,k,v,mask|0,out  i: B,A,S,dh,ldq,ldk,ldv,ldo  f: scale */
 #define TP_OP_AVGPOOL2D 15   /* p: x,y   i: N,H,W,C,k,stride,pad,y_pitch|0   NHWC window average, padding counted */
 #define TP_OP_COPY2D 16      /* p: src,dst   i: rows,width,src_pitch,dst_pitch   (elements) */
+#define TP_OP_SCALE_CHANNELS 17 /* p: x,scale,y   i: N,HW,C   y[n,p,c] = x[n,p,c] * scale[n,c] (NHWC) */
 
 typedef struct tp_config {
     uint32_t struct_size;       /* sizeof(tp_config) */

@@ -257,6 +257,69 @@ class MobileNetV2(nn.Module):
         return self.classifier(x.mean((2, 3)))
 
 
+# (expand ratio, kernel, stride, in, out, layers) of EfficientNet-B0 (Tan & Le 2019, table 1)
+EFFICIENTNET_B0 = ((1, 3, 1, 32, 16, 1), (6, 3, 2, 16, 24, 2), (6, 5, 2, 24, 40, 2), (6, 3, 2, 40, 80, 3),
+                   (6, 5, 1, 80, 112, 3), (6, 5, 2, 112, 192, 4), (6, 3, 1, 192, 320, 1))
+
+
+class _SqueezeExcite(nn.Module):
+    def __init__(self, channels, squeeze):
+        super().__init__()
+        self.fc1 = nn.Conv2d(channels, squeeze, 1)
+        self.fc2 = nn.Conv2d(squeeze, channels, 1)
+
+    def forward(self, x):
+        s = x.mean((2, 3), keepdim=True)
+        return x * torch.sigmoid(self.fc2(F.silu(self.fc1(s))))
+
+
+class _MBConv(nn.Module):
+    """block.0 expand 1x1 (absent for ratio 1), then depthwise k x k, squeeze-excite (squeeze width
+    = block input / 4), linear 1x1 projection; identity shortcut when stride 1 and in == out."""
+
+    def __init__(self, cin, cout, k, stride, expand):
+        super().__init__()
+        hidden = cin * expand
+        layers = []
+        if expand != 1:
+            layers.append(_ConvBN(cin, hidden, 1))
+        layers.append(_ConvBN(hidden, hidden, k, stride, groups=hidden))
+        layers.append(_SqueezeExcite(hidden, max(1, cin // 4)))
+        layers.append(_ConvBN(hidden, cout, 1))
+        self.block = nn.Sequential(*layers)
+        self.residual = stride == 1 and cin == cout
+
+    def forward(self, x):
+        y = x
+        for m in self.block:
+            if isinstance(m, _SqueezeExcite):
+                y = m(y)
+            elif m is self.block[-1]:
+                y = m(y)
+            else:
+                y = F.silu(m(y))
+        return x + y if self.residual else y
+
+
+class EfficientNetB0(nn.Module):
+    def __init__(self, num_classes=1000):
+        super().__init__()
+        feats = [_ConvBN(3, 32, 3, 2)]
+        for t, k, s, cin, cout, n in EFFICIENTNET_B0:
+            stage = [_MBConv(cin if i == 0 else cout, cout, k, s if i == 0 else 1, t) for i in range(n)]
+            feats.append(nn.Sequential(*stage))
+        feats.append(_ConvBN(320, 1280, 1))
+        self.features = nn.Sequential(*feats)
+        self.classifier = nn.Linear(1280, num_classes)
+
+    def forward(self, x):
+        x = F.silu(self.features[0](x))
+        for stage in list(self.features)[1:-1]:
+            x = stage(x)
+        x = F.silu(self.features[-1](x))
+        return self.classifier(x.mean((2, 3)))
+
+
 def load_numpy_state(module, weights):
     """Strictly load a {name: np.ndarray} dict (BN `num_batches_tracked` buffers excepted)."""
     sd = {k: torch.from_numpy(v.copy()) for k, v in weights.items()}

@@ -7,7 +7,7 @@ import torch
 
 from oracle import models as om
 from tests.harness import assert_close
-from torpor_amd.functions import bert, densenet, mobilenet, resnet
+from torpor_amd.functions import bert, densenet, efficientnet, mobilenet, resnet
 
 pytestmark = pytest.mark.gpu
 LOGIT_RTOL = 1e-3   # north-star bar: rel 1e-3 (fp32) on logits
@@ -183,6 +183,23 @@ def test_mobilenet_v2(gpu_server, image, batch):
         want = model(torch.from_numpy(x)).numpy()
     e = assert_close(logits, want, LOGIT_RTOL, "mobilenet_v2 logits")
     print(f"mobilenet_v2 b{batch} {image}px: rel err {e:.2e}")
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+@pytest.mark.parametrize("image,batch", [(96, 2), (224, 1)])
+def test_efficientnet_b0(gpu_server, image, batch):
+    """EfficientNet-B0 (tests/endpoint.py:34-35): depthwise 3x3 / 5x5, SiLU, squeeze-and-excitation."""
+    weights = _perturb_bn(efficientnet.init_weights(seed=12), seed=13)
+    x = torch.randn(batch, 3, image, image, generator=torch.Generator().manual_seed(14)).numpy()
+    fn = efficientnet.EfficientNetB0(gpu_server, 15, batch=batch, weights=weights, image=image)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.EfficientNetB0(), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, "efficientnet_b0 logits")
+    print(f"efficientnet_b0 b{batch} {image}px: rel err {e:.2e}")
     _check_swap_identity(gpu_server, fn, weights)
     _cycle(gpu_server, fn, [x], [logits])
     fn.unload()

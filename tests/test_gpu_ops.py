@@ -8,7 +8,7 @@ from oracle import ops as ref
 from tests.harness import OpSession, assert_close
 from torpor_amd.server import (NCHW, NHWC, OP_ADD, OP_ATTENTION, OP_AVGPOOL, OP_BIAS_ACT, OP_EMBEDDING, OP_FILL, OP_GELU,
                                OP_LAYERNORM, OP_MAXPOOL, OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_RELU, OP_SOFTMAX,
-                               OP_SUM, OP_AVGPOOL2D, OP_COPY2D, ACT_RELU, ACT_RELU6, ACT_SILU, ACT_SIGMOID, TorporError)
+                               OP_SUM, OP_AVGPOOL2D, OP_COPY2D, OP_SCALE_CHANNELS, ACT_RELU, ACT_RELU6, ACT_SILU, ACT_SIGMOID, TorporError)
 
 pytestmark = pytest.mark.gpu
 
@@ -116,6 +116,12 @@ def test_new_activations_window_average_and_strided_views(gpu_server):
         got = t.read(wv, wide.shape)
         assert_close(got[..., 4:16], want, 2e-6, "avgpool2d into a slice")
         assert (got[..., :4] == 7).all() and (got[..., 16:] == 7).all()
+        # squeeze-and-excitation gating: every pixel of image n scaled per channel
+        gate = rng.uniform(0, 1, (2, 12)).astype(np.float32)
+        gv = t.act(gate)
+        sv = t.empty(img.nbytes)
+        t.s.launch(t.fid, OP_SCALE_CHANNELS, [iv, gv, sv], [2, 9 * 8, 12])
+        np.testing.assert_array_equal(t.read(sv, img.shape), img * gate[:, None, None, :])
         # strided copy: columns 3..10 of x into columns 1..8 of a 12-wide matrix
         dst = np.zeros((17, 12), np.float32)
         dv = t.act(dst)

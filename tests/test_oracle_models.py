@@ -212,3 +212,31 @@ def test_mobilenet_v2_counts():
     assert len(blocks) == 17 and sum(b.residual for b in blocks) == 10
     dw = [c for b in blocks for c in b.modules() if isinstance(c, torch.nn.Conv2d) and c.groups > 1]
     assert len(dw) == 17 and all(c.groups == c.in_channels == c.out_channels for c in dw)
+
+
+def test_efficientnet_b0_counts():
+    """5,288,548 parameters and 0.39 G multiply-accumulates per 224x224 image (published); 16 MBConv
+    blocks, squeeze width = block input / 4, 9 identity shortcuts; the product-side weight generator
+    loads strictly."""
+    model = om.EfficientNetB0().eval()
+    assert sum(p.numel() for p in model.parameters()) == 5288548
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000)
+    assert round(m / 1e9, 2) == 0.39
+    blocks = [b for b in model.modules() if isinstance(b, om._MBConv)]
+    assert len(blocks) == 16 and sum(b.residual for b in blocks) == 9
+    se = [s_ for s_ in model.modules() if isinstance(s_, om._SqueezeExcite)]
+    assert [s_.fc1.out_channels for s_ in se][:4] == [8, 4, 6, 6]
+    from torpor_amd.functions import efficientnet as peff
+    om.load_numpy_state(om.EfficientNetB0(), peff.init_weights())
+
+
+def test_squeeze_excite_matches_functional_definition():
+    torch.manual_seed(5)
+    se = om._SqueezeExcite(12, 3).eval()
+    x = torch.randn(2, 12, 5, 4)
+    with torch.no_grad():
+        s_ = x.mean((2, 3))
+        g = torch.sigmoid(F.linear(F.silu(F.linear(s_, se.fc1.weight.flatten(1), se.fc1.bias)), se.fc2.weight.flatten(1),
+                                   se.fc2.bias))
+        assert torch.allclose(se(x), x * g[:, :, None, None], atol=1e-6)

@@ -1232,6 +1232,14 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             if (!launch) return 0;
             return tpk::launch_copy2d(F(0), Fm(1), rows, (int)width, sp, dp, compute_);
         }
+        case TP_OP_SCALE_CHANNELS: {
+            if (!need(3, 3, 0)) return TP_EINVAL;
+            const int64_t N = I[0], HW = I[1], C = I[2];
+            if (N < 1 || HW < 1 || C < 1 || N > 0x7fffffff || C > 0x7fffffff) return TP_EINVAL;
+            if ((r = R(0, false, N * HW * C)) || (r = R(1, false, N * C)) || (r = R(2, false, N * HW * C))) return r;
+            if (!launch) return 0;
+            return tpk::launch_scale_channels(F(0), F(1), Fm(2), (int)N, HW, (int)C, compute_);
+        }
         case TP_OP_ATTENTION: {
             if (!need(5, 8, 1)) return TP_EINVAL;
             const int64_t B = I[0], A = I[1], S = I[2], dh = I[3];
@@ -1307,6 +1315,7 @@ static void op_work(const Op& op, double* flops, double* bytes, const char** nam
                 case TP_OP_FILL: *bytes = 4.0 * (double)I[0]; *name = "fill"; break;
                 case TP_OP_AVGPOOL2D: *bytes = 4.0 * (double)(I[0] * I[1] * I[2] * I[3]) * 1.25; *name = "avgpool2d"; break;
                 case TP_OP_COPY2D: *bytes = 8.0 * (double)(I[0] * I[1]); *name = "copy2d"; break;
+                case TP_OP_SCALE_CHANNELS: *bytes = 8.0 * (double)(I[0] * I[1] * I[2]); *name = "scale_channels"; break;
                 case TP_OP_ATTENTION:
                     *flops = 4.0 * (double)(I[0] * I[1]) * (double)(I[2] * I[2]) * (double)I[3];
                     *bytes = 16.0 * (double)(I[0] * I[2]) * (double)(I[1] * I[3]);

@@ -78,6 +78,8 @@ int launch_bn_inference(const float* x, float* y, const float* g, const float* b
 // count_include_pad=True); y_pitch = floats between output pixels (0 = C).
 int launch_avgpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, long y_pitch,
                      hipStream_t s);
+// y[n][p][c] = x[n][p][c] * s[n][c], NHWC with HW pixels per image (squeeze-and-excitation gating)
+int launch_scale_channels(const float* x, const float* sc, float* y, int N, long HW, int C, hipStream_t s);
 // dst[r*dst_pitch + c] = src[r*src_pitch + c], r < rows, c < width
 int launch_copy2d(const float* src, float* dst, long rows, int width, long src_pitch, long dst_pitch, hipStream_t s);
 int launch_relu(const float* x, float* y, long n, hipStream_t s);

@@ -151,6 +151,23 @@ int launch_avgpool2d(const float* x, float* y, int N, int H, int W, int C, int k
     return (int)hipGetLastError();
 }
 
+// y[n][p][c] = x[n][p][c] * s[n][c]  (squeeze-and-excitation gating, NHWC)
+__global__ __launch_bounds__(256) void scale_channels_kernel(const float* __restrict__ x, const float* __restrict__ sc,
+                                                             float* __restrict__ y, long total, long hwc, int C) {
+    const long st = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += st) {
+        const long n = i / hwc;
+        const int c = (int)(i % C);
+        y[i] = x[i] * sc[n * C + c];
+    }
+}
+int launch_scale_channels(const float* x, const float* sc, float* y, int N, long HW, int C, hipStream_t s) {
+    if (!x || !sc || !y || N < 1 || HW < 1 || C < 1) return K_EINVAL;
+    const long total = (long)N * HW * C;
+    hipLaunchKernelGGL(scale_channels_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, x, sc, y, total, HW * C, C);
+    return (int)hipGetLastError();
+}
+
 __global__ __launch_bounds__(256) void copy2d_kernel(const float* __restrict__ src, float* __restrict__ dst, long total,
                                                      int width, long src_pitch, long dst_pitch) {
     const long st = (long)gridDim.x * blockDim.x;

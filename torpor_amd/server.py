@@ -17,7 +17,8 @@ ACK_OK, ACK_INAVAIL = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH, ACT_RELU6, ACT_SILU, ACT_SIGMOID = 0, 1, 2, 3, 4, 5, 6
 NCHW, NHWC = 0, 1
 (OP_RELU, OP_ADD, OP_BIAS_ACT, OP_GELU, OP_MAXPOOL, OP_AVGPOOL, OP_LAYERNORM, OP_SOFTMAX, OP_EMBEDDING,
- OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION, OP_AVGPOOL2D, OP_COPY2D) = range(1, 17)
+ OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION, OP_AVGPOOL2D, OP_COPY2D,
+ OP_SCALE_CHANNELS) = range(1, 18)
 FLAG_HOST_ONLY = 1
 
 
