@@ -48,13 +48,14 @@ EXTRA_WORKLOADS = {
     "densenet201-b1": ("densenet", "densenet201", 1, None),
     "mobilenetv2-b1": ("mobilenet", "mobilenet_v2", 1, None),
     "efficientnet-b0-b1": ("efficientnet", "efficientnet_b0", 1, None),
+    "inception-v3-b1": ("inception", "inception_v3", 1, None),
     "bert-large-qa-b1-s512": ("bert-qa", "bert-large", 1, 512),   # the reference endpoint's own call
 }
 
 
 def make_function(server, fid, name, seed=0):
     import torch
-    from torpor_amd.functions import bert, densenet, efficientnet, mobilenet, resnet
+    from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet
 
     family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     g = torch.Generator().manual_seed(0)
@@ -62,6 +63,10 @@ def make_function(server, fid, name, seed=0):
         weights = densenet.init_weights(arch, seed=seed)
         fn = densenet.DenseNet(server, fid, arch, batch=batch, weights=weights)
         inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
+    elif family == "inception":
+        weights = inception.init_weights(seed=seed)
+        fn = inception.InceptionV3(server, fid, batch=batch, weights=weights)
+        inputs = [torch.randn(batch, 3, 299, 299, generator=g).numpy()]
     elif family == "efficientnet":
         weights = efficientnet.init_weights(seed=seed)
         fn = efficientnet.EfficientNetB0(server, fid, batch=batch, weights=weights)
@@ -198,9 +203,10 @@ def cpu_baseline(name, weights, inputs, first):
     family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     cores = int(os.environ.get("OMP_NUM_THREADS") or torch.get_num_threads())
     torch.set_num_threads(cores)
-    if family in ("resnet", "densenet", "mobilenet", "efficientnet"):
+    if family in ("resnet", "densenet", "mobilenet", "efficientnet", "inception"):
         net = {"resnet": lambda: om.ResNet(arch), "densenet": lambda: om.DenseNet(arch),
-               "mobilenet": lambda: om.MobileNetV2(), "efficientnet": lambda: om.EfficientNetB0()}[family]()
+               "mobilenet": lambda: om.MobileNetV2(), "efficientnet": lambda: om.EfficientNetB0(),
+               "inception": lambda: om.InceptionV3()}[family]()
         model = om.load_numpy_state(net, weights)
         x = torch.from_numpy(inputs[0])
         fwd = lambda: (model(x),)

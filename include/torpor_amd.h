@@ -79,7 +79,7 @@ typedef struct tp_server tp_server;
 #define TP_OP_ADD 2          /* p: a,b,y        i: n, relu */
 #define TP_OP_BIAS_ACT 3     /* p: x,bias,y     i: rows, C, act */
 #define TP_OP_GELU 4         /* p: x,y          i: n */
-#define TP_OP_MAXPOOL 5      /* p: x,y          i: N,H,W,C,k,stride,pad,layout */
+#define TP_OP_MAXPOOL 5      /* p: x,y          i: N,H,W,C,k,stride,pad,layout[,y_pitch (NHWC, 0 = C)] */
 #define TP_OP_AVGPOOL 6      /* p: x,y          i: N,HW,C,layout   (global average) */
 #define TP_OP_LAYERNORM 7    /* p: x,res|0,gamma,beta,y  i: rows,width  f: eps */
 #define TP_OP_SOFTMAX 8      /* p: x,mask|0,y   i: rows,width,rows_per_mask  f: scale */

@@ -320,6 +320,134 @@ class EfficientNetB0(nn.Module):
         return self.classifier(x.mean((2, 3)))
 
 
+class _BasicConv(nn.Module):
+    """conv (no bias) + batch-norm (eps 1e-3) + relu, torchvision's BasicConv2d."""
+
+    def __init__(self, cin, cout, k, stride=1, padding=0):
+        super().__init__()
+        self.conv = nn.Conv2d(cin, cout, k, stride, padding, bias=False)
+        self.bn = nn.BatchNorm2d(cout, eps=0.001)
+
+    def forward(self, x):
+        return F.relu(self.bn(self.conv(x)))
+
+
+class _IncA(nn.Module):
+    def __init__(self, cin, pool):
+        super().__init__()
+        self.branch1x1 = _BasicConv(cin, 64, 1)
+        self.branch5x5_1 = _BasicConv(cin, 48, 1)
+        self.branch5x5_2 = _BasicConv(48, 64, 5, padding=2)
+        self.branch3x3dbl_1 = _BasicConv(cin, 64, 1)
+        self.branch3x3dbl_2 = _BasicConv(64, 96, 3, padding=1)
+        self.branch3x3dbl_3 = _BasicConv(96, 96, 3, padding=1)
+        self.branch_pool = _BasicConv(cin, pool, 1)
+
+    def forward(self, x):
+        return torch.cat([self.branch1x1(x), self.branch5x5_2(self.branch5x5_1(x)),
+                          self.branch3x3dbl_3(self.branch3x3dbl_2(self.branch3x3dbl_1(x))),
+                          self.branch_pool(F.avg_pool2d(x, 3, 1, 1))], 1)
+
+
+class _IncB(nn.Module):
+    def __init__(self, cin):
+        super().__init__()
+        self.branch3x3 = _BasicConv(cin, 384, 3, stride=2)
+        self.branch3x3dbl_1 = _BasicConv(cin, 64, 1)
+        self.branch3x3dbl_2 = _BasicConv(64, 96, 3, padding=1)
+        self.branch3x3dbl_3 = _BasicConv(96, 96, 3, stride=2)
+
+    def forward(self, x):
+        return torch.cat([self.branch3x3(x), self.branch3x3dbl_3(self.branch3x3dbl_2(self.branch3x3dbl_1(x))),
+                          F.max_pool2d(x, 3, 2)], 1)
+
+
+class _IncC(nn.Module):
+    def __init__(self, cin, c7):
+        super().__init__()
+        self.branch1x1 = _BasicConv(cin, 192, 1)
+        self.branch7x7_1 = _BasicConv(cin, c7, 1)
+        self.branch7x7_2 = _BasicConv(c7, c7, (1, 7), padding=(0, 3))
+        self.branch7x7_3 = _BasicConv(c7, 192, (7, 1), padding=(3, 0))
+        self.branch7x7dbl_1 = _BasicConv(cin, c7, 1)
+        self.branch7x7dbl_2 = _BasicConv(c7, c7, (7, 1), padding=(3, 0))
+        self.branch7x7dbl_3 = _BasicConv(c7, c7, (1, 7), padding=(0, 3))
+        self.branch7x7dbl_4 = _BasicConv(c7, c7, (7, 1), padding=(3, 0))
+        self.branch7x7dbl_5 = _BasicConv(c7, 192, (1, 7), padding=(0, 3))
+        self.branch_pool = _BasicConv(cin, 192, 1)
+
+    def forward(self, x):
+        b7 = self.branch7x7_3(self.branch7x7_2(self.branch7x7_1(x)))
+        d = self.branch7x7dbl_1(x)
+        for m in (self.branch7x7dbl_2, self.branch7x7dbl_3, self.branch7x7dbl_4, self.branch7x7dbl_5):
+            d = m(d)
+        return torch.cat([self.branch1x1(x), b7, d, self.branch_pool(F.avg_pool2d(x, 3, 1, 1))], 1)
+
+
+class _IncD(nn.Module):
+    def __init__(self, cin):
+        super().__init__()
+        self.branch3x3_1 = _BasicConv(cin, 192, 1)
+        self.branch3x3_2 = _BasicConv(192, 320, 3, stride=2)
+        self.branch7x7x3_1 = _BasicConv(cin, 192, 1)
+        self.branch7x7x3_2 = _BasicConv(192, 192, (1, 7), padding=(0, 3))
+        self.branch7x7x3_3 = _BasicConv(192, 192, (7, 1), padding=(3, 0))
+        self.branch7x7x3_4 = _BasicConv(192, 192, 3, stride=2)
+
+    def forward(self, x):
+        b = self.branch7x7x3_4(self.branch7x7x3_3(self.branch7x7x3_2(self.branch7x7x3_1(x))))
+        return torch.cat([self.branch3x3_2(self.branch3x3_1(x)), b, F.max_pool2d(x, 3, 2)], 1)
+
+
+class _IncE(nn.Module):
+    def __init__(self, cin):
+        super().__init__()
+        self.branch1x1 = _BasicConv(cin, 320, 1)
+        self.branch3x3_1 = _BasicConv(cin, 384, 1)
+        self.branch3x3_2a = _BasicConv(384, 384, (1, 3), padding=(0, 1))
+        self.branch3x3_2b = _BasicConv(384, 384, (3, 1), padding=(1, 0))
+        self.branch3x3dbl_1 = _BasicConv(cin, 448, 1)
+        self.branch3x3dbl_2 = _BasicConv(448, 384, 3, padding=1)
+        self.branch3x3dbl_3a = _BasicConv(384, 384, (1, 3), padding=(0, 1))
+        self.branch3x3dbl_3b = _BasicConv(384, 384, (3, 1), padding=(1, 0))
+        self.branch_pool = _BasicConv(cin, 192, 1)
+
+    def forward(self, x):
+        t = self.branch3x3_1(x)
+        d = self.branch3x3dbl_2(self.branch3x3dbl_1(x))
+        return torch.cat([self.branch1x1(x), self.branch3x3_2a(t), self.branch3x3_2b(t), self.branch3x3dbl_3a(d),
+                          self.branch3x3dbl_3b(d), self.branch_pool(F.avg_pool2d(x, 3, 1, 1))], 1)
+
+
+class InceptionV3(nn.Module):
+    """Inception-v3 (Szegedy et al. 2016) as served in eval mode: torchvision's layer names, no
+    auxiliary classifier, no input re-normalisation; 299x299 inputs."""
+
+    def __init__(self, num_classes=1000):
+        super().__init__()
+        self.Conv2d_1a_3x3 = _BasicConv(3, 32, 3, stride=2)
+        self.Conv2d_2a_3x3 = _BasicConv(32, 32, 3)
+        self.Conv2d_2b_3x3 = _BasicConv(32, 64, 3, padding=1)
+        self.Conv2d_3b_1x1 = _BasicConv(64, 80, 1)
+        self.Conv2d_4a_3x3 = _BasicConv(80, 192, 3)
+        self.Mixed_5b, self.Mixed_5c, self.Mixed_5d = _IncA(192, 32), _IncA(256, 64), _IncA(288, 64)
+        self.Mixed_6a = _IncB(288)
+        self.Mixed_6b, self.Mixed_6c, self.Mixed_6d, self.Mixed_6e = _IncC(768, 128), _IncC(768, 160), _IncC(768, 160), _IncC(768, 192)
+        self.Mixed_7a = _IncD(768)
+        self.Mixed_7b, self.Mixed_7c = _IncE(1280), _IncE(2048)
+        self.fc = nn.Linear(2048, num_classes)
+
+    def forward(self, x):
+        x = self.Conv2d_2b_3x3(self.Conv2d_2a_3x3(self.Conv2d_1a_3x3(x)))
+        x = F.max_pool2d(x, 3, 2)
+        x = self.Conv2d_4a_3x3(self.Conv2d_3b_1x1(x))
+        x = F.max_pool2d(x, 3, 2)
+        for m in (self.Mixed_5b, self.Mixed_5c, self.Mixed_5d, self.Mixed_6a, self.Mixed_6b, self.Mixed_6c, self.Mixed_6d,
+                  self.Mixed_6e, self.Mixed_7a, self.Mixed_7b, self.Mixed_7c):
+            x = m(x)
+        return self.fc(x.mean((2, 3)))
+
+
 def load_numpy_state(module, weights):
     """Strictly load a {name: np.ndarray} dict (BN `num_batches_tracked` buffers excepted)."""
     sd = {k: torch.from_numpy(v.copy()) for k, v in weights.items()}

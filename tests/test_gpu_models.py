@@ -7,7 +7,7 @@ import torch
 
 from oracle import models as om
 from tests.harness import assert_close
-from torpor_amd.functions import bert, densenet, efficientnet, mobilenet, resnet
+from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet
 
 pytestmark = pytest.mark.gpu
 LOGIT_RTOL = 1e-3   # north-star bar: rel 1e-3 (fp32) on logits
@@ -200,6 +200,24 @@ def test_efficientnet_b0(gpu_server, image, batch):
         want = model(torch.from_numpy(x)).numpy()
     e = assert_close(logits, want, LOGIT_RTOL, "efficientnet_b0 logits")
     print(f"efficientnet_b0 b{batch} {image}px: rel err {e:.2e}")
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+@pytest.mark.parametrize("image,batch", [(139, 2), (299, 1)])
+def test_inception_v3(gpu_server, image, batch):
+    """Inception-v3 (tests/endpoint.py:32-33): asymmetric convolutions, window pooling, branches
+    written straight into channel slices of the block output."""
+    weights = _perturb_bn(inception.init_weights(seed=15), seed=16)
+    x = torch.randn(batch, 3, image, image, generator=torch.Generator().manual_seed(17)).numpy()
+    fn = inception.InceptionV3(gpu_server, 16, batch=batch, weights=weights, image=image)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.InceptionV3(), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, "inception_v3 logits")
+    print(f"inception_v3 b{batch} {image}px: rel err {e:.2e}")
     _check_swap_identity(gpu_server, fn, weights)
     _cycle(gpu_server, fn, [x], [logits])
     fn.unload()

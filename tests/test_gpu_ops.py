@@ -88,6 +88,24 @@ def test_bias_act_and_layouts(gpu_server):
         np.testing.assert_array_equal(t.read(iv, img.shape), img)
 
 
+@pytest.mark.parametrize("N,H,W,C", [(2, 40, 33, 70), (1, 112, 112, 96), (3, 16, 16, 8), (8, 7, 7, 2048), (2, 4, 4, 5),
+                                     (2, 3, 5, 130)])
+def test_global_avgpool_large_maps(gpu_server, N, H, W, C):
+    """Maps of 16 pixels and more take the two-stage (sliced) reduction, smaller ones one thread
+    per channel."""
+    rng = np.random.default_rng(H + C)
+    x = _rand(rng, N, H, W, C) + 0.5
+    with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
+        xv = t.act(x)
+        av = t.empty(N * C * 4)
+        t.s.launch(t.fid, OP_AVGPOOL, [xv, av], [N, H * W, C, NHWC])
+        got = t.read(av, (N, C))
+        t.s.launch(t.fid, OP_AVGPOOL, [xv, av], [N, H * W, C, NHWC])
+        again = t.read(av, (N, C))
+    assert_close(got, ref.avgpool(x, nhwc=True), 2e-6, "global avgpool")
+    np.testing.assert_array_equal(got, again)   # fixed summation order
+
+
 def test_new_activations_window_average_and_strided_views(gpu_server):
     """relu6 / silu / sigmoid, k x k average pooling (also into a channel slice of a wider tensor),
     2-D strided copy, and batch-norm over the first channels of a wider tensor."""

@@ -240,3 +240,23 @@ def test_squeeze_excite_matches_functional_definition():
         g = torch.sigmoid(F.linear(F.silu(F.linear(s_, se.fc1.weight.flatten(1), se.fc1.bias)), se.fc2.weight.flatten(1),
                                    se.fc2.bias))
         assert torch.allclose(se(x), x * g[:, :, None, None], atol=1e-6)
+
+
+def test_inception_v3_counts():
+    """23,834,568 parameters without the auxiliary classifier (27,161,264 published with it, whose own
+    share is 3,326,696) and 5.71 G multiply-accumulates per 299x299 image; 94 conv + batch-norm pairs;
+    output widths of the Mixed blocks 256, 288, 288, 768 x5, 1280, 2048, 2048."""
+    model = om.InceptionV3().eval()
+    assert sum(p.numel() for p in model.parameters()) == 23834568 == 27161264 - 3326696
+    m, y = _macs(model, torch.zeros(1, 3, 299, 299))
+    assert y.shape == (1, 1000) and round(m / 1e9, 2) == 5.71
+    assert sum(1 for c in model.modules() if isinstance(c, torch.nn.Conv2d)) == 94
+    widths, x = [], torch.zeros(1, 192, 35, 35)
+    with torch.no_grad():
+        for name in ("Mixed_5b", "Mixed_5c", "Mixed_5d", "Mixed_6a", "Mixed_6b", "Mixed_6c", "Mixed_6d", "Mixed_6e",
+                     "Mixed_7a", "Mixed_7b", "Mixed_7c"):
+            x = getattr(model, name)(x)
+            widths.append(x.shape[1])
+    assert widths == [256, 288, 288, 768, 768, 768, 768, 768, 1280, 2048, 2048] and x.shape[2:] == (8, 8)
+    from torpor_amd.functions import inception as pinc
+    om.load_numpy_state(om.InceptionV3(), pinc.init_weights())

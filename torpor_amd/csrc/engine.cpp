@@ -1161,16 +1161,18 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             if (N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || st < 1 || H + 2 * pad < k || W + 2 * pad < k)
                 return TP_EINVAL;
             const int64_t Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
-            if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, N * Ho * Wo * C))) return r;
+            const int64_t yp = (op.ni > 8 && I[8]) ? I[8] : C;   // NHWC: elements between output pixels
+            if (yp < C || (yp != C && !I[7])) return TP_EINVAL;
+            if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, (N * Ho * Wo - 1) * yp + C))) return r;
             if (!launch) return 0;
             return tpk::launch_maxpool2d(F(0), Fm(1), (int)N, (int)H, (int)W, (int)C, (int)k, (int)st, (int)pad,
-                                         (int)I[7], compute_);
+                                         (int)I[7], yp, compute_);
         }
         case TP_OP_AVGPOOL:
             if (!need(2, 4, 0)) return TP_EINVAL;
             if ((r = R(0, false, I[0] * I[1] * I[2])) || (r = R(1, false, I[0] * I[2]))) return r;
             if (!launch) return 0;
-            return tpk::launch_global_avgpool(F(0), Fm(1), (int)I[0], (int)I[1], (int)I[2], (int)I[3], compute_);
+            return tpk::launch_global_avgpool(F(0), Fm(1), (int)I[0], (int)I[1], (int)I[2], (int)I[3], ws, compute_);
         case TP_OP_LAYERNORM:
             if (!need(5, 2, 1)) return TP_EINVAL;
             if ((r = R(0, false, I[0] * I[1])) || (r = R(1, true, I[0] * I[1])) || (r = R(2, false, I[1])) ||

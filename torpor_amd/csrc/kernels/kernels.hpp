@@ -88,9 +88,11 @@ int launch_bias_act(const float* x, const float* bias, float* y, long rows, int 
 int launch_gelu(const float* x, float* y, long n, hipStream_t s);
 int launch_nchw_to_nhwc(const float* x, float* y, int N, int C, int H, int W, hipStream_t s);
 int launch_nhwc_to_nchw(const float* x, float* y, int N, int C, int H, int W, hipStream_t s);
+// y_pitch: NHWC only, floats between output pixels (0 = C)
 int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, int nhwc,
-                     hipStream_t s);
-int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, hipStream_t s);
+                     long y_pitch, hipStream_t s);
+int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, const Workspace& ws,
+                          hipStream_t s);
 int launch_layernorm(const float* x, const float* residual, const float* gamma, const float* beta, float* y,
                      long rows, int width, float eps, hipStream_t s);
 // y[row] = softmax(scale * x[row] + mask[(row / rows_per_mask) * width ...]) over `width`

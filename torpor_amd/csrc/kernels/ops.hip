@@ -322,7 +322,7 @@ int launch_nhwc_to_nchw(const float* x, float* y, int N, int C, int H, int W, hi
 // ---------------------------------------------------------------- pooling
 __global__ __launch_bounds__(256) void maxpool_kernel(const float* __restrict__ x, float* __restrict__ y, int N, int H,
                                                       int W, int C, int Ho, int Wo, int k, int stride, int pad,
-                                                      int nhwc) {
+                                                      int nhwc, long y_pitch) {
     const long total = (long)N * Ho * Wo * C;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         int c, wo, ho;
@@ -353,18 +353,20 @@ __global__ __launch_bounds__(256) void maxpool_kernel(const float* __restrict__ 
                 m = fmaxf(m, x[xi]);
             }
         }
-        y[i] = m;
+        y[nhwc ? (i / C) * y_pitch + c : i] = m;
     }
 }
 int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, int nhwc,
-                     hipStream_t s) {
+                     long y_pitch, hipStream_t s) {
     if (!x || !y || N <= 0 || H <= 0 || W <= 0 || C <= 0 || k <= 0 || stride <= 0 || pad < 0 || pad * 2 > k)
         return K_EINVAL;
+    if (y_pitch == 0) y_pitch = C;
+    if (y_pitch < C || (y_pitch != C && !nhwc)) return K_EINVAL;
     const int Ho = (H + 2 * pad - k) / stride + 1, Wo = (W + 2 * pad - k) / stride + 1;
     if (Ho <= 0 || Wo <= 0) return K_EINVAL;
     const long total = (long)N * Ho * Wo * C;
     hipLaunchKernelGGL(maxpool_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, x, y, N, H, W, C, Ho, Wo, k,
-                       stride, pad, nhwc);
+                       stride, pad, nhwc, y_pitch);
     return (int)hipGetLastError();
 }
 
@@ -392,8 +394,49 @@ __global__ __launch_bounds__(256) void avgpool_nchw_kernel(const float* __restri
     s = wave_sum(s);
     if (lane == 0) y[row] = s / (float)HW;
 }
-int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, hipStream_t s) {
+// NHWC maps of 16 pixels and more: the pixels of an image are cut into S slices; a workgroup sums one slice
+// for 64 channels (4 pixel phases x 64 lanes, coalesced along channels), the second kernel adds
+// the S partial sums in a fixed order.
+__global__ __launch_bounds__(256) void avgpool_partial_kernel(const float* __restrict__ x, float* __restrict__ part,
+                                                              int HW, int C, int S) {
+    __shared__ float red[4][64];
+    const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cx, sl = blockIdx.y, n = blockIdx.z;
+    const int per = (HW + S - 1) / S;
+    const int p0 = sl * per, p1 = (p0 + per < HW) ? p0 + per : HW;
+    float acc = 0.f;
+    if (c < C) {
+        const float* px = x + (long)n * HW * C + c;
+        for (int q = p0 + ry; q < p1; q += 4) acc += px[(long)q * C];
+    }
+    red[ry][cx] = acc;
+    __syncthreads();
+    if (ry == 0 && c < C) part[((long)n * S + sl) * C + c] = (red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]);
+}
+__global__ __launch_bounds__(256) void avgpool_final_kernel(const float* __restrict__ part, float* __restrict__ y,
+                                                            long total, int C, int S, float inv) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long n = i / C;
+        const int c = (int)(i - n * C);
+        float acc = 0.f;
+        for (int sl = 0; sl < S; ++sl) acc += part[(n * S + sl) * C + c];
+        y[i] = acc * inv;
+    }
+}
+int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, const Workspace& ws,
+                          hipStream_t s) {
     if (!x || !y || N <= 0 || HW <= 0 || C <= 0) return K_EINVAL;
+    if (nhwc && HW >= 16 && ws.ptr) {
+        int S = HW >= 512 ? (HW + 63) / 64 : (HW + 7) / 8;
+        if (S > 64) S = 64;
+        if ((size_t)N * S * C * sizeof(float) <= ws.bytes && N <= 65535) {
+            hipLaunchKernelGGL(avgpool_partial_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)S, (unsigned)N),
+                               dim3(256), 0, s, x, ws.ptr, HW, C, S);
+            hipLaunchKernelGGL(avgpool_final_kernel, dim3(grid_for((long)N * C, 256)), dim3(256), 0, s, ws.ptr, y,
+                               (long)N * C, C, S, 1.0f / (float)HW);
+            return (int)hipGetLastError();
+        }
+    }
     if (nhwc) {
         hipLaunchKernelGGL(avgpool_nhwc_kernel, dim3(grid_for((long)N * C, 256)), dim3(256), 0, s, x, y, N, HW, C);
     } else {
