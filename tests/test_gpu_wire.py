@@ -73,3 +73,26 @@ def test_bert_small_over_the_wire(gpu_wire_server):
         h2, p2 = fn.invoke([ids])
         assert np.array_equal(h2, hidden) and np.array_equal(p2, pooled)
         fn.unload()
+
+
+def test_densenet_and_mobilenet_over_the_wire(gpu_wire_server):
+    """The wire fields added for channel-slice views (conv x_pitch / y_pitch, batch-norm x_pitch,
+    groups) and the op ids of window pooling / strided copy: results over the wire must equal the
+    in-process C-ABI path bit for bit."""
+    from torpor_amd.functions import densenet, mobilenet
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, 3, 64, 64, generator=g).numpy()
+    for fid, make, weights in (
+            (9, lambda s, f, w: densenet.DenseNet(s, f, "densenet121", batch=1, weights=w, image=64),
+             densenet.init_weights("densenet121", seed=4)),
+            (10, lambda s, f, w: mobilenet.MobileNetV2(s, f, batch=1, weights=w, image=64), mobilenet.init_weights(seed=4))):
+        with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as local:
+            (want_local,) = make(local, 0, weights).register([x])
+        with wire.RemoteServer(gpu_wire_server, client_id=fid) as rs:
+            fn = make(rs, fid, weights)
+            (first,) = fn.register([x])
+            assert np.array_equal(first, want_local), "wire path differs from the in-process path"
+            assert fn.unload()[0] == ACK_OK
+            (cold,) = fn.invoke([x])
+            assert np.array_equal(cold, first)
+            assert fn.unload()[0] == ACK_OK
