@@ -27,6 +27,7 @@ CASES = [
     (1, 13, 11, 5, 7, 3, 1, 1, NCHW, NCHW, "conv_generic"),       # odd sizes, NCHW both
     (1, 9, 9, 12, 20, 5, 2, 2, NHWC, NCHW, "conv_generic"),       # 5x5, mixed layouts
     (1, 10, 10, 12, 16, 3, 1, 0, NHWC, NHWC, "conv_generic"),     # Cin % 8 != 0
+    (2, 12, 12, 48, 64, 5, 1, 2, NHWC, NHWC, "conv_generic"),     # Inception's 5x5
 ]
 
 
@@ -104,6 +105,35 @@ def test_conv_rejects_bad_shapes(gpu_server):
         with pytest.raises(TorporError):
             t.s.stream_synchronize(t.fid)
         t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1)
+
+
+@pytest.mark.parametrize("kh,kw,stride,Cin,Cout,H,W", [
+    (1, 7, 1, 16, 24, 17, 17), (7, 1, 1, 48, 70, 17, 17), (1, 3, 1, 24, 40, 8, 8), (3, 1, 1, 16, 64, 8, 9),
+    (1, 7, 1, 256, 32, 5, 7),   # splits over channels
+])
+def test_conv_tap_shapes(gpu_server, kh, kw, stride, Cin, Cout, H, W):
+    """The asymmetric convolutions of Inception on the MFMA taps kernel ("same" padding),
+    with the fused batch-norm + ReLU of a BasicConv2d."""
+    rng = np.random.default_rng(kh * 10 + kw + Cin)
+    N, ph, pw = 2, kh // 2, kw // 2
+    x = _rand(rng, N, H, W, Cin)
+    w = _rand(rng, Cout, Cin, kh, kw) * np.float32(1.0 / np.sqrt(Cin * kh * kw))
+    g, b, mu = _rand(rng, Cout), _rand(rng, Cout), _rand(rng, Cout)
+    var = rng.uniform(0.5, 2.0, Cout).astype(np.float32)
+    Ho, Wo = (H + 2 * ph - kh) // stride + 1, (W + 2 * pw - kw) // stride + 1
+    with OpSession(gpu_server, [w, g, b, mu, var]) as t:
+        xv = t.act(x)
+        yv = t.empty(N * Ho * Wo * Cout * 4)
+        t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, kh, kw, stride=stride, pad=(ph, pw))
+        assert t.s.last_kernel() == f"conv_taps_{kh}x{kw}_64x64", t.s.last_kernel()
+        plain = t.read(yv, (N, Ho, Wo, Cout))
+        t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, kh, kw, stride=stride, pad=(ph, pw), bn=tuple(t.w[1:5]),
+                 bn_eps=1e-3, act=ACT_RELU)
+        fused = t.read(yv, (N, Ho, Wo, Cout))
+    want = ref.conv2d(x, w, (stride, stride), (ph, pw), x_nhwc=True, y_nhwc=True)
+    assert_close(plain, want, RTOL, f"conv {kh}x{kw}")
+    z = ref.bn(want, g, b, mu, var, 1e-3, Cout, nhwc=True, relu=True)
+    assert_close(fused, z, 5e-5, f"conv {kh}x{kw} + bn + relu")
 
 
 @pytest.mark.parametrize("C,k,stride,HW", [(32, 3, 1, 14), (24, 3, 2, 15), (16, 5, 2, 9), (8, 3, 1, 5)])

@@ -9,7 +9,7 @@
 // residual / activation.
 //
 //   1x1, NHWC, Cin%4==0, pad 0      -> the dense GEMM kernel with a row gather
-//   3x3, NHWC, Cin%8==0             -> conv3x3_fast_kernel (K-block = 8 channels x 9 taps)
+//   3x3, 1x7, 7x1, 1x3, 3x1; NHWC, Cin%8==0 -> conv_taps_kernel (K-block = 8 channels x taps)
 //   everything else (7x7 stem, NCHW) -> conv_generic_kernel (scalar gathers)
 #include "kernels.hpp"
 #include "mfma_tile.hpp"
@@ -44,19 +44,21 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
     return xcd * q + (xcd < rem ? xcd : rem) + local;
 }
 
-// K-block = 8 input channels x 9 taps, ordered k_local = tap*8 + c in LDS.
+// KH x KW taps (T = KH*KW; 3x3, and the 1x7 / 7x1 / 1x3 / 3x1 shapes of Inception), NHWC,
+// Cin % 8 == 0.  K-block = 8 input channels x T taps, ordered k_local = tap*8 + c in LDS.
 // Activation side: for (pixel, tap) the 8 channels are 32 contiguous bytes of
 // the NHWC input (two dwordx4 loads by two neighbouring threads).  Weight side:
-// for one output channel the 8x9 block is 72 contiguous floats of the
-// [Cout][Cin][3][3] tensor; each thread loads 36 of them (4 channels x 9 taps)
+// for one output channel the 8 x T block is 8T contiguous floats of the
+// [Cout][Cin][KH][KW] tensor; each thread loads 4T of them (4 channels x T taps)
 // with dwordx4 and transposes in registers to the tap-major LDS order.
 //
-// WGK > 1 (3 or 9: the nine k-groups of a K-block split evenly) lets extra wavefronts share one
-// output tile; with few output tiles this replaces a split over workgroups, whose partial sums
-// go through memory and a reduction launch.
-template <class C>
-__global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x3_fast_kernel(const ConvDev p) {
-    static_assert(C::BK == 72, "3x3 fast path uses K-blocks of 72");
+// WGK > 1 (3 or 9 for 3x3: the nine k-groups of a K-block split evenly) lets extra wavefronts
+// share one output tile; with few output tiles this replaces a split over workgroups, whose
+// partial sums go through memory and a reduction launch.
+template <class C, int KH, int KW>
+__global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_taps_kernel(const ConvDev p) {
+    constexpr int T = KH * KW;
+    static_assert(C::BK == 8 * T, "K-block = 8 channels x taps");
     static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
     __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, red_floats<C>() + stage_floats<C>())];
     float* As = lds;
@@ -74,14 +76,14 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x
     // Branch-free operand fetch: rows past the last pixel are clamped to it (computed, then
     // dropped at the store) and taps that fall into the padding read from a page of zeros with
     // a zero channel step, so every load in the loop is unconditional.
-    constexpr int NVA = (C::BM * 18 + C::THREADS - 1) / C::THREADS;
+    constexpr int NVA = (C::BM * 2 * T + C::THREADS - 1) / C::THREADS;
     const float* pa[NVA];
     int stepA[NVA];
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
         int idx = i * C::THREADS + tid;
-        if (idx > C::BM * 18 - 1) idx = C::BM * 18 - 1;
-        const int row = idx / 18, t2 = idx - row * 18;
+        if (idx > C::BM * 2 * T - 1) idx = C::BM * 2 * T - 1;
+        const int row = idx / (2 * T), t2 = idx - row * (2 * T);
         const int tap = t2 >> 1, cq = t2 & 1;
         long grow = m0 + row;
         if (grow > p.M - 1) grow = p.M - 1;
@@ -89,8 +91,8 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x
         const long tt = grow / p.Wo;
         const int ho = (int)(tt % p.Ho);
         const long n = tt / p.Ho;
-        const int hi = ho * p.sh - p.ph + tap / 3;
-        const int wi = wo * p.sw - p.pw + tap % 3;
+        const int hi = ho * p.sh - p.ph + tap / KW;
+        const int wi = wo * p.sw - p.pw + tap % KW;
         const bool inside = hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
         pa[i] = inside ? p.x + n * p.xs_n + (long)hi * p.xs_h + (long)wi * p.xs_w + cq * 4 : p.zeros;
         stepA[i] = inside ? 1 : 0;
@@ -99,12 +101,12 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x
     const int wcol = tid >> 1, wcq = tid & 1;
     long wc = n0 + wcol;
     if (wc > p.Cout - 1) wc = p.Cout - 1;
-    const float* __restrict__ wbase = p.w + (wc * (long)p.Cin + wcq * 4) * 9;
+    const float* __restrict__ wbase = p.w + (wc * (long)p.Cin + wcq * 4) * T;
 
     f32x16 acc[C::TM][C::TN];
     zero_acc<C>(acc);
     f32x4 ra[NVA];
-    f32x4 rw[9];
+    f32x4 rw[T];
 
     auto load_regs = [&](int c0) {
         if (c0 > cend - 8) c0 = cend - 8;  // look-ahead past the end re-reads the last block
@@ -112,24 +114,24 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv3x
         for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + c0 * stepA[i]);
         if (tid < C::BN * 2) {
 #pragma unroll
-            for (int j = 0; j < 9; ++j) rw[j] = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * 9 + j * 4);
+            for (int j = 0; j < T; ++j) rw[j] = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * T + j * 4);
         }
     };
     auto store_lds = [&]() {
 #pragma unroll
         for (int i = 0; i < NVA; ++i) {
             const int idx = i * C::THREADS + tid;
-            const int row = idx / 18, t2 = idx - row * 18;
-            if (idx < C::BM * 18) *reinterpret_cast<f32x4*>(As + row * C::LDK + t2 * 4) = ra[i];
+            const int row = idx / (2 * T), t2 = idx - row * (2 * T);
+            if (idx < C::BM * 2 * T) *reinterpret_cast<f32x4*>(As + row * C::LDK + t2 * 4) = ra[i];
         }
         if (tid < C::BN * 2) {
-            // rw holds w[c][tap] for c = 0..3 (this thread's channel quad), flat index c*9 + tap
+            // rw holds w[c][tap] for c = 0..3 (this thread's channel quad), flat index c*T + tap
 #pragma unroll
-            for (int tap = 0; tap < 9; ++tap) {
+            for (int tap = 0; tap < T; ++tap) {
                 f32x4 v;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const int f = c * 9 + tap;
+                    const int f = c * T + tap;
                     v[c] = rw[f >> 2][f & 3];
                 }
                 *reinterpret_cast<f32x4*>(Bs + wcol * C::LDK + tap * 8 + wcq * 4) = v;
@@ -400,9 +402,31 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         p.ep.ncols = a.Cout;
     }
 
-    const bool fast3 = a.KH == 3 && a.KW == 3 && a.x_nhwc && (a.Cin % 8 == 0) && (xp % 4 == 0) && aligned16c(a.x) &&
-                       aligned16c(a.w) && ws.zeros != nullptr;
-    if (fast3) {
+    const bool taps_ok = a.x_nhwc && (a.Cin % 8 == 0) && (xp % 4 == 0) && aligned16c(a.x) && aligned16c(a.w) &&
+                         ws.zeros != nullptr;
+    const bool fast3 = a.KH == 3 && a.KW == 3 && taps_ok;
+    const int other_taps = !taps_ok ? 0 : (a.KH == 1 && a.KW == 7) ? 1 : (a.KH == 7 && a.KW == 1) ? 2
+                           : (a.KH == 1 && a.KW == 3) ? 3 : (a.KH == 3 && a.KW == 1) ? 4 : 0;
+    if (other_taps) {
+        // the asymmetric shapes (Inception): one 64x64 tile shape, split over channel blocks.  (5x5 stays on
+        // the general kernel: a 200-wide K-block leaves one workgroup per CU and measured 2x slower.)
+        const int T = a.KH * a.KW;
+        p.tiles_m = (int)((M + 63) / 64);
+        p.tiles_n = (a.Cout + 63) / 64;
+        long kper_k = p.K;
+        p.splits = choose_splits((long)p.tiles_m * p.tiles_n, p.K, 8 * T, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
+        p.kper = kper_k / T;
+        dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
+        switch (other_taps) {
+            case 1: hipLaunchKernelGGL((conv_taps_kernel<TileCfg<64, 64, 56, 2, 2>, 1, 7>), grid, dim3(256), 0, s, p); break;
+            case 2: hipLaunchKernelGGL((conv_taps_kernel<TileCfg<64, 64, 56, 2, 2>, 7, 1>), grid, dim3(256), 0, s, p); break;
+            case 3: hipLaunchKernelGGL((conv_taps_kernel<TileCfg<64, 64, 24, 2, 2>, 1, 3>), grid, dim3(256), 0, s, p); break;
+            default: hipLaunchKernelGGL((conv_taps_kernel<TileCfg<64, 64, 24, 2, 2>, 3, 1>), grid, dim3(256), 0, s, p); break;
+        }
+        static const char* const nm[5] = {"", "conv_taps_1x7_64x64", "conv_taps_7x1_64x64", "conv_taps_1x3_64x64",
+                                          "conv_taps_3x1_64x64"};
+        set_last_kernel(nm[other_taps]);
+    } else if (fast3) {
         const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);
         const long t64 = ((M + 63) / 64) * ((a.Cout + 63) / 64);
         static const int forced = getenv("TORPOR_CONV3_CFG") ? atoi(getenv("TORPOR_CONV3_CFG")) : -1;
@@ -429,23 +453,23 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
         switch (cfg) {
             case 0:
-                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3L>), grid, dim3(Conv3L::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3L, 3, 3>), grid, dim3(Conv3L::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_128x128");
                 break;
             case 1:
-                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3M>), grid, dim3(Conv3M::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3M, 3, 3>), grid, dim3(Conv3M::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_64x64");
                 break;
             case 2:
-                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3S>), grid, dim3(Conv3S::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3S, 3, 3>), grid, dim3(Conv3S::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_64x64_k3");
                 break;
             case 3:
-                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3T>), grid, dim3(Conv3T::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3T, 3, 3>), grid, dim3(Conv3T::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_32x32_k9");
                 break;
             default:
-                hipLaunchKernelGGL((conv3x3_fast_kernel<Conv3U>), grid, dim3(Conv3U::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3U, 3, 3>), grid, dim3(Conv3U::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_32x32_k3");
                 break;
         }
