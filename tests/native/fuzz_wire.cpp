@@ -1,0 +1,120 @@
+// Host-side robustness check, built with AddressSanitizer + UndefinedBehaviorSanitizer on the host pass
+// (tests/test_sanitize_host.py): the wire front end's message handlers are fed (a) well-formed
+// request sequences, (b) the same bytes with random mutations, (c) random bytes, against an engine
+// created with TP_FLAG_HOST_ONLY (no device is touched).  Nothing may crash, leak or trip a
+// sanitizer; malformed input must come back as error codes.
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <string>
+
+#define main torpor_server_main   // the front end's handlers live in an anonymous namespace of its one file
+#include "../../torpor_amd/csrc/wire/server_main.cpp"
+#undef main
+
+namespace {
+
+std::string query(int type, const std::string& body, int client) {
+    pb::Writer q;
+    q.i32(1, type);
+    q.message(2, body);
+    q.i32(3, client);
+    pb::Writer l;
+    l.message(1, q.out);
+    return l.out;
+}
+std::string signal_msg(int type, const char* fn, const char* payload) {
+    pb::Writer w;
+    w.i32(1, type);
+    w.str(2, fn);
+    w.str(3, payload);
+    return w.out;
+}
+
+}  // namespace
+
+int main() {
+    tp_config cfg;
+    std::memset(&cfg, 0, sizeof cfg);
+    cfg.struct_size = sizeof cfg;
+    cfg.flags = TP_FLAG_HOST_ONLY;
+    cfg.mem_limit_bytes = 64ull << 20;
+    cfg.pool_bytes = 96ull << 20;
+    Server S;
+    if (tp_server_create(&cfg, &S.eng) != 0) {
+        std::fprintf(stderr, "tp_server_create failed\n");
+        return 2;
+    }
+    std::mt19937_64 rng(12345);
+    std::vector<std::string> corpus;
+
+    // a well-formed registration: ExecuteAfterLoad, malloc, upload, device synchronise
+    bool dfr = false;
+    corpus.push_back(signal_msg(TP_REQ_EXECUTE_AFTER_LOAD, "3", "1"));
+    (void)handle_signal(S, corpus.back(), &dfr);
+    {
+        pb::Writer m;
+        m.u64(1, 4096);
+        corpus.push_back(query(Q_MALLOC, m.out, 3));
+        pb::Writer c;  // a convolution descriptor with every field present
+        c.u64(4, 1);
+        c.u64(6, 2);
+        c.u64(13, 3);
+        for (int f = 20; f <= 33; ++f) c.i32(f, 3);
+        c.u64(35, 8);
+        c.u64(36, 8);
+        corpus.push_back(query(Q_CONV, c.out, 3));
+        pb::Writer l;
+        l.i32(20, TP_OP_LAYERNORM);
+        corpus.push_back(query(Q_LAUNCH, l.out, 3));
+        pb::Writer g;
+        for (int f = 1; f <= 20; ++f) g.u64(f, 1 + f);
+        corpus.push_back(query(Q_GEMM, g.out, 3));
+        corpus.push_back(query(Q_SGEMM, g.out, 3));
+        corpus.push_back(query(Q_SGEMM_BATCHED, g.out, 3));
+        corpus.push_back(query(Q_BN, g.out, 3));
+        corpus.push_back(query(Q_MEMCPY, g.out, 3));
+        corpus.push_back(query(Q_MEMCPY_ASYNC, g.out, 3));
+        corpus.push_back(query(Q_MEMSET_ASYNC, g.out, 3));
+        corpus.push_back(query(Q_REPLAY, g.out, 3));
+        corpus.push_back(query(Q_FREE, g.out, 3));
+        corpus.push_back(query(Q_STREAM_SYNC, "", 3));
+        corpus.push_back(query(Q_DEVICE_SYNC, "", 3));
+    }
+    for (const auto& m : corpus) handle_query_list(S, m);
+
+    long handled = 0;
+    for (int it = 0; it < 20000; ++it) {
+        std::string m;
+        const int mode = (int)(rng() % 3);
+        if (mode == 0) {
+            m.resize(rng() % 96);
+            for (auto& ch : m) ch = (char)rng();
+        } else {
+            m = corpus[rng() % corpus.size()];
+            const int flips = 1 + (int)(rng() % 4);
+            for (int k = 0; k < flips && !m.empty(); ++k) {
+                const size_t pos = rng() % m.size();
+                if (mode == 1)
+                    m[pos] = (char)rng();
+                else
+                    m.erase(pos, 1 + rng() % 3);
+            }
+        }
+        if (rng() % 5 == 0) {
+            bool d = false;
+            (void)handle_signal(S, m, &d);
+        } else {
+            handle_query_list(S, m);
+        }
+        int32_t ack, resp;
+        while (tp_take_deferred_ack(S.eng, &ack, &resp) == 1) {
+        }
+        (void)tp_poll(S.eng);
+        ++handled;
+    }
+    tp_server_destroy(S.eng);
+    std::printf("fuzz ok: %ld messages\n", handled);
+    return 0;
+}

@@ -1,0 +1,42 @@
+"""Host code under AddressSanitizer + UndefinedBehaviorSanitizer: the engine (host-only mode), the
+C-ABI and the wire front end's message handlers are compiled with the sanitizers on the host pass
+and fed well-formed, mutated and random messages (tests/native/fuzz_wire.cpp).  CPU only."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HIPCC = "/opt/rocm/bin/hipcc"
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_wire_handlers_and_engine_under_sanitizers(tmp_path):
+    csrc = os.path.join(ROOT, "torpor_amd", "csrc")
+    san = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined"]
+    flags = ["--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops"] + san
+    objs = []
+    # the kernels come from the regular build (device code is not instrumented); host files are rebuilt
+    for src in ("engine.cpp", "capi.cpp"):
+        o = str(tmp_path / (src + ".o"))
+        subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", os.path.join(csrc, src), "-o", o],
+                              stderr=subprocess.DEVNULL)
+        objs.append(o)
+    for k in ("gemm", "conv", "ops", "attention"):
+        o = os.path.join(ROOT, "build", "obj", "kernels", k + ".hip.o")
+        if not os.path.exists(o):
+            pytest.skip("kernel objects not built (run make -C torpor_amd/csrc)")
+        objs.append(o)
+    drv = str(tmp_path / "fuzz_wire.o")
+    subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", os.path.join(ROOT, "tests", "native", "fuzz_wire.cpp"),
+                                             "-o", drv], stderr=subprocess.DEVNULL)
+    exe = str(tmp_path / "fuzz_wire")
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-o", exe, drv]
+                          + objs + ["-lpthread"], stderr=subprocess.DEVNULL)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TORPOR_IPC_DIR=str(tmp_path))
+    r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "fuzz ok" in r.stdout, (r.stdout[-2000:], r.stderr[-4000:])
+    shutil.rmtree(tmp_path, ignore_errors=True)

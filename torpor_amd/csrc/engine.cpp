@@ -1011,7 +1011,9 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
     void* q[12] = {nullptr};
     // the first 256 bytes of the scratch allocation stay zero for good (padding source of the
     // 3x3 convolution); split-K partial sums live behind them
-    const tpk::Workspace ws{workspace_ + 64, (size_t)cfg_.workspace_bytes - 256, workspace_};
+    // no device workspace in host-only mode (nothing is launched there)
+    const tpk::Workspace ws = workspace_ ? tpk::Workspace{workspace_ + 64, (size_t)cfg_.workspace_bytes - 256, workspace_}
+                                        : tpk::Workspace{};
     // Every operand is translated together with the byte span the kernel will touch, so an op
     // whose shapes do not fit its buffers is refused on the host instead of faulting the GPU.
     auto R = [&](int idx, bool optional, int64_t elems, int64_t elem_size = 4) -> int {
