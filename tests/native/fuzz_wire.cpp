@@ -115,6 +115,42 @@ int main() {
         ++handled;
     }
     tp_server_destroy(S.eng);
+
+    // the slab pool and the LRU evictor through their stand-alone handles: random alloc / release and
+    // add / lock / evict sequences, including stale offsets and unknown names
+    tp_pool* pool = tp_pool_create(64ull << 20);
+    std::vector<uint64_t> live;
+    for (int it = 0; it < 20000; ++it) {
+        const int op = (int)(rng() % 4);
+        if (op < 2) {
+            const uint64_t off = tp_pool_alloc(pool, 1 + rng() % (6ull << 20));
+            if (off != UINT64_MAX) live.push_back(off);
+        } else if (op == 2 && !live.empty()) {
+            const size_t k = rng() % live.size();
+            if (tp_pool_release(pool, live[k]) != 0) return 3;
+            live.erase(live.begin() + (long)k);
+        } else {
+            (void)tp_pool_release(pool, rng() % (64ull << 20));   // mostly not a live extent: must be refused
+            live.clear();                                          // (a hit frees one of ours; stop tracking)
+            tp_pool_destroy(pool);
+            pool = tp_pool_create(64ull << 20);
+        }
+    }
+    tp_pool_destroy(pool);
+    tp_lru* lru = tp_lru_create(1000);
+    char victims[256];
+    for (int it = 0; it < 20000; ++it) {
+        char name[8];
+        std::snprintf(name, sizeof name, "%d", (int)(rng() % 24));
+        int32_t nv = 0, over = 0;
+        switch (rng() % 5) {
+            case 0: case 1: (void)tp_lru_check_and_add(lru, name, 1 + rng() % 400, victims, sizeof victims, &nv, &over); break;
+            case 2: (void)tp_lru_lock(lru, name); break;
+            case 3: (void)tp_lru_unlock(lru, name); break;
+            default: (void)tp_lru_force_evict(lru, name); break;
+        }
+    }
+    tp_lru_destroy(lru);
     std::printf("fuzz ok: %ld messages\n", handled);
     return 0;
 }
