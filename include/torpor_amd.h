@@ -58,6 +58,7 @@ typedef struct tp_server tp_server;
 
 /* ---- tp_config.flags ---- */
 #define TP_FLAG_HOST_ONLY 1 /* no HIP calls: pool/LRU/state-machine logic only (CPU tests) */
+#define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
 
 /* ---- activation / epilogue ---- */
 #define TP_ACT_NONE 0
@@ -320,6 +321,48 @@ int tp_lru_force_evict(tp_lru* l, const char* function); /* 1 = was tracked, 0 =
 int tp_lru_lock(tp_lru* l, const char* function);
 int tp_lru_unlock(tp_lru* l, const char* function);
 uint64_t tp_lru_used(tp_lru* l);
+
+/* Control-plane policy objects for a node with several GPUs; decision logic only, no device calls.
+ * tp_evictor: the Evictor interface (evictor.hpp:14-26) with one budget per GPU.  TP_EVICT_LRU is LRUEvictor
+ *             (evictor.hpp:190-264); TP_EVICT_IA is InterferenceAwareEvictor (evictor.hpp:28-188): models of level
+ *             >= 1 that only one GPU holds are evicted after everything else.  Levels are those of the
+ *             ExecuteAfterLoad payload (controller.hpp:142-152), 0 light / 1 median / 2 heavy, default 0.
+ *             check_and_add writes victims as tp_lru_check_and_add does; order() writes the eviction order of one
+ *             GPU, first victim first.
+ * tp_sched:   executor states, residency and link tables of the controller, and its three decisions:
+ *             placement() (controller.hpp:271-294), TP_SCHED_RANDOM (controller.hpp:296-319) and TP_SCHED_IA
+ *             (controller.hpp:321-389).  status values are the reference's ExecutorStatus (-1 idle, 0 local, 1 peer
+ *             copy, 2..4 host-link swap of a light / median / heavy model, 5 cold start).  `draw` replaces rand()
+ *             of the random policy so that callers (and tests) own the random stream.  decide() returns 0 and
+ *             dst = -1 when no executor is idle. */
+#define TP_EVICT_LRU 0
+#define TP_EVICT_IA 1
+typedef struct tp_evictor tp_evictor;
+tp_evictor* tp_evictor_create(int32_t policy, int32_t gpu_count, uint64_t budget_bytes);
+void tp_evictor_destroy(tp_evictor* e);
+int tp_evictor_set_level(tp_evictor* e, const char* function, int32_t level);
+int tp_evictor_check_and_add(tp_evictor* e, int32_t gpu, const char* function, uint64_t size, char* victims,
+                             uint64_t cap, int32_t* n_victims, int32_t* over_budget);
+int tp_evictor_force_evict(tp_evictor* e, int32_t gpu, const char* function); /* 1 = was tracked */
+int tp_evictor_lock(tp_evictor* e, int32_t gpu, const char* function);
+int tp_evictor_unlock(tp_evictor* e, int32_t gpu, const char* function);
+uint64_t tp_evictor_used(tp_evictor* e, int32_t gpu);
+int tp_evictor_is_protected(tp_evictor* e, int32_t gpu, const char* function); /* TP_EVICT_IA: 1 = evicted last */
+int tp_evictor_order(tp_evictor* e, int32_t gpu, char* out, uint64_t cap);
+
+#define TP_SCHED_RANDOM 0
+#define TP_SCHED_IA 1
+typedef struct tp_sched tp_sched;
+tp_sched* tp_sched_create(int32_t gpu_count);
+void tp_sched_destroy(tp_sched* s);
+int tp_sched_set_sibling(tp_sched* s, int32_t gpu, int32_t other); /* shares the host link (PCIe switch) */
+int tp_sched_set_link(tp_sched* s, int32_t a, int32_t b, int32_t kind); /* -1 none, 0 self, 1 slow, 2 fast */
+int tp_sched_set_status(tp_sched* s, int32_t gpu, int32_t status);
+int tp_sched_set_level(tp_sched* s, const char* function, int32_t level);
+int tp_sched_set_resident(tp_sched* s, const char* function, int32_t gpu, int32_t resident);
+int tp_sched_placement(tp_sched* s); /* GPU for a cold start, -1 if none idle */
+int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t draw, int32_t* dst_gpu,
+                    int32_t* src_gpu, int32_t* status);
 
 #ifdef __cplusplus
 }

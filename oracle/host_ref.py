@@ -3,11 +3,23 @@
   LruRef      include/server/evictor.hpp:190-264 (LRUEvictor), single GPU.  One difference is
               made explicit: where the reference would loop forever (nothing unlocked left to
               evict, evictor.hpp:211-224) `check_and_add` stops evicting and inserts anyway.
+  IaRef       include/server/evictor.hpp:28-188 (InterferenceAwareEvictor), any number of GPUs,
+              kept in the reference's own shape (two recency lists per GPU).  Same explicit
+              difference: the search of the protected list stops when nothing unlocked is left
+              (the reference would loop forever, evictor.hpp:85-97).
+  SchedRef    include/server/controller.hpp:271-389: round-robin placement and the random /
+              interference-aware scheduling decisions over executor states, residency and the
+              PCIe-sibling and peer-link tables (defaults: the reference's 4-GPU tables,
+              controller.hpp:117-118).
   signal_*    proto3 wire bytes of proto/signal.proto:5-30, written from the protobuf encoding
               spec (varint field keys, length-delimited strings, default values omitted).
 
 Pinning: LruRef is checked against a brute-force list model on random traces
-(tests/test_host_logic.py); the codec against the known-answer byte strings derived by hand from
+(tests/test_host_logic.py); IaRef against LruRef where the two policies must coincide (one GPU,
+one level), against the policy's defining invariant (a model of level >= 1 is protected exactly
+when one GPU holds it) on random multi-GPU traces, and on hand-worked traces; SchedRef on
+hand-worked cases over the reference's 4-GPU tables and against exhaustive properties (never a
+busy GPU, a resident idle GPU always wins, the sibling-status minimum); the codec against the known-answer byte strings derived by hand from
 the proto3 spec and against the installed `google.protobuf` runtime with a descriptor built in
 code (tests/test_wire.py).
 """
@@ -48,6 +60,141 @@ class LruRef:
 
     def unlock(self, func):
         self.locked.discard(func)
+
+
+class IaRef:
+    """Two recency lists per GPU; index 0 of a list is the most recent entry (evictor.hpp:181-186)."""
+
+    def __init__(self, gpu_count, budget):
+        self.budget = budget
+        self.first = [[] for _ in range(gpu_count)]     # protected: [name, size], evicted last
+        self.second = [[] for _ in range(gpu_count)]
+        self.locked = [set() for _ in range(gpu_count)]
+        self.cur = [0] * gpu_count
+        self.gpus = {}                                   # model_to_gpus
+        self.level = {}                                  # model_level_map (controller.hpp:472)
+
+    @staticmethod
+    def _find(lst, func):
+        return next((i for i, e in enumerate(lst) if e[0] == func), None)
+
+    def _move(self, src, dst, func):
+        i = self._find(src, func)
+        if i is None:
+            return False
+        dst.insert(0, src.pop(i))
+        return True
+
+    def check_and_add(self, gpu, func, sz):
+        if gpu in self.gpus.get(func, set()):            # evictor.hpp:43-60
+            if not self._move(self.first[gpu], self.first[gpu], func):
+                self._move(self.second[gpu], self.second[gpu], func)
+            return []
+        victims = []
+        for lst in (self.second[gpu], self.first[gpu]):  # evictor.hpp:65-97
+            while self.cur[gpu] + sz >= self.budget:
+                i = next((k for k in range(len(lst) - 1, -1, -1) if lst[k][0] not in self.locked[gpu]), None)
+                if i is None:
+                    break
+                name, size = lst.pop(i)
+                victims.append(name)
+                self.cur[gpu] -= size
+        holders = self.gpus.setdefault(func, set())
+        heavy = self.level.get(func, 0) >= 1
+        if heavy and not holders:                        # evictor.hpp:99-103
+            self.first[gpu].insert(0, [func, sz])
+        else:                                            # evictor.hpp:104-122
+            self.second[gpu].insert(0, [func, sz])
+            if heavy:
+                for g in sorted(holders):
+                    self._move(self.first[g], self.second[g], func)
+        holders.add(gpu)
+        self.cur[gpu] += sz
+        for mod in victims:                              # evictor.hpp:126-144
+            left = self.gpus.setdefault(mod, set())
+            left.discard(gpu)
+            if self.level.get(mod, 0) >= 1 and len(left) == 1:
+                g = next(iter(left))
+                self._move(self.second[g], self.first[g], mod)
+        return victims
+
+    def force_evict(self, gpu, func):                    # evictor.hpp:149-170
+        hit = False
+        for lst in (self.first[gpu], self.second[gpu]):
+            i = self._find(lst, func)
+            if i is not None:
+                self.cur[gpu] -= lst.pop(i)[1]
+                hit = True
+                break
+        self.gpus.setdefault(func, set()).discard(gpu)
+        return hit
+
+    def lock(self, gpu, func):                           # evictor.hpp:172-174
+        self.locked[gpu].add(func)
+
+    def unlock(self, gpu, func):                         # evictor.hpp:176-180
+        self.locked[gpu].discard(func)
+
+    def order(self, gpu):
+        """Eviction order, first victim first."""
+        return [e[0] for e in reversed(self.second[gpu])] + [e[0] for e in reversed(self.first[gpu])]
+
+
+class SchedRef:
+    AVAIL, LOCAL, PEER, HOST_LIGHT, HOST_MEDIAN, HOST_HEAVY, COLD = -1, 0, 1, 2, 3, 4, 5   # controller.hpp:18-24
+
+    def __init__(self, gpu_count=4, sibling=(1, 0, 3, 2),
+                 link=((0, 1, 1, 2), (1, 0, 2, 1), (1, 2, 0, 2), (2, 1, 2, 0))):   # controller.hpp:117-118
+        self.n = gpu_count
+        self.status = [self.AVAIL] * gpu_count
+        self.sibling = list(sibling)
+        self.link = [list(r) for r in link]
+        self.resident = {}
+        self.level = {}
+        self.rr = 0
+
+    def _host_status(self, func):                        # controller.hpp:26-32
+        lv = self.level.get(func, 0)
+        return lv + self.HOST_LIGHT if 0 <= lv <= 2 else self.HOST_MEDIAN
+
+    def placement(self):                                 # controller.hpp:271-294
+        if self.status[self.rr] == self.AVAIL:
+            g = self.rr
+            self.rr = (self.rr + 1) % self.n
+            return g
+        return next((i for i in range(self.n) if self.status[i] == self.AVAIL), -1)
+
+    def random_schedule(self, func, draw):               # controller.hpp:296-319 ; draw stands for rand()
+        idle = [i for i in range(self.n) if self.status[i] == self.AVAIL]
+        if not idle:
+            return (-1, -1, -1)
+        for g in sorted(self.resident.get(func, ())):
+            if self.status[g] == self.AVAIL:
+                return (g, -1, self.LOCAL)
+        return (idle[draw % len(idle)], -1, self._host_status(func))
+
+    def interference_aware_schedule(self, func):         # controller.hpp:321-389
+        idle = [i for i in range(self.n) if self.status[i] == self.AVAIL]
+        if not idle:
+            return (-1, -1, -1)
+        holders = sorted(self.resident.get(func, ()))
+        if holders:
+            for g in holders:
+                if self.status[g] == self.AVAIL:
+                    return (g, -1, self.LOCAL)
+            dst, src = idle[0], holders[0]
+            for i in idle:                               # controller.hpp:347-355: the inner break only
+                for j in holders:
+                    if self.link[i][j] == 2:
+                        dst, src = i, j
+                        break
+            return (dst, src, self.PEER)
+        best, best_status = idle[0], self.status[self.sibling[idle[0]]]
+        for g in idle:                                   # controller.hpp:379-385
+            if self.status[self.sibling[g]] < best_status:
+                best_status = self.status[self.sibling[g]]
+                best = g
+        return (best, -1, self._host_status(func))
 
 
 def _varint(v):

@@ -293,6 +293,32 @@ def test_eviction_under_budget_and_deterministic_offsets(host_server):
     assert s.pool_stats()["used"] == 0
 
 
+def _register_level(s, fid, level):
+    fn = resnet.ResNet(s, fid, "resnet50", batch=1, seed=fid, image=32, level=level)
+    with pytest.raises(TorporError):
+        fn.register([np.zeros((1, 3, 32, 32), np.float32)])
+    return fn
+
+
+def test_model_levels_select_the_two_class_policy_or_plain_lru():
+    """controller.hpp:103-109, 142-152: by default a light model (level 0) is evicted before median / heavy
+    ones whatever its recency; with the LRU policy the level is ignored."""
+    for lru in (False, True):
+        s = Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20, request_timeout_ms=200,
+                   evict_lru=lru)
+        f1 = _register_level(s, 1, 1)
+        _register_level(s, 2, 2), _register_level(s, 3, 0)
+        assert [s.resident(i) for i in (1, 2, 3)] == [True, True, True]
+        assert s.signal(REQ_EXECUTE, 1, "")[0] == ACK_OK      # recency now 2 < 3 < 1; the budget holds three models
+        packed, outbuf, _ = f1.pack([np.zeros((1, 3, 32, 32), np.float32)])
+        with pytest.raises(TorporError):                      # host-only: completes the request without data
+            s.replay(1, packed, outbuf)
+        _register_level(s, 4, 1)
+        # two-class: the light model 3 goes although 2 is older; LRU: the oldest, 2
+        assert [s.resident(i) for i in (1, 2, 3, 4)] == ([True, False, True, True] if lru else [True, True, False, True])
+        s.close()
+
+
 def test_request_timeout_completes_the_request(host_server):
     """cuda_server.hpp:257-264: an Execute that sends no ops is force-completed after the timeout
     (200 ms here) and the executor becomes available again."""

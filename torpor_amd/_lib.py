@@ -157,6 +157,27 @@ SYMBOLS = {
     "tp_lru_lock": (C.c_int, [_P, C.c_char_p]),
     "tp_lru_unlock": (C.c_int, [_P, C.c_char_p]),
     "tp_lru_used": (_U64, [_P]),
+    "tp_evictor_create": (_P, [_I32, _I32, _U64]),
+    "tp_evictor_destroy": (None, [_P]),
+    "tp_evictor_set_level": (C.c_int, [_P, C.c_char_p, _I32]),
+    "tp_evictor_check_and_add": (C.c_int, [_P, _I32, C.c_char_p, _U64, C.c_char_p, _U64, C.POINTER(_I32),
+                                           C.POINTER(_I32)]),
+    "tp_evictor_force_evict": (C.c_int, [_P, _I32, C.c_char_p]),
+    "tp_evictor_lock": (C.c_int, [_P, _I32, C.c_char_p]),
+    "tp_evictor_unlock": (C.c_int, [_P, _I32, C.c_char_p]),
+    "tp_evictor_used": (_U64, [_P, _I32]),
+    "tp_evictor_is_protected": (C.c_int, [_P, _I32, C.c_char_p]),
+    "tp_evictor_order": (C.c_int, [_P, _I32, C.c_char_p, _U64]),
+    "tp_sched_create": (_P, [_I32]),
+    "tp_sched_destroy": (None, [_P]),
+    "tp_sched_set_sibling": (C.c_int, [_P, _I32, _I32]),
+    "tp_sched_set_link": (C.c_int, [_P, _I32, _I32, _I32]),
+    "tp_sched_set_status": (C.c_int, [_P, _I32, _I32]),
+    "tp_sched_set_level": (C.c_int, [_P, C.c_char_p, _I32]),
+    "tp_sched_set_resident": (C.c_int, [_P, C.c_char_p, _I32, _I32]),
+    "tp_sched_placement": (C.c_int, [_P]),
+    "tp_sched_decide": (C.c_int, [_P, _I32, C.c_char_p, C.c_uint32, C.POINTER(_I32), C.POINTER(_I32),
+                                  C.POINTER(_I32)]),
 }
 
 _lib = None

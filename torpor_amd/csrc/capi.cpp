@@ -1,9 +1,11 @@
 // extern "C" surface of the engine (include/torpor_amd.h).  Nothing here throws across the
 // boundary: allocation failures and engine errors come back as integer codes.
+#include <algorithm>
 #include <cstring>
 #include <new>
 
 #include "engine.hpp"
+#include "scheduler.hpp"
 #include "kernels/kernels.hpp"
 
 struct tp_server {
@@ -514,5 +516,153 @@ int tp_lru_unlock(tp_lru* l, const char* function) {
     TP_GUARD_END
 }
 uint64_t tp_lru_used(tp_lru* l) { return l ? l->lru.cur_size() : 0; }
+
+static void join_names(const std::vector<std::string>& v, char* out, uint64_t cap) {
+    if (!out || !cap) return;
+    std::string joined;
+    for (size_t i = 0; i < v.size(); ++i) {
+        if (i) joined += '\n';
+        joined += v[i];
+    }
+    std::strncpy(out, joined.c_str(), cap - 1);
+    out[cap - 1] = '\0';
+}
+
+struct tp_evictor {
+    int policy = TP_EVICT_IA;
+    tp::IaEvictor ia;
+    std::vector<tp::LruEvictor> lru;  // evictor.hpp:190-264 keeps one list per GPU
+    bool ok(int gpu) const { return gpu >= 0 && gpu < ia.gpu_count(); }
+};
+tp_evictor* tp_evictor_create(int32_t policy, int32_t gpu_count, uint64_t budget_bytes) {
+    if ((policy != TP_EVICT_LRU && policy != TP_EVICT_IA) || gpu_count < 1 || gpu_count > 64) return nullptr;
+    try {
+        auto* e = new tp_evictor;
+        e->policy = policy;
+        e->ia = tp::IaEvictor(gpu_count, budget_bytes);
+        e->lru.assign((size_t)gpu_count, tp::LruEvictor(budget_bytes));
+        return e;
+    } catch (...) {
+        return nullptr;
+    }
+}
+void tp_evictor_destroy(tp_evictor* e) { delete e; }
+int tp_evictor_set_level(tp_evictor* e, const char* function, int32_t level) {
+    TP_GUARD_BEGIN
+    if (!e || !function) return TP_EINVAL;
+    e->ia.set_level(function, level);
+    return 0;
+    TP_GUARD_END
+}
+int tp_evictor_check_and_add(tp_evictor* e, int32_t gpu, const char* function, uint64_t size, char* victims,
+                             uint64_t cap, int32_t* n_victims, int32_t* over_budget) {
+    TP_GUARD_BEGIN
+    if (!e || !function || !e->ok(gpu)) return TP_EINVAL;
+    bool over = false;
+    auto v = e->policy == TP_EVICT_IA ? e->ia.check_and_add(gpu, function, size, &over)
+                                      : e->lru[(size_t)gpu].check_and_add(function, size, &over);
+    if (n_victims) *n_victims = (int32_t)v.size();
+    if (over_budget) *over_budget = over ? 1 : 0;
+    join_names(v, victims, cap);
+    return 0;
+    TP_GUARD_END
+}
+int tp_evictor_force_evict(tp_evictor* e, int32_t gpu, const char* function) {
+    TP_GUARD_BEGIN
+    if (!e || !function || !e->ok(gpu)) return TP_EINVAL;
+    return (e->policy == TP_EVICT_IA ? e->ia.force_evict(gpu, function) : e->lru[(size_t)gpu].force_evict(function)) ? 1 : 0;
+    TP_GUARD_END
+}
+int tp_evictor_lock(tp_evictor* e, int32_t gpu, const char* function) {
+    TP_GUARD_BEGIN
+    if (!e || !function || !e->ok(gpu)) return TP_EINVAL;
+    if (e->policy == TP_EVICT_IA) e->ia.lock(gpu, function);
+    else e->lru[(size_t)gpu].lock(function);
+    return 0;
+    TP_GUARD_END
+}
+int tp_evictor_unlock(tp_evictor* e, int32_t gpu, const char* function) {
+    TP_GUARD_BEGIN
+    if (!e || !function || !e->ok(gpu)) return TP_EINVAL;
+    if (e->policy == TP_EVICT_IA) e->ia.unlock(gpu, function);
+    else e->lru[(size_t)gpu].unlock(function);
+    return 0;
+    TP_GUARD_END
+}
+uint64_t tp_evictor_used(tp_evictor* e, int32_t gpu) {
+    if (!e || !e->ok(gpu)) return 0;
+    return e->policy == TP_EVICT_IA ? e->ia.cur_size(gpu) : e->lru[(size_t)gpu].cur_size();
+}
+int tp_evictor_is_protected(tp_evictor* e, int32_t gpu, const char* function) {
+    TP_GUARD_BEGIN
+    if (!e || !function || !e->ok(gpu)) return TP_EINVAL;
+    return e->policy == TP_EVICT_IA && e->ia.is_protected(gpu, function) ? 1 : 0;
+    TP_GUARD_END
+}
+int tp_evictor_order(tp_evictor* e, int32_t gpu, char* out, uint64_t cap) {
+    TP_GUARD_BEGIN
+    if (!e || !e->ok(gpu)) return TP_EINVAL;
+    std::vector<std::string> v;
+    if (e->policy == TP_EVICT_IA) v = e->ia.order(gpu);
+    else {
+        v = e->lru[(size_t)gpu].order();  // most recent first
+        std::reverse(v.begin(), v.end());
+    }
+    join_names(v, out, cap);
+    return (int)v.size();
+    TP_GUARD_END
+}
+
+struct tp_sched {
+    tp::Scheduler s;
+};
+tp_sched* tp_sched_create(int32_t gpu_count) {
+    if (gpu_count < 1 || gpu_count > 64) return nullptr;
+    try {
+        auto* s = new tp_sched;
+        s->s.reset(gpu_count);
+        return s;
+    } catch (...) {
+        return nullptr;
+    }
+}
+void tp_sched_destroy(tp_sched* s) { delete s; }
+int tp_sched_set_sibling(tp_sched* s, int32_t gpu, int32_t other) {
+    return s && s->s.set_sibling(gpu, other) ? 0 : TP_EINVAL;
+}
+int tp_sched_set_link(tp_sched* s, int32_t a, int32_t b, int32_t kind) {
+    return s && kind >= -1 && kind <= 2 && s->s.set_link(a, b, kind) ? 0 : TP_EINVAL;
+}
+int tp_sched_set_status(tp_sched* s, int32_t gpu, int32_t status) {
+    return s && status >= -1 && status <= 5 && s->s.set_status(gpu, status) ? 0 : TP_EINVAL;
+}
+int tp_sched_set_level(tp_sched* s, const char* function, int32_t level) {
+    TP_GUARD_BEGIN
+    if (!s || !function) return TP_EINVAL;
+    s->s.set_level(function, level);
+    return 0;
+    TP_GUARD_END
+}
+int tp_sched_set_resident(tp_sched* s, const char* function, int32_t gpu, int32_t resident) {
+    TP_GUARD_BEGIN
+    if (!s || !function || gpu < 0 || gpu >= s->s.gpu_count()) return TP_EINVAL;
+    s->s.set_resident(function, gpu, resident != 0);
+    return 0;
+    TP_GUARD_END
+}
+int tp_sched_placement(tp_sched* s) { return s ? s->s.placement() : TP_EINVAL; }
+int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t draw, int32_t* dst_gpu,
+                    int32_t* src_gpu, int32_t* status) {
+    TP_GUARD_BEGIN
+    if (!s || !function || (policy != TP_SCHED_RANDOM && policy != TP_SCHED_IA)) return TP_EINVAL;
+    const tp::ScheduleDecision d = policy == TP_SCHED_IA
+                                       ? s->s.interference_aware_schedule(function)
+                                       : s->s.random_schedule(function, [draw](int n) { return (int)(draw % (uint32_t)n); });
+    if (dst_gpu) *dst_gpu = d.dst_gpu;
+    if (src_gpu) *src_gpu = d.src_gpu;
+    if (status) *status = d.status;
+    return 0;
+    TP_GUARD_END
+}
 
 }  // extern "C"

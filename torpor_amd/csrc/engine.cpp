@@ -48,6 +48,10 @@ int Engine::init() {
     // memory_manager.hpp:42-44 adds 5 GiB of slack above the eviction budget; 1 GiB is enough
     // here because allocations are whole-model extents, not per-tensor blocks.
     if (cfg_.pool_bytes == 0) cfg_.pool_bytes = cfg_.mem_limit_bytes + (1ull << 30);
+    {
+        const char* pol = std::getenv("EVICT_POLICY");  // controller.hpp:103-109
+        lru_.two_class = !((cfg_.flags & TP_FLAG_EVICT_LRU) || (pol && std::string(pol) == "LRU"));
+    }
     lru_.set_budget(cfg_.mem_limit_bytes);
     pool_.reset(cfg_.pool_bytes);
 
@@ -790,7 +794,7 @@ void Engine::evict_model(Model& m) {
 // controller.hpp:392-400
 bool Engine::check_eviction(Model& m) {
     bool over = false;
-    auto victims = lru_.check_and_add(std::to_string(m.id), m.total_bytes(), &over);
+    auto victims = lru_.check_and_add(std::to_string(m.id), m.total_bytes(), m.level, &over);
     for (auto& v : victims) {
         Model* vm = find(std::atoi(v.c_str()));
         if (vm) evict_model(*vm);

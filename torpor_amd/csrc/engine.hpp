@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "../../include/torpor_amd.h"
+#include "ia_evictor.hpp"
 #include "lru.hpp"
 #include "pool.hpp"
 
@@ -211,7 +212,26 @@ private:
     tp_config cfg_;
     std::mutex mu_;
     SlabPool pool_;
-    LruEvictor lru_;
+    // controller.hpp:103-109: EVICT_POLICY=LRU selects the plain LRU, anything else the two-class policy.
+    // With one GPU and every model at the default level (Median) both make the same decisions.
+    struct EvictPolicy {
+        bool two_class = true;
+        LruEvictor lru;
+        IaEvictor ia{1, 0};
+        void set_budget(uint64_t b) { lru.set_budget(b); ia.set_budget(b); }
+        uint64_t budget() const { return two_class ? ia.budget() : lru.budget(); }
+        uint64_t cur_size() const { return two_class ? ia.cur_size(0) : lru.cur_size(); }
+        size_t size() const { return two_class ? ia.size(0) : lru.size(); }
+        std::vector<std::string> check_and_add(const std::string& f, uint64_t sz, int level, bool* over) {
+            if (!two_class) return lru.check_and_add(f, sz, over);
+            ia.set_level(f, level);
+            return ia.check_and_add(0, f, sz, over);
+        }
+        bool force_evict(const std::string& f) { return two_class ? ia.force_evict(0, f) : lru.force_evict(f); }
+        bool peek_victim(const std::string& keep, std::string* out) const {
+            return two_class ? ia.peek_victim(0, keep, out) : lru.peek_victim(keep, out);
+        }
+    } lru_;
     uint8_t* arena_ = nullptr;
     float* workspace_ = nullptr;
     hipStream_t compute_ = nullptr, copy_ = nullptr, copy2_ = nullptr;

@@ -20,6 +20,7 @@ NCHW, NHWC = 0, 1
  OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION, OP_AVGPOOL2D, OP_COPY2D,
  OP_SCALE_CHANNELS) = range(1, 18)
 FLAG_HOST_ONLY = 1
+FLAG_EVICT_LRU = 2   # plain LRU instead of the two-class policy (as env EVICT_POLICY=LRU)
 
 
 def _chk(code, what):
@@ -34,7 +35,7 @@ def _as_bytes_view(a):
 
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
-                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0):
+                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False):
         self._l = _lib.lib()
         cfg = _lib.Config()
         cfg.struct_size = C.sizeof(_lib.Config)
@@ -44,7 +45,7 @@ class Server:
         cfg.chunk_bytes = chunk_bytes
         cfg.chunk_max_bytes = chunk_max_bytes
         cfg.workspace_bytes = workspace_bytes
-        cfg.flags = FLAG_HOST_ONLY if host_only else 0
+        cfg.flags = (FLAG_HOST_ONLY if host_only else 0) | (FLAG_EVICT_LRU if evict_lru else 0)
         cfg.request_timeout_ms = request_timeout_ms
         cfg.copy_streams = copy_streams
         h = C.c_void_p()
