@@ -1,0 +1,500 @@
+"""Request router: the layer that calls the server's signal boundary.
+
+What the reference's scripts/router.py does around the GPU server, without its docker / HTTP
+plumbing: functions are launched (ExecuteAfterLoad with the model level as payload,
+router.py:381-387), requests arrive from senders, wait in a FIFO queue (router.py:156-216) or
+in the SLO-aware pair of queues (router.py:218-378), are batched per function up to `-b`
+(router.py:186-189, 352-355) and dispatched with an Execute signal; completions feed the
+per-function statistics [requests within the deadline, requests, summed latency]
+(router.py:481-489) from which the SLO-aware policy re-ranks functions every two seconds
+(router.py:495-498) and adapts its admission factor alpha every 20 re-rankings.
+
+The reference runs one manager process per GPU and lets several functions execute at once on
+different GPUs; with one GPU the executor serves one request at a time, so `Router.pump`
+dispatches synchronously: drain the inbox, then run one batch to completion.
+
+Senders (scripts/sender_fix_rate.py, scripts/sender_from_trace.py) are functions that return
+the arrival list [(seconds since the previous request, function)], and `keepalive_p99`
+is tools/export_keepalive.py:24-27.
+"""
+import argparse
+import collections
+import json
+import time
+
+import numpy as np
+
+# scripts/router.py:39 ; levels from get_mixed_model_level (router.py:44-53)
+MIXED_MODELS = ("resnet50", "resnet101", "resnet152", "densenet169", "densenet201", "inception", "efficientnet",
+                "bertqa")
+
+
+def mixed_model_name(func_id, models=MIXED_MODELS):
+    return models[func_id % len(models)]
+
+
+def mixed_model_level(func_id, models=MIXED_MODELS):
+    i = func_id % len(models)
+    if i < 3:
+        return 1
+    if i < 7:
+        return 0
+    return 2 if i == 7 else 1
+
+
+# ----------------------------------------------------------------------------------------- policies
+class _Stats:
+    """Per function: [requests that met the deadline, requests, summed latency] (router.py:133-136)."""
+
+    def __init__(self):
+        self.stat = {}
+        self.avail = {}
+
+    def add(self, f):
+        self.stat[f] = [0, 0, 0.0]
+        self.avail[f] = True
+
+    def record(self, f, latencies, deadline):       # router.py:481-489
+        s = self.stat[f]
+        for lat in latencies:
+            s[2] += lat
+            s[1] += 1
+            if lat <= deadline:
+                s[0] += 1
+        self.avail[f] = True
+
+    def slo_ratio(self, slo):
+        """Share of the functions with at least one request whose hit rate reaches the target."""
+        seen = [s for s in self.stat.values() if s[1] > 0]
+        if not seen:
+            return None
+        return sum(1 for s in seen if s[0] / s[1] >= slo) / len(seen)
+
+
+class FifoPolicy:
+    """Arrival order; batches are runs of the same function at the head (router.py:156-216)."""
+    name = "fifo"
+
+    def __init__(self, stats, slo):
+        self.stats, self.slo = stats, slo
+        self.queue = collections.deque()
+
+    def add_function(self, f):
+        pass
+
+    def insert(self, f, arrival):
+        self.queue.append((f, arrival))
+
+    def __len__(self):
+        return len(self.queue)
+
+    def next_batch(self, limit):
+        if not self.queue:
+            return None
+        f, arr = self.queue.popleft()
+        arrivals = [arr]
+        while self.queue and self.queue[0][0] == f and len(arrivals) < limit(f):
+            arrivals.append(self.queue.popleft()[1])
+        return f, arrivals
+
+    def update(self):
+        return self.stats.slo_ratio(self.slo)
+
+
+class SloAwarePolicy:
+    """Two queues (router.py:218-378).
+
+    A function's urgency is  mean latency x (slo x requests - requests on time): the time it would
+    take to serve the on-time requests it is short of.  High-priority requests are kept most urgent
+    first, low-priority ones least urgent first; dispatch takes the first request of a function
+    that has none in flight, high queue before low.  `update` re-ranks: functions are sorted by
+    urgency / (1 - slo), and the least urgent ones whose positive urgencies add up to at most
+    alpha x (sum of positive urgencies) are high priority, the rest low - with alpha < 1 the
+    functions furthest from their target are sacrificed so that the others meet theirs.  Every
+    `window` updates alpha doubles (capped at 1) if the share of functions meeting the target rose
+    by 4 % or more, halves if it fell by more than 4 %, and creeps up by 1 % otherwise.
+
+    Positions in the queues come from a binary search with the urgencies of the moment, as in the
+    reference (router.py:229-248); the queues are re-sorted only by `update`, so between updates the
+    probe sequence decides where a request lands and is kept the same: mid = (lo + hi) // 2.
+    """
+    name = "sa"
+
+    def __init__(self, stats, slo, window=20, diff_threshold=0.04, scale=2.0, low_scale=1.01):
+        self.stats, self.slo = stats, slo
+        self.high_q, self.low_q = [], []
+        self.high, self.low = set(), set()
+        self.alpha = 1.0
+        self.window, self.diff_threshold, self.scale, self.low_scale = window, diff_threshold, scale, low_scale
+        self._updates = 0
+        self._old_ratio = 0.0
+
+    def add_function(self, f):          # router.py:475-479: new functions start as high priority
+        self.high.add(f)
+
+    def urgency(self, f):               # router.py:224-225
+        met, n, total = self.stats.stat[f]
+        return (total / n) * (self.slo * n - met) if n > 0 else 0
+
+    def insert(self, f, arrival):
+        if f in self.high:
+            q, before = self.high_q, lambda other, mine: other < mine
+        elif f in self.low:
+            q, before = self.low_q, lambda other, mine: other >= mine
+        else:
+            return False
+        mine = self.urgency(f)
+        lo, hi = 0, len(q)
+        while lo < hi:
+            mid = (lo + hi) // 2
+            if before(self.urgency(q[mid][0]), mine):
+                hi = mid
+            else:
+                lo = mid + 1
+        q.insert(lo, (f, arrival))
+        return True
+
+    def __len__(self):
+        return len(self.high_q) + len(self.low_q)
+
+    def _first_available(self):
+        for q in (self.high_q, self.low_q):
+            for i, (f, _) in enumerate(q):
+                if self.stats.avail[f]:
+                    return q, i
+        return None, None
+
+    def next_batch(self, limit):
+        q, i = self._first_available()
+        if q is None:
+            return None
+        f, arr = q.pop(i)
+        arrivals = [arr]
+        while len(arrivals) < limit(f):
+            q, i = self._first_available()
+            if q is None or q[i][0] != f:
+                break
+            arrivals.append(q.pop(i)[1])
+        return f, arrivals
+
+    def update(self):                   # router.py:318-376
+        self._updates += 1
+        slo = self.slo
+        ranked = [(f, (s[2] / s[1]) * (slo * s[1] - s[0]) / (1 - slo)) for f, s in self.stats.stat.items() if s[1] > 0]
+        ranked.sort(key=lambda x: x[1])
+        budget = sum(v for _, v in ranked if v >= 0) * self.alpha
+        border, acc = -1, 0
+        for i, (_, v) in enumerate(ranked):
+            if v > 0:
+                acc += v
+                if acc > budget:
+                    border = i - 1
+                    break
+        if acc <= budget:
+            border = len(ranked) - 1
+        for i, (f, _) in enumerate(ranked):
+            if i <= border:
+                self.high.add(f)
+                self.low.discard(f)
+            else:
+                self.high.discard(f)
+                self.low.add(f)
+        old_high, old_low = self.high_q, self.low_q
+        self.high_q, self.low_q = [], []
+        for f, arr in old_high:
+            self.insert(f, arr)
+        for f, arr in old_low:
+            self.insert(f, arr)
+        ratio = self.stats.slo_ratio(slo)
+        if ratio is None:
+            return None
+        if self._updates >= self.window:
+            diff = (ratio - self._old_ratio) / self._old_ratio if self._old_ratio > 0 else self.diff_threshold
+            if diff >= self.diff_threshold:
+                self.alpha = min(1, self.alpha * self.scale)
+                self._old_ratio = ratio
+            elif diff < -self.diff_threshold:
+                self.alpha = self.alpha / self.scale
+                self._old_ratio = ratio
+            else:
+                self.alpha = min(1, self.alpha * self.low_scale)
+            self._updates = 0
+        return ratio
+
+
+# ------------------------------------------------------------------------------------------- router
+class Router:
+    """`backend.launch(func_id, level)` registers a function and `backend.execute(func_id, n)` serves
+    a batch of n requests of it, blocking until the answers are back (see `FunctionBackend`)."""
+
+    UPDATE_PERIOD_S = 2.0               # router.py:495
+
+    def __init__(self, backend, slo_percentile=0.98, deadline_s=0.1, batch_limit=1, policy="sa", clock=time.monotonic,
+                 deadlines=None, batch_limits=None):
+        self.backend = backend
+        self.slo = slo_percentile
+        self.deadline_s = deadline_s
+        self.deadlines = dict(deadlines or {})          # per-function overrides (router.py:18: 0.2 s for BERT)
+        self.batch_limit = batch_limit
+        self.batch_limits = dict(batch_limits or {})    # router.py:20,186
+        self.clock = clock
+        self.stats = _Stats()
+        self.policy = SloAwarePolicy(self.stats, self.slo) if policy == "sa" else FifoPolicy(self.stats, self.slo)
+        self.inbox = collections.deque()
+        self.unhealthy = set()                          # router.py:491-493
+        self.latencies = collections.defaultdict(list)
+        self.batches = collections.Counter()
+        self._last_update = None
+        self.slo_history = []
+
+    def launch(self, func_id, level=None):
+        """router.py:381-387 + the manager's reply (router.py:475-479)."""
+        self.backend.launch(func_id, mixed_model_level(func_id) if level is None else level)
+        self.stats.add(func_id)
+        self.policy.add_function(func_id)
+
+    def force_evict(self, func_id):     # router.py:408-412
+        self.backend.unload(func_id)
+
+    def load_all(self):                 # router.py:462-468
+        for f in self.stats.stat:
+            self.backend.load(f)
+
+    def submit(self, func_id, arrival=None):
+        """A request from a sender (router.py:429-437)."""
+        if func_id in self.unhealthy:
+            return False
+        self.inbox.append((func_id, self.clock() if arrival is None else arrival))
+        return True
+
+    def _limit(self, f):
+        return self.batch_limits.get(f, self.batch_limit)
+
+    def pump(self):
+        """One turn of the scheduling loop: queue what has arrived, re-rank when due, then dispatch one
+        batch and wait for it.  Returns the number of requests served."""
+        now = self.clock()
+        if self._last_update is None:
+            self._last_update = now
+        while self.inbox:
+            f, arr = self.inbox.popleft()
+            self.policy.insert(f, arr)
+        if now - self._last_update > self.UPDATE_PERIOD_S:
+            self._last_update = now
+            ratio = self.policy.update()
+            if ratio is not None:
+                self.slo_history.append((now, ratio, getattr(self.policy, "alpha", None), len(self.policy)))
+        got = self.policy.next_batch(self._limit)
+        if got is None:
+            return 0
+        f, arrivals = got
+        self.stats.avail[f] = False
+        try:
+            self.backend.execute(f, len(arrivals))
+        except Exception:
+            self.unhealthy.add(f)       # router.py:104-106: a function that fails is taken out of service
+            self.stats.avail[f] = True
+            raise
+        end = self.clock()
+        lats = [end - a for a in arrivals]
+        self.stats.record(f, lats, self.deadlines.get(f, self.deadline_s))
+        self.latencies[f].extend(lats)
+        self.batches[len(arrivals)] += 1
+        return len(arrivals)
+
+    def queued(self):
+        return len(self.policy) + len(self.inbox)
+
+    def summary(self):
+        all_lat = np.sort(np.concatenate([np.asarray(v) for v in self.latencies.values()])) if self.latencies else np.zeros(0)
+
+        def pct(q):
+            return float(all_lat[min(len(all_lat) - 1, int(round(q * (len(all_lat) - 1))))]) * 1e3 if len(all_lat) else None
+
+        per_func = {f: s[0] / s[1] for f, s in self.stats.stat.items() if s[1] > 0}
+        return dict(policy=self.policy.name, requests=int(len(all_lat)), p50_ms=pct(0.5), p99_ms=pct(0.99),
+                    mean_ms=float(all_lat.mean() * 1e3) if len(all_lat) else None,
+                    functions_meeting_slo=self.stats.slo_ratio(self.slo),
+                    requests_within_deadline=(sum(s[0] for s in self.stats.stat.values()) /
+                                              max(1, sum(s[1] for s in self.stats.stat.values()))),
+                    worst_function_hit_rate=min(per_func.values()) if per_func else None,
+                    alpha=getattr(self.policy, "alpha", None), batches=dict(self.batches), queued=self.queued())
+
+
+def serve_arrivals(router, arrivals, clock=time.monotonic, drain=True):
+    """Open-loop replay of an arrival list [(gap_s, function)] against the wall clock: requests are
+    submitted when due, whatever the backlog (sender_from_trace.py:51-57)."""
+    t0 = clock()
+    due, i, n = 0.0, 0, len(arrivals)
+    if n:
+        due = float(arrivals[0][0])
+    while i < n or (drain and router.queued()):
+        now = clock() - t0
+        while i < n and due <= now:
+            router.submit(int(arrivals[i][1]), t0 + due)
+            i += 1
+            if i < n:
+                due += float(arrivals[i][0])
+        if router.pump() == 0 and i < n:
+            while clock() - t0 < due:
+                pass
+    return clock() - t0
+
+
+# ------------------------------------------------------------------------------------------ senders
+def fixed_rate_arrivals(func_num, rate_per_min, mins, rng):
+    """scripts/sender_fix_rate.py:46-56: every function at `rate_per_min`; per minute, as many gaps as
+    requests, each drawn (in milliseconds) from a Poisson law whose mean is the mean gap."""
+    out = []
+    overall = int(rate_per_min * func_num)
+    for _ in range(mins):
+        gaps = rng.poisson(60 * 1000 / overall, overall)
+        funcs = rng.choice(func_num, overall)
+        out += [(g / 1000, int(f)) for g, f in zip(gaps, funcs)]
+    return out
+
+
+def trace_arrivals(patterns, func_num, rng):
+    """scripts/sender_from_trace.py:19-32: each function follows one row of `patterns` (requests per
+    minute, one column per minute), rows drawn with replacement."""
+    patterns = np.asarray(patterns)
+    rows = patterns[rng.choice(len(patterns), func_num)]
+    out = []
+    for minute in range(patterns.shape[1]):
+        rates = rows[:, minute].astype(np.float64)
+        overall = int(rates.sum())
+        if overall <= 0:
+            continue
+        gaps = rng.poisson(60 * 1000 / overall, overall)
+        funcs = rng.choice(func_num, overall, p=rates / rates.sum())
+        out += [(g / 1000, int(f)) for g, f in zip(gaps, funcs)]
+    return out
+
+
+def synthetic_rate_patterns(n, mins, rng, mean_rpm=10.0):
+    """Stand-in for the reference's trace sample (tools/samples.npy: 203 functions x 31 minutes of
+    requests per minute, mean about 10, range 0..33): a per-function base rate with Poisson
+    minute-to-minute variation."""
+    base = rng.gamma(shape=6.0, scale=mean_rpm / 6.0, size=n)
+    return rng.poisson(base[:, None], size=(n, mins)).astype(np.int64)
+
+
+def keepalive_p99(arrivals):
+    """tools/export_keepalive.py:13-27: per function, the 99th percentile of its inter-arrival times."""
+    t, stamps = 0.0, collections.defaultdict(list)
+    for gap, f in arrivals:
+        t += gap
+        stamps[int(f)].append(t)
+    return {f: float(np.percentile(np.diff(s), 99)) for f, s in stamps.items() if len(s) > 1}
+
+
+# ------------------------------------------------------------------------------------------ backend
+class FunctionBackend:
+    """Functions of `torpor_amd.functions` behind a server (in-process `Server` or wire `Client`).
+
+    The reference's function container runs the model at batch = number of batched requests
+    (tests/endpoint.py:84-92).  Op streams here are recorded per shape, so a function is registered
+    at the router's batch limit and a smaller batch runs with the remaining rows left as they were."""
+
+    def __init__(self, server, factory, example_inputs):
+        self.server, self.factory, self.example_inputs = server, factory, example_inputs
+        self.fn = {}
+        self.first = {}                 # answers of the registration run
+
+    def launch(self, func_id, level):
+        fn = self.factory(self.server, func_id, level)
+        inputs = self.example_inputs(fn)
+        first = fn.register(inputs)
+        fn._weights = None              # the server's pinned store holds the authoritative copy now
+        packed, outbuf, views = fn.pack(inputs)
+        self.fn[func_id] = (fn, packed, outbuf, views)
+        self.first[func_id] = [np.array(a, copy=True) for a in first]
+
+    def outputs(self, func_id):
+        """Answers of the last request of the function."""
+        fn, _, _, views = self.fn[func_id]
+        return fn.postprocess(views)
+
+    def execute(self, func_id, n):
+        fn, packed, outbuf, _ = self.fn[func_id]
+        ack, _, deferred = self.server.signal(1, func_id, "")
+        if ack != 0 or deferred:
+            raise RuntimeError(f"execute {func_id}: ack={ack} deferred={deferred}")
+        self.server.replay(func_id, packed, outbuf)
+
+    def unload(self, func_id):
+        self.server.signal(3, func_id, "")
+
+    def load(self, func_id):
+        self.server.signal(2, func_id, "")
+
+
+def build_function(server, func_id, level, model, batch):
+    """One of the reference's served models (tests/endpoint.py:16-40) with seeded random weights."""
+    from .functions import bert, densenet, efficientnet, inception, mobilenet, resnet
+    name = mixed_model_name(func_id) if model == "mixed" else model
+    if name in ("resnet50", "resnet101", "resnet152"):
+        return resnet.ResNet(server, func_id, name, batch=batch, seed=func_id, level=level)
+    if name in ("densenet121", "densenet169", "densenet201"):
+        return densenet.DenseNet(server, func_id, name, batch=batch, seed=func_id, level=level)
+    if name == "inception":
+        return inception.InceptionV3(server, func_id, batch=batch, seed=func_id, level=level)
+    if name == "efficientnet":
+        return efficientnet.EfficientNetB0(server, func_id, batch=batch, seed=func_id, level=level)
+    if name == "mobilenet":
+        return mobilenet.MobileNetV2(server, func_id, batch=batch, seed=func_id, level=level)
+    if name in ("bert", "bert-base"):
+        return bert.Bert(server, func_id, "bert-base", batch=batch, seq=128, seed=func_id, level=level)
+    if name == "bertqa":
+        w = bert.init_weights("bert-large", seed=func_id, qa_head=True)
+        return bert.Bert(server, func_id, "bert-large", batch=batch, seq=512, weights=w, level=level, token_types=True)
+    raise ValueError(f"unknown model {name}")
+
+
+def ones_inputs(fn):
+    """The reference's endpoints feed all-ones inputs (tests/endpoint.py:53,66)."""
+    return [np.ones(shape, dtype=dt) for shape, dt in fn.input_specs()]
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="serve a synthetic request trace through the router on one GPU")
+    ap.add_argument("-m", default="resnet152", help="model name or 'mixed' (router.py:502)")
+    ap.add_argument("-f", type=int, default=1, help="number of functions")
+    ap.add_argument("-t", type=int, default=98, help="SLO percentile")
+    ap.add_argument("-d", type=int, default=100, help="latency deadline in ms (BERT question answering: twice that)")
+    ap.add_argument("-b", type=int, default=1, help="batch size limit")
+    ap.add_argument("-p", default="sa", choices=["sa", "fifo"])
+    ap.add_argument("--rate", type=float, default=0.0, help="requests per minute per function; 0: trace patterns")
+    ap.add_argument("--mins", type=int, default=1)
+    ap.add_argument("--patterns", default=None, help=".npy of requests per minute [functions x minutes]")
+    ap.add_argument("--speedup", type=float, default=1.0, help="divide every gap by this")
+    ap.add_argument("--mem-gb", type=float, default=24.0)
+    ap.add_argument("--seed", type=int, default=0)
+    a = ap.parse_args(argv)
+
+    from .server import Server
+    rng = np.random.default_rng(a.seed)
+    if a.rate > 0:
+        arrivals = fixed_rate_arrivals(a.f, a.rate, a.mins, rng)
+    else:
+        pat = np.load(a.patterns) if a.patterns else synthetic_rate_patterns(203, a.mins, rng)
+        arrivals = trace_arrivals(pat[:, :a.mins], a.f, rng)
+    arrivals = [(g / a.speedup, f) for g, f in arrivals]
+    limit = int(a.mem_gb * 2 ** 30)
+    with Server(mem_limit_bytes=limit, pool_bytes=limit + (2 << 30)) as server:
+        backend = FunctionBackend(server, lambda s, fid, lv: build_function(s, fid, lv, a.m, a.b), ones_inputs)
+        qa = {f for f in range(a.f) if a.m == "mixed" and mixed_model_name(f) == "bertqa"}
+        router = Router(backend, a.t / 100, a.d / 1000, a.b, a.p, deadlines={f: 2 * a.d / 1000 for f in qa},
+                        batch_limits={f: 1 for f in qa})
+        for f in range(a.f):
+            router.launch(f, mixed_model_level(f) if a.m == "mixed" else 1)
+        for f in range(a.f):
+            router.force_evict(f)
+        wall = serve_arrivals(router, arrivals)
+        out = router.summary()
+        out.update(wall_s=wall, offered=len(arrivals), model=a.m, functions=a.f, pool=server.pool_stats())
+        print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
