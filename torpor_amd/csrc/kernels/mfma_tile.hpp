@@ -202,20 +202,96 @@ __device__ __forceinline__ bool reduce_k_slices(f32x16 (&acc)[C::TM][C::TN], flo
     return true;
 }
 
+// Vector form of the accumulator write-out for the common case: row-major output with 16-byte
+// aligned rows, no beta term, whole 32-column blocks in range.  Each 32x32 block goes through the
+// wavefront's LDS staging block and comes back transposed to "four consecutive columns per
+// lane", so one step writes eight rows with 128-bit stores (4 steps per block instead of 16 with
+// 32-bit stores).  The loop body has no conditional load: a load under a branch makes the
+// compiler wait for every outstanding memory operation at the join, stores of the previous step
+// included, which serialised the old loop on the store round trip.  RES: add a residual tensor
+// (rows clamped for the load, the store is predicated).  RAW: split-K partial sums, no epilogue.
+template <class C, bool RES, bool RAW>
+__device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
+                                               long M, float* __restrict__ out, long pitch, const Epilogue& e,
+                                               float* __restrict__ stage) {
+    const int r = lane & 31;
+    const int h = lane >> 5;
+    const int cq = (lane & 7) * 4;  // this lane's four columns within the block
+    const int rq = lane >> 3;       // and its row within each group of eight
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+        const long col = n0 + wn * C::WTN + j * 32 + cq;
+        float cs[4] = {1.f, 1.f, 1.f, 1.f}, ct[4] = {0.f, 0.f, 0.f, 0.f};
+        if (!RAW) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) epilogue_column(e, col + c, cs[c], ct[c]);
+        }
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) stage[((v >> 2) * 8 + h * 4 + (v & 3)) * 32 + r] = acc[i][j][v];
+            wave_lds_sync();
+            const long row0 = m0 + wm * C::WTM + i * 32 + rq;
+#pragma unroll 1
+            for (int it = 0; it < 4; ++it) {
+                const long row = row0 + it * 8;
+                f32x4 x = *reinterpret_cast<const f32x4*>(stage + (it * 8 + rq) * 32 + cq);
+                f32x4 res;
+                if (RES) {
+                    const long rr = row < M ? row : M - 1;
+                    res = *reinterpret_cast<const f32x4*>(e.residual + rr * e.ldr + col);
+                }
+                if (!RAW) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float y = x[c] * e.alpha;
+                        y = y * cs[c] + ct[c];
+                        if (RES) y += res[c];
+                        x[c] = apply_act(y, e.act);
+                    }
+                }
+                if (row < M) *reinterpret_cast<f32x4*>(out + row * pitch + col) = x;
+            }
+            wave_lds_sync();
+        }
+    }
+}
+
+__device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 // Write the accumulators.  `partial` != nullptr: raw sums go to the split-K workspace slice
 // [M][N]; otherwise the epilogue is applied and C is written.
 //
 // Each 32x32 accumulator block first goes to `stage` (1024 floats of LDS private to this
 // wavefront; the caller guarantees that every wavefront has finished reading the operand
-// tiles), then a rolled 16-step loop writes two rows per step.  The rolled loop keeps one copy
-// of the epilogue in the program instead of one per accumulator register: the unrolled form
-// was tens of thousands of instructions, whose fetch alone cost up to a third of a GEMM.
+// tiles).  Wavefronts whose columns are all in range and whose output rows are 16-byte aligned
+// take store_tile_vec; the rest (NCHW outputs, a beta term, ragged right edge, odd pitches) a
+// rolled 16-step loop that writes two rows per step.  Rolled or short loops keep one copy of the
+// epilogue in the program instead of one per accumulator register: the unrolled form was tens of
+// thousands of instructions, whose fetch alone cost up to a third of a GEMM.
 template <class C>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
                                            long M, long N, float* __restrict__ Cout, const Epilogue& e,
                                            float* __restrict__ partial, float* __restrict__ stage) {
     const int r = lane & 31;
     const int h = lane >> 5;
+    if (n0 + (wn + 1) * C::WTN <= N) {  // the same for every lane of the wavefront
+        if (partial) {
+            if ((N & 3) == 0 && aligned16_dev(partial)) {
+                store_tile_vec<C, false, true>(acc, wm, wn, lane, m0, n0, M, partial, N, e, stage);
+                return;
+            }
+        } else if (!e.out_nchw && e.beta == 0.f && (e.ldc & 3) == 0 && aligned16_dev(Cout)) {
+            if (!e.residual) {
+                store_tile_vec<C, false, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage);
+                return;
+            }
+            if ((e.ldr & 3) == 0 && aligned16_dev(e.residual)) {
+                store_tile_vec<C, true, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage);
+                return;
+            }
+        }
+    }
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const long col = n0 + wn * C::WTN + j * 32 + r;
