@@ -575,7 +575,9 @@ void Engine::choose_copy_plan(Model& m) {
     if (compute_us <= 0) compute_us = est;
     const double bytes = (double)m.image_bytes;
     const double t1 = std::max(bytes / 54.0e3, compute_us + kernels * 1.2);
-    const double t2 = std::max(bytes / 56.5e3, compute_us + kernels * 2.4);
+    // (measured on ResNet-152 batch 8: kernels that share the device with two copy streams run
+    // about 15 % longer, on top of the per-launch cost)
+    const double t2 = std::max(bytes / 56.5e3, compute_us * 1.15 + kernels * 2.4);
     m.ncopy = (t2 <= t1) ? 2 : 1;
     if (copy_streams_cfg_ == 1 || copy_streams_cfg_ == 2) m.ncopy = copy_streams_cfg_;
     m.chunk_max = cfg_.chunk_max_bytes;
