@@ -616,7 +616,10 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, long* kper_out) {
     int splits = 1;
     const long kblocks = (K + bk - 1) / bk;
-    if (tiles < g_num_cu && kblocks >= 8) {
+    static const int forced = getenv("TORPOR_SPLITS") ? atoi(getenv("TORPOR_SPLITS")) : 0;
+    if (forced > 0 && kblocks >= 2L * forced && (size_t)forced * (size_t)M * (size_t)N * sizeof(float) <= ws_bytes) {
+        splits = forced;
+    } else if (tiles < g_num_cu && kblocks >= 8) {
         long want = (2L * g_num_cu + tiles - 1) / tiles;
         long maxs = kblocks / 4;  // keep at least 4 K-blocks per split
         if (want > maxs) want = maxs;
