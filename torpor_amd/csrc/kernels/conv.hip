@@ -55,14 +55,16 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
 // WGK > 1 (3 or 9 for 3x3: the nine k-groups of a K-block split evenly) lets extra wavefronts
 // share one output tile; with few output tiles this replaces a split over workgroups, whose
 // partial sums go through memory and a reduction launch.
-template <class C, int KH, int KW>
+//
+// STAGES = 2 keeps two K-blocks in LDS: the block fetched during the previous iteration is
+// written to the idle stage before the MFMAs of the current one are issued, so LDS writes and
+// matrix work overlap and an iteration has one barrier instead of two.
+template <class C, int KH, int KW, int STAGES = 2>
 __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_taps_kernel(const ConvDev p) {
     constexpr int T = KH * KW;
     static_assert(C::BK == 8 * T, "K-block = 8 channels x taps");
     static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
-    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, red_floats<C>() + stage_floats<C>())];
-    float* As = lds;
-    float* Bs = lds + C::BM * C::LDK;
+    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, red_floats<C>() + stage_floats<C>())];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
     const int wm = wsp / C::WGN, wn = wsp % C::WGN;
@@ -117,7 +119,9 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
             for (int j = 0; j < T; ++j) rw[j] = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * T + j * 4);
         }
     };
-    auto store_lds = [&]() {
+    auto store_lds = [&](int stage) {
+        float* As = lds + stage * C::LDS_FLOATS;
+        float* Bs = As + C::BM * C::LDK;
 #pragma unroll
         for (int i = 0; i < NVA; ++i) {
             const int idx = i * C::THREADS + tid;
@@ -140,12 +144,28 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     };
 
     load_regs(cbeg);
-    for (int c0 = cbeg; c0 < cend; c0 += 8) {
-        store_lds();
+    if (STAGES == 2) {
+        store_lds(0);
+        load_regs(cbeg + 8);
         __syncthreads();
-        load_regs(c0 + 8);
-        mma_block<C>(As, Bs, acc, wm, wn, lane, wk);
-        __syncthreads();
+        int cur = 0;
+        for (int c0 = cbeg; c0 < cend; c0 += 8) {
+            // the other stage was last read before the barrier that ended the previous iteration
+            store_lds(cur ^ 1);
+            load_regs(c0 + 16);
+            const float* As = lds + cur * C::LDS_FLOATS;
+            mma_block<C>(As, As + C::BM * C::LDK, acc, wm, wn, lane, wk);
+            __syncthreads();
+            cur ^= 1;
+        }
+    } else {
+        for (int c0 = cbeg; c0 < cend; c0 += 8) {
+            store_lds(0);
+            __syncthreads();
+            load_regs(c0 + 8);
+            mma_block<C>(lds, lds + C::BM * C::LDK, acc, wm, wn, lane, wk);
+            __syncthreads();
+        }
     }
     if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
@@ -453,11 +473,15 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
         switch (cfg) {
             case 0:
-                hipLaunchKernelGGL((conv_taps_kernel<Conv3L, 3, 3>), grid, dim3(Conv3L::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3L, 3, 3, 1>), grid, dim3(Conv3L::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_128x128");
                 break;
             case 1:
-                hipLaunchKernelGGL((conv_taps_kernel<Conv3M, 3, 3>), grid, dim3(Conv3M::THREADS), 0, s, p);
+                // two LDS stages halve the workgroups a CU can hold: only when all of them still fit at once
+                if (tiles * p.splits <= 2L * num_cu())
+                    hipLaunchKernelGGL((conv_taps_kernel<Conv3M, 3, 3, 2>), grid, dim3(Conv3M::THREADS), 0, s, p);
+                else
+                    hipLaunchKernelGGL((conv_taps_kernel<Conv3M, 3, 3, 1>), grid, dim3(Conv3M::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_64x64");
                 break;
             case 2:
@@ -465,11 +489,11 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
                 set_last_kernel("conv3x3_fast_64x64_k3");
                 break;
             case 3:
-                hipLaunchKernelGGL((conv_taps_kernel<Conv3T, 3, 3>), grid, dim3(Conv3T::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3T, 3, 3, 1>), grid, dim3(Conv3T::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_32x32_k9");
                 break;
             default:
-                hipLaunchKernelGGL((conv_taps_kernel<Conv3U, 3, 3>), grid, dim3(Conv3U::THREADS), 0, s, p);
+                hipLaunchKernelGGL((conv_taps_kernel<Conv3U, 3, 3, 1>), grid, dim3(Conv3U::THREADS), 0, s, p);
                 set_last_kernel("conv3x3_fast_32x32_k3");
                 break;
         }
