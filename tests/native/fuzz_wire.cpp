@@ -151,6 +151,53 @@ int main() {
         }
     }
     tp_lru_destroy(lru);
+
+    // the multi-GPU policy objects: random traces with out-of-range GPUs and unknown names mixed in
+    for (int policy = 0; policy < 2; ++policy) {
+        tp_evictor* ev = tp_evictor_create(policy, 4, 1000);
+        if (!ev) return 4;
+        for (int it = 0; it < 20000; ++it) {
+            char name[8];
+            std::snprintf(name, sizeof name, "%d", (int)(rng() % 24));
+            const int gpu = (int)(rng() % 6) - 1;   // -1 and 4 are invalid
+            int32_t nv = 0, over = 0;
+            switch (rng() % 8) {
+                case 0: case 1: case 2:
+                    (void)tp_evictor_check_and_add(ev, gpu, name, 1 + rng() % 400, victims, sizeof victims, &nv, &over);
+                    break;
+                case 3: (void)tp_evictor_lock(ev, gpu, name); break;
+                case 4: (void)tp_evictor_unlock(ev, gpu, name); break;
+                case 5: (void)tp_evictor_force_evict(ev, gpu, name); break;
+                case 6: (void)tp_evictor_set_level(ev, name, (int32_t)(rng() % 5) - 1); break;
+                default: (void)tp_evictor_order(ev, gpu, victims, 1 + rng() % sizeof victims); (void)tp_evictor_is_protected(ev, gpu, name); break;
+            }
+            uint64_t sum = 0;
+            for (int g = 0; g < 4; ++g) sum += tp_evictor_used(ev, g);
+            if (sum > 4ull * 24 * 400) return 5;
+        }
+        tp_evictor_destroy(ev);
+    }
+    tp_sched* sc = tp_sched_create(8);
+    if (!sc) return 6;
+    for (int it = 0; it < 20000; ++it) {
+        char name[8];
+        std::snprintf(name, sizeof name, "%d", (int)(rng() % 12));
+        const int gpu = (int)(rng() % 10) - 1;
+        int32_t d = 0, sr = 0, st = 0;
+        switch (rng() % 7) {
+            case 0: (void)tp_sched_set_status(sc, gpu, (int32_t)(rng() % 9) - 2); break;
+            case 1: (void)tp_sched_set_resident(sc, name, gpu, (int32_t)(rng() % 2)); break;
+            case 2: (void)tp_sched_set_level(sc, name, (int32_t)(rng() % 5) - 1); break;
+            case 3: (void)tp_sched_set_sibling(sc, gpu, (int32_t)(rng() % 10) - 1); break;
+            case 4: (void)tp_sched_set_link(sc, gpu, (int32_t)(rng() % 10) - 1, (int32_t)(rng() % 6) - 2); break;
+            case 5: { const int g = tp_sched_placement(sc); if (g < -1 || g > 7) return 7; break; }
+            default:
+                if (tp_sched_decide(sc, (int32_t)(rng() % 2), name, (uint32_t)rng(), &d, &sr, &st) != 0) return 8;
+                if (d < -1 || d > 7 || sr < -1 || sr > 7) return 9;
+                break;
+        }
+    }
+    tp_sched_destroy(sc);
     std::printf("fuzz ok: %ld messages\n", handled);
     return 0;
 }
