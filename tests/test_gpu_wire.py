@@ -13,7 +13,7 @@ import torch
 from oracle import models as om
 from tests.harness import assert_close
 from torpor_amd import client as wire
-from torpor_amd.functions import bert, resnet
+from torpor_amd.functions import bert, mobilenet, resnet
 from torpor_amd.server import ACK_OK, Server
 
 pytestmark = pytest.mark.gpu
@@ -96,3 +96,32 @@ def test_densenet_and_mobilenet_over_the_wire(gpu_wire_server):
             (cold,) = fn.invoke([x])
             assert np.array_equal(cold, first)
             assert fn.unload()[0] == ACK_OK
+
+
+def test_router_over_the_wire(gpu_wire_server):
+    """The router with one wire connection per function (the reference's function containers are
+    separate clients of the server): FIFO trace, answers equal to the registration run."""
+    from torpor_amd import router as R
+
+    def factory(conn, fid, level):
+        if fid % 2:
+            return mobilenet.MobileNetV2(conn, fid, batch=1, seed=fid, level=level, image=64)
+        return resnet.ResNet(conn, fid, "resnet50", batch=1, seed=fid, level=level, image=64)
+
+    be = R.FunctionBackend(lambda fid: wire.RemoteServer(gpu_wire_server, client_id=fid), factory, R.ones_inputs)
+    r = R.Router(be, slo_percentile=0.9, deadline_s=0.1, batch_limit=1, policy="fifo")
+    try:
+        for f in (20, 21, 22):
+            r.launch(f, level=1)
+        for f in (20, 21, 22):
+            r.force_evict(f)
+        arrivals = [(0.002, 20 + (i * 7) % 3) for i in range(90)]
+        R.serve_arrivals(r, arrivals)
+        out = r.summary()
+        assert out["requests"] == 90 and out["queued"] == 0
+        for f in (20, 21, 22):
+            for a, b in zip(be.first[f], be.outputs(f)):
+                assert np.array_equal(a, b), f"function {f} changed its answer over the wire"
+            r.force_evict(f)
+    finally:
+        be.close()

@@ -397,12 +397,18 @@ class FunctionBackend:
     at the router's batch limit and a smaller batch runs with the remaining rows left as they were."""
 
     def __init__(self, server, factory, example_inputs):
-        self.server, self.factory, self.example_inputs = server, factory, example_inputs
+        # `server`: one in-process Server for every function, or a callable func_id -> connection
+        # (each function container of the reference is a client of its own: RemoteServer(dir, client_id))
+        self._owned = callable(server)
+        self.server_for = server if callable(server) else (lambda func_id: server)
+        self.factory, self.example_inputs = factory, example_inputs
         self.fn = {}
+        self.conn = {}
         self.first = {}                 # answers of the registration run
 
     def launch(self, func_id, level):
-        fn = self.factory(self.server, func_id, level)
+        self.conn[func_id] = self.server_for(func_id)
+        fn = self.factory(self.conn[func_id], func_id, level)
         inputs = self.example_inputs(fn)
         first = fn.register(inputs)
         fn._weights = None              # the server's pinned store holds the authoritative copy now
@@ -417,16 +423,23 @@ class FunctionBackend:
 
     def execute(self, func_id, n):
         fn, packed, outbuf, _ = self.fn[func_id]
-        ack, _, deferred = self.server.signal(1, func_id, "")
+        ack, _, deferred = self.conn[func_id].signal(1, func_id, "")
         if ack != 0 or deferred:
             raise RuntimeError(f"execute {func_id}: ack={ack} deferred={deferred}")
-        self.server.replay(func_id, packed, outbuf)
+        self.conn[func_id].replay(func_id, packed, outbuf)
 
     def unload(self, func_id):
-        self.server.signal(3, func_id, "")
+        self.conn[func_id].signal(3, func_id, "")
 
     def load(self, func_id):
-        self.server.signal(2, func_id, "")
+        self.conn[func_id].signal(2, func_id, "")
+
+    def close(self):
+        """Closes the per-function connections this backend opened (nothing for a shared server)."""
+        if self._owned:
+            for c in self.conn.values():
+                c.close()
+        self.conn.clear()
 
 
 def build_function(server, func_id, level, model, batch):
@@ -469,6 +482,9 @@ def main(argv=None):
     ap.add_argument("--patterns", default=None, help=".npy of requests per minute [functions x minutes]")
     ap.add_argument("--speedup", type=float, default=1.0, help="divide every gap by this")
     ap.add_argument("--mem-gb", type=float, default=24.0)
+    ap.add_argument("--connect", default=None, metavar="DIR",
+                    help="serve through a running torpor_server whose sockets are in DIR (one connection per function) "
+                         "instead of an in-process server")
     ap.add_argument("--seed", type=int, default=0)
     a = ap.parse_args(argv)
 
@@ -480,10 +496,10 @@ def main(argv=None):
         pat = np.load(a.patterns) if a.patterns else synthetic_rate_patterns(203, a.mins, rng)
         arrivals = trace_arrivals(pat[:, :a.mins], a.f, rng)
     arrivals = [(g / a.speedup, f) for g, f in arrivals]
-    limit = int(a.mem_gb * 2 ** 30)
-    with Server(mem_limit_bytes=limit, pool_bytes=limit + (2 << 30)) as server:
-        backend = FunctionBackend(server, lambda s, fid, lv: build_function(s, fid, lv, a.m, a.b), ones_inputs)
-        qa = {f for f in range(a.f) if a.m == "mixed" and mixed_model_name(f) == "bertqa"}
+    qa = {f for f in range(a.f) if a.m == "mixed" and mixed_model_name(f) == "bertqa"}
+
+    def serve(server_or_factory, stats):
+        backend = FunctionBackend(server_or_factory, lambda s, fid, lv: build_function(s, fid, lv, a.m, a.b), ones_inputs)
         router = Router(backend, a.t / 100, a.d / 1000, a.b, a.p, deadlines={f: 2 * a.d / 1000 for f in qa},
                         batch_limits={f: 1 for f in qa})
         for f in range(a.f):
@@ -492,8 +508,17 @@ def main(argv=None):
             router.force_evict(f)
         wall = serve_arrivals(router, arrivals)
         out = router.summary()
-        out.update(wall_s=wall, offered=len(arrivals), model=a.m, functions=a.f, pool=server.pool_stats())
+        out.update(wall_s=wall, offered=len(arrivals), model=a.m, functions=a.f, **stats())
+        backend.close()
         print(json.dumps(out))
+
+    if a.connect:
+        from .client import RemoteServer
+        serve(lambda fid: RemoteServer(a.connect, client_id=fid), lambda: {"transport": "wire"})
+    else:
+        limit = int(a.mem_gb * 2 ** 30)
+        with Server(mem_limit_bytes=limit, pool_bytes=limit + (2 << 30)) as server:
+            serve(server, lambda: {"transport": "in-process", "pool": server.pool_stats()})
 
 
 if __name__ == "__main__":
