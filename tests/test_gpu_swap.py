@@ -73,3 +73,27 @@ def test_gate_orders_compute_after_copy():
             assert s.swap_stats(0)["gate_waits"] > 50
             (gb,) = b.invoke([xb])
             assert np.array_equal(gb, yb)
+
+
+def test_graph_replays_match_eager_and_follow_the_placement(monkeypatch):
+    """TORPOR_GRAPH_MIN_OPS: warm requests launch the compute part of the program as one HIP graph.
+    Every replay of the graph must equal the eager answer, with other models' eager work and
+    synchronisations in between, and a swap-out / swap-in (new addresses) must re-capture."""
+    monkeypatch.setenv("TORPOR_GRAPH_MIN_OPS", "8")
+    with Server(mem_limit_bytes=300 << 20, pool_bytes=512 << 20) as s:
+        fa, xa, ya = _mk(s, 0, seed=3)
+        fb, xb, yb = _mk(s, 1, seed=4)
+        for rnd in range(3):
+            for i in range(5):                      # the second warm request captures, the rest replay
+                (got,) = fa.invoke([xa])
+                assert np.array_equal(got, ya), (rnd, i)
+                (gb,) = fb.invoke([xb], replay=False)    # eager, op by op, between the replays
+                assert np.array_equal(gb, yb)
+            x2 = xa + 1.0                            # new inputs through the same graph
+            (g2,) = fa.invoke([x2])
+            (e2,) = fa.invoke([x2], replay=False)
+            assert np.array_equal(g2, e2) and not np.array_equal(g2, ya)
+            assert fa.unload()[0] == ACK_OK          # placement is dropped ...
+            _mk(s, 2 + rnd, seed=5 + rnd)            # ... and the pool re-used, so it comes back elsewhere or not
+            (cold,) = fa.invoke([xa])
+            assert np.array_equal(cold, ya)

@@ -68,6 +68,7 @@ int Engine::init() {
     HIPCHK(hipStreamCreateWithFlags(&copy_, hipStreamNonBlocking));
     HIPCHK(hipStreamCreateWithFlags(&copy2_, hipStreamNonBlocking));
     copy_streams_cfg_ = (int)env_u64("TORPOR_COPY_STREAMS", (uint64_t)cfg_.copy_streams);  // 0 = per model
+    graph_min_ops_ = (int)env_u64("TORPOR_GRAPH_MIN_OPS", 0);
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&h2d_stage_), 16ull << 20, hipHostMallocDefault));
     h2d_cap_ = 16ull << 20;
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&d2h_stage_), 8ull << 20, hipHostMallocDefault));
@@ -94,6 +95,7 @@ Engine::~Engine() {
             for (auto ev : m.chunk_ev) (void)hipEventDestroy(ev);
             if (m.t0) (void)hipEventDestroy(m.t0);
             if (m.t1) (void)hipEventDestroy(m.t1);
+            drop_graph(m);
         }
     }
     if (!host_only()) {
@@ -751,6 +753,7 @@ int Engine::swap_in(Model& m) {
     }
     m.w_dev = arena_ + m.w_pool_off;
     m.a_dev = arena_ + m.a_pool_off;
+    drop_graph(m);  // the captured launches hold the old addresses
     build_chunks(m);  // the plan follows the latest forward-time figure
     m.resident = true;
     m.fully_loaded = false;
@@ -786,6 +789,7 @@ void Engine::evict_model(Model& m) {
     if (m.a_pool_off != UINT64_MAX) pool_.release(m.a_pool_off);
     m.w_pool_off = m.a_pool_off = UINT64_MAX;
     m.w_dev = m.a_dev = nullptr;
+    drop_graph(m);
     m.resident = false;
     m.fully_loaded = false;
     m.copy_state.store(CS_IDLE);
@@ -818,6 +822,7 @@ void Engine::start_cold(int id, int level) {
             for (auto ev : old->chunk_ev) (void)hipEventDestroy(ev);
             if (old->t0) (void)hipEventDestroy(old->t0);
             if (old->t1) (void)hipEventDestroy(old->t1);
+            drop_graph(*old);
         }
         models_.erase(id);
     }
@@ -1491,6 +1496,65 @@ int Engine::op_compute(int client, const Op& op) {
     return 0;
 }
 
+void Engine::drop_graph(Model& m) {
+    if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
+    m.graph_exec = nullptr;
+    m.graph_begin = m.graph_end = -1;
+    m.graph_state = 0;
+    m.warm_streak = 0;
+}
+
+// Captures the longest run of compute ops of the recorded program on the compute stream.  The
+// model is fully loaded (no gate waits), the run holds no copy from or to the host and no memset
+// (memset nodes are kept out of graphs on purpose), and capture is thread-local: the copy thread
+// may be issuing another model's transfers meanwhile.
+int Engine::build_graph(Model& m) {
+    auto graphable = [](const Op& op) {
+        return op.kind == OPK_GEMM || op.kind == OPK_CONV || op.kind == OPK_BN || op.kind == OPK_LAUNCH || op.kind == OPK_D2D;
+    };
+    int best_b = -1, best_e = -1;
+    const int n = (int)m.program.size();
+    for (int i = 0; i < n;) {
+        if (!graphable(m.program[(size_t)i])) {
+            ++i;
+            continue;
+        }
+        int j = i;
+        while (j < n && graphable(m.program[(size_t)j])) ++j;
+        if (j - i > best_e - best_b) best_b = i, best_e = j;
+        i = j;
+    }
+    m.graph_state = -1;
+    if (best_b < 0 || best_e - best_b < graph_min_ops_) return 0;
+    if (hipStreamBeginCapture(compute_, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int r = 0;
+    for (int i = best_b; i < best_e && !r; ++i) r = exec_op(m, m.program[(size_t)i], nullptr, true);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(compute_, &g);
+    if (r || e != hipSuccess || !g) {
+        if (std::getenv("TORPOR_GRAPH_DEBUG")) std::fprintf(stderr, "graph: capture failed r=%d e=%d\n", r, (int)e);
+        if (g) (void)hipGraphDestroy(g);
+        (void)hipGetLastError();
+        return r ? r : (int)e;
+    }
+    hipGraphExec_t ge = nullptr;
+    e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess || !ge) {
+        (void)hipGetLastError();
+        return (int)e;
+    }
+    m.graph_exec = ge;
+    m.graph_begin = best_b;
+    m.graph_end = best_e;
+    m.graph_state = 1;
+    if (std::getenv("TORPOR_GRAPH_DEBUG")) std::fprintf(stderr, "graph: model %d ops [%d, %d)\n", m.id, best_b, best_e);
+    return 0;
+}
+
 int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uint64_t out_bytes) {
     std::lock_guard<std::mutex> lk(mu_);
     int err = 0;
@@ -1507,7 +1571,25 @@ int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uin
     rc.out_bytes = out_bytes;
     int ret = 0;
     bool completed = false;
-    for (const Op& op : m->program) {
+    // Warm requests at an unchanged placement launch the compute part of the program as one HIP
+    // graph (captured on the second such request); everything else goes op by op.
+    bool graphed = false;
+    if (warm && graph_min_ops_ > 0 && !profiling_ && !host_only()) {
+        if (m->graph_state == 0 && ++m->warm_streak >= 2) (void)build_graph(*m);
+        graphed = m->graph_state == 1;
+    }
+    const int n_ops = (int)m->program.size();
+    for (int i = 0; i < n_ops; ++i) {
+        if (graphed && i == m->graph_begin) {
+            hipError_t e = hipGraphLaunch(m->graph_exec, compute_);
+            if (e != hipSuccess) {
+                ret = (int)e;
+                break;
+            }
+            i = m->graph_end - 1;
+            continue;
+        }
+        const Op& op = m->program[(size_t)i];
         int r = exec_op(*m, op, &rc, true);
         if (r && !ret) ret = r;
         if (r) break;

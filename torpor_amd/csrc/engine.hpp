@@ -104,6 +104,11 @@ struct Model {
     int ncopy = 2;            // copy streams used by the current swap-in plan
     uint64_t chunk_max = 0;   // largest transfer group of the current plan
     double warm_us = 0;       // best warm replay so far (host wall clock), 0 = none yet
+    // captured compute segment of the recorded program (warm replays at an unchanged placement)
+    hipGraphExec_t graph_exec = nullptr;
+    int graph_begin = -1, graph_end = -1;  // program[graph_begin, graph_end) is what the graph launches
+    int graph_state = 0;                   // 0 none yet, 1 ready, -1 not usable for this model
+    int warm_streak = 0;                   // warm replays since the placement last changed
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing_valid = false;
     // recorded program
@@ -202,6 +207,8 @@ private:
     int build_image(Model& m, bool by_access);
     void build_chunks(Model& m);
     void choose_copy_plan(Model& m);
+    void drop_graph(Model& m);
+    int build_graph(Model& m);
     void wait_copy_idle(Model& m);
     void copy_main();
     int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
@@ -237,6 +244,7 @@ private:
     hipStream_t compute_ = nullptr, copy_ = nullptr, copy2_ = nullptr;
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
+    int graph_min_ops_ = 0;  // 0: warm replays launch op by op; n: capture compute runs of at least n ops
     std::unordered_map<int, std::unique_ptr<Model>> models_;
 
     int active_ = -1;
