@@ -152,6 +152,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         cold_ms_p50=pctl(cold, 0.5), cold_ms_p99=pctl(cold, 0.99), cold_ms_min=min(cold),
         warm_ms_p50=pctl(warm, 0.5), warm_ms_min=min(warm),
         cold_over_warm=pctl(cold, 0.5) / pctl(warm, 0.5),
+        exposed_swap_ms=pctl(cold, 0.5) - pctl(warm, 0.5),   # the part of the swap-in that compute did not hide
         weight_bytes=info["image_bytes"], act_bytes=info["act_bytes"], ops=info["n_ops"], chunks=info["n_chunks"],
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
