@@ -72,8 +72,12 @@ def serve(server, fleet, seconds, rate, seed, check_every=500):
     st0 = server.pool_stats()
     lat_hit, lat_miss, by_arch, swap_bytes, swap_ms = [], [], {}, 0, 0.0
     t0 = time.perf_counter()
+    next_note = 30.0
     for i in range(n_req):
         now = time.perf_counter() - t0
+        if now >= next_note:        # a line every half minute, so that a long run is seen to be alive
+            print(f"[{now:6.0f} s] {i} of {n_req} requests served", file=sys.stderr, flush=True)
+            next_note += 30.0
         if now < arrivals[i]:
             while time.perf_counter() - t0 < arrivals[i]:
                 pass
