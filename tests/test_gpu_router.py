@@ -16,6 +16,45 @@ def _factory(server, fid, level):
     return resnet.ResNet(server, fid, "resnet50", batch=2, seed=fid, level=level, image=64)
 
 
+def _same_rows(first, got, f):
+    """Full batches replay the recorded stream (same bits); a smaller batch runs other tile shapes,
+    so its rows agree with the registered run to rounding (inputs are all ones: every row is alike)."""
+    if got.shape == first.shape:
+        assert np.array_equal(first, got), f"function {f} changed its answer"
+    else:
+        ref = first[:got.shape[0]]
+        assert np.abs(got - ref).max() <= 1e-4 * max(np.abs(ref).max(), 1e-6), f"function {f}: rows differ"
+
+
+def test_fewer_rows_than_the_registered_batch():
+    """`invoke_rows` runs a request at its own batch size inside the buffers of the registered one:
+    same bits as a function registered at that size, and the oracle's answer."""
+    import torch
+    from oracle import models as om
+    from tests.harness import assert_close
+    w = resnet.init_weights("resnet50", seed=11)
+    x = np.random.default_rng(11).standard_normal((4, 3, 64, 64)).astype(np.float32)
+    model = om.load_numpy_state(om.ResNet("resnet50"), w)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
+        big = resnet.ResNet(s, 0, "resnet50", batch=4, weights=w, image=64)
+        (y4,) = big.register([x])
+        assert_close(y4, want, 1e-3, "batch 4")
+        for rows in (1, 2, 3):
+            small = resnet.ResNet(s, rows, "resnet50", batch=rows, weights=w, image=64)
+            (ys,) = small.register([x[:rows]])
+            (got,) = big.invoke_rows([x[:rows]], rows)
+            assert got.shape == (rows, 1000) and np.array_equal(got, ys), rows
+            assert_close(got, want[:rows], 1e-3, f"{rows} rows")
+        (again,) = big.invoke([x])                         # the recorded stream is untouched
+        assert np.array_equal(again, y4)
+        (cold,) = (big.unload(), big.invoke_rows([x[1:3]], 2))[1]   # also from the swapped-out state
+        assert_close(cold, want[1:3], 1e-3, "rows 1..2 cold")
+        with pytest.raises(ValueError):
+            big.invoke_rows([x], 5)
+
+
 @pytest.mark.parametrize("policy", ["sa", "fifo"])
 def test_router_serves_a_fleet_under_memory_pressure(policy):
     with Server(mem_limit_bytes=260 << 20, pool_bytes=512 << 20) as s:
@@ -34,10 +73,15 @@ def test_router_serves_a_fleet_under_memory_pressure(policy):
         assert out["requests"] == 600 and out["queued"] == 0 and wall < 60
         st1 = s.pool_stats()
         assert st1["swap_ins"] - st0["swap_ins"] >= 6 and st1["evictions"] > st0["evictions"]   # 3 ResNets exceed the budget
+        assert set(out["batches"]) <= {1, 2}
         for f in range(6):
             for a, b in zip(be.first[f], be.outputs(f)):      # the last request served during the trace
-                assert np.array_equal(a, b), f"function {f} changed its answer"
-            be.execute(f, 1)
+                _same_rows(a, b, f)
+            be.execute(f, 2)                                  # full batch: the recorded op stream, same bits
             for a, b in zip(be.first[f], be.outputs(f)):
                 assert np.array_equal(a, b), f"function {f} changed its answer"
+            be.execute(f, 1)                                  # one request: issued op by op at batch 1
+            for a, b in zip(be.first[f], be.outputs(f)):
+                assert b.shape[0] == 1
+                _same_rows(a, b, f)
         assert sum(k * v for k, v in out["batches"].items()) == 600

@@ -393,8 +393,9 @@ class FunctionBackend:
     """Functions of `torpor_amd.functions` behind a server (in-process `Server` or wire `Client`).
 
     The reference's function container runs the model at batch = number of batched requests
-    (tests/endpoint.py:84-92).  Op streams here are recorded per shape, so a function is registered
-    at the router's batch limit and a smaller batch runs with the remaining rows left as they were."""
+    (tests/endpoint.py:84-92).  A function is registered at the router's batch limit; a full batch
+    replays the recorded op stream in one call, a smaller one is issued op by op at its own size
+    (`Function.invoke_rows`)."""
 
     def __init__(self, server, factory, example_inputs):
         # `server`: one in-process Server for every function, or a callable func_id -> connection
@@ -405,6 +406,8 @@ class FunctionBackend:
         self.fn = {}
         self.conn = {}
         self.first = {}                 # answers of the registration run
+        self.inputs = {}
+        self.last = {}                  # answers of the last request when it ran below the registered batch
 
     def launch(self, func_id, level):
         self.conn[func_id] = self.server_for(func_id)
@@ -414,19 +417,28 @@ class FunctionBackend:
         fn._weights = None              # the server's pinned store holds the authoritative copy now
         packed, outbuf, views = fn.pack(inputs)
         self.fn[func_id] = (fn, packed, outbuf, views)
+        self.inputs[func_id] = inputs
         self.first[func_id] = [np.array(a, copy=True) for a in first]
+        self.last[func_id] = None
 
     def outputs(self, func_id):
         """Answers of the last request of the function."""
+        if self.last[func_id] is not None:
+            return self.last[func_id]
         fn, _, _, views = self.fn[func_id]
         return fn.postprocess(views)
 
     def execute(self, func_id, n):
         fn, packed, outbuf, _ = self.fn[func_id]
+        batch = getattr(fn, "batch", n)
+        if 0 < n < batch:               # fewer requests than the registered batch: run at that size
+            self.last[func_id] = fn.invoke_rows([a[:n] for a in self.inputs[func_id]], n)
+            return
         ack, _, deferred = self.conn[func_id].signal(1, func_id, "")
         if ack != 0 or deferred:
             raise RuntimeError(f"execute {func_id}: ack={ack} deferred={deferred}")
         self.conn[func_id].replay(func_id, packed, outbuf)
+        self.last[func_id] = None
 
     def unload(self, func_id):
         self.conn[func_id].signal(3, func_id, "")
