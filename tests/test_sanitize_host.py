@@ -34,8 +34,9 @@ def test_wire_handlers_and_engine_under_sanitizers(tmp_path):
     subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", os.path.join(ROOT, "tests", "native", "fuzz_wire.cpp"),
                                              "-o", drv], stderr=subprocess.DEVNULL)
     exe = str(tmp_path / "fuzz_wire")
-    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-o", exe, drv]
-                          + objs + ["-lpthread"], stderr=subprocess.DEVNULL)
+    # link step: the sanitizer runtimes for the host objects only (device code is never instrumented)
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950"] + san + ["-o", exe, drv] + objs + ["-lpthread"],
+                          stderr=subprocess.DEVNULL)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TORPOR_IPC_DIR=str(tmp_path))
     r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "fuzz ok" in r.stdout, (r.stdout[-2000:], r.stderr[-4000:])
