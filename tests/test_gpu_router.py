@@ -55,6 +55,30 @@ def test_fewer_rows_than_the_registered_batch():
             big.invoke_rows([x], 5)
 
 
+def test_fewer_rows_bert_and_mobilenet():
+    """The same for a transformer (rows = sequences) and a depthwise network."""
+    from torpor_amd.functions import bert
+    cfg = dict(layers=2, hidden=128, heads=2, ffn=256)
+    wb = bert.init_weights(seed=3, vocab=400, max_pos=64, cfg=cfg)
+    ids = np.random.default_rng(3).integers(0, 400, (4, 48))
+    wm = mobilenet.init_weights(seed=6)
+    xm = np.random.default_rng(6).standard_normal((3, 3, 64, 64)).astype(np.float32)
+    with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
+        big = bert.Bert(s, 0, batch=4, seq=48, weights=wb, cfg=cfg)
+        big.register([ids])
+        for rows in (1, 3):
+            small = bert.Bert(s, 10 + rows, batch=rows, seq=48, weights=wb, cfg=cfg)
+            want = small.register([ids[:rows]])
+            got = big.invoke_rows([ids[:rows]], rows)
+            assert all(np.array_equal(a, b) for a, b in zip(got, want)), rows
+        mb = mobilenet.MobileNetV2(s, 1, batch=3, weights=wm, image=64)
+        mb.register([xm])
+        small = mobilenet.MobileNetV2(s, 21, batch=2, weights=wm, image=64)
+        (want,) = small.register([xm[:2]])
+        (got,) = mb.invoke_rows([xm[:2]], 2)
+        assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("policy", ["sa", "fifo"])
 def test_router_serves_a_fleet_under_memory_pressure(policy):
     with Server(mem_limit_bytes=260 << 20, pool_bytes=512 << 20) as s:
