@@ -341,7 +341,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             store_lds(ra1, rb1, 1);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);
+            if (k0 + C::BK < kend) mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);  // odd block count
             store_lds(ra0, rb0, 0);
             __syncthreads();
         }
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             store_lds(ra1, rb1, 0);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
+            if (k0 + C::BK < kend) mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);  // odd block count
             __syncthreads();
         }
     }
@@ -688,7 +688,9 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         if (batch == 1 && cfg < 3) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
         dim3 grid(plan_xcd_grid(p, a.M, a.N), 1, p.splits > 1 ? p.splits : batch);
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
-        const bool clean = allow_clean && a.K >= 64 && a.K % 64 == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
+        // whole K-blocks; the 32-wide tiles take them in pairs, an odd last one is handled in the loop
+        const long kq = cfg >= 3 ? 64 : 32;
+        const bool clean = allow_clean && a.K >= kq && a.K % kq == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
