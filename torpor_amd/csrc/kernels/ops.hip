@@ -423,9 +423,48 @@ __global__ __launch_bounds__(256) void avgpool_final_kernel(const float* __restr
         y[i] = acc * inv;
     }
 }
+// NHWC maps of 16 to 256 pixels in one launch: a workgroup takes 64 channels of one image as 16 lanes of
+// four channels (128-bit loads) x 16 pixel phases, so a thread's chain of loads is HW / 16 long, and adds the
+// phases through LDS in a fixed order.
+__global__ __launch_bounds__(256) void avgpool_small_kernel(const float* __restrict__ x, float* __restrict__ y, int HW,
+                                                            int C, float inv) {
+    __shared__ float red[16][64];
+    const int cq = threadIdx.x & 15, ph = threadIdx.x >> 4;
+    const int c = blockIdx.x * 64 + cq * 4, n = blockIdx.y;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    if (c < C) {  // C % 4 == 0: the four channels are in range together
+        const float* px = x + (long)n * HW * C + c;
+        for (int q = ph; q < HW; q += 16) {
+            const float4 v = *reinterpret_cast<const float4*>(px + (long)q * C);
+            a0 += v.x;
+            a1 += v.y;
+            a2 += v.z;
+            a3 += v.w;
+        }
+    }
+    red[ph][cq * 4 + 0] = a0;
+    red[ph][cq * 4 + 1] = a1;
+    red[ph][cq * 4 + 2] = a2;
+    red[ph][cq * 4 + 3] = a3;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int cc = blockIdx.x * 64 + threadIdx.x;
+        if (cc < C) {
+            float acc = 0.f;
+#pragma unroll
+            for (int p = 0; p < 16; ++p) acc += red[p][threadIdx.x];
+            y[(long)n * C + cc] = acc * inv;
+        }
+    }
+}
 int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nhwc, const Workspace& ws,
                           hipStream_t s) {
     if (!x || !y || N <= 0 || HW <= 0 || C <= 0) return K_EINVAL;
+    if (nhwc && HW >= 16 && HW <= 256 && N <= 65535 && (C & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        hipLaunchKernelGGL(avgpool_small_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)N), dim3(256), 0, s, x, y, HW, C,
+                           1.0f / (float)HW);
+        return (int)hipGetLastError();
+    }
     if (nhwc && HW >= 16 && ws.ptr) {
         int S = HW >= 512 ? (HW + 63) / 64 : (HW + 7) / 8;
         if (S > 64) S = 64;
