@@ -136,7 +136,8 @@ def test_conv_tap_shapes(gpu_server, kh, kw, stride, Cin, Cout, H, W):
     assert_close(fused, z, 5e-5, f"conv {kh}x{kw} + bn + relu")
 
 
-@pytest.mark.parametrize("C,k,stride,HW", [(32, 3, 1, 14), (24, 3, 2, 15), (16, 5, 2, 9), (8, 3, 1, 5)])
+@pytest.mark.parametrize("C,k,stride,HW", [(32, 3, 1, 14), (24, 3, 2, 15), (16, 5, 2, 9), (8, 3, 1, 5), (12, 7, 1, 9),
+                                           (40, 5, 1, 6)])
 def test_depthwise(gpu_server, C, k, stride, HW):
     """groups == channels (MobileNet-style), with the fused batch-norm + relu6 epilogue."""
     from torpor_amd.server import ACT_RELU6
@@ -151,7 +152,8 @@ def test_depthwise(gpu_server, C, k, stride, HW):
         xv = t.act(x)
         yv = t.empty(N * Ho * Ho * C * 4)
         t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=C)
-        assert t.s.last_kernel() == "depthwise_nhwc"
+        # 3x3 / 5x5 run the branch-free vector kernel, other sizes the general one
+        assert t.s.last_kernel() == {3: "depthwise_3x3", 5: "depthwise_5x5"}.get(k, "depthwise_nhwc")
         plain = t.read(yv, (N, Ho, Ho, C))
         t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=C,
                  bn=tuple(t.w[1:5]), bn_eps=1e-5, act=ACT_RELU6)

@@ -304,6 +304,67 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const DwDev p) {
     }
 }
 
+// The same for fixed K x K taps (3x3, 5x5), weights 16-byte aligned, row-major output with aligned
+// rows and no beta term: the 4*K*K weights of the channel quad are fetched up front as vectors,
+// every tap's load is unconditional (out-of-range taps read a clamped address and are zeroed by
+// a select), so all K*K loads of a thread are in flight together, and the result leaves as one
+// 128-bit store.
+template <int KS>
+__global__ __launch_bounds__(256) void depthwise_taps_kernel(const DwDev p) {
+    constexpr int T = KS * KS;
+    const long st = (long)gridDim.x * blockDim.x;
+    const int C4 = p.C >> 2;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total; i += st) {
+        const int c = (int)(i % C4) * 4;
+        long t = i / C4;
+        const long row = t;
+        const int wo = (int)(t % p.Wo);
+        t /= p.Wo;
+        const int ho = (int)(t % p.Ho);
+        const long n = t / p.Ho;
+        f32x4 wv[T];  // flat [channel j][tap]: element j*T + tap
+        const f32x4* wq = reinterpret_cast<const f32x4*>(p.w + (long)c * T);
+#pragma unroll
+        for (int q = 0; q < T; ++q) wv[q] = wq[q];
+        f32x4 xv[T];
+        bool ok[T];
+        const int hi0 = ho * p.sh - p.ph, wi0 = wo * p.sw - p.pw;
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < KS; ++kw) {
+                const int hi = hi0 + kh, wi = wi0 + kw;
+                const int tap = kh * KS + kw;
+                ok[tap] = hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
+                const int hc = hi < 0 ? 0 : (hi >= p.H ? p.H - 1 : hi);
+                const int wc = wi < 0 ? 0 : (wi >= p.W ? p.W - 1 : wi);
+                xv[tap] = *reinterpret_cast<const f32x4*>(p.x + ((n * p.H + hc) * p.W + wc) * p.xp + c);
+            }
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int tap = 0; tap < T; ++tap) {  // same order of additions as the general kernel
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int f = j * T + tap;
+                const float xw = xv[tap][j] * wv[f >> 2][f & 3];
+                acc[j] += ok[tap] ? xw : 0.f;
+            }
+        }
+        f32x4 res = {0.f, 0.f, 0.f, 0.f};
+        if (p.ep.residual) res = *reinterpret_cast<const f32x4*>(p.ep.residual + row * p.ep.ldr + c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float cs, ct;
+            epilogue_column(p.ep, c + j, cs, ct);
+            float v = acc[j] * p.ep.alpha;
+            v = v * cs + ct;
+            if (p.ep.residual) v += res[j];
+            acc[j] = apply_act(v, p.ep.act);
+        }
+        *reinterpret_cast<f32x4*>(p.y + row * p.ep.ldc + c) = acc;
+    }
+}
+
 static int launch_depthwise(const ConvArgs& a, int Ho, int Wo, long xp, long yp, hipStream_t s) {
     if (a.groups != a.Cin || a.Cin != a.Cout) return K_EUNSUPPORTED;  // only groups == channels
     if (!a.x_nhwc || !a.y_nhwc || a.Cin % 4 != 0 || xp % 4 != 0) return K_EUNSUPPORTED;
@@ -331,8 +392,19 @@ static int launch_depthwise(const ConvArgs& a, int Ho, int Wo, long xp, long yp,
     p.ep = make_epilogue(ea, yp);
     long blocks = (p.total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(depthwise_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p);
-    set_last_kernel("depthwise_nhwc");
+    const bool vec = a.KH == a.KW && (a.KH == 3 || a.KH == 5) && p.ep.beta == 0.f && (yp & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.w) & 15) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15) == 0 &&
+                     (!p.ep.residual || ((p.ep.ldr & 3) == 0 && (reinterpret_cast<uintptr_t>(p.ep.residual) & 15) == 0));
+    if (vec && a.KH == 3) {
+        hipLaunchKernelGGL(depthwise_taps_kernel<3>, dim3((unsigned)blocks), dim3(256), 0, s, p);
+        set_last_kernel("depthwise_3x3");
+    } else if (vec) {
+        hipLaunchKernelGGL(depthwise_taps_kernel<5>, dim3((unsigned)blocks), dim3(256), 0, s, p);
+        set_last_kernel("depthwise_5x5");
+    } else {
+        hipLaunchKernelGGL(depthwise_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p);
+        set_last_kernel("depthwise_nhwc");
+    }
     return (int)hipGetLastError();
 }
 
