@@ -329,28 +329,31 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     };
 
     const float* As0 = lds;
+    const long kpairs = kbeg + (kend - kbeg) / (2 * C::BK) * (2 * C::BK);  // end of the whole pairs of K-blocks
     if (STAGES == 2) {
         const float* As1 = lds + C::LDS_FLOATS;
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
         store_lds(ra0, rb0, 0);
         __syncthreads();
-        for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
+        for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
             load_regs(ra0, rb0, k0 + 2 * C::BK);
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             store_lds(ra1, rb1, 1);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            if (k0 + C::BK < kend) mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);  // odd block count
+            mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             store_lds(ra0, rb0, 0);
             __syncthreads();
         }
+        // an odd last K-block is in stage 0 by now (kept out of the loop: a branch there costs 10 %)
+        if (kpairs < kend) mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
     } else {
         // one LDS stage, two barriers per K-block: half the LDS footprint, so twice as many
         // workgroups stay resident and hide each other's barrier and memory latency
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
-        for (long k0 = kbeg; k0 < kend; k0 += 2 * C::BK) {
+        for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
             store_lds(ra0, rb0, 0);
             __syncthreads();
             load_regs(ra0, rb0, k0 + 2 * C::BK);
@@ -359,7 +362,13 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             store_lds(ra1, rb1, 0);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
-            if (k0 + C::BK < kend) mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);  // odd block count
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
+            __syncthreads();
+        }
+        if (kpairs < kend) {  // odd last K-block: it is in the first register set
+            store_lds(ra0, rb0, 0);
+            __syncthreads();
+            mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
         }
     }
