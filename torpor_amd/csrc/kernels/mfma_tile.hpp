@@ -202,6 +202,8 @@ __device__ __forceinline__ bool reduce_k_slices(f32x16 (&acc)[C::TM][C::TN], flo
     return true;
 }
 
+__device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 // Vector form of the accumulator write-out for the common case: row-major output with 16-byte
 // aligned rows, no beta term, whole 32-column blocks in range.  Each 32x32 block goes through the
 // wavefront's LDS staging block and comes back transposed to "four consecutive columns per
@@ -218,13 +220,38 @@ __device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int 
     const int h = lane >> 5;
     const int cq = (lane & 7) * 4;  // this lane's four columns within the block
     const int rq = lane >> 3;       // and its row within each group of eight
+    const bool colvec = !RAW && (!e.bias || aligned16_dev(e.bias)) &&
+                        (!e.bn_scale || (aligned16_dev(e.bn_scale) && aligned16_dev(e.bn_var) && aligned16_dev(e.bn_mean) &&
+                                         aligned16_dev(e.bn_bias)));
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const long col = n0 + wn * C::WTN + j * 32 + cq;
         float cs[4] = {1.f, 1.f, 1.f, 1.f}, ct[4] = {0.f, 0.f, 0.f, 0.f};
         if (!RAW) {
+            if (colvec) {
+                // the constants of the four columns as vectors: one round trip for the bias and one for the
+                // four batch-norm arrays, instead of one per scalar load under its own branch
+                f32x4 b = {0.f, 0.f, 0.f, 0.f};
+                if (e.bias) b = *reinterpret_cast<const f32x4*>(e.bias + col);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) epilogue_column(e, col + c, cs[c], ct[c]);
+                for (int c = 0; c < 4; ++c) ct[c] = b[c];
+                if (e.bn_scale) {
+                    const f32x4 g = *reinterpret_cast<const f32x4*>(e.bn_scale + col);
+                    const f32x4 vr = *reinterpret_cast<const f32x4*>(e.bn_var + col);
+                    const f32x4 mu = *reinterpret_cast<const f32x4*>(e.bn_mean + col);
+                    const f32x4 bb = *reinterpret_cast<const f32x4*>(e.bn_bias + col);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {  // same arithmetic as epilogue_column
+                        const float inv = 1.0f / sqrtf(vr[c] + e.bn_eps);
+                        const float gg = g[c] * inv;
+                        cs[c] = gg;
+                        ct[c] = (b[c] - mu[c]) * gg + bb[c];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) epilogue_column(e, col + c, cs[c], ct[c]);
+            }
         }
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
@@ -256,8 +283,6 @@ __device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int 
         }
     }
 }
-
-__device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Write the accumulators.  `partial` != nullptr: raw sums go to the split-K workspace slice
 // [M][N]; otherwise the epilogue is applied and C is written.
