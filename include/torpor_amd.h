@@ -334,7 +334,9 @@ uint64_t tp_lru_used(tp_lru* l);
  *             (controller.hpp:321-389).  status values are the reference's ExecutorStatus (-1 idle, 0 local, 1 peer
  *             copy, 2..4 host-link swap of a light / median / heavy model, 5 cold start).  `draw` replaces rand()
  *             of the random policy so that callers (and tests) own the random stream.  decide() returns 0 and
- *             dst = -1 when no executor is idle. */
+ *             dst = -1 when no executor is idle.
+ * Neither object locks: the reference calls its evictor and scheduler from the controller thread only
+ * (controller.hpp:128-216), and so must a caller of these. */
 #define TP_EVICT_LRU 0
 #define TP_EVICT_IA 1
 typedef struct tp_evictor tp_evictor;
