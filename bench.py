@@ -16,6 +16,7 @@ pinned-host -> HBM link peak, and "cpu_baseline" is the PyTorch CPU forward of t
 seeded model timed on this box's host cores (oracle/models.py, a reported baseline only).
 """
 import argparse
+import gc
 import json
 import os
 import re
@@ -120,6 +121,8 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
     for _ in range(warmup):
         cold_step()
     server.stream_synchronize(fid)
+    gc.collect()
+    gc.disable()   # as timeit does: a collection inside a timed step is the interpreter's, not the path's
     cold, swap_gbps, swap_ms = [], [], []
     t_begin = time.perf_counter()
     for _ in range(steps):
@@ -127,6 +130,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         st = server.swap_stats(fid)   # waits for the tail of the copy: part of the step
         swap_ms.append(st["copy_ms"])
         streams = st["copy_streams"]
+        gathers = st["host_gathers"]
         swap_gbps.append(st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
     server.stream_synchronize(fid)
     t_total = time.perf_counter() - t_begin
@@ -140,6 +144,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
     for _ in range(max(3, warmup)):
         warm_step()
     warm = [warm_step() for _ in range(max(steps, 20))]
+    gc.enable()
 
     # per-kernel roofline accounting over timed warm requests
     server.profile_begin()
@@ -156,7 +161,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         weight_bytes=info["image_bytes"], act_bytes=info["act_bytes"], ops=info["n_ops"], chunks=info["n_chunks"],
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
-        copy_streams=streams, steps_total_s=t_total,
+        copy_streams=streams, host_gathers=gathers, steps_total_s=t_total,
     )
     return res, kstats, empty_us, (fn, inputs, weights, first)
 

@@ -59,6 +59,7 @@ typedef struct tp_server tp_server;
 /* ---- tp_config.flags ---- */
 #define TP_FLAG_HOST_ONLY 1 /* no HIP calls: pool/LRU/state-machine logic only (CPU tests) */
 #define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
+#define TP_FLAG_NO_HOST_GATHER 4 /* embedding lookups always wait for their table's transfer group, as env TORPOR_HOST_GATHER=0 */
 
 /* ---- activation / epilogue ---- */
 #define TP_ACT_NONE 0
@@ -180,7 +181,7 @@ typedef struct tp_swap_stats {
     uint32_t chunks;
     uint32_t gate_waits; /* compute-stream waits issued during the last request */
     uint32_t copy_streams; /* streams the last swap-in alternated over */
-    uint32_t reserved0;
+    uint32_t host_gathers; /* lookups of the last request that read their table in place from the host store */
 } tp_swap_stats;
 
 /* ------------------------------------------------------------------ lifecycle

@@ -3,7 +3,7 @@ swap-in / swap-out, prefetch (Load), gate ordering with a poisoned pool."""
 import numpy as np
 import pytest
 
-from torpor_amd.functions import resnet
+from torpor_amd.functions import bert, resnet
 from torpor_amd.server import ACK_INAVAIL, ACK_OK, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD, Server
 
 pytestmark = pytest.mark.gpu
@@ -97,3 +97,31 @@ def test_graph_replays_match_eager_and_follow_the_placement(monkeypatch):
             _mk(s, 2 + rnd, seed=5 + rnd)            # ... and the pool re-used, so it comes back elsewhere or not
             (cold,) = fa.invoke([xa])
             assert np.array_equal(cold, ya)
+
+
+@pytest.mark.parametrize("host_gather", [True, False])
+def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather):
+    """The word-embedding table is looked up by row, so it is the last tensor of the image, and a
+    cold request reads its rows from the pinned host store while the table is still on its way;
+    with the option off the lookup waits for the table.  Either way cold answers equal warm ones
+    bit for bit and the device copy ends up identical to the host store."""
+    cfg = dict(layers=2, hidden=512, heads=8, ffn=1024)
+    weights = bert.init_weights(seed=21, vocab=30522, max_pos=128, cfg=cfg)   # table: 62 MB of 71
+    ids = np.random.default_rng(4).integers(0, 30522, (2, 64))
+    with Server(mem_limit_bytes=1 << 30, host_gather=host_gather) as s:
+        fn = bert.Bert(s, 3, batch=2, seq=64, weights=weights, cfg=cfg)
+        first = fn.register([ids])
+        off = {k: s.weight_offset(3, va) for k, va in fn.w.items()}
+        assert off["embeddings.word_embeddings.weight"] == max(off.values())
+        assert off["embeddings.position_embeddings.weight"] < off["encoder.layer.0.output.dense.weight"]
+        for _ in range(3):
+            fn.unload()
+            cold = fn.invoke([ids])
+            st = s.swap_stats(3)
+            assert st["host_gathers"] == (1 if host_gather else 0)
+            warm = fn.invoke([ids])
+            assert s.swap_stats(3)["host_gathers"] == 0
+            for a, b, c in zip(first, cold, warm):
+                assert np.array_equal(a, b) and np.array_equal(a, c)
+            assert np.array_equal(s.readback_weights(3), s.host_weights(3))
+        fn.unload()

@@ -319,6 +319,27 @@ def test_model_levels_select_the_two_class_policy_or_plain_lru():
         s.close()
 
 
+def test_tables_looked_up_by_index_are_last_in_the_image():
+    """First-access order (model_repo.hpp:102-109) with one exception: the word-embedding table,
+    read first but only a few rows of it, follows every tensor the forward pass streams through.
+    The other embedding operands (position and type tables, LayerNorm) keep their early place."""
+    from torpor_amd.functions import bert
+    cfg = dict(layers=2, hidden=64, heads=2, ffn=128)
+    weights = bert.init_weights(seed=1, vocab=500, max_pos=32, cfg=cfg)
+    with Server(host_only=True, mem_limit_bytes=64 << 20, pool_bytes=128 << 20) as s:
+        fn = bert.Bert(s, 0, batch=1, seq=16, weights=weights, cfg=cfg)
+        with pytest.raises(TorporError) as e:
+            fn.register([np.zeros((1, 16), np.int64)])
+        assert e.value.code == -19
+        off = {k: s.weight_offset(0, va) for k, va in fn.w.items()}
+        assert off["embeddings.word_embeddings.weight"] == max(off.values())
+        assert off["embeddings.position_embeddings.weight"] == 0
+        first_layer = min(v for k, v in off.items() if k.startswith("encoder.layer.0."))
+        assert off["embeddings.LayerNorm.weight"] < first_layer
+        last = max(v for k, v in off.items() if k.startswith("pooler."))
+        assert last < off["embeddings.word_embeddings.weight"]
+
+
 def test_request_timeout_completes_the_request(host_server):
     """cuda_server.hpp:257-264: an Execute that sends no ops is force-completed after the timeout
     (200 ms here) and the executor becomes available again."""

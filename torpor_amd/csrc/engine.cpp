@@ -69,10 +69,22 @@ int Engine::init() {
     HIPCHK(hipStreamCreateWithFlags(&copy2_, hipStreamNonBlocking));
     copy_streams_cfg_ = (int)env_u64("TORPOR_COPY_STREAMS", (uint64_t)cfg_.copy_streams);  // 0 = per model
     graph_min_ops_ = (int)env_u64("TORPOR_GRAPH_MIN_OPS", 0);
+    d2h_kernel_ = (int)env_u64("TORPOR_D2H_KERNEL", 2);  // 0 never, 1 always, 2 while a swap-in is running
+    host_gather_ = !(cfg_.flags & TP_FLAG_NO_HOST_GATHER) && env_u64("TORPOR_HOST_GATHER", 1) != 0;
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&h2d_stage_), 16ull << 20, hipHostMallocDefault));
     h2d_cap_ = 16ull << 20;
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&d2h_stage_), 8ull << 20, hipHostMallocDefault));
     d2h_cap_ = 8ull << 20;
+    {  // first use of the copy kernel and of device writes into the pinned buffer, off the request path
+        void* stage_dev = nullptr;
+        if (hipHostGetDevicePointer(&stage_dev, d2h_stage_, 0) == hipSuccess && stage_dev) {
+            (void)tpk::launch_copy(workspace_, stage_dev, 4096, compute_);
+            HIPCHK(hipStreamSynchronize(compute_));
+        } else {
+            (void)hipGetLastError();
+            d2h_kernel_ = 0;
+        }
+    }
     copy_thread_ = std::thread(&Engine::copy_main, this);
     return 0;
 }
@@ -216,7 +228,16 @@ int Engine::gate(Model& m, const Xlat& x) {
     return 0;
 }
 
-int Engine::resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out) {
+// Has transfer group `idx` of the running swap-in arrived?  Never blocks.
+bool Engine::landed(Model& m, uint32_t idx) {
+    if (idx < m.gated_upto) return true;
+    if (m.issued.load(std::memory_order_acquire) <= idx) return false;
+    if (hipEventQuery(m.chunk_ev[idx]) != hipSuccess) return false;
+    return !(m.ncopy == 2 && idx > 0 && idx - 1 >= m.gated_upto && hipEventQuery(m.chunk_ev[idx - 1]) != hipSuccess);
+}
+
+// `gather`: the kernel looks rows of this operand up by index instead of streaming it.
+int Engine::resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out, bool gather) {
     *out = nullptr;
     if (va == 0) return optional ? 0 : TP_EFAULT;
     Xlat x;
@@ -224,7 +245,24 @@ int Engine::resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** 
     if (r) return r;
     if (x.weight) {
         // memory_manager.hpp:273-284 / model_repo.hpp:102-109: first-access order, tracked run only
-        if (mode_ == MODE_TRACK && x.param->access_rank < 0) x.param->access_rank = m.next_rank++;
+        if (mode_ == MODE_TRACK) {
+            if (x.param->access_rank < 0) x.param->access_rank = m.next_rank++;
+            if (gather) x.param->gathered = true;
+        }
+        // A table whose transfer group has not arrived is read where it lies in the pinned host
+        // store: the few rows a request needs cross the link at once, the table itself follows
+        // after every tensor the forward pass streams through.
+        if (gather && host_gather_ && x.param->gathered && m.host_image_dev && !m.fully_loaded && !host_only() &&
+            m.copy_state.load(std::memory_order_acquire) != CS_IDLE) {
+            auto it = std::lower_bound(m.chunk_end.begin(), m.chunk_end.end(), x.image_end);
+            if (it == m.chunk_end.end()) return TP_EFAULT;
+            if (!landed(m, (uint32_t)(it - m.chunk_end.begin()))) {
+                if (m.copy_error.load()) return m.copy_error.load();
+                *out = m.host_image_dev + (static_cast<uint8_t*>(x.p) - m.w_dev);
+                m.stats.host_gathers++;
+                return 0;
+            }
+        }
         r = gate(m, x);
         if (r) return r;
     }
@@ -383,7 +421,17 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
             r = ensure_stage(&d2h_stage_, &d2h_cap_, bytes);
             if (r) return r;
         }
-        HIPCHK(hipMemcpyAsync(d2h_stage_ + d2h_pos_, p, bytes, hipMemcpyDeviceToHost, compute_));
+        // While a swap-in is running the copy engines hold its queued transfer groups, and a
+        // device-to-host copy handed to them would wait for all of those; a copy kernel writing
+        // into the pinned buffer goes the other way over the link without queueing behind them.
+        void* stage_dev = nullptr;
+        if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+            hipHostGetDevicePointer(&stage_dev, d2h_stage_, 0) == hipSuccess && stage_dev) {
+            int kr = tpk::launch_copy(p, static_cast<uint8_t*>(stage_dev) + d2h_pos_, bytes, compute_);
+            if (kr) return kr;
+        } else {
+            HIPCHK(hipMemcpyAsync(d2h_stage_ + d2h_pos_, p, bytes, hipMemcpyDeviceToHost, compute_));
+        }
         pending_d2h_.push_back({dst, d2h_pos_, bytes});
         d2h_pos_ = align_up(d2h_pos_ + bytes, 256);
     }
@@ -526,6 +574,8 @@ int Engine::build_image(Model& m, bool by_access) {
         std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) {
             const int ra = m.params[a].access_rank, rb = m.params[b].access_rank;
             if ((ra >= 0) != (rb >= 0)) return ra >= 0;
+            // index-looked-up tables after everything the forward pass streams through
+            if (m.params[a].gathered != m.params[b].gathered) return !m.params[a].gathered;
             if (ra >= 0 && ra != rb) return ra < rb;
             return m.params[a].voff < m.params[b].voff;
         });
@@ -551,6 +601,12 @@ int Engine::build_image(Model& m, bool by_access) {
     for (size_t i = 0; i < m.params.size(); ++i) m.params[i].image_off = new_off[i];
     host_free(m.host_image);
     m.host_image = img;
+    m.host_image_dev = nullptr;
+    if (!host_only()) {
+        void* dp = nullptr;
+        if (hipHostGetDevicePointer(&dp, img, 0) == hipSuccess) m.host_image_dev = static_cast<uint8_t*>(dp);
+        else (void)hipGetLastError();
+    }
     m.image_bytes = off;
     return 1;  // image changed
 }
@@ -600,6 +656,17 @@ void Engine::build_chunks(Model& m) {
         pos = end;
         if (sz < m.chunk_max) sz = std::min(sz * 2, m.chunk_max);
     }
+    // first group that holds nothing but tables looked up by index (they are last in the image)
+    m.defer_from = UINT32_MAX;
+    uint64_t table_off = UINT64_MAX;
+    for (const Param& p : m.params)
+        if (p.gathered) table_off = std::min(table_off, p.image_off);
+    if (host_gather_ && table_off != UINT64_MAX)
+        for (size_t i = 0; i < m.chunk_end.size(); ++i)
+            if ((i ? m.chunk_end[i - 1] : 0) >= table_off) {
+                m.defer_from = (uint32_t)i;
+                break;
+            }
     if (!host_only()) {
         while (m.chunk_ev.size() < m.chunk_end.size()) {
             hipEvent_t ev = nullptr;
@@ -694,6 +761,11 @@ void Engine::copy_main() {
                 const uint64_t end = m->chunk_end[i];
                 // alternate streams so that one group's DMA set-up hides behind the other's transfer
                 hipStream_t cs = (m->ncopy == 2 && (i & 1)) ? copy2_ : copy_;
+                // The link is not shared evenly between two streams and one may run several groups
+                // ahead.  Its first group of deferred tables waits for the other stream's last group
+                // of streamed tensors, so that the stream that lags gets the whole link for those.
+                if (m->ncopy == 2 && (i == m->defer_from || i == m->defer_from + 1) && i >= 2)
+                    (void)hipStreamWaitEvent(cs, m->chunk_ev[i == m->defer_from ? i - 1 : i - 2], 0);
                 e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
                 if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
                 if (e != hipSuccess) {
@@ -850,6 +922,7 @@ int Engine::start_execute(int id) {
     active_ = id;
     mode_ = MODE_EXEC;
     m->stats.gate_waits = 0;
+    m->stats.host_gathers = 0;
     req_start_ = Clock::now();
     if (was_resident)
         exec_status_ = ES_LOCAL;
@@ -1205,7 +1278,8 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         case TP_OP_EMBEDDING:
             if (!need(6, 5, 0)) return TP_EINVAL;
             if (I[1] < 1 || I[2] < 1 || I[3] < 1 || I[4] < 1) return TP_EINVAL;
-            if ((r = R(0, false, I[0], 8)) || (r = R(1, true, I[0], 8)) || (r = R(2, false, I[3] * I[2])) ||
+            if ((r = R(0, false, I[0], 8)) || (r = R(1, true, I[0], 8)) ||
+                (r = resolve(m, op.p[2], (uint64_t)(I[3] * I[2]) * 4, false, &q[2], /*gather=*/true)) ||
                 (r = R(3, true, I[1] * I[2])) || (r = R(4, true, I[4] * I[2])) || (r = R(5, false, I[0] * I[2])))
                 return r;
             if (!launch) return 0;

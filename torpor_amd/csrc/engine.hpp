@@ -57,6 +57,10 @@ struct Param {  // one uploaded weight tensor (model_repo.hpp:31-36 ModelParamIn
     uint64_t size = 0;
     uint64_t image_off = 0;  // offset in the weight image (host store and device copy alike)
     int access_rank = -1;    // first-access position in the tracked run, -1 = never touched
+    // Rows of this tensor are looked up by index (an embedding table).  Such a tensor travels
+    // last in the weight image, and while its transfer group is still on its way a lookup reads
+    // the rows it needs straight from the pinned host store.
+    bool gathered = false;
 };
 struct WBlock {
     uint64_t voff, size;
@@ -80,6 +84,7 @@ struct Model {
     std::vector<Param> params;  // sorted by voff
     std::vector<uint8_t> staging;
     uint8_t* host_image = nullptr;
+    uint8_t* host_image_dev = nullptr;  // the same memory as kernels address it, null if not mapped
     uint64_t image_bytes = 0, param_bytes = 0;
     int next_rank = 0;
     std::vector<uint64_t> chunk_end;
@@ -101,6 +106,7 @@ struct Model {
     std::atomic<bool> cancel{false};
     std::atomic<int> copy_error{0};
     uint32_t gated_upto = 0;
+    uint32_t defer_from = UINT32_MAX;  // first transfer group made of deferred tables only
     int ncopy = 2;            // copy streams used by the current swap-in plan
     uint64_t chunk_max = 0;   // largest transfer group of the current plan
     double warm_us = 0;       // best warm replay so far (host wall clock), 0 = none yet
@@ -188,7 +194,8 @@ private:
     Model* active_model(int client, int* err);
     int translate(Model& m, uint64_t va, uint64_t span, Xlat* out);
     int gate(Model& m, const Xlat& x);
-    int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out);
+    int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out, bool gather = false);
+    bool landed(Model& m, uint32_t idx);
     int exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch);
     int exec_compute(Model& m, const Op& op, bool launch);
     int exec_compute_impl(Model& m, const Op& op, bool launch);
@@ -244,6 +251,8 @@ private:
     hipStream_t compute_ = nullptr, copy_ = nullptr, copy2_ = nullptr;
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
+    int d2h_kernel_ = 0;
+    bool host_gather_ = true;  // lookups may read a table in place from the host store during a swap-in
     int graph_min_ops_ = 0;  // 0: warm replays launch op by op; n: capture compute runs of at least n ops
     std::unordered_map<int, std::unique_ptr<Model>> models_;
 
