@@ -60,6 +60,7 @@ typedef struct tp_server tp_server;
 #define TP_FLAG_HOST_ONLY 1 /* no HIP calls: pool/LRU/state-machine logic only (CPU tests) */
 #define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
 #define TP_FLAG_NO_HOST_GATHER 4 /* embedding lookups always wait for their table's transfer group, as env TORPOR_HOST_GATHER=0 */
+#define TP_FLAG_NO_PACK 8 /* weights cross the link as they are instead of in the 28-bit transfer format, as env TORPOR_PACK=0 */
 
 /* ---- activation / epilogue ---- */
 #define TP_ACT_NONE 0

@@ -1,4 +1,5 @@
 #include "engine.hpp"
+#include "weight_pack.hpp"
 
 #include <algorithm>
 #include <cstdio>
@@ -69,6 +70,9 @@ int Engine::init() {
     HIPCHK(hipStreamCreateWithFlags(&copy2_, hipStreamNonBlocking));
     copy_streams_cfg_ = (int)env_u64("TORPOR_COPY_STREAMS", (uint64_t)cfg_.copy_streams);  // 0 = per model
     graph_min_ops_ = (int)env_u64("TORPOR_GRAPH_MIN_OPS", 0);
+    pack_ = !(cfg_.flags & TP_FLAG_NO_PACK) && env_u64("TORPOR_PACK", 1) != 0;
+    HIPCHK(hipStreamCreateWithFlags(&decode_, hipStreamNonBlocking));
+    HIPCHK(hipEventCreateWithFlags(&stage_free_ev_, hipEventDisableTiming));
     d2h_kernel_ = (int)env_u64("TORPOR_D2H_KERNEL", 2);  // 0 never, 1 always, 2 while a swap-in is running
     host_gather_ = !(cfg_.flags & TP_FLAG_NO_HOST_GATHER) && env_u64("TORPOR_HOST_GATHER", 1) != 0;
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&h2d_stage_), 16ull << 20, hipHostMallocDefault));
@@ -103,7 +107,9 @@ Engine::~Engine() {
     for (auto& kv : models_) {
         Model& m = *kv.second;
         host_free(m.host_image);
+        host_free(m.timg);
         if (!host_only()) {
+            for (auto ev : m.dma_ev) (void)hipEventDestroy(ev);
             for (auto ev : m.chunk_ev) (void)hipEventDestroy(ev);
             if (m.t0) (void)hipEventDestroy(m.t0);
             if (m.t1) (void)hipEventDestroy(m.t1);
@@ -116,6 +122,9 @@ Engine::~Engine() {
         if (d2h_stage_) (void)hipHostFree(d2h_stage_);
         if (workspace_) (void)hipFree(workspace_);
         if (arena_) (void)hipFree(arena_);
+        if (xfer_stage_) (void)hipFree(xfer_stage_);
+        if (stage_free_ev_) (void)hipEventDestroy(stage_free_ev_);
+        if (decode_) (void)hipStreamDestroy(decode_);
         if (compute_) (void)hipStreamDestroy(compute_);
         if (copy_) (void)hipStreamDestroy(copy_);
         if (copy2_) (void)hipStreamDestroy(copy2_);
@@ -611,6 +620,154 @@ int Engine::build_image(Model& m, bool by_access) {
     return 1;  // image changed
 }
 
+// ------------------------------------------------------------------ transfer image
+void Engine::free_transfer(Model& m) {
+    host_free(m.timg);
+    m.timg = nullptr;
+    m.timg_bytes = 0;
+    m.esc_index.clear();
+    for (auto& p : m.params) {
+        p.pack_base = -1;
+        p.t_off = 0;
+    }
+}
+
+// Builds what a swap-in sends over the link (weight_pack.hpp) once the image has its final order.
+// Tensors whose words compress go in the 28-bit format, the rest as they are; a model that would
+// save under 3 % keeps sending its image directly.
+int Engine::build_transfer(Model& m) {
+    free_transfer(m);
+    m.image_order.resize(m.params.size());
+    for (size_t i = 0; i < m.image_order.size(); ++i) m.image_order[i] = (uint32_t)i;
+    std::sort(m.image_order.begin(), m.image_order.end(),
+              [&](uint32_t a, uint32_t b) { return m.params[a].image_off < m.params[b].image_off; });
+    if (!pack_ || host_only() || m.image_bytes == 0 || m.image_bytes >= (16ull << 30)) return 0;
+    std::vector<int32_t> base(m.params.size(), -1);
+    uint64_t esc_total = 0;
+    for (uint32_t idx : m.image_order) {
+        const Param& p = m.params[idx];
+        if (p.gathered || p.size % 4 != 0 || p.size < 4096) continue;
+        uint32_t b = 0;
+        uint64_t outside = 0;
+        choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), p.size / 4, &b, &outside);
+        if (outside * 8 + packed_bytes(p.size / 4) <= p.size - p.size / 20) {
+            base[idx] = (int32_t)b;
+            esc_total += outside;
+        }
+    }
+    uint64_t off = align_up(esc_total * 8, kTensorAlign);
+    std::vector<uint64_t> t_off(m.params.size(), 0);
+    for (uint32_t idx : m.image_order) {
+        const Param& p = m.params[idx];
+        t_off[idx] = off;
+        off = align_up(off + (base[idx] >= 0 ? packed_bytes(p.size / 4) : p.size), kTensorAlign);
+    }
+    if (off > m.image_bytes - m.image_bytes / 32) return 0;
+    if (off > xfer_stage_cap_) {  // registration time: no swap-in may be using the area while it is replaced
+        for (auto& kv : models_)
+            while (kv.second->copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
+        (void)hipStreamSynchronize(copy_);
+        (void)hipStreamSynchronize(copy2_);
+        (void)hipStreamSynchronize(decode_);
+        if (xfer_stage_) (void)hipFree(xfer_stage_);
+        xfer_stage_ = nullptr;
+        xfer_stage_cap_ = 0;
+        const uint64_t cap = align_up(off, 2ull << 20);
+        if (hipMalloc(reinterpret_cast<void**>(&xfer_stage_), cap) != hipSuccess) {
+            (void)hipGetLastError();
+            xfer_stage_ = nullptr;
+            return 0;  // no room for a staging area: the image travels as it is
+        }
+        xfer_stage_cap_ = cap;
+    }
+    uint8_t* t = static_cast<uint8_t*>(host_alloc(off));
+    if (!t) return 0;
+    std::memset(t, 0, off);
+    std::vector<Escape> esc;
+    esc.reserve(esc_total);
+    static_assert(sizeof(Escape) == 8, "pairs of 32-bit words");
+    for (uint32_t idx : m.image_order) {
+        Param& p = m.params[idx];
+        p.t_off = t_off[idx];
+        p.pack_base = base[idx];
+        const uint8_t* src = m.host_image + p.image_off;
+        if (p.pack_base >= 0)
+            pack_words(reinterpret_cast<const uint32_t*>(src), p.size / 4, (uint32_t)p.pack_base, t + p.t_off,
+                       p.image_off / 4, &esc);
+        else
+            std::memcpy(t + p.t_off, src, p.size);
+    }
+    if (!esc.empty()) std::memcpy(t, esc.data(), esc.size() * sizeof(Escape));
+    m.esc_index.resize(esc.size());
+    for (size_t i = 0; i < esc.size(); ++i) m.esc_index[i] = esc[i].index;
+    m.timg = t;
+    m.timg_bytes = off;
+    return 1;
+}
+
+// Where image offset d (a multiple of the tensor alignment) lies in the transfer image.
+uint64_t Engine::xfer_off(const Model& m, uint64_t d) const {
+    size_t lo = 0, hi = m.image_order.size();
+    while (lo < hi) {
+        const size_t mid = (lo + hi) / 2;
+        if (m.params[m.image_order[mid]].image_off <= d) lo = mid + 1;
+        else hi = mid;
+    }
+    if (lo == 0) return m.image_order.empty() ? m.timg_bytes : m.params[m.image_order[0]].t_off;
+    const Param& p = m.params[m.image_order[lo - 1]];
+    const uint64_t rel = d - p.image_off;
+    if (rel >= p.size) return lo < m.image_order.size() ? m.params[m.image_order[lo]].t_off : m.timg_bytes;
+    return p.t_off + (p.pack_base >= 0 ? rel / 32 * 28 : rel);
+}
+
+// One transfer group of a packed swap-in: DMA into the staging area, then, on the expansion stream,
+// every tensor run of the group into its place, the out-of-window words patched, the group published.
+int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs) {
+    const uint64_t tb = i == 0 ? 0 : xfer_off(m, beg);
+    const uint64_t te = end >= m.image_bytes ? m.timg_bytes : xfer_off(m, end);
+    if (te < tb || te > xfer_stage_cap_) return TP_EFAULT;
+    hipError_t e = hipSuccess;
+    if (te > tb) e = hipMemcpyAsync(xfer_stage_ + tb, m.timg + tb, te - tb, hipMemcpyHostToDevice, cs);
+    if (e == hipSuccess) e = hipEventRecord(m.dma_ev[i], cs);
+    if (e == hipSuccess) e = hipStreamWaitEvent(decode_, m.dma_ev[i], 0);
+    if (e != hipSuccess) return (int)e;
+    size_t lo = 0, hi = m.image_order.size();
+    while (lo < hi) {
+        const size_t mid = (lo + hi) / 2;
+        if (m.params[m.image_order[mid]].image_off <= beg) lo = mid + 1;
+        else hi = mid;
+    }
+    tpk::UnpackArgs a;
+    int r = 0;
+    for (size_t k = lo ? lo - 1 : 0; k < m.image_order.size() && !r; ++k) {
+        const Param& p = m.params[m.image_order[k]];
+        if (p.image_off >= end) break;
+        const uint64_t from = std::max(beg, p.image_off), to = std::min(end, p.image_off + p.size);
+        if (to <= from) continue;
+        const uint64_t rel = from - p.image_off;
+        tpk::UnpackPiece& pc = a.piece[a.n++];
+        pc.src = xfer_stage_ + p.t_off + (p.pack_base >= 0 ? rel / 32 * 28 : rel);
+        pc.dst = m.w_dev + from;
+        pc.bytes = to - from;
+        pc.base = p.pack_base;
+        pc.first_block = 0;
+        if (a.n == tpk::kUnpackMaxPieces) {
+            r = tpk::launch_unpack(a, decode_);
+            a.n = 0;
+        }
+    }
+    if (!r && a.n) r = tpk::launch_unpack(a, decode_);
+    if (r) return r;
+    const auto e0 = std::lower_bound(m.esc_index.begin(), m.esc_index.end(), (uint32_t)(beg / 4));
+    const auto e1 = std::lower_bound(e0, m.esc_index.end(), (uint32_t)std::min<uint64_t>(end / 4, UINT32_MAX));
+    if (e1 > e0) {
+        r = tpk::launch_patch(reinterpret_cast<const uint32_t*>(xfer_stage_) + 2 * (e0 - m.esc_index.begin()),
+                              (uint64_t)(e1 - e0), reinterpret_cast<uint32_t*>(m.w_dev), decode_);
+        if (r) return r;
+    }
+    return (int)hipEventRecord(m.chunk_ev[i], decode_);
+}
+
 // One copy stream or two.  Measured on MI355X: a single stream loses ~15 us of DMA set-up per
 // hipMemcpyAsync (51 GB/s at 8 MiB groups, 55 GB/s at 32 MiB, of a 57 GB/s link); alternating
 // the groups over two streams hides that (56-57 GB/s at any group size) but every compute
@@ -673,6 +830,11 @@ void Engine::build_chunks(Model& m) {
             if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) break;
             m.chunk_ev.push_back(ev);
         }
+        while (m.timg && m.dma_ev.size() < m.chunk_end.size()) {
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) break;
+            m.dma_ev.push_back(ev);
+        }
         if (!m.t0) (void)hipEventCreate(&m.t0);
         if (!m.t1) (void)hipEventCreate(&m.t1);
     }
@@ -705,6 +867,8 @@ int Engine::finish_tracking(Model& m) {
     if (r < 0) return r;
     if (r == 1 && !host_only() && m.image_bytes)
         HIPCHK(hipMemcpy(m.w_dev, m.host_image, m.image_bytes, hipMemcpyHostToDevice));
+    r = build_transfer(m);
+    if (r < 0) return r;
     build_chunks(m);
     // fold the per-allocation activation extents of the tracked run into one arena
     if (!host_only()) HIPCHK(hipStreamSynchronize(compute_));
@@ -753,6 +917,10 @@ void Engine::copy_main() {
         // publish each group.  Publishing is an event record, not a host synchronisation.
         int err = 0;
         if (!m->cancel.load()) {
+            if (m->timg && stage_used_) {  // the staging area is shared: the previous expansion must be done with it
+                (void)hipStreamWaitEvent(copy_, stage_free_ev_, 0);
+                (void)hipStreamWaitEvent(copy2_, stage_free_ev_, 0);
+            }
             hipError_t e = hipEventRecord(m->t0, copy_);
             if (e != hipSuccess) err = (int)e;
             uint64_t beg = 0;
@@ -765,9 +933,13 @@ void Engine::copy_main() {
                 // ahead.  Its first group of deferred tables waits for the other stream's last group
                 // of streamed tensors, so that the stream that lags gets the whole link for those.
                 if (m->ncopy == 2 && (i == m->defer_from || i == m->defer_from + 1) && i >= 2)
-                    (void)hipStreamWaitEvent(cs, m->chunk_ev[i == m->defer_from ? i - 1 : i - 2], 0);
-                e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
-                if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
+                    (void)hipStreamWaitEvent(cs, (m->timg ? m->dma_ev : m->chunk_ev)[i == m->defer_from ? i - 1 : i - 2], 0);
+                if (m->timg) {
+                    e = (hipError_t)copy_chunk_packed(*m, i, beg, end, cs);
+                } else {
+                    e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
+                    if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
+                }
                 if (e != hipSuccess) {
                     err = (int)e;
                     break;
@@ -775,7 +947,11 @@ void Engine::copy_main() {
                 m->issued.store((uint32_t)i + 1, std::memory_order_release);
                 beg = end;
             }
-            if (!err) {
+            if (m->timg) {
+                (void)hipEventRecord(stage_free_ev_, decode_);
+                stage_used_ = true;
+                if (!err) (void)hipEventRecord(m->t1, decode_);  // the expansions follow the groups in order
+            } else if (!err) {
                 const size_t n = m->chunk_end.size();
                 if (m->ncopy == 2 && n >= 2) {  // t1 = both streams drained
                     const size_t last_odd = (n - 1) & 1 ? n - 1 : n - 2;
@@ -797,6 +973,7 @@ void Engine::wait_copy_idle(Model& m) {
     }
     (void)hipStreamSynchronize(copy_);
     (void)hipStreamSynchronize(copy2_);
+    (void)hipStreamSynchronize(decode_);
 }
 
 // memory_manager.hpp:213-227 sig_trans_thread + 451-507 check_and_malloc_model
@@ -834,7 +1011,7 @@ int Engine::swap_in(Model& m) {
     m.cancel.store(false);
     m.copy_error.store(0);
     m.stats.alloc_us = us_since(t0);
-    m.stats.bytes = m.image_bytes;
+    m.stats.bytes = m.timg ? m.timg_bytes : m.image_bytes;
     m.stats.chunks = (uint32_t)m.chunk_end.size();
     m.stats.copy_streams = (uint32_t)m.ncopy;
     ++swap_ins_;
@@ -890,7 +1067,9 @@ void Engine::start_cold(int id, int level) {
         evict_model(*old);
         wait_copy_idle(*old);
         host_free(old->host_image);
+        host_free(old->timg);
         if (!host_only()) {
+            for (auto ev : old->dma_ev) (void)hipEventDestroy(ev);
             for (auto ev : old->chunk_ev) (void)hipEventDestroy(ev);
             if (old->t0) (void)hipEventDestroy(old->t0);
             if (old->t1) (void)hipEventDestroy(old->t1);
@@ -1750,6 +1929,7 @@ int Engine::readback_weights(int client, void* dst, uint64_t bytes) {
     while (m->copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
     HIPCHK(hipStreamSynchronize(copy_));
     HIPCHK(hipStreamSynchronize(copy2_));
+    HIPCHK(hipStreamSynchronize(decode_));
     HIPCHK(hipStreamSynchronize(compute_));
     HIPCHK(hipMemcpy(dst, m->w_dev, bytes, hipMemcpyDeviceToHost));
     return 0;

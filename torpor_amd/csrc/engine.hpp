@@ -61,6 +61,9 @@ struct Param {  // one uploaded weight tensor (model_repo.hpp:31-36 ModelParamIn
     // last in the weight image, and while its transfer group is still on its way a lookup reads
     // the rows it needs straight from the pinned host store.
     bool gathered = false;
+    // place in the transfer image: as it is (pack_base < 0) or in the 28-bit format with that window base
+    uint64_t t_off = 0;
+    int32_t pack_base = -1;
 };
 struct WBlock {
     uint64_t voff, size;
@@ -86,6 +89,13 @@ struct Model {
     uint8_t* host_image = nullptr;
     uint8_t* host_image_dev = nullptr;  // the same memory as kernels address it, null if not mapped
     uint64_t image_bytes = 0, param_bytes = 0;
+    // What a swap-in sends when the weights compress: [words outside their window: (index, bits) pairs]
+    // [tensor payloads in image order].  Null when the image travels as it is.
+    uint8_t* timg = nullptr;
+    uint64_t timg_bytes = 0;
+    std::vector<uint32_t> esc_index;   // image word index of every pair, ascending
+    std::vector<uint32_t> image_order; // params[] indices by image_off
+    std::vector<hipEvent_t> dma_ev;    // transfer group arrived in the staging area (packed transfers)
     int next_rank = 0;
     std::vector<uint64_t> chunk_end;
     std::vector<hipEvent_t> chunk_ev;
@@ -196,6 +206,10 @@ private:
     int gate(Model& m, const Xlat& x);
     int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out, bool gather = false);
     bool landed(Model& m, uint32_t idx);
+    int build_transfer(Model& m);
+    uint64_t xfer_off(const Model& m, uint64_t image_off) const;
+    void free_transfer(Model& m);
+    int copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs);
     int exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch);
     int exec_compute(Model& m, const Op& op, bool launch);
     int exec_compute_impl(Model& m, const Op& op, bool launch);
@@ -249,6 +263,13 @@ private:
     uint8_t* arena_ = nullptr;
     float* workspace_ = nullptr;
     hipStream_t compute_ = nullptr, copy_ = nullptr, copy2_ = nullptr;
+    // packed transfers land in a staging area and are expanded into place on their own stream
+    hipStream_t decode_ = nullptr;
+    uint8_t* xfer_stage_ = nullptr;
+    uint64_t xfer_stage_cap_ = 0;
+    hipEvent_t stage_free_ev_ = nullptr;  // the last expansion that read the staging area
+    bool stage_used_ = false;
+    bool pack_ = true;
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
     int d2h_kernel_ = 0;

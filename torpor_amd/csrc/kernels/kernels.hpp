@@ -109,4 +109,24 @@ int launch_sum(const float* x, float* y, long n, hipStream_t s);  // y[0] = sum(
 int launch_fill(float* y, float v, long n, hipStream_t s);
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t s);
 
+// Expansion of transfer groups that arrived in the 28-bit weight format (or as they are).  A piece is
+// a run of one tensor: `bytes` bytes at dst, read from src either verbatim (base < 0) or as packed
+// groups of 8 words with exponent window base `base`.  dst and src are 16-byte aligned; a packed
+// piece starts on a group boundary.
+struct UnpackPiece {
+    const uint8_t* src;
+    uint8_t* dst;
+    uint64_t bytes;
+    int32_t base;
+    uint32_t first_block;  // filled by launch_unpack
+};
+constexpr int kUnpackMaxPieces = 24;
+struct UnpackArgs {
+    UnpackPiece piece[kUnpackMaxPieces];
+    int n = 0;
+};
+int launch_unpack(UnpackArgs& a, hipStream_t s);
+// image32[table[2i]] = table[2i+1] for i in [0, n): the words that did not fit their tensor's window
+int launch_patch(const uint32_t* table, uint64_t n, uint32_t* image32, hipStream_t s);
+
 }  // namespace tpk

@@ -765,4 +765,83 @@ int launch_sum(const float* x, float* y, long n, hipStream_t s) {
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------- 28-bit weight format
+// One workgroup expands 2048 words (8 KiB of the image): a lane takes one group, 7 dwords in, 8 out.
+constexpr int kUnpackBlockBytes = 8192;
+__global__ __launch_bounds__(256) void unpack_kernel(const UnpackArgs a) {
+    int k = 0;
+    while (k + 1 < a.n && a.piece[k + 1].first_block <= blockIdx.x) ++k;
+    const UnpackPiece& pc = a.piece[k];
+    const uint64_t off = (uint64_t)(blockIdx.x - pc.first_block) * kUnpackBlockBytes;
+    if (off >= pc.bytes) return;
+    const uint64_t left = pc.bytes - off;
+    uint8_t* __restrict__ dst = pc.dst + off;
+    if (pc.base < 0) {
+        const uint8_t* __restrict__ src = pc.src + off;
+        const uint64_t n = left < kUnpackBlockBytes ? left : kUnpackBlockBytes;
+        const uint64_t nv = n >> 4;
+        for (uint64_t i = threadIdx.x; i < nv; i += 256)
+            reinterpret_cast<f32x4*>(dst)[i] = reinterpret_cast<const f32x4*>(src)[i];
+        for (uint64_t i = (nv << 4) + threadIdx.x; i < n; i += 256) dst[i] = src[i];
+        return;
+    }
+    const uint64_t g = threadIdx.x;
+    if (g * 32 >= left) return;
+    const uint32_t* __restrict__ in = reinterpret_cast<const uint32_t*>(pc.src + off / 32 * 28) + g * 7;
+    uint32_t d[7];
+#pragma unroll
+    for (int j = 0; j < 7; ++j) d[j] = in[j];
+    uint32_t f[8];
+    f[0] = d[0] & 0xFFFFFFu;
+    f[1] = (d[0] >> 24) | ((d[1] & 0xFFFFu) << 8);
+    f[2] = (d[1] >> 16) | ((d[2] & 0xFFu) << 16);
+    f[3] = d[2] >> 8;
+    f[4] = d[3] & 0xFFFFFFu;
+    f[5] = (d[3] >> 24) | ((d[4] & 0xFFFFu) << 8);
+    f[6] = (d[4] >> 16) | ((d[5] & 0xFFu) << 16);
+    f[7] = d[5] >> 8;
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t code = (d[6] >> (4 * j)) & 0xFu;
+        w[j] = (f[j] & 0x7FFFFFu) | ((f[j] >> 23) << 31) | ((((uint32_t)pc.base + code) & 0xFFu) << 23);
+    }
+    uint32_t* __restrict__ out = reinterpret_cast<uint32_t*>(dst) + g * 8;
+    if (g * 32 + 32 <= left) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        reinterpret_cast<u32x4*>(out)[0] = u32x4{w[0], w[1], w[2], w[3]};
+        reinterpret_cast<u32x4*>(out)[1] = u32x4{w[4], w[5], w[6], w[7]};
+    } else {  // last group of a tensor whose word count is not a multiple of 8
+        const uint64_t words = (left - g * 32) / 4;
+        for (uint64_t j = 0; j < words; ++j) out[j] = w[j];
+    }
+}
+int launch_unpack(UnpackArgs& a, hipStream_t s) {
+    if (a.n < 0 || a.n > kUnpackMaxPieces) return K_EINVAL;
+    uint64_t blocks = 0;
+    for (int k = 0; k < a.n; ++k) {
+        UnpackPiece& pc = a.piece[k];
+        if (!pc.src || !pc.dst || !al16(pc.src) || !al16(pc.dst)) return K_EINVAL;
+        if (pc.base >= 0 && (pc.bytes % 4 != 0 || pc.base > 255)) return K_EINVAL;
+        pc.first_block = (uint32_t)blocks;
+        blocks += (pc.bytes + kUnpackBlockBytes - 1) / kUnpackBlockBytes;
+        if (blocks > 0x7FFFFFFFull) return K_EINVAL;
+    }
+    if (blocks == 0) return 0;
+    hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    return (int)hipGetLastError();
+}
+
+__global__ __launch_bounds__(256) void patch_kernel(const uint32_t* __restrict__ table, uint64_t n,
+                                                    uint32_t* __restrict__ image32) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
+        image32[table[2 * i]] = table[2 * i + 1];
+}
+int launch_patch(const uint32_t* table, uint64_t n, uint32_t* image32, hipStream_t s) {
+    if (!table || !image32) return K_EINVAL;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(patch_kernel, dim3(grid_for((long)n, 256)), dim3(256), 0, s, table, n, image32);
+    return (int)hipGetLastError();
+}
+
 }  // namespace tpk

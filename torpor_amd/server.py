@@ -21,6 +21,7 @@ NCHW, NHWC = 0, 1
  OP_SCALE_CHANNELS) = range(1, 18)
 FLAG_HOST_ONLY = 1
 FLAG_EVICT_LRU = 2   # plain LRU instead of the two-class policy (as env EVICT_POLICY=LRU)
+FLAG_NO_PACK = 8   # weights cross the link as they are
 FLAG_NO_HOST_GATHER = 4   # embedding lookups wait for their table instead of reading it from host memory
 
 
@@ -36,7 +37,7 @@ def _as_bytes_view(a):
 
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
-                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True):
+                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True, pack=True):
         self._l = _lib.lib()
         cfg = _lib.Config()
         cfg.struct_size = C.sizeof(_lib.Config)
@@ -47,7 +48,7 @@ class Server:
         cfg.chunk_max_bytes = chunk_max_bytes
         cfg.workspace_bytes = workspace_bytes
         cfg.flags = (FLAG_HOST_ONLY if host_only else 0) | (FLAG_EVICT_LRU if evict_lru else 0) | \
-            (0 if host_gather else FLAG_NO_HOST_GATHER)
+            (0 if host_gather else FLAG_NO_HOST_GATHER) | (0 if pack else FLAG_NO_PACK)
         cfg.request_timeout_ms = request_timeout_ms
         cfg.copy_streams = copy_streams
         h = C.c_void_p()
