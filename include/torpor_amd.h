@@ -368,6 +368,25 @@ int tp_sched_placement(tp_sched* s); /* GPU for a cold start, -1 if none idle */
 int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t draw, int32_t* dst_gpu,
                     int32_t* src_gpu, int32_t* status);
 
+/* ------------------------------------------------------------------ transfer format
+ * The lossless 28-bit format in which compressible weight tensors cross the host link
+ * (TP_FLAG_NO_PACK switches it off); no counterpart in the reference, which sends weights as they
+ * are (memory_manager.hpp:378-409).  A tensor is n 32-bit words of any content.  Packed: groups of
+ * 8 words in 28 bytes -- eight 24-bit little-endian fields (sign << 23 | mantissa), then one 32-bit
+ * word of eight 4-bit codes, word j in bits 4j..4j+3; code c < 15 stands for exponent base + c, code
+ * 15 for a word outside the window, listed as an (index, bits) pair.  The last group is zero-padded.
+ * Exposed so that the format can be checked on the host; the engine applies it on its own.
+ *   tp_pack_bound   bytes of the packed form of n words
+ *   tp_pack_words   chooses the window of 15 exponents holding the most words, packs, and writes up
+ *                   to pair_cap pairs; returns 0, or TP_ENOMEM when there are more pairs than that
+ *                   (*n_pairs then still holds the count)
+ *   tp_unpack_words the inverse, pairs applied */
+uint64_t tp_pack_bound(uint64_t n_words);
+int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* packed, int32_t* base, uint32_t* pairs,
+                  uint64_t pair_cap, uint64_t* n_pairs);
+int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
+                    uint32_t* words);
+
 #ifdef __cplusplus
 }
 #endif

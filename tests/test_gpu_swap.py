@@ -125,3 +125,39 @@ def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather
                 assert np.array_equal(a, b) and np.array_equal(a, c)
             assert np.array_equal(s.readback_weights(3), s.host_weights(3))
         fn.unload()
+
+
+@pytest.mark.parametrize("pack", [True, False])
+def test_packed_transfer_is_lossless_for_any_bits(pack):
+    """Weights cross the link in the 28-bit format and are expanded on the device.  Doctored tensors
+    (zeros, denormals, infinities, NaNs, exponents spread over 60 binades, one tensor of arbitrary
+    bits, one of zeros only) must come back bit for bit, swap-in after swap-in, and a request must
+    answer as it did at registration."""
+    weights = resnet.init_weights("resnet50", seed=5)
+    rng = np.random.default_rng(6)
+    flat = weights["layer1.0.conv1.weight"].reshape(-1).view(np.uint32)
+    flat[::97] = 0
+    flat[1::101] = 0x00000001
+    flat[2::103] = 0x7F800000
+    flat[3::107] = 0x7FC00001
+    flat[5::109] = 0xFF800000
+    big = weights["layer2.0.conv2.weight"]
+    weights["layer2.0.conv2.weight"] = rng.integers(0, 1 << 32, big.size, dtype=np.uint64).astype(np.uint32).view(np.float32).reshape(big.shape)
+    weights["layer3.0.conv1.weight"][:] = 0
+    w4 = weights["layer4.0.conv2.weight"]
+    w4 *= np.exp(rng.uniform(-20, 20, w4.shape)).astype(np.float32)
+    x = rng.standard_normal((1, 3, 64, 64)).astype(np.float32)
+    with Server(mem_limit_bytes=1 << 30, pack=pack) as s:
+        fn = resnet.ResNet(s, 2, "resnet50", batch=1, weights=weights, image=64)
+        first = fn.register([x])
+        host = s.host_weights(2).copy()
+        image = s.model_info(2)["image_bytes"]
+        assert np.array_equal(s.readback_weights(2), host)
+        for _ in range(3):
+            fn.unload()
+            cold = fn.invoke([x])
+            assert np.array_equal(first[0], cold[0], equal_nan=True)
+            assert np.array_equal(s.readback_weights(2), host)
+            sent = s.swap_stats(2)["bytes"]
+            assert (0.85 * image < sent < 0.93 * image) if pack else sent == image
+        fn.unload()

@@ -6,6 +6,7 @@
 
 #include "engine.hpp"
 #include "scheduler.hpp"
+#include "weight_pack.hpp"
 #include "kernels/kernels.hpp"
 
 struct tp_server {
@@ -661,6 +662,42 @@ int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t 
     if (dst_gpu) *dst_gpu = d.dst_gpu;
     if (src_gpu) *src_gpu = d.src_gpu;
     if (status) *status = d.status;
+    return 0;
+    TP_GUARD_END
+}
+
+// ------------------------------------------------------------------ transfer format
+uint64_t tp_pack_bound(uint64_t n_words) { return tp::packed_bytes(n_words); }
+
+int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* packed, int32_t* base, uint32_t* pairs,
+                  uint64_t pair_cap, uint64_t* n_pairs) {
+    TP_GUARD_BEGIN
+    if ((!words && n_words) || !packed || !base || (!pairs && pair_cap) || n_words > 0xFFFFFFFFull) return TP_EINVAL;
+    uint32_t b = 0;
+    uint64_t outside = 0;
+    tp::choose_window(words, n_words, &b, &outside);
+    std::vector<tp::Escape> esc;
+    tp::pack_words(words, n_words, b, packed, 0, &esc);
+    *base = (int32_t)b;
+    if (n_pairs) *n_pairs = esc.size();
+    if (esc.size() > pair_cap) return TP_ENOMEM;
+    for (size_t i = 0; i < esc.size(); ++i) {
+        pairs[2 * i] = esc[i].index;
+        pairs[2 * i + 1] = esc[i].bits;
+    }
+    return 0;
+    TP_GUARD_END
+}
+
+int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
+                    uint32_t* words) {
+    TP_GUARD_BEGIN
+    if (!packed || (!words && n_words) || base < 0 || base > 255 || (!pairs && n_pairs)) return TP_EINVAL;
+    tp::unpack_words(packed, n_words, (uint32_t)base, words);
+    for (uint64_t i = 0; i < n_pairs; ++i) {
+        if (pairs[2 * i] >= n_words) return TP_EINVAL;
+        words[pairs[2 * i]] = pairs[2 * i + 1];
+    }
     return 0;
     TP_GUARD_END
 }
