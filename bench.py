@@ -11,8 +11,9 @@ One JSON line is printed: the headline value is the cold-start p50 of the primar
 BERT-large batch 4 seq 384 (BASELINE.json configs[3]: the largest single-GPU configuration and,
 with ResNet-152, the one the north-star target is quoted on); the other single-GPU configs are
 reported under "workloads".  "roofline" is computed from per-launch HIP-event timings of the
-dominant kernel over timed warm requests, "swap" holds the swap-in GB/s against the measured
-pinned-host -> HBM link peak, and "cpu_baseline" is the PyTorch CPU forward of the same
+dominant kernel over timed warm requests, "swap" holds the swap-in GB/s (bytes that crossed the
+link; compressible tensors travel in a lossless 28-bit format) against the measured pinned-host ->
+HBM link peak, and "cpu_baseline" is the PyTorch CPU forward of the same
 seeded model timed on this box's host cores (oracle/models.py, a reported baseline only).
 """
 import argparse
@@ -131,7 +132,8 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         swap_ms.append(st["copy_ms"])
         streams = st["copy_streams"]
         gathers = st["host_gathers"]
-        swap_gbps.append(st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
+        swap_gbps.append(st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))   # bytes that crossed the link
+        link_bytes = st["bytes"]
     server.stream_synchronize(fid)
     t_total = time.perf_counter() - t_begin
     out = fn.postprocess([v.copy() for v in views])
@@ -161,6 +163,8 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         weight_bytes=info["image_bytes"], act_bytes=info["act_bytes"], ops=info["n_ops"], chunks=info["n_chunks"],
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
+        link_bytes=link_bytes,   # below weight_bytes when tensors travel in the 28-bit format
+        weights_gbps_p50=info["image_bytes"] / 1e9 / (pctl(swap_ms, 0.5) * 1e-3),   # weight bytes in place per second
         copy_streams=streams, host_gathers=gathers, steps_total_s=t_total,
     )
     return res, kstats, empty_us, (fn, inputs, weights, first)
@@ -300,7 +304,8 @@ def main():
         "config": {"workload": primary + " fp32, weights in pinned host store, not resident in HBM at start"},
         "swap": {"gbps": p["swap_gbps_p50"], "link_peak_gbps_measured": link,
                  "frac_of_measured_link": p["swap_frac_of_link"], "pcie_gen5_x16_nominal_gbps": PCIE_GEN5_X16_GBPS,
-                 "weight_bytes": p["weight_bytes"]},
+                 "weight_bytes": p["weight_bytes"], "link_bytes": p["link_bytes"],
+                 "weights_in_place_gbps": p["weights_gbps_p50"]},
         "warm_ms_p50": p["warm_ms_p50"],
         "cold_over_warm": p["cold_over_warm"],
         "roofline": roof[primary],
