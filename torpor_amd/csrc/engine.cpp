@@ -646,7 +646,7 @@ int Engine::build_transfer(Model& m) {
     uint64_t esc_total = 0;
     for (uint32_t idx : m.image_order) {
         const Param& p = m.params[idx];
-        if (p.gathered || p.size % 4 != 0 || p.size < 4096) continue;
+        if (p.size % 4 != 0 || p.size < 4096) continue;
         uint32_t b = 0;
         uint64_t outside = 0;
         choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), p.size / 4, &b, &outside);
@@ -788,7 +788,7 @@ void Engine::choose_copy_plan(Model& m) {
         kernels += (op.kind == OPK_GEMM || op.kind == OPK_CONV) ? 1.5 : 1.0;
     }
     if (compute_us <= 0) compute_us = est;
-    const double bytes = (double)m.image_bytes;
+    const double bytes = (double)(m.timg ? m.timg_bytes : m.image_bytes);  // what crosses the link
     const double t1 = std::max(bytes / 54.0e3, compute_us + kernels * 1.2);
     // (measured on ResNet-152 batch 8: kernels that share the device with two copy streams run
     // about 15 % longer, on top of the per-launch cost)
