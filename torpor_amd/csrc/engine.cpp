@@ -1909,6 +1909,9 @@ int Engine::swap_stats(int client, tp_swap_stats* out) {
     if (!out) return TP_EINVAL;
     Model* m = find(client);
     if (!m) return TP_ENOENT;
+    // the copy thread may still be handing the last groups to the streams (it never takes mu_)
+    while (!host_only() && m->timing_valid && m->copy_state.load(std::memory_order_acquire) == CS_RUNNING)
+        std::this_thread::yield();
     if (!host_only() && m->timing_valid && m->copy_state.load() == CS_ISSUED && !m->cancel.load()) {
         if (hipEventSynchronize(m->t1) == hipSuccess) {
             float ms = 0.f;
