@@ -391,7 +391,18 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
         if (r) return r;
     }
     std::memcpy(h2d_stage_ + h2d_pos_, src, bytes);
-    HIPCHK(hipMemcpyAsync(x.p, h2d_stage_ + h2d_pos_, bytes, hipMemcpyHostToDevice, compute_));
+    // During a swap-in the copy engines belong to the weight stream: a request input handed to them
+    // queues among its transfer groups and disturbs how they alternate over the engines.  A copy
+    // kernel reads the pinned buffer instead (alignment of the destination permitting).
+    void* stage_dev = nullptr;
+    const bool by_kernel = (d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+                           hipHostGetDevicePointer(&stage_dev, h2d_stage_, 0) == hipSuccess && stage_dev;
+    if (by_kernel) {
+        int kr = tpk::launch_copy(static_cast<uint8_t*>(stage_dev) + h2d_pos_, x.p, bytes, compute_);
+        if (kr) return kr;
+    } else {
+        HIPCHK(hipMemcpyAsync(x.p, h2d_stage_ + h2d_pos_, bytes, hipMemcpyHostToDevice, compute_));
+    }
     h2d_pos_ = align_up(h2d_pos_ + bytes, 256);
     return 0;
 }
@@ -726,14 +737,19 @@ uint64_t Engine::xfer_off(const Model& m, uint64_t d) const {
 
 // One transfer group of a packed swap-in: DMA into the staging area, then, on the expansion stream,
 // every tensor run of the group into its place, the out-of-window words patched, the group published.
-int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs) {
-    const uint64_t tb = i == 0 ? 0 : xfer_off(m, beg);
-    const uint64_t te = end >= m.image_bytes ? m.timg_bytes : xfer_off(m, end);
-    if (te < tb || te > xfer_stage_cap_) return TP_EFAULT;
-    hipError_t e = hipSuccess;
-    if (te > tb) e = hipMemcpyAsync(xfer_stage_ + tb, m.timg + tb, te - tb, hipMemcpyHostToDevice, cs);
-    if (e == hipSuccess) e = hipEventRecord(m.dma_ev[i], cs);
-    if (e == hipSuccess) e = hipStreamWaitEvent(decode_, m.dma_ev[i], 0);
+int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs, bool do_dma,
+                              bool do_expand) {
+    if (do_dma) {
+        const uint64_t tb = i == 0 ? 0 : xfer_off(m, beg);
+        const uint64_t te = end >= m.image_bytes ? m.timg_bytes : xfer_off(m, end);
+        if (te < tb || te > xfer_stage_cap_) return TP_EFAULT;
+        hipError_t e = hipSuccess;
+        if (te > tb) e = hipMemcpyAsync(xfer_stage_ + tb, m.timg + tb, te - tb, hipMemcpyHostToDevice, cs);
+        if (e == hipSuccess) e = hipEventRecord(m.dma_ev[i], cs);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (!do_expand) return 0;
+    hipError_t e = hipStreamWaitEvent(decode_, m.dma_ev[i], 0);
     if (e != hipSuccess) return (int)e;
     size_t lo = 0, hi = m.image_order.size();
     while (lo < hi) {
@@ -927,10 +943,9 @@ void Engine::copy_main() {
             }
             hipError_t e = hipEventRecord(m->t0, copy_);
             if (e != hipSuccess) err = (int)e;
-            uint64_t beg = 0;
-            for (size_t i = 0; i < m->chunk_end.size() && !err; ++i) {
-                if (m->cancel.load()) break;
-                const uint64_t end = m->chunk_end[i];
+            // A group is handed over in two steps: its DMA (and, sent as it is, its event), then --
+            // for a packed transfer -- its expansion and event on the expansion stream.
+            auto dma = [&](size_t i, uint64_t beg, uint64_t end) -> int {
                 // alternate streams so that one group's DMA set-up hides behind the other's transfer
                 hipStream_t cs = (m->ncopy == 2 && (i & 1)) ? copy2_ : copy_;
                 // The link is not shared evenly between two streams and one may run several groups
@@ -938,17 +953,37 @@ void Engine::copy_main() {
                 // of streamed tensors, so that the stream that lags gets the whole link for those.
                 if (m->ncopy == 2 && (i == m->defer_from || i == m->defer_from + 1) && i >= 2)
                     (void)hipStreamWaitEvent(cs, (m->timg ? m->dma_ev : m->chunk_ev)[i == m->defer_from ? i - 1 : i - 2], 0);
-                if (m->timg) {
-                    e = (hipError_t)copy_chunk_packed(*m, i, beg, end, cs);
-                } else {
-                    e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
-                    if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
-                }
-                if (e != hipSuccess) {
-                    err = (int)e;
-                    break;
-                }
-                m->issued.store((uint32_t)i + 1, std::memory_order_release);
+                if (m->timg) return copy_chunk_packed(*m, i, beg, end, cs, /*dma=*/true, /*expand=*/false);
+                hipError_t e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
+                if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
+                return (int)e;
+            };
+            auto publish = [&](size_t i, uint64_t beg, uint64_t end) -> int {
+                int r = m->timg ? copy_chunk_packed(*m, i, beg, end, nullptr, false, true) : 0;
+                if (!r) m->issued.store((uint32_t)i + 1, std::memory_order_release);
+                return r;
+            };
+            const size_t n_groups = m->chunk_end.size();
+            size_t i = 0;
+            uint64_t beg = 0;
+            // With two streams the first two DMAs go out back to back, before anything else is
+            // submitted.  Measured: when the second stream's first copy is submitted while the first
+            // stream's is already moving (25 us later), the whole swap-in runs at 52.5 GB/s instead of
+            // 56.5 GB/s; submitted together, both streams settle into the faster pattern.
+            if (m->ncopy == 2 && n_groups >= 2 && !err && !m->cancel.load()) {
+                const uint64_t e0 = m->chunk_end[0], e1 = m->chunk_end[1];
+                err = dma(0, 0, e0);
+                if (!err) err = dma(1, e0, e1);
+                if (!err) err = publish(0, 0, e0);
+                if (!err) err = publish(1, e0, e1);
+                i = 2;
+                beg = e1;
+            }
+            for (; i < n_groups && !err; ++i) {
+                if (m->cancel.load()) break;
+                const uint64_t end = m->chunk_end[i];
+                err = dma(i, beg, end);
+                if (!err) err = publish(i, beg, end);
                 beg = end;
             }
             if (m->timg) {

@@ -209,7 +209,7 @@ private:
     int build_transfer(Model& m);
     uint64_t xfer_off(const Model& m, uint64_t image_off) const;
     void free_transfer(Model& m);
-    int copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs);
+    int copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs, bool do_dma, bool do_expand);
     int exec_op(Model& m, const Op& op, ReplayCtx* rc, bool launch);
     int exec_compute(Model& m, const Op& op, bool launch);
     int exec_compute_impl(Model& m, const Op& op, bool launch);
