@@ -175,8 +175,9 @@ typedef struct tp_model_info {
 } tp_model_info;
 
 typedef struct tp_swap_stats {
-    uint64_t bytes;      /* weight bytes moved by the last swap-in of this model */
-    double copy_ms;      /* first copy issued -> last copy landed, on the copy stream */
+    uint64_t bytes;      /* bytes the last swap-in of this model moved over the host link (below the image size when
+                            tensors travel in the 28-bit transfer format) */
+    double copy_ms;      /* first copy issued -> last group in place (landed and, if packed, expanded) */
     double alloc_us;     /* host time to (re)acquire pool extents ("CheckMalloc", memory_manager.hpp:499-501) */
     double evict_us;     /* host time of the last swap-out (memory_manager.hpp:258) */
     uint32_t chunks;
