@@ -102,7 +102,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
     fn, inputs, weights = make_function(server, fid, name)
     first = fn.register(inputs)
     info = server.model_info(fid)
-    packed, outbuf, views = fn.pack(inputs)
+    packed, outbuf, views = fn.pack(inputs, pinned=True)   # results land in pinned memory, as a serving loop would have it
 
     def cold_step():
         fn.unload()

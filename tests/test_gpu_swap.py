@@ -161,3 +161,21 @@ def test_packed_transfer_is_lossless_for_any_bits(pack):
             sent = s.swap_stats(2)["bytes"]
             assert (0.85 * image < sent < 0.93 * image) if pack else sent == image
         fn.unload()
+
+
+def test_results_into_pinned_buffers_equal_results_through_staging(gpu_server):
+    """tp_host_alloc: a result whose destination lies in such a buffer is written by the device itself
+    (by copy kernel while a swap-in runs, by the copy engine otherwise); same bytes as the staged path."""
+    s = gpu_server
+    fn, x, y = _mk(s, 7, seed=31)
+    packed, out_plain, views_plain = fn.pack([x])
+    _, out_pinned, views_pinned = fn.pack([x], pinned=True)
+    for cold in (False, True, True, False):
+        for out in (out_pinned, out_plain):
+            if cold:
+                fn.unload()
+            out[:] = 0
+            assert s.signal(REQ_EXECUTE, 7, "")[0] == ACK_OK
+            s.replay(7, packed, out)
+        assert np.array_equal(views_plain[0], y) and np.array_equal(views_pinned[0], y)
+    fn.unload()

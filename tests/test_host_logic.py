@@ -340,6 +340,20 @@ def test_tables_looked_up_by_index_are_last_in_the_image():
         assert last < off["embeddings.word_embeddings.weight"]
 
 
+def test_pinned_result_buffers_are_tracked(host_server):
+    import ctypes as C
+    from torpor_amd import _lib
+    L, h = _lib.lib(), host_server._h
+    p = C.c_void_p()
+    assert L.tp_host_alloc(h, 0, C.byref(p)) == -22 and L.tp_host_alloc(h, 64, None) == -22
+    assert L.tp_host_alloc(h, 4096, C.byref(p)) == 0 and p.value
+    a = host_server.host_empty(100)
+    a[:] = 7
+    assert a.sum() == 700
+    assert L.tp_host_free(h, C.c_void_p(p.value + 8)) == -22      # not the start of a buffer
+    assert L.tp_host_free(h, p) == 0 and L.tp_host_free(h, p) == -22
+
+
 def test_request_timeout_completes_the_request(host_server):
     """cuda_server.hpp:257-264: an Execute that sends no ops is force-completed after the timeout
     (200 ms here) and the executor becomes available again."""

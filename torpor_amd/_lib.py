@@ -178,6 +178,8 @@ SYMBOLS = {
     "tp_sched_placement": (C.c_int, [_P]),
     "tp_sched_decide": (C.c_int, [_P, _I32, C.c_char_p, C.c_uint32, C.POINTER(_I32), C.POINTER(_I32),
                                   C.POINTER(_I32)]),
+    "tp_host_alloc": (C.c_int, [_P, _U64, C.POINTER(_P)]),
+    "tp_host_free": (C.c_int, [_P, _P]),
     "tp_pack_bound": (_U64, [_U64]),
     "tp_pack_words": (C.c_int, [_P, _U64, _P, C.POINTER(_I32), _P, _U64, C.POINTER(_U64)]),
     "tp_unpack_words": (C.c_int, [_P, _U64, _I32, _P, _U64, _P]),

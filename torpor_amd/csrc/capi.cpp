@@ -350,6 +350,19 @@ int tp_replay(tp_server* s, int32_t client, const void* input, uint64_t input_by
     TP_GUARD_END
 }
 
+int tp_host_alloc(tp_server* s, uint64_t bytes, void** ptr) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.user_host_alloc(bytes, ptr);
+    TP_GUARD_END
+}
+int tp_host_free(tp_server* s, void* ptr) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.user_host_free(ptr);
+    TP_GUARD_END
+}
+
 int tp_model_resident(tp_server* s, int32_t client) {
     TP_GUARD_BEGIN
     ENG(s);

@@ -116,6 +116,8 @@ Engine::~Engine() {
             drop_graph(m);
         }
     }
+    for (auto& kv : user_pinned_) host_free(reinterpret_cast<void*>(kv.first));
+    user_pinned_.clear();
     if (!host_only()) {
         for (auto e : prof_events_) (void)hipEventDestroy(e);
         if (h2d_stage_) (void)hipHostFree(h2d_stage_);
@@ -430,6 +432,24 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
     int r = resolve(m, src, bytes, false, &p);
     if (r) return r;
     if (!host_only() && bytes) {
+        // a destination inside a pinned result buffer of ours is written by the device itself
+        auto ub = user_pinned_.upper_bound(reinterpret_cast<uintptr_t>(dst));
+        if (ub != user_pinned_.begin()) {
+            --ub;
+            const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
+            if (d >= ub->first && d - ub->first + bytes <= ub->second) {
+                void* dst_dev = nullptr;
+                if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+                    hipHostGetDevicePointer(&dst_dev, dst, 0) == hipSuccess && dst_dev) {
+                    int kr = tpk::launch_copy(p, dst_dev, bytes, compute_);
+                    if (kr) return kr;
+                } else {
+                    HIPCHK(hipMemcpyAsync(dst, p, bytes, hipMemcpyDeviceToHost, compute_));
+                }
+                d2h_seen_ = true;
+                return 0;
+            }
+        }
         if (d2h_pos_ + bytes > d2h_cap_) {
             if (!pending_d2h_.empty()) {
                 // pending copies still point into the old buffer: deliver them first
@@ -456,6 +476,26 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
         d2h_pos_ = align_up(d2h_pos_ + bytes, 256);
     }
     d2h_seen_ = true;
+    return 0;
+}
+
+int Engine::user_host_alloc(uint64_t bytes, void** ptr) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!ptr || bytes == 0) return TP_EINVAL;
+    void* p = host_alloc(bytes);
+    if (!p) return TP_ENOMEM;
+    user_pinned_[reinterpret_cast<uintptr_t>(p)] = bytes;
+    *ptr = p;
+    return 0;
+}
+
+int Engine::user_host_free(void* ptr) {
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = user_pinned_.find(reinterpret_cast<uintptr_t>(ptr));
+    if (it == user_pinned_.end()) return TP_EINVAL;
+    if (!host_only()) (void)hipStreamSynchronize(compute_);  // a result may still be on its way into it
+    host_free(ptr);
+    user_pinned_.erase(it);
     return 0;
 }
 

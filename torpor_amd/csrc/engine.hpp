@@ -162,6 +162,8 @@ public:
     int op_free(int client, uint64_t va);
     int op_h2d(int client, uint64_t dst, const void* src, uint64_t bytes);
     int op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes);
+    int user_host_alloc(uint64_t bytes, void** ptr);
+    int user_host_free(void* ptr);
     int op_d2h(int client, void* dst, uint64_t src, uint64_t bytes);
     int op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes);
     int op_memset(int client, uint64_t dst, int value, uint64_t bytes);
@@ -287,6 +289,7 @@ private:
 
     uint8_t* h2d_stage_ = nullptr;
     uint64_t h2d_cap_ = 0, h2d_pos_ = 0;
+    std::map<uintptr_t, uint64_t> user_pinned_;  // result buffers handed out by user_host_alloc: base -> bytes
     uint8_t* d2h_stage_ = nullptr;
     uint64_t d2h_cap_ = 0, d2h_pos_ = 0;
     std::vector<PendingD2H> pending_d2h_;

@@ -137,14 +137,16 @@ class Function:
         finally:
             self.batch, self.out_specs = saved
 
-    def pack(self, inputs):
+    def pack(self, inputs, pinned=False):
         """Request inputs as one byte string and one output buffer with per-output views,
-        in the order the recorded H2D / D2H copies consume them."""
+        in the order the recorded H2D / D2H copies consume them.  `pinned`: the output buffer is
+        pinned memory of the server (results land in it without a staging copy; it lives as long as
+        the server)."""
         specs = self.input_specs()
         parts = [np.ascontiguousarray(a, dtype=dt).reshape(-1).view(np.uint8) for a, (_, dt) in zip(inputs, specs)]
         packed = np.concatenate(parts) if len(parts) > 1 else parts[0]
         sizes = [int(np.prod(shape)) * np.dtype(dt).itemsize for shape, dt in self.out_specs]
-        outbuf = np.empty(sum(sizes), dtype=np.uint8)
+        outbuf = self.s.host_empty(sum(sizes)) if pinned else np.empty(sum(sizes), dtype=np.uint8)
         views, pos = [], 0
         for (shape, dt), n in zip(self.out_specs, sizes):
             views.append(outbuf[pos:pos + n].view(dt).reshape(shape))

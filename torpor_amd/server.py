@@ -223,6 +223,14 @@ class Server:
     def last_kernel(self):
         return self._l.tp_last_kernel().decode()
 
+    def host_empty(self, nbytes):
+        """uint8 array over pinned host memory of the server: a request result whose destination lies
+        in it is written by the device directly.  Valid until the server is closed."""
+        p = C.c_void_p()
+        _chk(self._l.tp_host_alloc(self._h, max(1, nbytes), C.byref(p)), "tp_host_alloc")
+        buf = (C.c_uint8 * max(1, nbytes)).from_address(p.value)
+        return np.frombuffer(buf, dtype=np.uint8, count=nbytes)
+
     def measure_h2d(self, nbytes=256 << 20, iters=10):
         g = C.c_double()
         _chk(self._l.tp_measure_h2d(self._h, nbytes, iters, C.byref(g)), "tp_measure_h2d")
