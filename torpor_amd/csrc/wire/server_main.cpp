@@ -61,6 +61,23 @@ struct Server {
     std::map<int, std::vector<StagedD2H>> staged;        // client id -> D2H copies awaiting the next sync
     std::vector<zmtp::Conn*> waiting_ack;                // REP peers whose request was queued
     bool verbose = false;
+    // Replay results are received in pinned memory of the engine (tp_host_alloc): the device writes
+    // them there itself, and the reply message is built from it.  Grown on demand, freed with the engine.
+    uint8_t* reply_buf = nullptr;
+    uint64_t reply_cap = 0;
+    uint8_t* reply_room(uint64_t bytes) {
+        if (bytes <= reply_cap) return reply_buf;
+        if (reply_buf) (void)tp_host_free(eng, reply_buf);
+        reply_buf = nullptr;
+        reply_cap = 0;
+        void* p = nullptr;
+        uint64_t cap = 1ull << 20;
+        while (cap < bytes) cap *= 2;
+        if (tp_host_alloc(eng, cap, &p) != 0) return nullptr;
+        reply_buf = static_cast<uint8_t*>(p);
+        reply_cap = cap;
+        return reply_buf;
+    }
 };
 
 std::string generic_response(int err) {
@@ -367,15 +384,15 @@ bool handle_query(Server& S, int type, const pb::View& q, int client, std::strin
                 else if (f == 2 && r.read_u64(wt, &u)) out_bytes = u;
                 else if (f != 2) r.skip(wt);
             }
-            std::vector<uint8_t> out;
             int err = out_bytes > (1ull << 32) ? TP_EINVAL : 0;
+            uint8_t* out = nullptr;
             if (!err) {
-                out.resize(out_bytes);
-                err = tp_replay(S.eng, client, payload.p, payload.n, out.data(), out_bytes);
+                out = S.reply_room(out_bytes ? out_bytes : 1);
+                err = out ? tp_replay(S.eng, client, payload.p, payload.n, out, out_bytes) : TP_ENOMEM;
             }
             pb::Writer w;
             w.i32(1, err);
-            if (!err) w.bytes(2, out.data(), out.size());
+            if (!err) w.bytes(2, out, out_bytes);
             *reply = w.out;
             return true;
         }
