@@ -100,11 +100,12 @@ def test_graph_replays_match_eager_and_follow_the_placement(monkeypatch):
 
 
 @pytest.mark.parametrize("host_gather", [True, False])
-def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather):
+def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather, monkeypatch):
     """The word-embedding table is looked up by row, so it is the last tensor of the image, and a
     cold request reads its rows from the pinned host store while the table is still on its way;
     with the option off the lookup waits for the table.  Either way cold answers equal warm ones
     bit for bit and the device copy ends up identical to the host store."""
+    monkeypatch.delenv("TORPOR_HOST_GATHER", raising=False)   # the flag under test, not the environment
     cfg = dict(layers=2, hidden=512, heads=8, ffn=1024)
     weights = bert.init_weights(seed=21, vocab=30522, max_pos=128, cfg=cfg)   # table: 62 MB of 71
     ids = np.random.default_rng(4).integers(0, 30522, (2, 64))
@@ -128,11 +129,12 @@ def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather
 
 
 @pytest.mark.parametrize("pack", [True, False])
-def test_packed_transfer_is_lossless_for_any_bits(pack):
+def test_packed_transfer_is_lossless_for_any_bits(pack, monkeypatch):
     """Weights cross the link in the 28-bit format and are expanded on the device.  Doctored tensors
     (zeros, denormals, infinities, NaNs, exponents spread over 60 binades, one tensor of arbitrary
     bits, one of zeros only) must come back bit for bit, swap-in after swap-in, and a request must
     answer as it did at registration."""
+    monkeypatch.delenv("TORPOR_PACK", raising=False)
     weights = resnet.init_weights("resnet50", seed=5)
     rng = np.random.default_rng(6)
     flat = weights["layer1.0.conv1.weight"].reshape(-1).view(np.uint32)
