@@ -395,6 +395,11 @@ int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* packed, int3
                   uint64_t pair_cap, uint64_t* n_pairs);
 int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
                     uint32_t* words);
+/* The same expansion by the device kernels a swap-in uses (through the engine's workspace, on the compute
+ * stream, synchronous): lets the kernels be checked against tp_unpack_words on arbitrary input.
+ * TP_EINVAL when packed form, pairs and result do not fit the workspace together. */
+int tp_unpack_words_device(tp_server* s, const uint8_t* packed, uint64_t n_words, int32_t base,
+                           const uint32_t* pairs, uint64_t n_pairs, uint32_t* words);
 
 #ifdef __cplusplus
 }

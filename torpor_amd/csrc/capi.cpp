@@ -715,4 +715,15 @@ int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const
     TP_GUARD_END
 }
 
+int tp_unpack_words_device(tp_server* s, const uint8_t* packed, uint64_t n_words, int32_t base,
+                           const uint32_t* pairs, uint64_t n_pairs, uint32_t* words) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    if (!packed || (!words && n_words) || base < 0 || base > 255 || (!pairs && n_pairs)) return TP_EINVAL;
+    for (uint64_t i = 0; i < n_pairs; ++i)
+        if (pairs[2 * i] >= n_words) return TP_EINVAL;
+    return E.unpack_on_device(packed, n_words, base, pairs, n_pairs, words);
+    TP_GUARD_END
+}
+
 }  // extern "C"

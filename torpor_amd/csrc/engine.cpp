@@ -89,6 +89,25 @@ int Engine::init() {
             d2h_kernel_ = 0;
         }
     }
+    {
+        // First use of the copy streams (queue and copy-engine set-up, about 6 ms) happens here
+        // rather than inside the first swap-in: a few copies on both streams, issued as a swap-in
+        // issues them, into the upper half of the workspace.
+        uint8_t* ws = reinterpret_cast<uint8_t*>(workspace_);
+        const uint64_t half = cfg_.workspace_bytes / 2;
+        const uint64_t n = std::min<uint64_t>(std::min<uint64_t>(half / 2, h2d_cap_ / 2), 8ull << 20) & ~uint64_t(255);
+        if (n) {
+            for (int rep = 0; rep < 24; ++rep) {
+                HIPCHK(hipMemcpyAsync(ws + half, h2d_stage_, n, hipMemcpyHostToDevice, copy_));
+                HIPCHK(hipMemcpyAsync(ws + half + n, h2d_stage_ + n, n, hipMemcpyHostToDevice, copy2_));
+            }
+            (void)tpk::launch_copy(ws + half, ws + half + n, 4096, decode_);
+            HIPCHK(hipStreamSynchronize(copy_));
+            HIPCHK(hipStreamSynchronize(copy2_));
+            HIPCHK(hipStreamSynchronize(decode_));
+            HIPCHK(hipMemset(ws + half, 0, 2 * n));  // the workspace is handed to the kernels zeroed
+        }
+    }
     copy_thread_ = std::thread(&Engine::copy_main, this);
     return 0;
 }
@@ -496,6 +515,45 @@ int Engine::user_host_free(void* ptr) {
     if (!host_only()) (void)hipStreamSynchronize(compute_);  // a result may still be on its way into it
     host_free(ptr);
     user_pinned_.erase(it);
+    return 0;
+}
+
+// Test hook: the expansion kernels of a packed swap-in on caller-supplied input.
+int Engine::unpack_on_device(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs,
+                             uint64_t n_pairs, uint32_t* words) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (host_only()) return TP_ENODEV;
+    if (n_words == 0) return 0;
+    if (active_ >= 0) return TP_EBUSY;  // the workspace belongs to the running request
+    const uint64_t pb = align_up(packed_bytes(n_words), 256), eb = align_up(n_pairs * 8, 256), wb = align_up(n_words * 4, 256);
+    const uint64_t room = cfg_.workspace_bytes - 4096;
+    if (pb + eb + wb > room) return TP_EINVAL;
+    uint8_t* d_packed = reinterpret_cast<uint8_t*>(workspace_) + 4096;
+    uint8_t* d_pairs = d_packed + pb;
+    uint8_t* d_words = d_pairs + eb;
+    HIPCHK(hipStreamSynchronize(compute_));
+    HIPCHK(hipMemcpy(d_packed, packed, packed_bytes(n_words), hipMemcpyHostToDevice));
+    if (n_pairs) HIPCHK(hipMemcpy(d_pairs, pairs, n_pairs * 8, hipMemcpyHostToDevice));
+    HIPCHK(hipMemset(d_words, 0xA5, wb));
+    tpk::UnpackArgs a;
+    a.n = 1;
+    a.piece[0].src = d_packed;
+    a.piece[0].dst = d_words;
+    a.piece[0].bytes = n_words * 4;
+    a.piece[0].base = base;
+    a.piece[0].first_block = 0;
+    int r = tpk::launch_unpack(a, compute_);
+    if (!r && n_pairs)
+        r = tpk::launch_patch(reinterpret_cast<const uint32_t*>(d_pairs), n_pairs, reinterpret_cast<uint32_t*>(d_words), compute_);
+    if (r) return r;
+    HIPCHK(hipStreamSynchronize(compute_));
+    // one word past the end must be untouched (the last group is written word by word)
+    uint32_t guard = 0;
+    if (n_words * 4 < wb) {
+        HIPCHK(hipMemcpy(&guard, d_words + n_words * 4, 4, hipMemcpyDeviceToHost));
+        if (guard != 0xA5A5A5A5u) return TP_EFAULT;
+    }
+    HIPCHK(hipMemcpy(words, d_words, n_words * 4, hipMemcpyDeviceToHost));
     return 0;
 }
 

@@ -164,6 +164,8 @@ public:
     int op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes);
     int user_host_alloc(uint64_t bytes, void** ptr);
     int user_host_free(void* ptr);
+    int unpack_on_device(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
+                         uint32_t* words);
     int op_d2h(int client, void* dst, uint64_t src, uint64_t bytes);
     int op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes);
     int op_memset(int client, uint64_t dst, int value, uint64_t bytes);
