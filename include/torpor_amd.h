@@ -60,7 +60,7 @@ typedef struct tp_server tp_server;
 #define TP_FLAG_HOST_ONLY 1 /* no HIP calls: pool/LRU/state-machine logic only (CPU tests) */
 #define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
 #define TP_FLAG_NO_HOST_GATHER 4 /* embedding lookups always wait for their table's transfer group, as env TORPOR_HOST_GATHER=0 */
-#define TP_FLAG_NO_PACK 8 /* weights cross the link as they are instead of in the 28-bit transfer format, as env TORPOR_PACK=0 */
+#define TP_FLAG_NO_PACK 8 /* weights cross the link as they are instead of in the packed transfer format, as env TORPOR_PACK=0 */
 
 /* ---- activation / epilogue ---- */
 #define TP_ACT_NONE 0
@@ -176,7 +176,7 @@ typedef struct tp_model_info {
 
 typedef struct tp_swap_stats {
     uint64_t bytes;      /* bytes the last swap-in of this model moved over the host link (below the image size when
-                            tensors travel in the 28-bit transfer format) */
+                            tensors travel in the packed transfer format) */
     double copy_ms;      /* first copy issued -> last group in place (landed and, if packed, expanded) */
     double alloc_us;     /* host time to (re)acquire pool extents ("CheckMalloc", memory_manager.hpp:499-501) */
     double evict_us;     /* host time of the last swap-out (memory_manager.hpp:258) */
@@ -378,28 +378,38 @@ int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t 
                     int32_t* src_gpu, int32_t* status);
 
 /* ------------------------------------------------------------------ transfer format
- * The lossless 28-bit format in which compressible weight tensors cross the host link
- * (TP_FLAG_NO_PACK switches it off); no counterpart in the reference, which sends weights as they
- * are (memory_manager.hpp:378-409).  A tensor is n 32-bit words of any content.  Packed: groups of
- * 8 words in 28 bytes -- eight 24-bit little-endian fields (sign << 23 | mantissa), then one 32-bit
- * word of eight 4-bit codes, word j in bits 4j..4j+3; code c < 15 stands for exponent base + c, code
- * 15 for a word outside the window, listed as an (index, bits) pair.  The last group is zero-padded.
- * Exposed so that the format can be checked on the host; the engine applies it on its own.
- *   tp_pack_bound   bytes of the packed form of n words
- *   tp_pack_words   chooses the window of 15 exponents holding the most words, packs, and writes up
- *                   to pair_cap pairs; returns 0, or TP_ENOMEM when there are more pairs than that
- *                   (*n_pairs then still holds the count)
- *   tp_unpack_words the inverse, pairs applied */
+ * The lossless format in which compressible weight tensors cross the host link (TP_FLAG_NO_PACK
+ * switches it off); no counterpart in the reference, which sends weights as they are
+ * (memory_manager.hpp:378-409).  A tensor is n 32-bit words of any content.
+ *   payload: units of 64 words in 216 bytes -- eight groups of eight 24-bit little-endian fields
+ *            (sign << 23 | mantissa), then 24 bytes of exponent codes: group g of the unit in bits
+ *            24g..24g+23, word j of the group in bits 3j..3j+2 of those.  Code c < 7 stands for
+ *            exponent base + c, code 7 for "next byte of the extension stream".  The last unit is
+ *            padded with zero words (code 0).
+ *   extension stream: the exponent bytes of the words with code 7, in word order.
+ *   block table: entry b = number of extension bytes that belong to words before word 2048 b
+ *            (the device expands blocks of 2048 words independently).
+ * Exposed so that the format can be checked on the host and the device kernel on its own; the engine
+ * applies it by itself.
+ *   tp_pack_bound / tp_pack_blocks   payload bytes / block-table entries for n words
+ *   tp_pack_words    chooses the window of 7 exponents that holds the most words and packs; returns
+ *                    TP_ENOMEM when the extension stream needs more than ext_cap bytes (*n_ext still
+ *                    holds the count)
+ *   tp_unpack_words  the inverse on the host
+ *   tp_unpack_words_device  the inverse by the kernel a swap-in uses (through the engine's workspace,
+ *                    synchronous), for words [w_from, w_to) only -- w_from a multiple of 64, w_to a
+ *                    multiple of 64 or n_words -- as for a transfer group that ends inside a tensor;
+ *                    the other words come back as 0xA5A5A5A5.  TP_EINVAL when it does not fit the
+ *                    workspace. */
 uint64_t tp_pack_bound(uint64_t n_words);
-int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* packed, int32_t* base, uint32_t* pairs,
-                  uint64_t pair_cap, uint64_t* n_pairs);
-int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
+uint64_t tp_pack_blocks(uint64_t n_words);
+int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* payload, int32_t* base, uint8_t* ext,
+                  uint64_t ext_cap, uint64_t* n_ext, uint32_t* block_tab);
+int tp_unpack_words(const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext, uint64_t n_ext,
                     uint32_t* words);
-/* The same expansion by the device kernels a swap-in uses (through the engine's workspace, on the compute
- * stream, synchronous): lets the kernels be checked against tp_unpack_words on arbitrary input.
- * TP_EINVAL when packed form, pairs and result do not fit the workspace together. */
-int tp_unpack_words_device(tp_server* s, const uint8_t* packed, uint64_t n_words, int32_t base,
-                           const uint32_t* pairs, uint64_t n_pairs, uint32_t* words);
+int tp_unpack_words_device(tp_server* s, const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext,
+                           uint64_t n_ext, const uint32_t* block_tab, uint64_t w_from, uint64_t w_to,
+                           uint32_t* words);
 
 #ifdef __cplusplus
 }

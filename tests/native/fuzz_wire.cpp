@@ -199,21 +199,25 @@ int main() {
     }
     tp_sched_destroy(sc);
 
-    // the 28-bit transfer format: exactly sized buffers, every length, weight-like and arbitrary words
+    // the packed transfer format: exactly sized buffers, every length, weight-like and arbitrary words
     for (int it = 0; it < 3000; ++it) {
-        const uint64_t n = rng() % 300;
-        std::vector<uint32_t> w(n), back(n, 0xDEADBEEFu), pairs(2 * n);
+        const uint64_t n = it < 2990 ? rng() % 300 : 2040 + rng() % 4200;
+        std::vector<uint32_t> w(n), back(n, 0xDEADBEEFu), tab((size_t)tp_pack_blocks(n));
         const int kind = (int)(rng() % 3);
         for (auto& v : w)
             v = kind == 0 ? (uint32_t)rng()
                           : (uint32_t)(((rng() % 2) << 31) | ((uint64_t)(120 + rng() % (kind == 1 ? 6 : 40)) << 23) | (rng() & 0x7FFFFF));
-        std::vector<uint8_t> packed((size_t)tp_pack_bound(n));
+        std::vector<uint8_t> payload((size_t)tp_pack_bound(n)), ext(n);
         int32_t base = -1;
-        uint64_t np = 0;
+        uint64_t ne = 0;
         uint8_t dummy = 0;
-        if (tp_pack_words(w.data(), n, packed.empty() ? &dummy : packed.data(), &base, pairs.data(), n, &np) != 0) return 10;
-        if (tp_unpack_words(packed.empty() ? &dummy : packed.data(), n, base, pairs.data(), np, back.data()) != 0) return 11;
+        uint32_t dummy32 = 0;
+        if (tp_pack_words(w.data(), n, payload.empty() ? &dummy : payload.data(), &base, ext.data(), n, &ne,
+                          tab.empty() ? &dummy32 : tab.data()) != 0)
+            return 10;
+        if (tp_unpack_words(payload.empty() ? &dummy : payload.data(), n, base, ext.data(), ne, back.data()) != 0) return 11;
         if (w != back) return 12;
+        if (ne && tp_unpack_words(payload.data(), n, base, ext.data(), ne - 1, back.data()) == 0) return 13;  // short stream
     }
     std::printf("fuzz ok: %ld messages\n", handled);
     return 0;

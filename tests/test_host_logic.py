@@ -354,8 +354,9 @@ def test_pinned_result_buffers_are_tracked(host_server):
     assert L.tp_host_free(h, p) == 0 and L.tp_host_free(h, p) == -22
     # the device expansion hook needs a device
     w = np.zeros(8, np.uint32)
-    packed = np.zeros(28, np.uint8)
-    assert L.tp_unpack_words_device(h, packed.ctypes.data, 8, 0, None, 0, w.ctypes.data) == -19
+    payload = np.zeros(216, np.uint8)
+    tab = np.zeros(1, np.uint32)
+    assert L.tp_unpack_words_device(h, payload.ctypes.data, 8, 0, None, 0, tab.ctypes.data, 0, 8, w.ctypes.data) == -19
 
 
 def test_request_timeout_completes_the_request(host_server):

@@ -181,9 +181,10 @@ SYMBOLS = {
     "tp_host_alloc": (C.c_int, [_P, _U64, C.POINTER(_P)]),
     "tp_host_free": (C.c_int, [_P, _P]),
     "tp_pack_bound": (_U64, [_U64]),
-    "tp_pack_words": (C.c_int, [_P, _U64, _P, C.POINTER(_I32), _P, _U64, C.POINTER(_U64)]),
+    "tp_pack_blocks": (_U64, [_U64]),
+    "tp_pack_words": (C.c_int, [_P, _U64, _P, C.POINTER(_I32), _P, _U64, C.POINTER(_U64), _P]),
     "tp_unpack_words": (C.c_int, [_P, _U64, _I32, _P, _U64, _P]),
-    "tp_unpack_words_device": (C.c_int, [_P, _P, _U64, _I32, _P, _U64, _P]),
+    "tp_unpack_words_device": (C.c_int, [_P, _P, _U64, _I32, _P, _U64, _P, _U64, _U64, _P]),
 }
 
 _lib = None

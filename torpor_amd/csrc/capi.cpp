@@ -681,48 +681,47 @@ int tp_sched_decide(tp_sched* s, int32_t policy, const char* function, uint32_t 
 
 // ------------------------------------------------------------------ transfer format
 uint64_t tp_pack_bound(uint64_t n_words) { return tp::packed_bytes(n_words); }
+uint64_t tp_pack_blocks(uint64_t n_words) { return tp::packed_blocks(n_words); }
 
-int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* packed, int32_t* base, uint32_t* pairs,
-                  uint64_t pair_cap, uint64_t* n_pairs) {
+int tp_pack_words(const uint32_t* words, uint64_t n_words, uint8_t* payload, int32_t* base, uint8_t* ext,
+                  uint64_t ext_cap, uint64_t* n_ext, uint32_t* block_tab) {
     TP_GUARD_BEGIN
-    if ((!words && n_words) || !packed || !base || (!pairs && pair_cap) || n_words > 0xFFFFFFFFull) return TP_EINVAL;
+    if ((!words && n_words) || !payload || !base || (!ext && ext_cap) || (!block_tab && n_words)) return TP_EINVAL;
     uint32_t b = 0;
     uint64_t outside = 0;
     tp::choose_window(words, n_words, &b, &outside);
-    std::vector<tp::Escape> esc;
-    tp::pack_words(words, n_words, b, packed, 0, &esc);
+    std::memset(payload, 0, tp::packed_bytes(n_words));
+    std::vector<uint8_t> e;
+    tp::pack_words(words, n_words, b, payload, &e, block_tab);
     *base = (int32_t)b;
-    if (n_pairs) *n_pairs = esc.size();
-    if (esc.size() > pair_cap) return TP_ENOMEM;
-    for (size_t i = 0; i < esc.size(); ++i) {
-        pairs[2 * i] = esc[i].index;
-        pairs[2 * i + 1] = esc[i].bits;
-    }
+    if (n_ext) *n_ext = e.size();
+    if (e.size() > ext_cap) return TP_ENOMEM;
+    if (!e.empty()) std::memcpy(ext, e.data(), e.size());
     return 0;
     TP_GUARD_END
 }
 
-int tp_unpack_words(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
+int tp_unpack_words(const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext, uint64_t n_ext,
                     uint32_t* words) {
     TP_GUARD_BEGIN
-    if (!packed || (!words && n_words) || base < 0 || base > 255 || (!pairs && n_pairs)) return TP_EINVAL;
-    tp::unpack_words(packed, n_words, (uint32_t)base, words);
-    for (uint64_t i = 0; i < n_pairs; ++i) {
-        if (pairs[2 * i] >= n_words) return TP_EINVAL;
-        words[pairs[2 * i]] = pairs[2 * i + 1];
-    }
-    return 0;
+    if (!payload || (!words && n_words) || base < 0 || base > 255 || (!ext && n_ext)) return TP_EINVAL;
+    return tp::unpack_words(payload, n_words, (uint32_t)base, ext, n_ext, words) == UINT64_MAX ? TP_EINVAL : 0;
     TP_GUARD_END
 }
 
-int tp_unpack_words_device(tp_server* s, const uint8_t* packed, uint64_t n_words, int32_t base,
-                           const uint32_t* pairs, uint64_t n_pairs, uint32_t* words) {
+int tp_unpack_words_device(tp_server* s, const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext,
+                           uint64_t n_ext, const uint32_t* block_tab, uint64_t w_from, uint64_t w_to,
+                           uint32_t* words) {
     TP_GUARD_BEGIN
     ENG(s);
-    if (!packed || (!words && n_words) || base < 0 || base > 255 || (!pairs && n_pairs)) return TP_EINVAL;
-    for (uint64_t i = 0; i < n_pairs; ++i)
-        if (pairs[2 * i] >= n_words) return TP_EINVAL;
-    return E.unpack_on_device(packed, n_words, base, pairs, n_pairs, words);
+    if (!payload || (!words && n_words) || base < 0 || base > 255 || (!ext && n_ext) || (!block_tab && n_words))
+        return TP_EINVAL;
+    if (w_from > w_to || w_to > n_words || (w_from & 63) || ((w_to & 63) && w_to != n_words)) return TP_EINVAL;
+    {  // the stream must hold what the codes ask for: expand on the host first
+        std::vector<uint32_t> probe(n_words);
+        if (tp::unpack_words(payload, n_words, (uint32_t)base, ext, n_ext, probe.data()) == UINT64_MAX) return TP_EINVAL;
+    }
+    return E.unpack_on_device(payload, n_words, base, ext, n_ext, block_tab, w_from, w_to, words);
     TP_GUARD_END
 }
 

@@ -518,43 +518,45 @@ int Engine::user_host_free(void* ptr) {
     return 0;
 }
 
-// Test hook: the expansion kernels of a packed swap-in on caller-supplied input.
-int Engine::unpack_on_device(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs,
-                             uint64_t n_pairs, uint32_t* words) {
+// Test hook: the expansion kernel of a packed swap-in on caller-supplied input.  Words outside
+// [w_from, w_to) come back as 0xA5A5A5A5.
+int Engine::unpack_on_device(const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext, uint64_t n_ext,
+                             const uint32_t* block_tab, uint64_t w_from, uint64_t w_to, uint32_t* words) {
     std::lock_guard<std::mutex> lk(mu_);
     if (host_only()) return TP_ENODEV;
     if (n_words == 0) return 0;
     if (active_ >= 0) return TP_EBUSY;  // the workspace belongs to the running request
-    const uint64_t pb = align_up(packed_bytes(n_words), 256), eb = align_up(n_pairs * 8, 256), wb = align_up(n_words * 4, 256);
-    const uint64_t room = cfg_.workspace_bytes - 4096;
-    if (pb + eb + wb > room) return TP_EINVAL;
-    uint8_t* d_packed = reinterpret_cast<uint8_t*>(workspace_) + 4096;
-    uint8_t* d_pairs = d_packed + pb;
-    uint8_t* d_words = d_pairs + eb;
+    const uint64_t pb = align_up(packed_bytes(n_words), 256), eb = align_up(n_ext + 1, 256),
+                   tb = align_up(packed_blocks(n_words) * 4, 256), wb = align_up(n_words * 4 + 4, 256);
+    if (cfg_.workspace_bytes < 8192 || pb + eb + tb + wb > cfg_.workspace_bytes - 4096) return TP_EINVAL;
+    uint8_t* d_payload = reinterpret_cast<uint8_t*>(workspace_) + 4096;
+    uint8_t* d_ext = d_payload + pb;
+    uint8_t* d_tab = d_ext + eb;
+    uint8_t* d_words = d_tab + tb;
     HIPCHK(hipStreamSynchronize(compute_));
-    HIPCHK(hipMemcpy(d_packed, packed, packed_bytes(n_words), hipMemcpyHostToDevice));
-    if (n_pairs) HIPCHK(hipMemcpy(d_pairs, pairs, n_pairs * 8, hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(d_payload, payload, packed_bytes(n_words), hipMemcpyHostToDevice));
+    if (n_ext) HIPCHK(hipMemcpy(d_ext, ext, n_ext, hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(d_tab, block_tab, packed_blocks(n_words) * 4, hipMemcpyHostToDevice));
     HIPCHK(hipMemset(d_words, 0xA5, wb));
     tpk::UnpackArgs a;
     a.n = 1;
-    a.piece[0].src = d_packed;
+    a.piece[0].src = d_payload;
     a.piece[0].dst = d_words;
-    a.piece[0].bytes = n_words * 4;
+    a.piece[0].bytes = 0;
+    a.piece[0].w_from = w_from;
+    a.piece[0].w_to = w_to;
+    a.piece[0].ext = d_ext;
+    a.piece[0].tab = reinterpret_cast<const uint32_t*>(d_tab);
     a.piece[0].base = base;
     a.piece[0].first_block = 0;
     int r = tpk::launch_unpack(a, compute_);
-    if (!r && n_pairs)
-        r = tpk::launch_patch(reinterpret_cast<const uint32_t*>(d_pairs), n_pairs, reinterpret_cast<uint32_t*>(d_words), compute_);
     if (r) return r;
     HIPCHK(hipStreamSynchronize(compute_));
-    // one word past the end must be untouched (the last group is written word by word)
-    uint32_t guard = 0;
-    if (n_words * 4 < wb) {
-        HIPCHK(hipMemcpy(&guard, d_words + n_words * 4, 4, hipMemcpyDeviceToHost));
-        if (guard != 0xA5A5A5A5u) return TP_EFAULT;
-    }
     HIPCHK(hipMemcpy(words, d_words, n_words * 4, hipMemcpyDeviceToHost));
-    return 0;
+    uint32_t guard = 0;  // the word past the end must be untouched (the last group is written word by word)
+    HIPCHK(hipMemcpy(&guard, d_words + n_words * 4, 4, hipMemcpyDeviceToHost));
+    HIPCHK(hipMemset(reinterpret_cast<uint8_t*>(workspace_) + 4096, 0, pb + eb + tb + wb));
+    return guard == 0xA5A5A5A5u ? 0 : TP_EFAULT;
 }
 
 int Engine::op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes) {
@@ -734,10 +736,9 @@ void Engine::free_transfer(Model& m) {
     host_free(m.timg);
     m.timg = nullptr;
     m.timg_bytes = 0;
-    m.esc_index.clear();
     for (auto& p : m.params) {
         p.pack_base = -1;
-        p.t_off = 0;
+        p.t_off = p.tab_off = p.ext_off = 0;
     }
 }
 
@@ -756,24 +757,28 @@ int Engine::build_transfer(Model& m) {
     // DenseNet-169/201: cold equal or up to 0.04 ms slower with the format than without).
     if (m.warm_us > 0 && (double)m.image_bytes / 54.0e3 < 0.8 * m.warm_us) return 0;
     std::vector<int32_t> base(m.params.size(), -1);
-    uint64_t esc_total = 0;
-    for (uint32_t idx : m.image_order) {
-        const Param& p = m.params[idx];
-        if (p.size % 4 != 0 || p.size < 4096) continue;
-        uint32_t b = 0;
-        uint64_t outside = 0;
-        choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), p.size / 4, &b, &outside);
-        if (outside * 8 + packed_bytes(p.size / 4) <= p.size - p.size / 20) {
-            base[idx] = (int32_t)b;
-            esc_total += outside;
-        }
-    }
-    uint64_t off = align_up(esc_total * 8, kTensorAlign);
+    std::vector<uint64_t> n_ext(m.params.size(), 0), tab_off(m.params.size(), 0), ext_off(m.params.size(), 0);
     std::vector<uint64_t> t_off(m.params.size(), 0);
+    uint64_t off = 0;
     for (uint32_t idx : m.image_order) {
         const Param& p = m.params[idx];
         t_off[idx] = off;
-        off = align_up(off + (base[idx] >= 0 ? packed_bytes(p.size / 4) : p.size), kTensorAlign);
+        if (p.size % 4 == 0 && p.size >= 4096) {
+            uint32_t b = 0;
+            uint64_t outside = 0;
+            const uint64_t nw = p.size / 4;
+            choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), nw, &b, &outside);
+            if (packed_bytes(nw) + packed_blocks(nw) * 4 + outside <= p.size - p.size / 20) {
+                // a packed tensor's region: block table, extension stream, payload -- the first two
+                // arrive with the tensor's first bytes, whichever transfer group carries them
+                base[idx] = (int32_t)b;
+                n_ext[idx] = outside;
+                tab_off[idx] = off;
+                ext_off[idx] = off + packed_blocks(nw) * 4;
+                t_off[idx] = align_up(ext_off[idx] + outside, kTensorAlign);
+            }
+        }
+        off = align_up(t_off[idx] + (base[idx] >= 0 ? packed_bytes(p.size / 4) : p.size), kTensorAlign);
     }
     if (off > m.image_bytes - m.image_bytes / 32) return 0;
     if (off > xfer_stage_cap_) {  // registration time: no swap-in may be using the area while it is replaced
@@ -796,23 +801,28 @@ int Engine::build_transfer(Model& m) {
     uint8_t* t = static_cast<uint8_t*>(host_alloc(off));
     if (!t) return 0;
     std::memset(t, 0, off);
-    std::vector<Escape> esc;
-    esc.reserve(esc_total);
-    static_assert(sizeof(Escape) == 8, "pairs of 32-bit words");
+    std::vector<uint8_t> ext;
     for (uint32_t idx : m.image_order) {
         Param& p = m.params[idx];
         p.t_off = t_off[idx];
         p.pack_base = base[idx];
+        p.tab_off = tab_off[idx];
+        p.ext_off = ext_off[idx];
         const uint8_t* src = m.host_image + p.image_off;
-        if (p.pack_base >= 0)
-            pack_words(reinterpret_cast<const uint32_t*>(src), p.size / 4, (uint32_t)p.pack_base, t + p.t_off,
-                       p.image_off / 4, &esc);
-        else
+        if (p.pack_base >= 0) {
+            ext.clear();
+            pack_words(reinterpret_cast<const uint32_t*>(src), p.size / 4, (uint32_t)p.pack_base, t + p.t_off, &ext,
+                       reinterpret_cast<uint32_t*>(t + p.tab_off));
+            if (ext.size() != n_ext[idx]) {  // the two passes disagree: never send a stream that does not decode
+                host_free(t);
+                free_transfer(m);
+                return 0;
+            }
+            if (!ext.empty()) std::memcpy(t + p.ext_off, ext.data(), ext.size());
+        } else {
             std::memcpy(t + p.t_off, src, p.size);
+        }
     }
-    if (!esc.empty()) std::memcpy(t, esc.data(), esc.size() * sizeof(Escape));
-    m.esc_index.resize(esc.size());
-    for (size_t i = 0; i < esc.size(); ++i) m.esc_index[i] = esc[i].index;
     m.timg = t;
     m.timg_bytes = off;
     return 1;
@@ -826,11 +836,13 @@ uint64_t Engine::xfer_off(const Model& m, uint64_t d) const {
         if (m.params[m.image_order[mid]].image_off <= d) lo = mid + 1;
         else hi = mid;
     }
-    if (lo == 0) return m.image_order.empty() ? m.timg_bytes : m.params[m.image_order[0]].t_off;
+    if (lo == 0) return 0;
     const Param& p = m.params[m.image_order[lo - 1]];
     const uint64_t rel = d - p.image_off;
-    if (rel >= p.size) return lo < m.image_order.size() ? m.params[m.image_order[lo]].t_off : m.timg_bytes;
-    return p.t_off + (p.pack_base >= 0 ? rel / 32 * 28 : rel);
+    auto region = [](const Param& q) { return q.pack_base >= 0 ? q.tab_off : q.t_off; };
+    if (rel >= p.size) return lo < m.image_order.size() ? region(m.params[m.image_order[lo]]) : m.timg_bytes;
+    if (rel == 0) return region(p);
+    return p.t_off + (p.pack_base >= 0 ? rel / 256 * kPackUnitBytes : rel);
 }
 
 // One transfer group of a packed swap-in: DMA into the staging area, then, on the expansion stream,
@@ -862,13 +874,25 @@ int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hi
         if (p.image_off >= end) break;
         const uint64_t from = std::max(beg, p.image_off), to = std::min(end, p.image_off + p.size);
         if (to <= from) continue;
-        const uint64_t rel = from - p.image_off;
         tpk::UnpackPiece& pc = a.piece[a.n++];
-        pc.src = xfer_stage_ + p.t_off + (p.pack_base >= 0 ? rel / 32 * 28 : rel);
-        pc.dst = m.w_dev + from;
-        pc.bytes = to - from;
         pc.base = p.pack_base;
         pc.first_block = 0;
+        if (p.pack_base >= 0) {
+            pc.src = xfer_stage_ + p.t_off;
+            pc.dst = m.w_dev + p.image_off;
+            pc.bytes = 0;
+            pc.w_from = (from - p.image_off) / 4;
+            pc.w_to = (to - p.image_off) / 4;
+            pc.ext = xfer_stage_ + p.ext_off;
+            pc.tab = reinterpret_cast<const uint32_t*>(xfer_stage_ + p.tab_off);
+        } else {
+            pc.src = xfer_stage_ + p.t_off + (from - p.image_off);
+            pc.dst = m.w_dev + from;
+            pc.bytes = to - from;
+            pc.w_from = pc.w_to = 0;
+            pc.ext = nullptr;
+            pc.tab = nullptr;
+        }
         if (a.n == tpk::kUnpackMaxPieces) {
             r = tpk::launch_unpack(a, decode_);
             a.n = 0;
@@ -876,13 +900,6 @@ int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hi
     }
     if (!r && a.n) r = tpk::launch_unpack(a, decode_);
     if (r) return r;
-    const auto e0 = std::lower_bound(m.esc_index.begin(), m.esc_index.end(), (uint32_t)(beg / 4));
-    const auto e1 = std::lower_bound(e0, m.esc_index.end(), (uint32_t)std::min<uint64_t>(end / 4, UINT32_MAX));
-    if (e1 > e0) {
-        r = tpk::launch_patch(reinterpret_cast<const uint32_t*>(xfer_stage_) + 2 * (e0 - m.esc_index.begin()),
-                              (uint64_t)(e1 - e0), reinterpret_cast<uint32_t*>(m.w_dev), decode_);
-        if (r) return r;
-    }
     return (int)hipEventRecord(m.chunk_ev[i], decode_);
 }
 

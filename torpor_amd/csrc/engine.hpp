@@ -61,8 +61,10 @@ struct Param {  // one uploaded weight tensor (model_repo.hpp:31-36 ModelParamIn
     // last in the weight image, and while its transfer group is still on its way a lookup reads
     // the rows it needs straight from the pinned host store.
     bool gathered = false;
-    // place in the transfer image: as it is (pack_base < 0) or in the 28-bit format with that window base
+    // place in the transfer image: as it is (pack_base < 0) or packed with that window base, its block
+    // table and extension stream right before its payload
     uint64_t t_off = 0;
+    uint64_t tab_off = 0, ext_off = 0;
     int32_t pack_base = -1;
 };
 struct WBlock {
@@ -89,11 +91,10 @@ struct Model {
     uint8_t* host_image = nullptr;
     uint8_t* host_image_dev = nullptr;  // the same memory as kernels address it, null if not mapped
     uint64_t image_bytes = 0, param_bytes = 0;
-    // What a swap-in sends when the weights compress: [words outside their window: (index, bits) pairs]
-    // [tensor payloads in image order].  Null when the image travels as it is.
+    // What a swap-in sends when the weights compress: the tensors in image order, each as it is or as
+    // [block table][extension stream][payload].  Null when the image travels as it is.
     uint8_t* timg = nullptr;
     uint64_t timg_bytes = 0;
-    std::vector<uint32_t> esc_index;   // image word index of every pair, ascending
     std::vector<uint32_t> image_order; // params[] indices by image_off
     std::vector<hipEvent_t> dma_ev;    // transfer group arrived in the staging area (packed transfers)
     int next_rank = 0;
@@ -164,8 +165,8 @@ public:
     int op_d2h_async(int client, void* dst, uint64_t src, uint64_t bytes);
     int user_host_alloc(uint64_t bytes, void** ptr);
     int user_host_free(void* ptr);
-    int unpack_on_device(const uint8_t* packed, uint64_t n_words, int32_t base, const uint32_t* pairs, uint64_t n_pairs,
-                         uint32_t* words);
+    int unpack_on_device(const uint8_t* payload, uint64_t n_words, int32_t base, const uint8_t* ext, uint64_t n_ext,
+                         const uint32_t* block_tab, uint64_t w_from, uint64_t w_to, uint32_t* words);
     int op_d2h(int client, void* dst, uint64_t src, uint64_t bytes);
     int op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes);
     int op_memset(int client, uint64_t dst, int value, uint64_t bytes);

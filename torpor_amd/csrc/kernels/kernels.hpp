@@ -109,14 +109,18 @@ int launch_sum(const float* x, float* y, long n, hipStream_t s);  // y[0] = sum(
 int launch_fill(float* y, float v, long n, hipStream_t s);
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t s);
 
-// Expansion of transfer groups that arrived in the 28-bit weight format (or as they are).  A piece is
-// a run of one tensor: `bytes` bytes at dst, read from src either verbatim (base < 0) or as packed
-// groups of 8 words with exponent window base `base`.  dst and src are 16-byte aligned; a packed
-// piece starts on a group boundary.
+// Expansion of transfer groups into the weight image.  A piece is a run of one tensor.  Raw
+// (base < 0): `bytes` bytes from src to dst, both 16-byte aligned.  Packed (weight_pack.hpp): src is
+// the tensor's payload and dst the tensor's place in the image; words [w_from, w_to) are expanded
+// (w_from a multiple of 64; w_to a multiple of 64 or the tensor's word count), reading the codes of
+// the same 2048-word block before w_from as well, which an earlier transfer group has delivered.
 struct UnpackPiece {
     const uint8_t* src;
     uint8_t* dst;
     uint64_t bytes;
+    uint64_t w_from, w_to;
+    const uint8_t* ext;   // the tensor's extension stream
+    const uint32_t* tab;  // the tensor's block table
     int32_t base;
     uint32_t first_block;  // filled by launch_unpack
 };
@@ -126,7 +130,5 @@ struct UnpackArgs {
     int n = 0;
 };
 int launch_unpack(UnpackArgs& a, hipStream_t s);
-// image32[table[2i]] = table[2i+1] for i in [0, n): the words that did not fit their tensor's window
-int launch_patch(const uint32_t* table, uint64_t n, uint32_t* image32, hipStream_t s);
 
 }  // namespace tpk

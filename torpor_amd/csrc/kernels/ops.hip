@@ -765,18 +765,22 @@ int launch_sum(const float* x, float* y, long n, hipStream_t s) {
     return (int)hipGetLastError();
 }
 
-// ---------------------------------------------------------------- 28-bit weight format
-// One workgroup expands 2048 words (8 KiB of the image): a lane takes one group, 7 dwords in, 8 out.
+// ---------------------------------------------------------------- weight transfer format
+// One workgroup handles one 2048-word block of a tensor (8 KiB of the image): a lane takes one group
+// of eight words, 6 dwords of fields and 24 bits of codes in, two 128-bit stores out.  The rank of a
+// lane's first out-of-window word in the tensor's extension stream is the block-table entry plus a
+// prefix sum over the lanes before it.
 constexpr int kUnpackBlockBytes = 8192;
 __global__ __launch_bounds__(256) void unpack_kernel(const UnpackArgs a) {
     int k = 0;
     while (k + 1 < a.n && a.piece[k + 1].first_block <= blockIdx.x) ++k;
     const UnpackPiece& pc = a.piece[k];
-    const uint64_t off = (uint64_t)(blockIdx.x - pc.first_block) * kUnpackBlockBytes;
-    if (off >= pc.bytes) return;
-    const uint64_t left = pc.bytes - off;
-    uint8_t* __restrict__ dst = pc.dst + off;
+    const uint64_t lb = blockIdx.x - pc.first_block;
     if (pc.base < 0) {
+        const uint64_t off = lb * kUnpackBlockBytes;
+        if (off >= pc.bytes) return;
+        const uint64_t left = pc.bytes - off;
+        uint8_t* __restrict__ dst = pc.dst + off;
         const uint8_t* __restrict__ src = pc.src + off;
         const uint64_t n = left < kUnpackBlockBytes ? left : kUnpackBlockBytes;
         const uint64_t nv = n >> 4;
@@ -785,34 +789,63 @@ __global__ __launch_bounds__(256) void unpack_kernel(const UnpackArgs a) {
         for (uint64_t i = (nv << 4) + threadIdx.x; i < n; i += 256) dst[i] = src[i];
         return;
     }
-    const uint64_t g = threadIdx.x;
-    if (g * 32 >= left) return;
-    const uint32_t* __restrict__ in = reinterpret_cast<const uint32_t*>(pc.src + off / 32 * 28) + g * 7;
-    uint32_t d[7];
-#pragma unroll
-    for (int j = 0; j < 7; ++j) d[j] = in[j];
+    __shared__ uint32_t wave_total[4];
+    const uint64_t bi = pc.w_from / 2048 + lb;
+    const uint64_t word0 = bi * 2048 + (uint64_t)threadIdx.x * 8;
+    const bool have = word0 < pc.w_to;  // this group has arrived
     uint32_t f[8];
-    f[0] = d[0] & 0xFFFFFFu;
-    f[1] = (d[0] >> 24) | ((d[1] & 0xFFFFu) << 8);
-    f[2] = (d[1] >> 16) | ((d[2] & 0xFFu) << 16);
-    f[3] = d[2] >> 8;
-    f[4] = d[3] & 0xFFFFFFu;
-    f[5] = (d[3] >> 24) | ((d[4] & 0xFFFFu) << 8);
-    f[6] = (d[4] >> 16) | ((d[5] & 0xFFu) << 16);
-    f[7] = d[5] >> 8;
+    uint32_t codes = 0;
+    if (have) {
+        const uint64_t unit = word0 >> 6;
+        const uint32_t g = (uint32_t)(word0 & 63) >> 3;
+        const uint32_t* __restrict__ up = reinterpret_cast<const uint32_t*>(pc.src + unit * 216);
+        const uint32_t* __restrict__ fp = up + g * 6;
+        uint32_t d[6];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) d[j] = fp[j];
+        f[0] = d[0] & 0xFFFFFFu;
+        f[1] = (d[0] >> 24) | ((d[1] & 0xFFFFu) << 8);
+        f[2] = (d[1] >> 16) | ((d[2] & 0xFFu) << 16);
+        f[3] = d[2] >> 8;
+        f[4] = d[3] & 0xFFFFFFu;
+        f[5] = (d[3] >> 24) | ((d[4] & 0xFFFFu) << 8);
+        f[6] = (d[4] >> 16) | ((d[5] & 0xFFu) << 16);
+        f[7] = d[5] >> 8;
+        const uint32_t bit = 24 * g, di = bit >> 5, sh = bit & 31;
+        const uint64_t two = (uint64_t)up[48 + di] | ((uint64_t)up[48 + (di < 5 ? di + 1 : 5)] << 32);
+        codes = (uint32_t)(two >> sh) & 0xFFFFFFu;
+    }
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) cnt += ((codes >> (3 * j)) & 7u) == 7u ? 1u : 0u;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t x = cnt;
+#pragma unroll
+    for (int dlt = 1; dlt < 64; dlt <<= 1) {
+        const uint32_t y = __shfl_up(x, dlt, 64);
+        if (lane >= dlt) x += y;
+    }
+    if (lane == 63) wave_total[wave] = x;
+    __syncthreads();
+    uint32_t rank = x - cnt;
+    for (int w = 0; w < wave; ++w) rank += wave_total[w];
+    if (!have || word0 < pc.w_from) return;
+    const uint8_t* __restrict__ ext = pc.ext + pc.tab[bi] + rank;
     uint32_t w[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const uint32_t code = (d[6] >> (4 * j)) & 0xFu;
-        w[j] = (f[j] & 0x7FFFFFu) | ((f[j] >> 23) << 31) | ((((uint32_t)pc.base + code) & 0xFFu) << 23);
+        const uint32_t code = (codes >> (3 * j)) & 7u;
+        uint32_t e = (uint32_t)pc.base + code;
+        if (code == 7u) e = *ext++;
+        w[j] = (f[j] & 0x7FFFFFu) | ((f[j] >> 23) << 31) | ((e & 0xFFu) << 23);
     }
-    uint32_t* __restrict__ out = reinterpret_cast<uint32_t*>(dst) + g * 8;
-    if (g * 32 + 32 <= left) {
+    uint32_t* __restrict__ out = reinterpret_cast<uint32_t*>(pc.dst) + word0;
+    if (word0 + 8 <= pc.w_to) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         reinterpret_cast<u32x4*>(out)[0] = u32x4{w[0], w[1], w[2], w[3]};
         reinterpret_cast<u32x4*>(out)[1] = u32x4{w[4], w[5], w[6], w[7]};
     } else {  // last group of a tensor whose word count is not a multiple of 8
-        const uint64_t words = (left - g * 32) / 4;
+        const uint64_t words = pc.w_to - word0;
         for (uint64_t j = 0; j < words; ++j) out[j] = w[j];
     }
 }
@@ -822,25 +855,17 @@ int launch_unpack(UnpackArgs& a, hipStream_t s) {
     for (int k = 0; k < a.n; ++k) {
         UnpackPiece& pc = a.piece[k];
         if (!pc.src || !pc.dst || !al16(pc.src) || !al16(pc.dst)) return K_EINVAL;
-        if (pc.base >= 0 && (pc.bytes % 4 != 0 || pc.base > 255)) return K_EINVAL;
         pc.first_block = (uint32_t)blocks;
-        blocks += (pc.bytes + kUnpackBlockBytes - 1) / kUnpackBlockBytes;
+        if (pc.base < 0) {
+            blocks += (pc.bytes + kUnpackBlockBytes - 1) / kUnpackBlockBytes;
+        } else {
+            if (pc.base > 255 || !pc.tab || pc.w_to < pc.w_from || (pc.w_from & 63)) return K_EINVAL;
+            if (pc.w_to > pc.w_from) blocks += (pc.w_to + 2047) / 2048 - pc.w_from / 2048;
+        }
         if (blocks > 0x7FFFFFFFull) return K_EINVAL;
     }
     if (blocks == 0) return 0;
     hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
-    return (int)hipGetLastError();
-}
-
-__global__ __launch_bounds__(256) void patch_kernel(const uint32_t* __restrict__ table, uint64_t n,
-                                                    uint32_t* __restrict__ image32) {
-    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
-        image32[table[2 * i]] = table[2 * i + 1];
-}
-int launch_patch(const uint32_t* table, uint64_t n, uint32_t* image32, hipStream_t s) {
-    if (!table || !image32) return K_EINVAL;
-    if (n == 0) return 0;
-    hipLaunchKernelGGL(patch_kernel, dim3(grid_for((long)n, 256)), dim3(256), 0, s, table, n, image32);
     return (int)hipGetLastError();
 }
 
