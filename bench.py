@@ -12,7 +12,7 @@ BERT-large batch 4 seq 384 (BASELINE.json configs[3]: the largest single-GPU con
 with ResNet-152, the one the north-star target is quoted on); the other single-GPU configs are
 reported under "workloads".  "roofline" is computed from per-launch HIP-event timings of the
 dominant kernel over timed warm requests, "swap" holds the swap-in GB/s (bytes that crossed the
-link; compressible tensors travel in a lossless 28-bit format) against the measured pinned-host ->
+link; compressible tensors travel in a lossless 27-bit format) against the measured pinned-host ->
 HBM link peak, and "cpu_baseline" is the PyTorch CPU forward of the same
 seeded model timed on this box's host cores (oracle/models.py, a reported baseline only).
 """
@@ -163,7 +163,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         weight_bytes=info["image_bytes"], act_bytes=info["act_bytes"], ops=info["n_ops"], chunks=info["n_chunks"],
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
-        link_bytes=link_bytes,   # below weight_bytes when tensors travel in the 28-bit format
+        link_bytes=link_bytes,   # below weight_bytes when tensors travel in the packed format
         weights_gbps_p50=info["image_bytes"] / 1e9 / (pctl(swap_ms, 0.5) * 1e-3),   # weight bytes in place per second
         copy_streams=streams, host_gathers=gathers, steps_total_s=t_total,
     )

@@ -61,7 +61,7 @@ def _cycle(server, fn, inputs, first):
         assert np.array_equal(a, b), "cold (swap-in) request differs from the first run"
     st = server.swap_stats(fn.fid)
     image = server.model_info(fn.fid)["image_bytes"]
-    assert 0.8 * image < st["bytes"] <= image and st["copy_ms"] > 0   # link bytes: 28-bit format or as they are
+    assert 0.8 * image < st["bytes"] <= image and st["copy_ms"] > 0   # link bytes: packed or as they are
     return st
 
 

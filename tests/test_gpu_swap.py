@@ -130,7 +130,7 @@ def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather
 
 @pytest.mark.parametrize("pack", [True, False])
 def test_packed_transfer_is_lossless_for_any_bits(pack, monkeypatch):
-    """Weights cross the link in the 28-bit format and are expanded on the device.  Doctored tensors
+    """Weights cross the link in the packed format and are expanded on the device.  Doctored tensors
     (zeros, denormals, infinities, NaNs, exponents spread over 60 binades, one tensor of arbitrary
     bits, one of zeros only) must come back bit for bit, swap-in after swap-in, and a request must
     answer as it did at registration."""

@@ -743,7 +743,7 @@ void Engine::free_transfer(Model& m) {
 }
 
 // Builds what a swap-in sends over the link (weight_pack.hpp) once the image has its final order.
-// Tensors whose words compress go in the 28-bit format, the rest as they are; a model that would
+// Tensors whose words compress go in the packed format, the rest as they are; a model that would
 // save under 3 % keeps sending its image directly.
 int Engine::build_transfer(Model& m) {
     free_transfer(m);
