@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 
 from torpor_amd.functions import bert, resnet
+from torpor_amd.functions.base import Function
 from torpor_amd.server import ACK_INAVAIL, ACK_OK, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD, Server
 
 pytestmark = pytest.mark.gpu
@@ -181,3 +182,59 @@ def test_results_into_pinned_buffers_equal_results_through_staging(gpu_server):
             s.replay(7, packed, out)
         assert np.array_equal(views_plain[0], y) and np.array_equal(views_pinned[0], y)
     fn.unload()
+
+
+class _Chain(Function):
+    """y = x W^T applied `depth` times with one square weight: a long run of device work behind very
+    few calls, so that the request's host side is over long before the device is."""
+
+    def __init__(self, server, fid, seed, n=2048, depth=24):
+        super().__init__(server, fid)
+        self.n, self.depth, self.batch = n, depth, 1
+        rng = np.random.default_rng(seed)
+        self._w = (rng.standard_normal((n, n)) / np.sqrt(n)).astype(np.float32)
+
+    def weights(self):
+        return {"w": self._w}
+
+    def input_specs(self):
+        return [((self.n, self.n), np.float32)]
+
+    def forward(self, inputs):
+        n = self.n
+        a, b = inputs[0], self.alloc(4 * n * n)
+        for _ in range(self.depth):
+            self.s.gemm(self.fid, a.va, self.w["w"], b.va, n, n, n, n, n, n)
+            a, b = b, a
+        return [(a, (n, n), np.float32)]
+
+
+def test_memory_of_a_finished_request_is_not_reused_while_its_kernels_run():
+    """A request is over for the controller once its result copy is queued (cuda_server.hpp:1044), which
+    can be milliseconds before the device has run it.  The next request may evict that model at once;
+    its weights, activations and result must stay intact until the device is done with them."""
+    with Server(mem_limit_bytes=80 << 20, pool_bytes=256 << 20) as s:
+        a, b = _Chain(s, 0, seed=1), _Chain(s, 1, seed=2)
+        x = np.random.default_rng(3).standard_normal((a.n, a.n)).astype(np.float32)
+        (ya,) = a.register([x])
+        (yb,) = b.register([x])                      # the budget holds one model: this evicts 0
+        assert not s.resident(0) and s.resident(1)
+        assert np.abs(ya).max() > 0 and not np.array_equal(ya, yb)
+        for _ in range(3):
+            # request for model 0, issued op by op, left unsynchronised after the result copy
+            assert s.signal(REQ_EXECUTE, 0, "") == (ACK_OK, 0, False)
+            a._alloc_pos = 0
+            buf = a.alloc(x.nbytes)
+            s.h2d(0, buf.va, x)
+            ((out, shape, dt),) = a.forward([buf])
+            got_a = np.empty(shape, dt)
+            s.d2h_async(0, got_a, out.va)
+            # the executor is free again: model 1 is started at once, which evicts model 0
+            assert s.signal(REQ_EXECUTE, 1, "") == (ACK_OK, 0, False)
+            assert not s.resident(0) and s.resident(1)
+            packed, outbuf, views = b.pack([x])
+            s.replay(1, packed, outbuf)
+            s.stream_synchronize(0)
+            assert np.array_equal(got_a, ya), "model 0's result was damaged by the swap-in that followed it"
+            assert np.array_equal(views[0], yb)
+            assert np.array_equal(s.readback_weights(1), s.host_weights(1))

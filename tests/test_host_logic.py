@@ -293,6 +293,28 @@ def test_eviction_under_budget_and_deterministic_offsets(host_server):
     assert s.pool_stats()["used"] == 0
 
 
+def test_load_while_busy_never_evicts_the_running_model():
+    """controller.hpp:208-215 accepts Load while an executor is busy; the model that is running must
+    not be the victim of the eviction that makes room for it."""
+    s = Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20, request_timeout_ms=60000)
+    try:
+        fns = [_register(s, i, seed=i) for i in range(1, 5)]
+        assert [s.resident(i) for i in range(1, 5)] == [False, True, True, True]
+        assert s.signal(REQ_EXECUTE, 2, "") == (ACK_OK, 0, False)       # LRU order, oldest first: 3, 4, 2
+        for other in (1, 3, 4, 1, 3, 4):                                 # each Load evicts a model that is not 2
+            assert s.signal(REQ_LOAD, other, "")[0] == ACK_OK
+            assert s.resident(2) and s.resident(other)
+            assert sum(s.resident(i) for i in range(1, 5)) == 3
+        packed, outbuf, _ = fns[1].pack([np.zeros((1, 3, 32, 32), np.float32)])
+        with pytest.raises(TorporError):
+            s.replay(2, packed, outbuf)
+        # once the request is over the model is an ordinary candidate again: 2 is the oldest entry now
+        assert s.signal(REQ_LOAD, 1, "")[0] == ACK_OK
+        assert not s.resident(2)
+    finally:
+        s.close()
+
+
 def _register_level(s, fid, level):
     fn = resnet.ResNet(s, fid, "resnet50", batch=1, seed=fid, image=32, level=level)
     with pytest.raises(TorporError):

@@ -185,7 +185,10 @@ Model* Engine::active_model(int client, int* err) {
         return nullptr;
     }
     Model* m = find(active_);
-    if (!m) *err = TP_ENOENT;
+    if (!m)
+        *err = TP_ENOENT;
+    else
+        m->touch_seq = ++work_seq_;
     return m;
 }
 
@@ -634,6 +637,7 @@ int Engine::do_stream_sync(Model* m) {
     if (!host_only()) {
         hipError_t e = hipStreamSynchronize(compute_);
         if (e != hipSuccess) ret = (int)e;
+        else synced_seq_ = work_seq_;
         for (auto& pd : pending_d2h_)
             if (!ret) std::memcpy(pd.dst, d2h_stage_ + pd.stage_off, pd.bytes);
     } else if (d2h_seen_) {
@@ -666,6 +670,7 @@ int Engine::op_device_sync(int client) {
     if (!host_only()) {
         hipError_t e = hipStreamSynchronize(compute_);
         if (e != hipSuccess) ret = (int)e;
+        else synced_seq_ = work_seq_;
     }
     // cuda_server.hpp:959-961: the first device synchronisation after the uploads ends the
     // weight-loading phase; what is allocated from now on is not model memory.
@@ -1188,6 +1193,10 @@ void Engine::evict_model(Model& m) {
     if (!m.resident) return;
     const auto t0 = Clock::now();
     wait_copy_idle(m);
+    // A request counts as finished once its result copy is queued (cuda_server.hpp:1044), so the
+    // model's last kernels may still be running: its memory is not handed on before they are done.
+    if (!host_only() && m.touch_seq > synced_seq_ && hipStreamSynchronize(compute_) == hipSuccess)
+        synced_seq_ = work_seq_;
     if (m.w_pool_off != UINT64_MAX) pool_.release(m.w_pool_off);
     if (m.a_pool_off != UINT64_MAX) pool_.release(m.a_pool_off);
     m.w_pool_off = m.a_pool_off = UINT64_MAX;
@@ -1254,6 +1263,9 @@ int Engine::start_execute(int id) {
     // controller.hpp:414-417 + cuda_server.hpp:229-239
     active_ = id;
     mode_ = MODE_EXEC;
+    // A Load for another model may arrive while this one runs (controller.hpp:208-215 has no busy
+    // test): the running model is not a candidate for its eviction.
+    lru_.lock(std::to_string(id));
     m->stats.gate_waits = 0;
     m->stats.host_gathers = 0;
     req_start_ = Clock::now();
@@ -1273,6 +1285,7 @@ void Engine::complete_request() {
         if (r && !m->async_error) m->async_error = r;
     }
     const int status = exec_status_;
+    lru_.unlock(std::to_string(active_));
     active_ = -1;
     mode_ = MODE_NONE;
     if (m && m->state == MS_READY) {

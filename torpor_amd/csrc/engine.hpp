@@ -117,6 +117,7 @@ struct Model {
     std::atomic<bool> cancel{false};
     std::atomic<int> copy_error{0};
     uint32_t gated_upto = 0;
+    uint64_t touch_seq = 0;   // Engine::work_seq_ at this model's last data-plane call
     uint32_t defer_from = UINT32_MAX;  // first transfer group made of deferred tables only
     int ncopy = 2;            // copy streams used by the current swap-in plan
     uint64_t chunk_max = 0;   // largest transfer group of the current plan
@@ -264,6 +265,8 @@ private:
         bool peek_victim(const std::string& keep, std::string* out) const {
             return two_class ? ia.peek_victim(0, keep, out) : lru.peek_victim(keep, out);
         }
+        void lock(const std::string& f) { two_class ? ia.lock(0, f) : lru.lock(f); }
+        void unlock(const std::string& f) { two_class ? ia.unlock(0, f) : lru.unlock(f); }
     } lru_;
     uint8_t* arena_ = nullptr;
     float* workspace_ = nullptr;
@@ -289,6 +292,9 @@ private:
     std::deque<Queued> req_queue_;
     std::deque<std::pair<int, int>> deferred_acks_;
     bool d2h_seen_ = false;
+    // Data-plane calls are numbered; synced_seq_ is the number reached when the host last waited for
+    // the compute stream.  A model whose touch_seq is above it may still have work on the device.
+    uint64_t work_seq_ = 0, synced_seq_ = 0;
 
     uint8_t* h2d_stage_ = nullptr;
     uint64_t h2d_cap_ = 0, h2d_pos_ = 0;
