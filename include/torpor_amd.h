@@ -198,7 +198,11 @@ const char* tp_version(void);
  * One SignalRequest -> SignalAck exchange (controller.hpp:131-216).  `function` is the
  * decimal client id.  When the executor is busy the request is queued
  * (controller.hpp:156,177) and *deferred is set to 1: its ack appears later through
- * tp_take_deferred_ack, after the active request completes (controller.hpp:242-262). */
+ * tp_take_deferred_ack, after the active request completes (controller.hpp:242-262).
+ * Load and Unload are served while a request runs (controller.hpp:187-215); the function that is
+ * running is never the victim of the eviction a Load causes, and a function whose last request is
+ * still executing on the device (a request ends, for the controller, when its result copy is
+ * queued: cuda_server.hpp:1044) is swapped out only after the device has finished that work. */
 int tp_signal(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack, int32_t* resp,
               int32_t* deferred);
 int tp_take_deferred_ack(tp_server* s, int32_t* ack, int32_t* resp); /* 1 = ack produced, 0 = none */
