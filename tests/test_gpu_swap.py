@@ -238,3 +238,27 @@ def test_memory_of_a_finished_request_is_not_reused_while_its_kernels_run():
             assert np.array_equal(got_a, ya), "model 0's result was damaged by the swap-in that followed it"
             assert np.array_equal(views[0], yb)
             assert np.array_equal(s.readback_weights(1), s.host_weights(1))
+
+
+def test_executor_log_reports_every_swap_in(tmp_path, monkeypatch):
+    """The Transfer line of the executor log (memory_manager.hpp:425-431) carries what tp_swap_stats reports."""
+    import re
+    monkeypatch.setenv("TORPOR_LOG_DIR", str(tmp_path))
+    monkeypatch.setenv("EXECUTOR_LOG_LEVEL", "info")
+    with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
+        fn, x, y = _mk(s, 0, seed=5)
+        stats = []
+        for _ in range(3):
+            fn.unload()
+            (got,) = fn.invoke([x])
+            assert np.array_equal(got, y)
+            stats.append(s.swap_stats(0))
+        fn.unload()
+    lines = (tmp_path / "log_executor_0.txt").read_text().splitlines()
+    xfer = [re.search(r"Transfer model 0: (\d+) bytes over the link in (\d+) groups on (\d) streams, overall elasped (\d+) us", ln)
+            for ln in lines if "Transfer model" in ln]
+    assert len(xfer) == 3 and all(xfer)
+    for m, st in zip(xfer, stats):
+        assert int(m.group(1)) == st["bytes"] and int(m.group(2)) == st["chunks"] and int(m.group(3)) == st["copy_streams"]
+        assert abs(int(m.group(4)) - st["copy_ms"] * 1e3) <= 2
+    assert sum("Request of model 0 completed" in ln and "(swapped in)" in ln for ln in lines) == 3

@@ -4,6 +4,7 @@ controller / executor state machine of a host-only engine (TP_FLAG_HOST_ONLY: no
 compute - ops are validated, tracked and recorded but not launched)."""
 import ctypes as C
 import random
+import re
 
 import numpy as np
 import pytest
@@ -313,6 +314,38 @@ def test_load_while_busy_never_evicts_the_running_model():
         assert not s.resident(2)
     finally:
         s.close()
+
+
+def test_executor_log_has_the_reference_sections(tmp_path, monkeypatch):
+    """EXECUTOR_LOG_LEVEL (cuda_server.hpp:61-69) switches on log_executor_<gpu>.txt with the sections the
+    reference times: CheckMalloc (memory_manager.hpp:499-501), Evict (258), request completion
+    (cuda_server.hpp:294-295).  Unset, the engine writes nothing."""
+    monkeypatch.setenv("TORPOR_LOG_DIR", str(tmp_path))
+    monkeypatch.delenv("EXECUTOR_LOG_LEVEL", raising=False)
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20):
+        pass
+    assert not list(tmp_path.iterdir())
+    monkeypatch.setenv("EXECUTOR_LOG_LEVEL", "info")
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20) as s:
+        fn = _register(s, 7)
+        assert s.signal(REQ_UNLOAD, 7, "")[0] == ACK_OK
+        assert s.signal(REQ_EXECUTE, 7, "") == (ACK_OK, 0, False)
+        packed, outbuf, _ = fn.pack([np.zeros((1, 3, 32, 32), np.float32)])
+        with pytest.raises(TorporError):
+            s.replay(7, packed, outbuf)
+    text = (tmp_path / "log_executor_0.txt").read_text()
+    lines = text.splitlines()
+    assert all(re.match(r"\[\d{4}-\d\d-\d\d \d\d:\d\d:\d\d\.\d{6}\] \[info\] ", ln) for ln in lines), text
+    order = [next(i for i, ln in enumerate(lines) if key in ln) for key in
+             ("Executor 0 started", "Evict model 7 elasped", "CheckMalloc model 7 elasped", "Request of model 7 completed in")]
+    assert order == sorted(order)
+    assert "(swapped in)" in lines[order[-1]]
+    monkeypatch.setenv("EXECUTOR_LOG_LEVEL", "err")      # info lines are below this level
+    (tmp_path / "log_executor_0.txt").unlink()
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20) as s:
+        _register(s, 8)
+        s.signal(REQ_UNLOAD, 8, "")
+    assert (tmp_path / "log_executor_0.txt").read_text() == ""
 
 
 def _register_level(s, fid, level):

@@ -55,6 +55,10 @@ int Engine::init() {
     }
     lru_.set_budget(cfg_.mem_limit_bytes);
     pool_.reset(cfg_.pool_bytes);
+    log_.open(cfg_.device);
+    log_.write(ExecLog::INFO, "Executor %d started: budget %llu MiB, pool %llu MiB, first transfer group %llu KiB, %s eviction",
+               cfg_.device, (unsigned long long)(cfg_.mem_limit_bytes >> 20), (unsigned long long)(pool_.capacity() >> 20),
+               (unsigned long long)(cfg_.chunk_bytes >> 10), lru_.two_class ? "two-class" : "LRU");
 
     if (host_only()) {
         arena_ = reinterpret_cast<uint8_t*>(0x100000000000ull);
@@ -651,8 +655,10 @@ int Engine::do_stream_sync(Model* m) {
         if (!ret && m->async_error) ret = m->async_error;
         m->async_error = 0;
         if (!host_only() && m->resident && !m->fully_loaded && m->copy_state.load() == CS_ISSUED && m->t1 &&
-            hipEventQuery(m->t1) == hipSuccess)
+            hipEventQuery(m->t1) == hipSuccess) {
             m->fully_loaded = true;
+            log_transfer(*m);
+        }
     }
     return ret;
 }
@@ -1002,6 +1008,7 @@ int Engine::finish_loading(Model& m) {
 }
 
 int Engine::finish_tracking(Model& m) {
+    TraceRange trace("register: lay out and pack model", m.id);
     // memory_manager.hpp:73-80 unset_track_model_memory + the layout step described above
     int r = build_image(m, true);
     if (r < 0) return r;
@@ -1056,6 +1063,7 @@ void Engine::copy_main() {
         // memory_manager.hpp:378-409: walk the tensors in access order, one DMA per group, and
         // publish each group.  Publishing is an event record, not a host synchronisation.
         int err = 0;
+        TraceRange trace("swap-in: issue copies of model", m->id);
         if (!m->cancel.load()) {
             if (m->timg && stage_used_) {  // the staging area is shared: the previous expansion must be done with it
                 (void)hipStreamWaitEvent(copy_, stage_free_ev_, 0);
@@ -1124,6 +1132,19 @@ void Engine::copy_main() {
     }
 }
 
+// memory_manager.hpp:425-431: one line per finished swap-in, written when the engine first learns that
+// the last group has landed (a later synchronisation of the model, or its swap-out).
+void Engine::log_transfer(Model& m) {
+    if (!log_.on(ExecLog::INFO) || m.transfer_logged || host_only() || !m.timing_valid || !m.t0 || !m.t1) return;
+    if (m.cancel.load() || m.copy_error.load() || m.copy_state.load(std::memory_order_acquire) != CS_ISSUED) return;
+    if (hipEventQuery(m.t1) != hipSuccess) return;
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, m.t0, m.t1) != hipSuccess) return;
+    m.transfer_logged = true;
+    log_.write(ExecLog::INFO, "Transfer model %d: %llu bytes over the link in %u groups on %d streams, overall elasped %.0f us",
+               m.id, (unsigned long long)m.stats.bytes, m.stats.chunks, m.ncopy, ms * 1e3);
+}
+
 void Engine::wait_copy_idle(Model& m) {
     if (host_only()) return;
     if (m.copy_state.load(std::memory_order_acquire) == CS_RUNNING) {
@@ -1138,6 +1159,7 @@ void Engine::wait_copy_idle(Model& m) {
 // memory_manager.hpp:213-227 sig_trans_thread + 451-507 check_and_malloc_model
 int Engine::swap_in(Model& m) {
     if (m.resident) return 0;
+    TraceRange trace("swap-in: allocate model", m.id);
     const auto t0 = Clock::now();
     auto try_alloc = [&]() -> bool {
         m.w_pool_off = pool_.alloc(m.image_bytes);
@@ -1169,11 +1191,14 @@ int Engine::swap_in(Model& m) {
     m.issued.store(0);
     m.cancel.store(false);
     m.copy_error.store(0);
+    m.transfer_logged = false;
     m.stats.alloc_us = us_since(t0);
     m.stats.bytes = m.timg ? m.timg_bytes : m.image_bytes;
     m.stats.chunks = (uint32_t)m.chunk_end.size();
     m.stats.copy_streams = (uint32_t)m.ncopy;
     ++swap_ins_;
+    log_.write(ExecLog::INFO, "CheckMalloc model %d elasped %.0f us (%llu weight + %llu activation bytes)", m.id,
+               m.stats.alloc_us, (unsigned long long)m.image_bytes, (unsigned long long)m.act_bytes);
     if (host_only() || m.image_bytes == 0) {
         m.fully_loaded = true;
         return 0;
@@ -1191,8 +1216,11 @@ int Engine::swap_in(Model& m) {
 // memory_manager.hpp:240-259: metadata only, the host copy stays authoritative.
 void Engine::evict_model(Model& m) {
     if (!m.resident) return;
+    TraceRange trace("swap-out model", m.id);
     const auto t0 = Clock::now();
+    const bool was_running = m.copy_state.load(std::memory_order_acquire) == CS_RUNNING;
     wait_copy_idle(m);
+    if (!was_running) log_transfer(m);
     // A request counts as finished once its result copy is queued (cuda_server.hpp:1044), so the
     // model's last kernels may still be running: its memory is not handed on before they are done.
     if (!host_only() && m.touch_seq > synced_seq_ && hipStreamSynchronize(compute_) == hipSuccess)
@@ -1207,6 +1235,7 @@ void Engine::evict_model(Model& m) {
     m.copy_state.store(CS_IDLE);
     m.stats.evict_us = us_since(t0);
     ++evictions_;
+    log_.write(ExecLog::INFO, "Evict model %d elasped %.0f us", m.id, m.stats.evict_us);
 }
 
 // controller.hpp:392-400
@@ -1269,6 +1298,11 @@ int Engine::start_execute(int id) {
     m->stats.gate_waits = 0;
     m->stats.host_gathers = 0;
     req_start_ = Clock::now();
+    if (Roctx::get().available()) {
+        char name[64];
+        std::snprintf(name, sizeof name, "request of model %d (%s)", id, was_resident ? "resident" : "swapped out");
+        req_range_ = Roctx::get().start(name);
+    }
     if (was_resident)
         exec_status_ = ES_LOCAL;
     else
@@ -1285,6 +1319,11 @@ void Engine::complete_request() {
         if (r && !m->async_error) m->async_error = r;
     }
     const int status = exec_status_;
+    Roctx::get().stop(req_range_);
+    req_range_ = 0;
+    if (mode_ == MODE_EXEC)  // cuda_server.hpp:294-295
+        log_.write(ExecLog::INFO, "Request of model %d completed in %.3f ms (%s)", active_, us_since(req_start_) / 1000.0,
+                   status == ES_LOCAL ? "resident" : "swapped in");
     lru_.unlock(std::to_string(active_));
     active_ = -1;
     mode_ = MODE_NONE;
@@ -1982,6 +2021,7 @@ int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uin
     if (!m) return err;
     if (mode_ != MODE_EXEC) return TP_ESTATE;
     if (m->program.empty()) return TP_ENOENT;
+    TraceRange trace("replay of model", m->id);
     const bool warm = m->fully_loaded;
     const auto t_start = Clock::now();
     ReplayCtx rc;

@@ -28,6 +28,7 @@
 #include "ia_evictor.hpp"
 #include "lru.hpp"
 #include "pool.hpp"
+#include "trace.hpp"
 
 namespace tp {
 
@@ -129,6 +130,7 @@ struct Model {
     int warm_streak = 0;                   // warm replays since the placement last changed
     hipEvent_t t0 = nullptr, t1 = nullptr;
     bool timing_valid = false;
+    bool transfer_logged = false;  // the executor log has this swap-in's Transfer line
     // recorded program
     std::vector<Op> program;
     int async_error = 0;
@@ -237,6 +239,7 @@ private:
     void drop_graph(Model& m);
     int build_graph(Model& m);
     void wait_copy_idle(Model& m);
+    void log_transfer(Model& m);
     void copy_main();
     int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
     void* host_alloc(uint64_t bytes);
@@ -315,6 +318,9 @@ private:
     size_t prof_next_ = 0;
     std::vector<ProfRecord> prof_records_;
     std::vector<tp_kernel_stat> prof_stats_;
+
+    ExecLog log_;
+    uint64_t req_range_ = 0;  // open "request" range of the marker trace, 0 = none
 
     std::thread copy_thread_;
     std::mutex cmu_;
