@@ -33,6 +33,40 @@ static uint64_t env_u64(const char* name, uint64_t dflt) {
 
 static void op_work(const Op& op, double* flops, double* bytes, const char** name);
 
+// Runs f(0) .. f(n-1) on up to TORPOR_HOST_THREADS (default 8) threads, the caller's included; tasks are
+// handed out one at a time.  Returns false if a task threw (the others still ran).
+template <class F>
+static bool parallel_for(size_t n, F&& f) {
+    static const size_t cap = [] {
+        const uint64_t hw = std::thread::hardware_concurrency();
+        const uint64_t want = env_u64("TORPOR_HOST_THREADS", 8);
+        return (size_t)std::max<uint64_t>(1, std::min<uint64_t>(want, hw ? hw : 1));
+    }();
+    std::atomic<size_t> next{0};
+    std::atomic<bool> ok{true};
+    auto work = [&] {
+        for (;;) {
+            const size_t i = next.fetch_add(1);
+            if (i >= n) return;
+            try {
+                f(i);
+            } catch (...) {
+                ok.store(false);
+            }
+        }
+    };
+    std::vector<std::thread> helpers;
+    const size_t want = std::min(cap, n);
+    try {
+        helpers.reserve(want);
+        for (size_t t = 1; t < want; ++t) helpers.emplace_back(work);
+    } catch (...) {  // no more threads to be had: go on with those that started
+    }
+    work();
+    for (auto& t : helpers) t.join();
+    return ok.load();
+}
+
 Engine::Engine(const tp_config& cfg) : cfg_(cfg) {}
 
 int Engine::init() {
@@ -723,12 +757,14 @@ int Engine::build_image(Model& m, bool by_access) {
     if (same && m.image_bytes == off) return 0;
     uint8_t* img = static_cast<uint8_t*>(host_alloc(off));
     if (!img) return TP_ENOMEM;
-    std::memset(img, 0, off ? off : 1);
-    for (size_t i = 0; i < m.params.size(); ++i) {
-        Param& p = m.params[i];
+    if (off == 0) img[0] = 0;
+    parallel_for(m.params.size(), [&](size_t i) {
+        const Param& p = m.params[i];
         const uint8_t* src = m.host_image ? m.host_image + p.image_off : m.staging.data() + p.voff;
         std::memcpy(img + new_off[i], src, p.size);
-    }
+        const uint64_t end = new_off[i] + p.size;  // the alignment gap behind the tensor reads as zeros
+        std::memset(img + end, 0, align_up(end, kTensorAlign) - end);
+    });
     for (size_t i = 0; i < m.params.size(); ++i) m.params[i].image_off = new_off[i];
     host_free(m.host_image);
     m.host_image = img;
@@ -771,14 +807,21 @@ int Engine::build_transfer(Model& m) {
     std::vector<uint64_t> n_ext(m.params.size(), 0), tab_off(m.params.size(), 0), ext_off(m.params.size(), 0);
     std::vector<uint64_t> t_off(m.params.size(), 0);
     uint64_t off = 0;
+    // one histogram pass per tensor picks its window; tensors are independent of each other
+    std::vector<uint32_t> win(m.params.size(), 0);
+    std::vector<uint64_t> win_out(m.params.size(), 0);
+    parallel_for(m.params.size(), [&](size_t i) {
+        const Param& p = m.params[i];
+        if (p.size % 4 == 0 && p.size >= 4096)
+            choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), p.size / 4, &win[i], &win_out[i]);
+    });
     for (uint32_t idx : m.image_order) {
         const Param& p = m.params[idx];
         t_off[idx] = off;
         if (p.size % 4 == 0 && p.size >= 4096) {
-            uint32_t b = 0;
-            uint64_t outside = 0;
+            const uint32_t b = win[idx];
+            const uint64_t outside = win_out[idx];
             const uint64_t nw = p.size / 4;
-            choose_window(reinterpret_cast<const uint32_t*>(m.host_image + p.image_off), nw, &b, &outside);
             if (packed_bytes(nw) + packed_blocks(nw) * 4 + outside <= p.size - p.size / 20) {
                 // a packed tensor's region: block table, extension stream, payload -- the first two
                 // arrive with the tensor's first bytes, whichever transfer group carries them
@@ -811,28 +854,51 @@ int Engine::build_transfer(Model& m) {
     }
     uint8_t* t = static_cast<uint8_t*>(host_alloc(off));
     if (!t) return 0;
-    std::memset(t, 0, off);
-    std::vector<uint8_t> ext;
     for (uint32_t idx : m.image_order) {
         Param& p = m.params[idx];
         p.t_off = t_off[idx];
         p.pack_base = base[idx];
         p.tab_off = tab_off[idx];
         p.ext_off = ext_off[idx];
+    }
+    // every tensor fills its own region of the transfer image; whatever lies between regions is zero
+    std::atomic<bool> agree{true};
+    const bool ran = parallel_for(m.image_order.size(), [&](size_t k) {
+        const uint32_t idx = m.image_order[k];
+        const Param& p = m.params[idx];
         const uint8_t* src = m.host_image + p.image_off;
+        const uint64_t region_beg = p.pack_base >= 0 ? p.tab_off : p.t_off;
+        const uint64_t region_end = k + 1 < m.image_order.size()
+                                        ? (m.params[m.image_order[k + 1]].pack_base >= 0 ? m.params[m.image_order[k + 1]].tab_off
+                                                                                         : m.params[m.image_order[k + 1]].t_off)
+                                        : off;
+        uint64_t filled_to = region_beg;
+        auto zero_to = [&](uint64_t upto) {
+            if (upto > filled_to) std::memset(t + filled_to, 0, upto - filled_to);
+        };
         if (p.pack_base >= 0) {
-            ext.clear();
-            pack_words(reinterpret_cast<const uint32_t*>(src), p.size / 4, (uint32_t)p.pack_base, t + p.t_off, &ext,
+            std::vector<uint8_t> ext;
+            const uint64_t nw = p.size / 4;
+            pack_words(reinterpret_cast<const uint32_t*>(src), nw, (uint32_t)p.pack_base, t + p.t_off, &ext,
                        reinterpret_cast<uint32_t*>(t + p.tab_off));
             if (ext.size() != n_ext[idx]) {  // the two passes disagree: never send a stream that does not decode
-                host_free(t);
-                free_transfer(m);
-                return 0;
+                agree.store(false);
+                return;
             }
             if (!ext.empty()) std::memcpy(t + p.ext_off, ext.data(), ext.size());
+            filled_to = p.ext_off + ext.size();
+            zero_to(p.t_off);
+            filled_to = p.t_off + packed_bytes(nw);
         } else {
             std::memcpy(t + p.t_off, src, p.size);
+            filled_to = p.t_off + p.size;
         }
+        zero_to(region_end);
+    });
+    if (!ran || !agree.load()) {
+        host_free(t);
+        free_transfer(m);
+        return 0;
     }
     m.timg = t;
     m.timg_bytes = off;
@@ -1009,11 +1075,18 @@ int Engine::finish_loading(Model& m) {
 
 int Engine::finish_tracking(Model& m) {
     TraceRange trace("register: lay out and pack model", m.id);
+    auto t_phase = Clock::now();
+    auto phase = [&](const char* what) {  // debug level: where a registration's time goes
+        log_.write(ExecLog::DEBUG, "Register model %d: %s elasped %.0f us", m.id, what, us_since(t_phase));
+        t_phase = Clock::now();
+    };
     // memory_manager.hpp:73-80 unset_track_model_memory + the layout step described above
     int r = build_image(m, true);
     if (r < 0) return r;
+    phase("image in access order");
     if (r == 1 && !host_only() && m.image_bytes)
         HIPCHK(hipMemcpy(m.w_dev, m.host_image, m.image_bytes, hipMemcpyHostToDevice));
+    phase("upload of the re-ordered image");
     build_chunks(m);
     // fold the per-allocation activation extents of the tracked run into one arena
     if (!host_only()) HIPCHK(hipStreamSynchronize(compute_));
@@ -1041,8 +1114,10 @@ int Engine::finish_tracking(Model& m) {
             if (pass == 1) m.warm_us = us_since(t0);
         }
         mode_ = saved_mode;
+        phase("two timed forward passes");
         r = build_transfer(m);  // needs the forward time: only a link-bound model gains from fewer bytes
         if (r < 0) return r;
+        phase("transfer image");
         build_chunks(m);
     }
     return 0;

@@ -54,7 +54,7 @@ inline void choose_window(const uint32_t* w, uint64_t n, uint32_t* base, uint64_
     *outside = n - best;
 }
 
-// Packs n words: payload (packed_bytes(n), zeroed by the caller), extension bytes appended to ext,
+// Packs n words: payload (packed_bytes(n), every byte of it written), extension bytes appended to ext,
 // block_tab[packed_blocks(n)] filled with the extension count before each block.
 inline void pack_words(const uint32_t* w, uint64_t n, uint32_t base, uint8_t* payload, std::vector<uint8_t>* ext,
                        uint32_t* block_tab) {
