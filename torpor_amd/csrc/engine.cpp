@@ -353,13 +353,10 @@ int Engine::op_malloc(int client, uint64_t bytes, uint64_t* va) {
     if (mode_ == MODE_LOAD) {  // weight block: cuda_server.hpp:969-970 with load flag set
         const uint64_t off = m->wbump;
         if (off + bytes > kVaOffMask) return TP_ENOMEM;
-        m->wbump = align_up(off + bytes, kTensorAlign);
+        const uint64_t bump = align_up(off + bytes, kTensorAlign);
+        if (!m->staging.resize(bump)) return TP_ENOMEM;  // nothing recorded for a block that has no room
+        m->wbump = bump;
         m->wblocks.push_back({off, bytes});
-        try {
-            m->staging.resize(m->wbump);
-        } catch (...) {
-            return TP_ENOMEM;
-        }
         *va = base | off;
         return 0;
     }
@@ -1060,7 +1057,7 @@ int Engine::finish_loading(Model& m) {
     for (auto& p : m.params) m.param_bytes += p.size;
     int r = build_image(m, false);
     if (r < 0) return r;
-    std::vector<uint8_t>().swap(m.staging);
+    m.staging.release();
     // cold start leaves the weights on the device (memory_manager.hpp:141), so the tracked
     // inference runs with a resident model
     m.w_pool_off = pool_.alloc(m.image_bytes);

@@ -12,9 +12,11 @@
 #pragma once
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <deque>
 #include <map>
 #include <memory>
@@ -77,6 +79,39 @@ struct ABlock {  // activation allocation
     uint64_t pool_off = UINT64_MAX;  // own extent while tracking, else inside the model's arena
 };
 
+// Bytes of a model's uploads until its weight image is laid out.  Grows with realloc: for blocks of this
+// size the C library moves pages instead of copying them, and nothing is filled in (only bytes that an
+// upload has written are ever read back).
+class UploadBuffer {
+public:
+    UploadBuffer() = default;
+    UploadBuffer(const UploadBuffer&) = delete;
+    UploadBuffer& operator=(const UploadBuffer&) = delete;
+    ~UploadBuffer() { release(); }
+    bool resize(uint64_t n) {
+        if (n > cap_) {
+            const uint64_t want = std::max<uint64_t>(n, cap_ + cap_ / 2);
+            void* q = std::realloc(p_, (size_t)want);
+            if (!q) return false;
+            p_ = static_cast<uint8_t*>(q);
+            cap_ = want;
+        }
+        size_ = n;
+        return true;
+    }
+    void release() {
+        std::free(p_);
+        p_ = nullptr;
+        size_ = cap_ = 0;
+    }
+    uint8_t* data() { return p_; }
+    uint64_t size() const { return size_; }
+
+private:
+    uint8_t* p_ = nullptr;
+    uint64_t size_ = 0, cap_ = 0;
+};
+
 enum ModelState : int { MS_LOADING = 0, MS_TRACKING = 1, MS_READY = 2 };
 enum CopyState : int { CS_IDLE = 0, CS_RUNNING = 1, CS_ISSUED = 2 };
 
@@ -88,7 +123,7 @@ struct Model {
     uint64_t wbump = 0;
     std::vector<WBlock> wblocks;
     std::vector<Param> params;  // sorted by voff
-    std::vector<uint8_t> staging;
+    UploadBuffer staging;
     uint8_t* host_image = nullptr;
     uint8_t* host_image_dev = nullptr;  // the same memory as kernels address it, null if not mapped
     uint64_t image_bytes = 0, param_bytes = 0;
