@@ -45,6 +45,7 @@ typedef struct tp_server tp_server;
 #define TP_ENOTACTIVE (-72)    /* client id is not the active function */
 #define TP_EUNSUPPORTED (-38)  /* shape / option not implemented */
 #define TP_EFAULT (-14)        /* virtual address does not translate */
+#define TP_ESCRATCH (-75)      /* the call needs more scratch memory than tp_gemm_noalloc's fixed buffer holds */
 
 /* ---- signal.proto enums (proto/signal.proto:5-30) ---- */
 #define TP_REQ_EXECUTE_AFTER_LOAD 0 /* register model */
@@ -255,6 +256,19 @@ int tp_bn_inference(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64
 int tp_bn_inference_pitched(tp_server* s, int32_t client, uint64_t x, uint64_t y, uint64_t scale, uint64_t bias,
                             uint64_t mean, uint64_t var, double eps, int64_t rows, int32_t channels, int64_t hw,
                             int32_t layout, int32_t relu, int64_t x_pitch);
+/* tp_gemm for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference.  The descriptor is tp_gemm's, except
+ * that x / y / c and the epilogue's pointers are raw device addresses on the current HIP device (not an
+ * engine's virtual addresses) and the work is enqueued on `stream` (a hipStream_t; NULL = the default
+ * stream); no tp_server is involved.  The call allocates nothing on host or device: the partial sums of
+ * a GEMM whose K range is split over workgroups go to a fixed TP_NOALLOC_SCRATCH_BYTES array that each
+ * GPU the library runs on holds until the process ends.  Results are bit-identical to tp_gemm's.
+ *   - a shape whose partial sums need more than that array is refused with TP_ESCRATCH (a split only
+ *     happens for fewer 64x64 output tiles than CUs, so m * n <= 1 Mi elements; at most 32 splits);
+ *   - all calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
+ *     race on it.  Calls on one stream are ordered and safe. */
+#define TP_NOALLOC_SCRATCH_BYTES (16u << 20)
+int tp_gemm_noalloc(const tp_gemm_desc* d, void* stream);
 /* cudaLaunchKernelService (cuda_server.hpp:1226-1310) by op id, pointer slots explicit. */
 int tp_launch(tp_server* s, int32_t client, int32_t op_id, const uint64_t* ptrs, int32_t n_ptrs,
               const int64_t* ints, int32_t n_ints, const float* floats, int32_t n_floats);

@@ -124,6 +124,7 @@ SYMBOLS = {
     "tp_sgemm_strided_batched": (C.c_int, [_P, _I32, _I32, _I32, _I32, _I32, _I32, C.c_float, _U64, _I32, _I64,
                                            _U64, _I32, _I64, C.c_float, _U64, _I32, _I64, _I32]),
     "tp_gemm": (C.c_int, [_P, _I32, C.POINTER(GemmDesc)]),
+    "tp_gemm_noalloc": (C.c_int, [C.POINTER(GemmDesc), _P]),
     "tp_conv_forward": (C.c_int, [_P, _I32, C.POINTER(ConvDesc)]),
     "tp_bn_inference": (C.c_int, [_P, _I32, _U64, _U64, _U64, _U64, _U64, _U64, C.c_double, _I64, _I32, _I64,
                                   _I32, _I32]),

@@ -644,13 +644,64 @@ int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, l
     return splits;
 }
 
-int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
-    if (a.M <= 0 || a.N <= 0 || a.K < 0 || !a.X || !a.Y || !a.C) return K_EINVAL;
-    if (a.nb0 < 1 || a.nb1 < 1) return K_EINVAL;
-    if (!((a.xs_k == 1) || (a.xs_r == 1)) || !((a.ys_k == 1) || (a.ys_c == 1))) return K_EINVAL;
-    if (a.gather && (a.Ho <= 0 || a.Wo <= 0 || a.H <= 0 || a.W <= 0)) return K_EINVAL;
-    const int batch = a.nb0 * a.nb1;
+// What launch_gemm decides from the shape alone: kernel family, tile and split of K over workgroups.
+struct GemmPlan {
+    bool fast = false, y_kc = false;
+    int cfg = 2, bm = 64, bn = 64;
+    int tiles_m = 0, tiles_n = 0;
+    int splits = 1;
+    long kper = 0;
+};
 
+static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
+    GemmPlan g;
+    const int batch = a.nb0 * a.nb1;
+    const bool x_fast = a.xs_k == 1 && (a.xs_r % 4 == 0) && (a.K % 4 == 0) && aligned16(a.X) && (a.xb0 % 4 == 0) &&
+                        (a.xb1 % 4 == 0);
+    g.y_kc = a.ys_k == 1 && (a.ys_c % 4 == 0) && (a.K % 4 == 0);
+    const bool y_cc = a.ys_c == 1 && a.ys_k != 1 && (a.ys_k % 4 == 0);
+    const bool y_fast = (g.y_kc || y_cc) && aligned16(a.Y) && (a.yb0 % 4 == 0) && (a.yb1 % 4 == 0);
+    g.fast = x_fast && y_fast;
+    if (g.fast) {
+        int cfg = choose_tile(a.M, a.N, a.K, batch, g.y_kc);
+        if (cfg >= 3 && !(a.K >= 128 && a.K % 128 == 0 && (g.y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
+        g.cfg = cfg;
+        g.bm = cfg == 4 ? 32 : cfg >= 2 ? 64 : 128;
+        g.bn = cfg == 0 ? 128 : cfg >= 3 ? 32 : 64;
+        g.tiles_m = (int)((a.M + g.bm - 1) / g.bm);
+        g.tiles_n = (int)((a.N + g.bn - 1) / g.bn);
+        const long tiles = (long)g.tiles_m * g.tiles_n * batch;
+        g.kper = ((a.K + 31) / 32) * 32;
+        if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws_bytes, &g.kper);
+    } else {
+        g.tiles_m = (int)((a.M + 63) / 64);
+        g.tiles_n = (int)((a.N + 63) / 64);
+        const long tiles = (long)g.tiles_m * g.tiles_n * batch;
+        g.kper = ((a.K + 15) / 16) * 16;
+        if (batch == 1) g.splits = choose_splits(tiles, a.K, 16, a.M, a.N, ws_bytes, &g.kper);
+    }
+    return g;
+}
+
+static bool gemm_args_ok(const GemmArgs& a) {
+    if (a.M <= 0 || a.N <= 0 || a.K < 0 || !a.X || !a.Y || !a.C) return false;
+    if (a.nb0 < 1 || a.nb1 < 1) return false;
+    if (!((a.xs_k == 1) || (a.xs_r == 1)) || !((a.ys_k == 1) || (a.ys_c == 1))) return false;
+    if (a.gather && (a.Ho <= 0 || a.Wo <= 0 || a.H <= 0 || a.W <= 0)) return false;
+    return true;
+}
+
+// Bytes of split-K partial sums launch_gemm would write for this call if the workspace were unbounded.
+long gemm_workspace_need(const GemmArgs& a) {
+    if (!gemm_args_ok(a)) return K_EINVAL;
+    const GemmPlan g = plan_gemm(a, ~(size_t)0);
+    return g.splits > 1 ? (long)g.splits * a.M * a.N * (long)sizeof(float) : 0;
+}
+
+int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
+    if (!gemm_args_ok(a)) return K_EINVAL;
+    const int batch = a.nb0 * a.nb1;
+    const GemmPlan g = plan_gemm(a, ws.ptr ? ws.bytes : 0);
     GemmDev p;
     p.X = a.X;
     p.Y = a.Y;
@@ -679,22 +730,14 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     p.ws = ws.ptr;
     p.ep = make_epilogue(a.ep, a.ldc);
 
-    const bool x_fast = a.xs_k == 1 && (a.xs_r % 4 == 0) && (a.K % 4 == 0) && aligned16(a.X) && (a.xb0 % 4 == 0) &&
-                        (a.xb1 % 4 == 0);
-    const bool y_kc = a.ys_k == 1 && (a.ys_c % 4 == 0) && (a.K % 4 == 0);
-    const bool y_cc = a.ys_c == 1 && a.ys_k != 1 && (a.ys_k % 4 == 0);
-    const bool y_fast = (y_kc || y_cc) && aligned16(a.Y) && (a.yb0 % 4 == 0) && (a.yb1 % 4 == 0);
+    p.tiles_m = g.tiles_m;
+    p.tiles_n = g.tiles_n;
+    p.splits = g.splits;
+    p.kper = g.kper;
+    const bool y_kc = g.y_kc;
 
-    if (x_fast && y_fast) {
-        int cfg = choose_tile(a.M, a.N, a.K, batch, y_kc);
-        if (cfg >= 3 && !(a.K >= 128 && a.K % 128 == 0 && (y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
-        const int bm = cfg == 4 ? 32 : cfg >= 2 ? 64 : 128, bn = cfg == 0 ? 128 : cfg >= 3 ? 32 : 64;
-        p.tiles_m = (int)((a.M + bm - 1) / bm);
-        p.tiles_n = (int)((a.N + bn - 1) / bn);
-        const long tiles = (long)p.tiles_m * p.tiles_n * batch;
-        p.splits = 1;
-        p.kper = ((a.K + 31) / 32) * 32;
-        if (batch == 1 && cfg < 3) p.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
+    if (g.fast) {
+        const int cfg = g.cfg;
         dim3 grid(plan_xcd_grid(p, a.M, a.N), 1, p.splits > 1 ? p.splits : batch);
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         // whole K-blocks; the 32-wide tiles take them in pairs, an odd last one is handled in the loop
@@ -727,12 +770,6 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
             variant = launch_fast<CfgM>(p, y_kc, clean, grid, s);
         g_last_kernel = names[cfg][y_kc ? 1 : 0][variant];
     } else {
-        p.tiles_m = (int)((a.M + 63) / 64);
-        p.tiles_n = (int)((a.N + 63) / 64);
-        const long tiles = (long)p.tiles_m * p.tiles_n * batch;
-        p.splits = 1;
-        p.kper = ((a.K + 15) / 16) * 16;
-        if (batch == 1) p.splits = choose_splits(tiles, a.K, 16, a.M, a.N, ws.ptr ? ws.bytes : 0, &p.kper);
         p.xr = p.xc = 0;
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits > 1 ? p.splits : batch);
         hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, s, p);

@@ -64,6 +64,9 @@ struct Workspace {
 
 void kernels_init(int device);  // caches CU count
 int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s);
+// Bytes of split-K partial sums launch_gemm writes for this call when the workspace is large enough to
+// hold them (0: the call uses no workspace); negative = the arguments are refused.
+long gemm_workspace_need(const GemmArgs& a);
 int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s);
 // introspection for tests/bench: which path the last launch on this thread took
 const char* last_kernel_name();

@@ -35,6 +35,18 @@ def _as_bytes_view(a):
     return a, a.ctypes.data_as(C.c_void_p), a.nbytes
 
 
+def gemm_noalloc(x, y, c, m, n, k, xs_r, ys_c, ldc, xs_k=1, ys_k=1, nb0=1, nb1=1, xb0=0, xb1=0, yb0=0, yb1=0,
+                 cb0=0, cb1=0, stream=0, **ep):
+    """tp_gemm_noalloc: the GEMM of Server.gemm on raw device addresses of the current HIP device, enqueued on
+    `stream` (a hipStream_t as an integer, 0 = default stream); allocates nothing.  Returns the status code."""
+    d = _lib.GemmDesc()
+    d.x, d.y, d.c, d.m, d.n, d.k = x, y, c, m, n, k
+    d.xs_r, d.xs_k, d.ys_c, d.ys_k, d.ldc = xs_r, xs_k, ys_c, ys_k, ldc
+    d.nb0, d.nb1, d.xb0, d.xb1, d.yb0, d.yb1, d.cb0, d.cb1 = nb0, nb1, xb0, xb1, yb0, yb1, cb0, cb1
+    Server._epilogue(d.ep, **ep)
+    return _lib.lib().tp_gemm_noalloc(C.byref(d), C.c_void_p(stream))
+
+
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
                  device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True, pack=True):
