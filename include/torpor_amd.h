@@ -207,6 +207,18 @@ const char* tp_version(void);
 int tp_signal(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack, int32_t* resp,
               int32_t* deferred);
 int tp_take_deferred_ack(tp_server* s, int32_t* ack, int32_t* resp); /* 1 = ack produced, 0 = none */
+/* The same two calls for a front end with many peers.  A queued signal gets a ticket (numbered from 1 in the
+ * order of queueing; 0 when the signal was answered at once) and its ack comes back with that ticket, so
+ * acks are matched to peers by ticket, not by position.  When the peer of a queued signal disconnects
+ * (the reference's REP socket simply loses the reply, controller.hpp:433-441, and the executor then sits
+ * in the orphaned request until the timeout of cuda_server.hpp:257-264) the front end cancels the ticket:
+ * 1 = it was still queued and is dropped, no ack will appear; 2 = its request had been started meanwhile:
+ * the pending ack is dropped and the request is completed at once (a half-finished registration is
+ * forgotten); 0 = unknown ticket or ack already taken. */
+int tp_signal_ticket(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack,
+                     int32_t* resp, int32_t* deferred, uint64_t* ticket);
+int tp_take_deferred_ack_ticket(tp_server* s, int32_t* ack, int32_t* resp, uint64_t* ticket);
+int tp_cancel_deferred(tp_server* s, uint64_t ticket);
 /* Request-timeout check of the executor loop (cuda_server.hpp:257-264); returns 1 when a
  * timed-out request was force-completed. */
 int tp_poll(tp_server* s);
@@ -215,6 +227,10 @@ int tp_poll(tp_server* s);
  * cudaMallocService / cudaFreeService (cuda_server.hpp:965-992, memory_manager.hpp:85-110). */
 int tp_malloc(tp_server* s, int32_t client, uint64_t bytes, uint64_t* vaddr);
 int tp_free(tp_server* s, int32_t client, uint64_t vaddr);
+/* 0 when [vaddr, vaddr + bytes) lies inside one block that the active function `client` may address now;
+ * no side effects.  For a front end that must set aside `bytes` of its own before the copy is validated
+ * (the reference mallocs `count` bytes unchecked, cuda_server.hpp:1007,1040). */
+int tp_check_address(tp_server* s, int32_t client, uint64_t vaddr, uint64_t bytes);
 /* cudaMemcpyService / cudaMemcpyAsyncService H2D (cuda_server.hpp:994-1037); while the
  * function is being registered the bytes go to the host weight store
  * (memory_manager.hpp:124-142, model_repo.hpp:151-168). */

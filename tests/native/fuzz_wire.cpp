@@ -3,6 +3,9 @@
 // request sequences, (b) the same bytes with random mutations, (c) random bytes, against an engine
 // created with TP_FLAG_HOST_ONLY (no device is touched).  Nothing may crash, leak or trip a
 // sanitizer; malformed input must come back as error codes.
+#include <sys/socket.h>
+
+#include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -52,7 +55,8 @@ int main() {
     // a well-formed registration: ExecuteAfterLoad, malloc, upload, device synchronise
     bool dfr = false;
     corpus.push_back(signal_msg(TP_REQ_EXECUTE_AFTER_LOAD, "3", "1"));
-    (void)handle_signal(S, corpus.back(), &dfr);
+    uint64_t ticket = 0;
+    (void)handle_signal(S, corpus.back(), &dfr, &ticket);
     {
         pb::Writer m;
         m.u64(1, 4096);
@@ -83,6 +87,47 @@ int main() {
         corpus.push_back(query(Q_DEVICE_SYNC, "", 3));
     }
     for (const auto& m : corpus) handle_query_list(S, m);
+    {
+        // device-to-host copies whose count the engine cannot vouch for (4 GiB, 2^64 - 1, a source that is
+        // no address) must be refused before the front end sets that much memory aside
+        const uint64_t counts[3] = {1ull << 32, ~0ull, 1ull << 31};
+        for (uint64_t cnt : counts)
+            for (int qt : {(int)Q_MEMCPY, (int)Q_MEMCPY_ASYNC}) {
+                pb::Writer c;
+                c.u64(1, KIND_D2H);
+                c.u64(2, 0x1234);
+                c.u64(3, 0x5678);
+                c.u64(4, cnt);
+                handle_query_list(S, query(qt, c.out, 3));
+            }
+        if (!S.staged[3].empty()) return 20;
+    }
+    {
+        // A peer that never reads: the writer gives up after its time budget (TORPOR_SEND_TIMEOUT_MS) and
+        // marks the connection failed instead of blocking the only server thread for ever.
+        setenv("TORPOR_SEND_TIMEOUT_MS", "200", 1);
+        int sv[2];
+        if (::socketpair(AF_UNIX, SOCK_STREAM, 0, sv) != 0) return 21;
+        int small = 4096;
+        (void)::setsockopt(sv[0], SOL_SOCKET, SO_SNDBUF, &small, sizeof small);
+        zmtp::Conn c(sv[0], zmtp::PUSH);
+        const auto t0 = std::chrono::steady_clock::now();
+        const bool sent = c.send({std::string(8u << 20, 'x')});
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        ::close(sv[1]);
+        if (sent || !c.failed() || ms > 5000.0) return 22;
+        // and a frame header that announces more than any legitimate message is refused at once
+        int sv2[2];
+        if (::socketpair(AF_UNIX, SOCK_STREAM, 0, sv2) != 0) return 23;
+        zmtp::Conn d(sv2[0], zmtp::PULL);
+        std::string hello = zmtp::greeting() + zmtp::ready_command(zmtp::PUSH);
+        hello.push_back(2);  // long frame
+        for (int sh = 56; sh >= 0; sh -= 8) hello.push_back((char)((zmtp::kMaxFrame + 1) >> sh));
+        if (::send(sv2[1], hello.data(), hello.size(), 0) != (ssize_t)hello.size()) return 24;
+        (void)d.pump();
+        ::close(sv2[1]);
+        if (!d.failed()) return 25;
+    }
 
     long handled = 0;
     for (int it = 0; it < 20000; ++it) {
@@ -104,12 +149,16 @@ int main() {
         }
         if (rng() % 5 == 0) {
             bool d = false;
-            (void)handle_signal(S, m, &d);
+            uint64_t tk = 0;
+            (void)handle_signal(S, m, &d, &tk);
+            if (d && rng() % 2) (void)tp_cancel_deferred(S.eng, tk);  // the peer went away while queued
+            if (rng() % 16 == 0) (void)tp_cancel_deferred(S.eng, rng() % 64);
         } else {
             handle_query_list(S, m);
         }
         int32_t ack, resp;
-        while (tp_take_deferred_ack(S.eng, &ack, &resp) == 1) {
+        uint64_t tk2 = 0;
+        while ((rng() % 2 ? tp_take_deferred_ack(S.eng, &ack, &resp) : tp_take_deferred_ack_ticket(S.eng, &ack, &resp, &tk2)) == 1) {
         }
         (void)tp_poll(S.eng);
         ++handled;

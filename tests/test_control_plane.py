@@ -6,6 +6,8 @@ import ctypes as C
 import itertools
 import random
 
+import numpy as np
+
 import pytest
 
 from oracle.host_ref import IaRef, LruRef, SchedRef
@@ -328,3 +330,121 @@ def test_default_topology_is_an_eight_gpu_all_to_all_node():
     s.l.tp_sched_set_status(s.h, 0, -1)                          # sibling of 0 is 1 (busy local), of 5 is 4 (busy local)
     s.l.tp_sched_set_status(s.h, 4, 4)
     assert s.decide(IA_POLICY, "g") == (0, -1, 2)                # GPU 5's sibling runs a heavy host swap
+
+
+# ------------------------------------------------------------ the engine's own victims vs the oracle
+def _tiny_function(s, fid, level, weight_mib):
+    """Registers a function of `weight_mib` MiB of weights and one 1 KiB activation through the C-ABI of a
+    host-only engine (no device): the LRU charges round_up(weights) + round_up(activations) slabs."""
+    from torpor_amd.server import ACK_OK, OP_RELU, REQ_EXECUTE_AFTER_LOAD
+    assert s.signal(REQ_EXECUTE_AFTER_LOAD, fid, str(level))[:2] == (ACK_OK, 0)
+    w = s.malloc(fid, weight_mib << 20)
+    s.h2d(fid, w, np.zeros((weight_mib << 20) // 4, np.float32))
+    s.device_synchronize(fid)
+    a = s.malloc(fid, 1024)
+    s.launch(fid, OP_RELU, [w, a], [256])
+    out = np.empty(256, np.float32)
+    s.d2h_async(fid, out, a)       # the request-finished marker: the registration completes here
+    try:
+        s.stream_synchronize(fid)
+    except Exception:              # host-only: no data to deliver (-19)
+        pass
+    return s.model_info(fid)["total_bytes"]
+
+
+@pytest.mark.parametrize("policy", ["two_class", "lru"])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_engine_victims_follow_the_oracle_on_levelled_traces(policy, seed):
+    """include/server/evictor.hpp:28-264 + controller.hpp:141-216,392-400 as the engine runs them: after every
+    Execute / Load / Unload signal (with requests left running in between, so that the active function is
+    locked) the set of resident functions and the charged bytes equal those of the oracle evictor fed the
+    same trace.  The pool is twice the budget, so the contiguous-extent fallback never adds victims."""
+    from oracle.host_ref import IaRef, LruRef
+    from torpor_amd.server import ACK_INAVAIL, ACK_OK, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD, Server
+
+    rng = np.random.default_rng(100 + seed)
+    budget = 96 << 20
+    two = policy == "two_class"
+    with Server(host_only=True, mem_limit_bytes=budget, pool_bytes=2 * budget + (64 << 20), request_timeout_ms=60000,
+                evict_lru=not two) as s:
+        ref = IaRef(1, budget) if two else LruRef(budget)
+        n = 14
+        level = {fid: int(rng.integers(0, 3)) for fid in range(n)}
+        size = {}
+
+        def ref_add(fid):
+            if two:
+                ref.level[fid] = level[fid]
+                return ref.check_and_add(0, fid, size[fid])
+            return ref.check_and_add(fid, size[fid])
+
+        def ref_resident(fid):
+            return (0 in ref.gpus.get(fid, set())) if two else (fid in ref.items)
+
+        def check(what):
+            got = [s.resident(f) for f in size]
+            want = [ref_resident(f) for f in size]
+            assert got == want, (what, got, want)
+            used = ref.cur[0] if two else ref.cur
+            assert s.pool_stats()["lru_used"] == used, what
+
+        for fid in range(n):
+            size[fid] = _tiny_function(s, fid, level[fid], int(rng.integers(2, 20)))
+            ref_add(fid)           # controller.hpp:223-227: the eviction check of a finished cold start
+            check(f"register {fid}")
+        active = None
+        for step in range(600):
+            fid = int(rng.integers(0, n))
+            r = rng.random()
+            if active is not None and r < 0.35:
+                assert s.model_info(active)["resident"] == 1
+                _finish(s, active)     # the running request ends
+                if two:
+                    ref.unlock(0, active)
+                else:
+                    ref.unlock(active)
+                active = None
+                check(f"step {step}: complete")
+            elif r < 0.6:
+                if active is None:
+                    assert s.signal(REQ_EXECUTE, fid)[:2] == (ACK_OK, 0)
+                    ref_add(fid)
+                    if two:
+                        ref.lock(0, fid)
+                    else:
+                        ref.lock(fid)
+                    active = fid
+                    check(f"step {step}: execute {fid}")
+            elif r < 0.85:
+                ack = s.signal(REQ_LOAD, fid)[0]
+                if fid == active:
+                    assert ack == ACK_INAVAIL
+                else:
+                    assert ack == ACK_OK
+                    ref_add(fid)
+                check(f"step {step}: load {fid}")
+            else:
+                ack = s.signal(REQ_UNLOAD, fid)[0]
+                if fid == active:
+                    assert ack == ACK_INAVAIL
+                else:
+                    assert ack == ACK_OK
+                    if two:
+                        ref.force_evict(0, fid)
+                    else:
+                        ref.force_evict(fid)
+                check(f"step {step}: unload {fid}")
+        st = s.pool_stats()
+        assert st["evictions"] > 50 and st["swap_ins"] > 50     # the budget did bind
+
+
+def _finish(s, fid):
+    """Ends the running request of `fid` the way a function does: one asynchronous device-to-host copy of
+    its activation (the completion marker, cuda_server.hpp:1044) and the stream synchronisation."""
+    from torpor_amd._lib import TorporError
+    va = (0x7A << 56) | (fid << 44) | (1 << 43)   # the function's first activation block
+    s.d2h_async(fid, np.empty(256, np.float32), va)
+    try:
+        s.stream_synchronize(fid)
+    except TorporError:
+        pass

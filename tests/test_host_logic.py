@@ -13,7 +13,8 @@ from oracle.host_ref import LruRef
 from torpor_amd import _lib
 from torpor_amd._lib import TorporError
 from torpor_amd.functions import resnet
-from torpor_amd.server import (ACK_INAVAIL, ACK_OK, OP_RELU, REQ_EXECUTE, REQ_EXECUTE_AFTER_LOAD, REQ_LOAD,
+from torpor_amd.server import (ACK_INAVAIL, ACK_OK, OP_ADD, OP_COPY2D, OP_NCHW_TO_NHWC, OP_RELU, REQ_EXECUTE,
+                               REQ_EXECUTE_AFTER_LOAD, REQ_LOAD,
                                REQ_UNLOAD, Server)
 
 SLAB = 2 << 20
@@ -473,3 +474,88 @@ def test_error_paths(host_server):
         s.stream_synchronize(20)                                     # sticky op errors + no device
     assert s.model_info(20)["registered"] == 1
     assert s.signal(REQ_UNLOAD, 20, "")[0] == ACK_OK
+
+
+def test_arguments_whose_spans_would_wrap_are_refused(host_server):
+    """Element counts and byte counts arrive unvalidated from wire clients; their products must not wrap
+    into a span that passes the bounds test (64-bit products of dims, off + span, the cast of a byte count
+    to a signed 64-bit integer)."""
+    s = host_server
+    assert s.signal(REQ_EXECUTE_AFTER_LOAD, 21, "1")[0] == ACK_OK
+    w = s.malloc(21, 1024)
+    s.h2d(21, w, np.zeros(256, np.float32))
+    s.device_synchronize(21)   # the upload phase ends
+    a = s.malloc(21, 1024)
+    b = s.malloc(21, 1024)
+
+    def refused(fn, *args, **kw):
+        with pytest.raises(TorporError) as e:
+            fn(*args, **kw)
+        assert e.value.code in (-22, -14, -12, -38), e.value.code
+    s.launch(21, OP_RELU, [a, b], [256])
+    refused(s.launch, 21, OP_RELU, [a, b], [257])
+    refused(s.launch, 21, OP_RELU, [a, b], [1 << 62])            # 2^62 elements x 4 bytes = 2^64
+    refused(s.launch, 21, OP_RELU, [a, b], [(1 << 62) + 1])
+    refused(s.launch, 21, OP_NCHW_TO_NHWC, [a, b], [1 << 16] * 4)  # N*C*H*W = 2^64
+    refused(s.launch, 21, OP_NCHW_TO_NHWC, [a, b], [1 << 15, 1 << 16, 1 << 16, 1 << 16])
+    refused(s.launch, 21, OP_NCHW_TO_NHWC, [a, b], [(1 << 32) + 1, 1, 1, 1])   # would be narrowed to int 1
+    refused(s.launch, 21, OP_COPY2D, [a, b], [1 << 40, 4, 1 << 40, 1 << 40])
+    refused(s.launch, 21, OP_ADD, [a, b, a], [-1, 0])
+    refused(s.d2d, 21, a, b, (1 << 64) - 1)
+    refused(s.d2d, 21, a, b, (1 << 63) + 16)
+    refused(s.d2d, 21, a + 8, b, (1 << 64) - 4)                  # off + span wraps to a small value
+    refused(s.memset, 21, a, 0, (1 << 64) - 1)
+    refused(s.memset, 21, a + 16, 0, (1 << 64) - 8)
+    refused(s.malloc, 21, (1 << 64) - 1)
+    refused(s.gemm, 21, a, w, b, 1 << 31, 1 << 31, 4, xs_r=4, ys_c=4, ldc=1 << 31)
+    refused(s.gemm, 21, a, w, b, 4, 4, 4, xs_r=(1 << 62), ys_c=4, ldc=4)
+    refused(s.gemm, 21, a, w, b, 2, 2, 2, xs_r=2, ys_c=2, ldc=2, nb0=1 << 20, nb1=1 << 20)
+    refused(s.conv, 21, a, w, b, 1 << 20, 1 << 20, 1 << 20, 1 << 4, 1, 1, 1)
+    refused(s.bn, 21, a, b, w, w, w, w, 1e-5, 1 << 50, 4)
+    s.d2d(21, a, b, 1024)                                         # what fits still passes
+    s.memset(21, a, 0, 1024)
+    s.gemm(21, a, w, b, 4, 4, 4, xs_r=4, ys_c=4, ldc=4)
+    out = np.empty(4, np.float32)
+    s.d2h_async(21, out, a)
+    with pytest.raises(TorporError):
+        s.stream_synchronize(21)
+    assert s.signal(REQ_UNLOAD, 21, "")[0] == ACK_OK
+
+
+def test_deferred_acks_carry_tickets_and_can_be_cancelled():
+    """Queued signals are matched to their acks by ticket; a cancelled ticket never produces an ack, and a
+    request that had been started for a peer that is gone is completed at once (controller.hpp:242-262 hands
+    the executor to the oldest queued signal)."""
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20, request_timeout_ms=60000) as s:
+        fns = {fid: _register(s, fid) for fid in (1, 2, 3, 4)}
+        assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)
+        t2 = s.signal_ticket(REQ_EXECUTE, 2)
+        t3 = s.signal_ticket(REQ_EXECUTE, 3)
+        t4 = s.signal_ticket(REQ_EXECUTE, 4)
+        assert [t[2] for t in (t2, t3, t4)] == [True] * 3
+        assert t2[3] < t3[3] < t4[3] and t2[3] >= 1
+        assert s.take_deferred_ack_ticket() is None
+        # the peer of the first queued signal goes away while still queued: no ack for it, ever
+        assert s.cancel_deferred(t2[3]) == 1
+        assert s.cancel_deferred(t2[3]) == 0
+        assert s.cancel_deferred(12345) == 0
+        x = np.zeros((1, 3, 32, 32), np.float32)
+
+        def drive(fid):     # the data plane of a request that the engine has already started
+            packed, outbuf, _ = fns[fid].pack([x])
+            with pytest.raises(TorporError) as e:
+                s.replay(fid, packed, outbuf)
+            assert e.value.code == -19              # host-only: the request completes, there is no data
+        drive(1)
+        assert s.take_deferred_ack_ticket() == (ACK_OK, 0, t3[3])   # function 3 was started, not 2
+        assert s.take_deferred_ack_ticket() is None
+        with pytest.raises(TorporError) as e:
+            s.malloc(2, 64)
+        assert e.value.code == -72                  # function 2 is not the active one
+        assert s.check_address(2, 0, 4) == -72
+        assert s.check_address(3, 0x1234, 4) == -14
+        # function 3 finishes, function 4 is started; its peer disappears before the ack is taken:
+        drive(3)
+        assert s.cancel_deferred(t4[3]) == 2        # ack dropped, the started request completed at once
+        assert s.take_deferred_ack_ticket() is None
+        assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)   # the executor is free again

@@ -171,3 +171,39 @@ def test_deferred_ack_and_timeout_over_the_wire(wire_server):
         assert 0.2 < time.time() - t0 < 5.0
         time.sleep(0.4)                                               # client 5's own request times out too
         assert a.signal(REQ_UNLOAD, 4)[0] == ACK_OK and b.signal(REQ_UNLOAD, 5)[0] == ACK_OK
+
+
+def test_ack_of_a_queued_peer_that_died_is_not_handed_to_the_next_one(wire_server):
+    """Two Execute signals are queued behind a running request; the first sender disconnects before its
+    ack.  The second must get the ack of *its own* request and find itself active (its data-plane calls
+    are accepted), not the orphaned ack of the dead peer's request."""
+    ids = (6, 7, 8)
+    conns = {cid: wire.RemoteServer(wire_server, client_id=cid) for cid in ids}
+    try:
+        for cid, rs in conns.items():
+            assert rs.signal(REQ_EXECUTE_AFTER_LOAD, cid, "1")[0] == ACK_OK
+            va = rs.malloc(cid, 1024)
+            rs.h2d(cid, va, np.ones(256, np.float32))
+            rs.device_synchronize(cid)
+            act = rs.malloc(cid, 1024)
+            rs.launch(cid, OP_RELU, [va, act], [256])
+            rs.d2h_async(cid, np.empty(256, np.float32), act)
+            with pytest.raises(wire.WireError):
+                rs.stream_synchronize(cid)
+        assert conns[6].signal(REQ_EXECUTE, 6)[:2] == (ACK_OK, 0)     # runs until its 300 ms timeout
+        # client 7 queues an Execute and goes away without waiting for the ack
+        conns[7].req.send([b"", wire.signal_request(REQ_EXECUTE, 7, "")])
+        time.sleep(0.05)
+        conns[7].close()
+        t0 = time.time()
+        assert conns[8].signal(REQ_EXECUTE, 8)[:2] == (ACK_OK, 0)     # answered when client 6's request ends
+        assert 0.1 < time.time() - t0 < 5.0
+        with pytest.raises(wire.WireError) as e:
+            conns[8].malloc(8, 1 << 20)
+        assert e.value.code == -12        # active (the frozen arena refuses); -72 would mean "not the active function"
+        time.sleep(0.4)
+        for cid in (6, 8):
+            assert conns[cid].signal(REQ_UNLOAD, cid)[0] == ACK_OK
+    finally:
+        for cid in (6, 8):
+            conns[cid].close()

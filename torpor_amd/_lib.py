@@ -109,6 +109,11 @@ SYMBOLS = {
     "tp_version": (C.c_char_p, []),
     "tp_signal": (C.c_int, [_P, _I32, C.c_char_p, C.c_char_p, C.POINTER(_I32), C.POINTER(_I32), C.POINTER(_I32)]),
     "tp_take_deferred_ack": (C.c_int, [_P, C.POINTER(_I32), C.POINTER(_I32)]),
+    "tp_signal_ticket": (C.c_int, [_P, _I32, C.c_char_p, C.c_char_p, C.POINTER(_I32), C.POINTER(_I32),
+                                   C.POINTER(_I32), C.POINTER(_U64)]),
+    "tp_take_deferred_ack_ticket": (C.c_int, [_P, C.POINTER(_I32), C.POINTER(_I32), C.POINTER(_U64)]),
+    "tp_cancel_deferred": (C.c_int, [_P, _U64]),
+    "tp_check_address": (C.c_int, [_P, _I32, _U64, _U64]),
     "tp_poll": (C.c_int, [_P]),
     "tp_malloc": (C.c_int, [_P, _I32, _U64, C.POINTER(_U64)]),
     "tp_free": (C.c_int, [_P, _I32, _U64]),

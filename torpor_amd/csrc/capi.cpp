@@ -94,6 +94,31 @@ int tp_take_deferred_ack(tp_server* s, int32_t* ack, int32_t* resp) {
     return E.take_deferred_ack(ack, resp);
     TP_GUARD_END
 }
+int tp_signal_ticket(tp_server* s, int32_t type, const char* function, const char* payload, int32_t* ack,
+                     int32_t* resp, int32_t* deferred, uint64_t* ticket) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.signal(type, function, payload, ack, resp, deferred, ticket);
+    TP_GUARD_END
+}
+int tp_take_deferred_ack_ticket(tp_server* s, int32_t* ack, int32_t* resp, uint64_t* ticket) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.take_deferred_ack(ack, resp, ticket);
+    TP_GUARD_END
+}
+int tp_cancel_deferred(tp_server* s, uint64_t ticket) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.cancel_deferred(ticket);
+    TP_GUARD_END
+}
+int tp_check_address(tp_server* s, int32_t client, uint64_t vaddr, uint64_t bytes) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.check_address(client, vaddr, bytes);
+    TP_GUARD_END
+}
 int tp_poll(tp_server* s) {
     TP_GUARD_BEGIN
     ENG(s);

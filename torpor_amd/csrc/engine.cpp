@@ -295,7 +295,8 @@ int Engine::translate(Model& m, uint64_t va, uint64_t span, Xlat* out) {
         if (it == m.ablocks.begin()) return TP_EFAULT;
         --it;
         ABlock& b = it->second;
-        if (off >= b.voff + b.size || off + span > b.voff + b.size) return TP_EFAULT;
+        // (off - b.voff) < b.size here, so neither side of the comparison can wrap
+        if (off >= b.voff + b.size || span > b.size - (off - b.voff)) return TP_EFAULT;
         // Once the arena is frozen every block keeps its place for good and later requests repeat
         // the tracked op stream without re-issuing its malloc/free calls, so liveness is only
         // enforced while the first inference is being tracked.
@@ -316,7 +317,7 @@ int Engine::translate(Model& m, uint64_t va, uint64_t span, Xlat* out) {
                                [](uint64_t o, const Param& p) { return o < p.voff; });
     if (it == m.params.begin()) return TP_EFAULT;
     --it;
-    if (off >= it->voff + it->size || off + span > it->voff + it->size) return TP_EFAULT;
+    if (off >= it->voff + it->size || span > it->size - (off - it->voff)) return TP_EFAULT;
     if (m.state == MS_LOADING || !m.resident) return TP_EFAULT;
     out->p = m.w_dev + it->image_off + (off - it->voff);
     out->weight = true;
@@ -401,6 +402,7 @@ int Engine::op_malloc(int client, uint64_t bytes, uint64_t* va) {
     Model* m = active_model(client, &err);
     if (!m) return err;
     if (bytes == 0) bytes = 1;
+    if (bytes > kVaOffMask) return TP_ENOMEM;  // larger than a function's address region: nothing below may wrap
     const uint64_t base = kVaTag | ((uint64_t)m->id << kVaClientShift);
     if (mode_ == MODE_LOAD) {  // weight block: cuda_server.hpp:969-970 with load flag set
         const uint64_t off = m->wbump;
@@ -422,6 +424,7 @@ int Engine::op_malloc(int client, uint64_t bytes, uint64_t* va) {
         return 0;
     }
     if (m->act_frozen) return TP_ENOMEM;  // arena is sized by the first (tracked) inference
+    if (m->abump + bytes > kVaOffMask) return TP_ENOMEM;
     ABlock b;
     b.voff = m->abump;
     b.size = bytes;
@@ -463,7 +466,7 @@ int Engine::ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need) {
 
 int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
     if (bytes == 0) return 0;
-    if (!src) return TP_EINVAL;
+    if (!src || bytes > kVaOffMask) return TP_EINVAL;
     if (mode_ == MODE_LOAD) {
         // memory_manager.hpp:124-142 + model_repo.hpp:151-168: capture into the host weight store
         if ((dst & kVaTagMask) != kVaTag || (int)((dst >> kVaClientShift) & kVaClientMask) != m.id ||
@@ -472,7 +475,7 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
         const uint64_t off = dst & kVaOffMask;
         bool inside = false;
         for (const WBlock& b : m.wblocks)
-            if (off >= b.voff && off + bytes <= b.voff + b.size) {
+            if (off >= b.voff && off - b.voff < b.size && bytes <= b.size - (off - b.voff)) {
                 inside = true;
                 break;
             }
@@ -536,7 +539,7 @@ int Engine::op_h2d(int client, uint64_t dst, const void* src, uint64_t bytes) {
 }
 
 int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
-    if (!dst && bytes) return TP_EINVAL;
+    if ((!dst && bytes) || bytes > kVaOffMask) return TP_EINVAL;
     void* p = nullptr;
     int r = resolve(m, src, bytes, false, &p);
     if (r) return r;
@@ -677,7 +680,7 @@ int Engine::op_d2h(int client, void* dst, uint64_t src, uint64_t bytes) {
     int err = 0;
     Model* m = active_model(client, &err);
     if (!m) return err;
-    if (!dst && bytes) return TP_EINVAL;
+    if ((!dst && bytes) || bytes > kVaOffMask) return TP_EINVAL;
     void* p = nullptr;
     int r = resolve(*m, src, bytes, false, &p);
     if (r) return r;
@@ -692,6 +695,7 @@ int Engine::op_d2d(int client, uint64_t dst, uint64_t src, uint64_t bytes) {
     int err = 0;
     Model* m = active_model(client, &err);
     if (!m) return err;
+    if (bytes > kVaOffMask) return TP_EINVAL;  // before the count is narrowed into the recorded op
     Op op;
     op.kind = OPK_D2D;
     op.p[0] = dst;
@@ -708,6 +712,7 @@ int Engine::op_memset(int client, uint64_t dst, int value, uint64_t bytes) {
     int err = 0;
     Model* m = active_model(client, &err);
     if (!m) return err;
+    if (bytes > kVaOffMask) return TP_EINVAL;
     Op op;
     op.kind = OPK_MEMSET;
     op.p[0] = dst;
@@ -1455,15 +1460,20 @@ void Engine::complete_request() {
         if (status == ES_COLD) check_eviction(*m);  // controller.hpp:223-227
     }
     exec_status_ = ES_AVAIL;
-    if (!req_queue_.empty()) {  // controller.hpp:242-262
+    start_next_queued();
+}
+
+// controller.hpp:242-262: the executor is free; the oldest queued signal gets it and its ack is produced
+void Engine::start_next_queued() {
+    while (exec_status_ == ES_AVAIL && !req_queue_.empty()) {
         Queued q = req_queue_.front();
         req_queue_.pop_front();
         if (q.cold) {
             start_cold(q.id, q.level);
-            deferred_acks_.emplace_back(TP_ACK_OK, 0);
+            deferred_acks_.push_back({TP_ACK_OK, 0, q.ticket, q.id});
         } else {
             int r = start_execute(q.id);
-            deferred_acks_.emplace_back(r ? TP_ACK_INAVAIL : TP_ACK_OK, 0);
+            deferred_acks_.push_back({r ? TP_ACK_INAVAIL : TP_ACK_OK, 0, q.ticket, q.id});
         }
     }
 }
@@ -1486,13 +1496,69 @@ int Engine::poll() {
     return poll_timeout_locked() ? 1 : 0;
 }
 
-int Engine::take_deferred_ack(int* ack, int* resp) {
+int Engine::take_deferred_ack(int* ack, int* resp, uint64_t* ticket) {
     std::lock_guard<std::mutex> lk(mu_);
     if (deferred_acks_.empty()) return 0;
-    if (ack) *ack = deferred_acks_.front().first;
-    if (resp) *resp = deferred_acks_.front().second;
+    if (ack) *ack = deferred_acks_.front().ack;
+    if (resp) *resp = deferred_acks_.front().resp;
+    if (ticket) *ticket = deferred_acks_.front().ticket;
     deferred_acks_.pop_front();
     return 1;
+}
+
+// The peer that sent a queued signal is gone.  Still queued: the entry is dropped and no ack will
+// appear for it (1).  Already started but its ack not yet taken: the ack is dropped and the request,
+// which nobody will drive, is completed at once instead of holding the executor until the request
+// timeout (2).  Unknown or already delivered: 0.
+int Engine::cancel_deferred(uint64_t ticket) {
+    std::lock_guard<std::mutex> lk(mu_);
+    for (auto it = req_queue_.begin(); it != req_queue_.end(); ++it)
+        if (it->ticket == ticket) {
+            req_queue_.erase(it);
+            return 1;
+        }
+    for (auto it = deferred_acks_.begin(); it != deferred_acks_.end(); ++it)
+        if (it->ticket == ticket) {
+            const int id = it->id;
+            const bool started = it->ack == TP_ACK_OK;
+            deferred_acks_.erase(it);
+            if (started && active_ == id) {
+                if (mode_ == MODE_LOAD || mode_ == MODE_TRACK) {
+                    // a registration nobody finishes: forget the half-built model
+                    Model* m = find(id);
+                    if (!host_only()) (void)hipStreamSynchronize(compute_);  // its tracked kernels may still run
+                    if (m) {
+                        for (auto& kv : m->ablocks)
+                            if (kv.second.pool_off != UINT64_MAX) pool_.release(kv.second.pool_off);
+                        if (m->w_pool_off != UINT64_MAX) pool_.release(m->w_pool_off);
+                        host_free(m->host_image);
+                        models_.erase(id);
+                    }
+                    active_ = -1;
+                    mode_ = MODE_NONE;
+                    exec_status_ = ES_AVAIL;
+                    start_next_queued();
+                } else {
+                    if (!host_only()) (void)hipStreamSynchronize(compute_);
+                    complete_request();
+                }
+            }
+            return 2;
+        }
+    return 0;
+}
+
+// Does [va, va + bytes) lie inside one block the active function `client` may address right now?
+// No side effects (no access-order rank, no gate wait): a front end asks before it sets aside
+// `bytes` of its own memory for a copy.
+int Engine::check_address(int client, uint64_t va, uint64_t bytes) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (active_ < 0 || mode_ == MODE_NONE) return TP_ESTATE;
+    if (client != active_) return TP_ENOTACTIVE;
+    Model* m = find(active_);
+    if (!m) return TP_ENOENT;
+    Xlat x;
+    return translate(*m, va, bytes, &x);
 }
 
 static bool parse_int(const char* s, int* out) {
@@ -1504,11 +1570,13 @@ static bool parse_int(const char* s, int* out) {
     return true;
 }
 
-int Engine::signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred) {
+int Engine::signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred,
+                   uint64_t* ticket) {
     std::lock_guard<std::mutex> lk(mu_);
     if (ack) *ack = TP_ACK_OK;
     if (resp) *resp = -1;
     if (deferred) *deferred = 0;
+    if (ticket) *ticket = 0;
     int id = -1;
     if (!parse_int(function, &id) || id < 0 || id > kMaxClient) return TP_EINVAL;  // cuda_server.hpp:221 stoi(func)
     poll_timeout_locked();
@@ -1523,8 +1591,9 @@ int Engine::signal(int type, const char* function, const char* payload, int* ack
                     if (ack) *ack = TP_ACK_INAVAIL;
                     return 0;
                 }
-                req_queue_.push_back({id, true, level});
+                req_queue_.push_back({id, true, level, ++ticket_seq_});
                 if (deferred) *deferred = 1;
+                if (ticket) *ticket = ticket_seq_;
                 return 0;
             }
             start_cold(id, level);
@@ -1533,8 +1602,9 @@ int Engine::signal(int type, const char* function, const char* payload, int* ack
         }
         case TP_REQ_EXECUTE: {  // controller.hpp:163-186
             if (busy) {
-                req_queue_.push_back({id, false, 1});
+                req_queue_.push_back({id, false, 1, ++ticket_seq_});
                 if (deferred) *deferred = 1;
+                if (ticket) *ticket = ticket_seq_;
                 return 0;
             }
             int r = start_execute(id);
@@ -1609,25 +1679,61 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
                                         : tpk::Workspace{};
     // Every operand is translated together with the byte span the kernel will touch, so an op
     // whose shapes do not fit its buffers is refused on the host instead of faulting the GPU.
-    auto R = [&](int idx, bool optional, int64_t elems, int64_t elem_size = 4) -> int {
+    // Spans are computed in 128-bit integers from arguments that have been range-checked first
+    // (anything a launcher narrows to int: at most INT32_MAX; counts, strides and pitches: at most
+    // the size of an address region), so that no product can wrap into a span that passes.
+    using i128 = __int128;
+    constexpr int64_t kIntMax = 0x7fffffff;
+    constexpr int64_t kLongMax = (int64_t)kVaOffMask;
+    auto R = [&](int idx, bool optional, i128 elems, int elem_size = 4) -> int {
         if (elems < 1) elems = 1;
+        if (elems > (i128)kLongMax) return TP_EFAULT;  // no block is that large
         return resolve(m, op.p[idx], (uint64_t)elems * (uint64_t)elem_size, optional, &q[idx]);
     };
-    const int64_t* I = op.i;
-    for (int k = 0; k < op.ni && k < 20; ++k)
-        if (I[k] < 0) return TP_EINVAL;
+    i128 I[20];
+    for (int k = 0; k < 20; ++k) I[k] = k < op.ni ? (i128)op.i[k] : (i128)0;
+    // arguments whose bit is set in long_mask may be as large as an address region, the others fit an int
+    auto ranges_ok = [&](uint32_t long_mask) {
+        for (int k = 0; k < op.ni && k < 20; ++k) {
+            if (op.i[k] < 0) return false;
+            if (op.i[k] > (((long_mask >> k) & 1u) ? kLongMax : kIntMax)) return false;
+        }
+        return true;
+    };
+    static const uint32_t kLaunchLong[] = {
+        /* 0 */ 0,
+        /* RELU */ 1u << 0, /* ADD */ 1u << 0, /* BIAS_ACT */ 1u << 0, /* GELU */ 1u << 0,
+        /* MAXPOOL */ 1u << 8, /* AVGPOOL */ 0, /* LAYERNORM */ 1u << 0, /* SOFTMAX */ (1u << 0) | (1u << 2),
+        /* EMBEDDING */ (1u << 0) | (1u << 3), /* NCHW_TO_NHWC */ 0, /* NHWC_TO_NCHW */ 0, /* SUM */ 1u << 0,
+        /* FILL */ 1u << 0, /* ATTENTION */ 0xF0u, /* AVGPOOL2D */ 1u << 7, /* COPY2D */ (1u << 0) | (1u << 2) | (1u << 3),
+        /* SCALE_CHANNELS */ 1u << 1};
+    {
+        uint32_t long_mask = 0;
+        switch (op.kind) {
+            case OPK_GEMM: long_mask = 0xF8u | 0xFC00u | (1u << 16); break;  // strides, ldc, batch strides, ldr
+            case OPK_CONV: long_mask = (1u << 13) | (1u << 15) | (1u << 16); break;  // ldr, x / y pitch
+            case OPK_BN: long_mask = (1u << 0) | (1u << 2) | (1u << 5); break;  // rows, hw, x pitch
+            case OPK_LAUNCH:
+                if (op.op_id > 0 && op.op_id < (int)(sizeof(kLaunchLong) / sizeof(kLaunchLong[0])))
+                    long_mask = kLaunchLong[op.op_id];
+                break;
+            default: break;
+        }
+        if (!ranges_ok(long_mask)) return TP_EINVAL;
+    }
     int r = 0;
     switch (op.kind) {
         case OPK_GEMM: {
-            const int64_t M = I[0], N = I[1], K = I[2];
-            const int64_t nb0 = I[8], nb1 = I[9];
+            const i128 M = I[0], N = I[1], K = I[2];
+            const i128 nb0 = I[8], nb1 = I[9];
             if (M < 1 || N < 1 || nb0 < 1 || nb1 < 1) return TP_EINVAL;
-            const int64_t kx = K > 0 ? K - 1 : 0;
-            const int64_t xs = (M - 1) * I[3] + kx * I[4] + (nb0 - 1) * I[10] + (nb1 - 1) * I[11] + 1;
-            const int64_t ys = (N - 1) * I[5] + kx * I[6] + (nb0 - 1) * I[12] + (nb1 - 1) * I[13] + 1;
-            const int64_t cs = (M - 1) * I[7] + N + (nb0 - 1) * I[14] + (nb1 - 1) * I[15];
+            if (nb0 * nb1 > 65535) return TP_EUNSUPPORTED;  // batches are the grid's z dimension
+            const i128 kx = K > 0 ? K - 1 : 0;
+            const i128 xs = (M - 1) * I[3] + kx * I[4] + (nb0 - 1) * I[10] + (nb1 - 1) * I[11] + 1;
+            const i128 ys = (N - 1) * I[5] + kx * I[6] + (nb0 - 1) * I[12] + (nb1 - 1) * I[13] + 1;
+            const i128 cs = (M - 1) * I[7] + N + (nb0 - 1) * I[14] + (nb1 - 1) * I[15];
             if (I[7] < N) return TP_EINVAL;
-            const int64_t ldr = I[16] ? I[16] : I[7];
+            const i128 ldr = I[16] ? I[16] : I[7];
             if (op.p[8] && (nb0 * nb1 != 1 || ldr < N)) return TP_EUNSUPPORTED;
             if ((r = R(0, false, xs)) || (r = R(1, false, ys)) || (r = R(2, false, cs))) return r;
             for (int k = 3; k < 8 && !r; ++k) r = R(k, true, N);
@@ -1640,41 +1746,41 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             g.X = static_cast<const float*>(q[0]);
             g.Y = static_cast<const float*>(q[1]);
             g.C = static_cast<float*>(q[2]);
-            g.M = M;
-            g.N = N;
-            g.K = K;
-            g.xs_r = I[3];
-            g.xs_k = I[4];
-            g.ys_c = I[5];
-            g.ys_k = I[6];
-            g.ldc = I[7];
+            g.M = (long)M;
+            g.N = (long)N;
+            g.K = (long)K;
+            g.xs_r = (long)I[3];
+            g.xs_k = (long)I[4];
+            g.ys_c = (long)I[5];
+            g.ys_k = (long)I[6];
+            g.ldc = (long)I[7];
             g.nb0 = (int)nb0;
             g.nb1 = (int)nb1;
-            g.xb0 = I[10];
-            g.xb1 = I[11];
-            g.yb0 = I[12];
-            g.yb1 = I[13];
-            g.cb0 = I[14];
-            g.cb1 = I[15];
+            g.xb0 = (long)I[10];
+            g.xb1 = (long)I[11];
+            g.yb0 = (long)I[12];
+            g.yb1 = (long)I[13];
+            g.cb0 = (long)I[14];
+            g.cb1 = (long)I[15];
             g.ep = ep_from(op, q, 3, 0, 16);
-            g.ep.ldr = ldr;
+            g.ep.ldr = (long)ldr;
             if (!launch) return 0;
             return tpk::launch_gemm(g, ws, compute_);
         }
         case OPK_CONV: {
-            const int64_t N = I[0], H = I[1], W = I[2], Cin = I[3], Cout = I[4], KH = I[5], KW = I[6];
-            const int64_t sh = I[7], sw = I[8], ph = I[9], pw = I[10];
+            const i128 N = I[0], H = I[1], W = I[2], Cin = I[3], Cout = I[4], KH = I[5], KW = I[6];
+            const i128 sh = I[7], sw = I[8], ph = I[9], pw = I[10];
             if (N < 1 || H < 1 || W < 1 || Cin < 1 || Cout < 1 || KH < 1 || KW < 1 || sh < 1 || sw < 1)
                 return TP_EINVAL;
-            const int64_t Ho = (H + 2 * ph - KH) / sh + 1, Wo = (W + 2 * pw - KW) / sw + 1;
+            const i128 Ho = (H + 2 * ph - KH) / sh + 1, Wo = (W + 2 * pw - KW) / sw + 1;
             if (H + 2 * ph < KH || W + 2 * pw < KW || Ho < 1 || Wo < 1) return TP_EINVAL;
-            const int64_t xpitch = op.ni > 15 ? I[15] : 0, ypitch = op.ni > 16 ? I[16] : 0;
-            const int64_t groups = (op.ni > 17 && I[17] > 0) ? I[17] : 1;
+            const i128 xpitch = op.ni > 15 ? I[15] : 0, ypitch = op.ni > 16 ? I[16] : 0;
+            const i128 groups = (op.ni > 17 && I[17] > 0) ? I[17] : 1;
             const bool x_nhwc = I[11] != 0, y_nhwc = I[12] != 0;
             if ((xpitch && (!x_nhwc || xpitch < Cin)) || (ypitch && (!y_nhwc || ypitch < Cout))) return TP_EINVAL;
             if (groups != 1 && (groups != Cin || Cin != Cout)) return TP_EUNSUPPORTED;
-            const int64_t ys = ypitch ? (N * Ho * Wo - 1) * ypitch + Cout : N * Ho * Wo * Cout;
-            const int64_t xs = xpitch ? (N * H * W - 1) * xpitch + Cin : N * H * W * Cin;
+            const i128 ys = ypitch ? (N * Ho * Wo - 1) * ypitch + Cout : N * Ho * Wo * Cout;
+            const i128 xs = xpitch ? (N * H * W - 1) * xpitch + Cin : N * H * W * Cin;
             if ((r = R(0, false, xs)) || (r = R(1, false, Cout * (Cin / groups) * KH * KW)) || (r = R(2, false, ys)))
                 return r;
             for (int k = 3; k < 8 && !r; ++k) r = R(k, true, Cout);
@@ -1700,8 +1806,8 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             c.pw = (int)pw;
             c.x_nhwc = (int)I[11];
             c.y_nhwc = (int)I[12];
-            c.x_pitch = xpitch;
-            c.y_pitch = ypitch;
+            c.x_pitch = (long)xpitch;
+            c.y_pitch = (long)ypitch;
             c.groups = (int)groups;
             c.ep = ep_from(op, q, 3, 0, 13);
             c.ep.ldr = 0;  // residual shares the layout and pitch of y
@@ -1709,10 +1815,10 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             return tpk::launch_conv2d(c, ws, compute_);
         }
         case OPK_BN: {
-            const int64_t rows = I[0], C = I[1];
-            const int64_t xpitch = op.ni > 5 ? I[5] : 0;
+            const i128 rows = I[0], C = I[1];
+            const i128 xpitch = op.ni > 5 ? I[5] : 0;
             if (C < 1 || (xpitch && xpitch < C)) return TP_EINVAL;
-            const int64_t xspan = (xpitch && rows > 0) ? (rows - 1) * xpitch + C : rows * C;
+            const i128 xspan = (xpitch && rows > 0) ? (rows - 1) * xpitch + C : rows * C;
             if ((r = R(0, false, xspan)) || (r = R(1, false, rows * C))) return r;
             for (int k = 2; k < 6 && !r; ++k) r = R(k, false, C);
             if (r) return r;
@@ -1752,11 +1858,11 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             return tpk::launch_bias_act(F(0), F(1), Fm(2), I[0], (int)I[1], (int)I[2], compute_);
         case TP_OP_MAXPOOL: {
             if (!need(2, 8, 0)) return TP_EINVAL;
-            const int64_t N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
+            const i128 N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
             if (N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || st < 1 || H + 2 * pad < k || W + 2 * pad < k)
                 return TP_EINVAL;
-            const int64_t Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
-            const int64_t yp = (op.ni > 8 && I[8]) ? I[8] : C;   // NHWC: elements between output pixels
+            const i128 Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
+            const i128 yp = (op.ni > 8 && I[8]) ? I[8] : C;   // NHWC: elements between output pixels
             if (yp < C || (yp != C && !I[7])) return TP_EINVAL;
             if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, (N * Ho * Wo - 1) * yp + C))) return r;
             if (!launch) return 0;
@@ -1777,7 +1883,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             return tpk::launch_layernorm(F(0), F(1), F(2), F(3), Fm(4), I[0], (int)I[1], op.f[0], compute_);
         case TP_OP_SOFTMAX: {
             if (!need(3, 3, 1)) return TP_EINVAL;
-            const int64_t rpm = I[2] > 0 ? I[2] : 1;
+            const i128 rpm = I[2] > 0 ? I[2] : 1;
             if ((r = R(0, false, I[0] * I[1])) || (r = R(1, true, ((I[0] + rpm - 1) / rpm) * I[1])) ||
                 (r = R(2, false, I[0] * I[1])))
                 return r;
@@ -1797,7 +1903,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         case TP_OP_NCHW_TO_NHWC:
         case TP_OP_NHWC_TO_NCHW: {
             if (!need(2, 4, 0)) return TP_EINVAL;
-            const int64_t n = I[0] * I[1] * I[2] * I[3];
+            const i128 n = I[0] * I[1] * I[2] * I[3];
             if ((r = R(0, false, n)) || (r = R(1, false, n))) return r;
             if (!launch) return 0;
             return op.op_id == TP_OP_NCHW_TO_NHWC
@@ -1811,12 +1917,12 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             return tpk::launch_sum(F(0), Fm(1), I[0], compute_);
         case TP_OP_AVGPOOL2D: {
             if (!need(2, 8, 0)) return TP_EINVAL;
-            const int64_t N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
+            const i128 N = I[0], H = I[1], W = I[2], C = I[3], k = I[4], st = I[5], pad = I[6];
             if (N < 1 || H < 1 || W < 1 || C < 1 || k < 1 || st < 1 || H + 2 * pad < k || W + 2 * pad < k)
                 return TP_EINVAL;
-            const int64_t yp = I[7] ? I[7] : C;
+            const i128 yp = I[7] ? I[7] : C;
             if (yp < C) return TP_EINVAL;
-            const int64_t Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
+            const i128 Ho = (H + 2 * pad - k) / st + 1, Wo = (W + 2 * pad - k) / st + 1;
             if ((r = R(0, false, N * H * W * C)) || (r = R(1, false, (N * Ho * Wo - 1) * yp + C))) return r;
             if (!launch) return 0;
             return tpk::launch_avgpool2d(F(0), Fm(1), (int)N, (int)H, (int)W, (int)C, (int)k, (int)st, (int)pad, yp,
@@ -1824,7 +1930,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         }
         case TP_OP_COPY2D: {
             if (!need(2, 4, 0)) return TP_EINVAL;
-            const int64_t rows = I[0], width = I[1], sp = I[2], dp = I[3];
+            const i128 rows = I[0], width = I[1], sp = I[2], dp = I[3];
             if (rows < 1 || width < 1 || sp < width || dp < width) return TP_EINVAL;
             if ((r = R(0, false, (rows - 1) * sp + width)) || (r = R(1, false, (rows - 1) * dp + width))) return r;
             if (!launch) return 0;
@@ -1832,7 +1938,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         }
         case TP_OP_SCALE_CHANNELS: {
             if (!need(3, 3, 0)) return TP_EINVAL;
-            const int64_t N = I[0], HW = I[1], C = I[2];
+            const i128 N = I[0], HW = I[1], C = I[2];
             if (N < 1 || HW < 1 || C < 1 || N > 0x7fffffff || C > 0x7fffffff) return TP_EINVAL;
             if ((r = R(0, false, N * HW * C)) || (r = R(1, false, N * C)) || (r = R(2, false, N * HW * C))) return r;
             if (!launch) return 0;
@@ -1840,7 +1946,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         }
         case TP_OP_ATTENTION: {
             if (!need(5, 8, 1)) return TP_EINVAL;
-            const int64_t B = I[0], A = I[1], S = I[2], dh = I[3];
+            const i128 B = I[0], A = I[1], S = I[2], dh = I[3];
             if (B < 1 || A < 1 || S < 1 || dh < 1 || B * S > 0x7fffffff || A * dh > 0x7fffffff) return TP_EINVAL;
             for (int k = 4; k < 8; ++k)
                 if (I[k] < A * dh) return TP_EINVAL;

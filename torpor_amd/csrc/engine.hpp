@@ -193,8 +193,11 @@ public:
     ~Engine();
     int init();
 
-    int signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred);
-    int take_deferred_ack(int* ack, int* resp);
+    int signal(int type, const char* function, const char* payload, int* ack, int* resp, int* deferred,
+               uint64_t* ticket = nullptr);
+    int take_deferred_ack(int* ack, int* resp, uint64_t* ticket = nullptr);
+    int cancel_deferred(uint64_t ticket);
+    int check_address(int client, uint64_t va, uint64_t bytes);
     int poll();
 
     int op_malloc(int client, uint64_t bytes, uint64_t* va);
@@ -234,6 +237,12 @@ private:
         int id;
         bool cold;
         int level;
+        uint64_t ticket;
+    };
+    struct DeferredAck {
+        int ack, resp;
+        uint64_t ticket;
+        int id;  // the function whose request this ack started
     };
     struct Xlat {
         uint8_t* p = nullptr;
@@ -266,6 +275,7 @@ private:
     void evict_model(Model& m);
     bool check_eviction(Model& m);
     void complete_request();
+    void start_next_queued();
     int finish_loading(Model& m);
     int finish_tracking(Model& m);
     int build_image(Model& m, bool by_access);
@@ -328,7 +338,8 @@ private:
     int exec_status_ = ES_AVAIL;
     std::chrono::steady_clock::time_point req_start_;
     std::deque<Queued> req_queue_;
-    std::deque<std::pair<int, int>> deferred_acks_;
+    std::deque<DeferredAck> deferred_acks_;
+    uint64_t ticket_seq_ = 0;  // queued signals are numbered from 1 in the order they were queued
     bool d2h_seen_ = false;
     // Data-plane calls are numbered; synced_seq_ is the number reached when the host last waited for
     // the compute stream.  A model whose touch_seq is above it may still have work on the device.

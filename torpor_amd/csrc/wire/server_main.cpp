@@ -59,7 +59,13 @@ struct Server {
     std::vector<std::unique_ptr<zmtp::Conn>> rep_conns, pull_conns;
     std::map<int, std::unique_ptr<zmtp::Conn>> pushers;  // client id -> PUSH connection
     std::map<int, std::vector<StagedD2H>> staged;        // client id -> D2H copies awaiting the next sync
-    std::vector<zmtp::Conn*> waiting_ack;                // REP peers whose request was queued
+    // REP peers whose signal was queued, by the engine's ticket for it.  Acks are matched to peers by
+    // ticket and peers are named by a tag that is never reused (a freed Conn's address can be).
+    struct Waiting {
+        uint64_t ticket, conn_tag;
+    };
+    std::vector<Waiting> waiting_ack;
+    uint64_t next_tag = 1;
     bool verbose = false;
     // Replay results are received in pinned memory of the engine (tp_host_alloc): the device writes
     // them there itself, and the reply message is built from it.  Grown on demand, freed with the engine.
@@ -158,8 +164,10 @@ bool handle_query(Server& S, int type, const pb::View& q, int client, std::strin
             } else if (kind == KIND_D2D) {
                 err = tp_memcpy_d2d(S.eng, client, dst, src, count);
             } else if (kind == KIND_D2H) {
+                // the engine vouches for source and count before this process sets `count` bytes aside
                 if (count > (1ull << 32)) {
                     err = TP_EINVAL;
+                } else if ((err = tp_check_address(S.eng, client, src, count)) != 0) {
                 } else if (type == Q_MEMCPY) {
                     back.resize(count);
                     err = tp_memcpy_d2h(S.eng, client, back.data(), src, count);
@@ -455,7 +463,7 @@ void handle_query_list(Server& S, const std::string& body) {
     }
 }
 
-std::string handle_signal(Server& S, const std::string& body, bool* deferred) {
+std::string handle_signal(Server& S, const std::string& body, bool* deferred, uint64_t* ticket) {
     pb::Reader r(body.data(), body.size());
     int f, wt, type = 0;
     uint64_t u;
@@ -469,7 +477,7 @@ std::string handle_signal(Server& S, const std::string& body, bool* deferred) {
         }
     }
     int32_t ack = TP_ACK_INAVAIL, resp = -1, dfr = 0;
-    const int rc = tp_signal(S.eng, type, function.c_str(), payload.c_str(), &ack, &resp, &dfr);
+    const int rc = tp_signal_ticket(S.eng, type, function.c_str(), payload.c_str(), &ack, &resp, &dfr, ticket);
     if (rc != 0) {
         ack = TP_ACK_INAVAIL;
         resp = -1;
@@ -482,11 +490,12 @@ std::string handle_signal(Server& S, const std::string& body, bool* deferred) {
     return w.out;
 }
 
-void accept_all(int lfd, zmtp::SockType t, std::vector<std::unique_ptr<zmtp::Conn>>& into) {
+void accept_all(Server& S, int lfd, zmtp::SockType t, std::vector<std::unique_ptr<zmtp::Conn>>& into) {
     for (;;) {
         const int fd = ::accept(lfd, nullptr, nullptr);
         if (fd < 0) break;
         into.push_back(std::make_unique<zmtp::Conn>(fd, t));
+        into.back()->tag = S.next_tag++;
     }
 }
 
@@ -540,8 +549,8 @@ int main() {
         for (auto& c : S.rep_conns) pfds.push_back({c->fd(), POLLIN, 0});
         for (auto& c : S.pull_conns) pfds.push_back({c->fd(), POLLIN, 0});
         ::poll(pfds.data(), pfds.size(), S.waiting_ack.empty() ? 50 : 1);
-        if (pfds[0].revents & POLLIN) accept_all(S.sig_listen, zmtp::REP, S.rep_conns);
-        if (pfds[1].revents & POLLIN) accept_all(S.srv_listen, zmtp::PULL, S.pull_conns);
+        if (pfds[0].revents & POLLIN) accept_all(S, S.sig_listen, zmtp::REP, S.rep_conns);
+        if (pfds[1].revents & POLLIN) accept_all(S, S.srv_listen, zmtp::PULL, S.pull_conns);
 
         for (auto& c : S.pull_conns) {
             c->pump();
@@ -558,9 +567,10 @@ int main() {
                 c->inbox().pop_front();
                 if (m.empty()) continue;
                 bool deferred = false;
-                const std::string ack = handle_signal(S, m.back(), &deferred);
+                uint64_t ticket = 0;
+                const std::string ack = handle_signal(S, m.back(), &deferred, &ticket);
                 if (deferred) {
-                    S.waiting_ack.push_back(c.get());  // answered when the active request completes
+                    S.waiting_ack.push_back({ticket, c->tag});  // answered when the active request completes
                 } else {
                     zmtp::Message reply(m.begin(), m.end() - 1);  // envelope (empty delimiter) first
                     reply.push_back(ack);
@@ -570,25 +580,35 @@ int main() {
         }
         (void)tp_poll(S.eng);  // request timeout (cuda_server.hpp:257-264)
         int32_t ack = 0, resp = 0;
-        while (!S.waiting_ack.empty() && tp_take_deferred_ack(S.eng, &ack, &resp) == 1) {
+        uint64_t ticket = 0;
+        while (tp_take_deferred_ack_ticket(S.eng, &ack, &resp, &ticket) == 1) {
             pb::Writer w;
             w.i32(1, ack);
             w.i32(2, resp);
-            zmtp::Conn* c = S.waiting_ack.front();
-            S.waiting_ack.erase(S.waiting_ack.begin());
-            bool alive = false;
-            for (auto& rc2 : S.rep_conns) alive = alive || rc2.get() == c;
-            if (alive) c->send({std::string(), w.out});
+            uint64_t tag = 0;
+            for (size_t k = 0; k < S.waiting_ack.size(); ++k)
+                if (S.waiting_ack[k].ticket == ticket) {
+                    tag = S.waiting_ack[k].conn_tag;
+                    S.waiting_ack.erase(S.waiting_ack.begin() + (long)k);
+                    break;
+                }
+            for (auto& rc2 : S.rep_conns)
+                if (tag && rc2->tag == tag) rc2->send({std::string(), w.out});
         }
         auto prune = [&](std::vector<std::unique_ptr<zmtp::Conn>>& v) {
             for (size_t i = 0; i < v.size();) {
                 if (v[i]->failed() && v[i]->inbox().empty()) {
+                    // A peer that waited for a deferred ack is gone: its queued signal is withdrawn, so
+                    // that the engine neither starts a request nobody will drive nor produces an ack
+                    // that another peer could be handed.
                     for (size_t k = 0; k < S.waiting_ack.size();)
-                        if (S.waiting_ack[k] == v[i].get())
-                            S.waiting_ack.erase(S.waiting_ack.begin() + k);
-                        else
+                        if (S.waiting_ack[k].conn_tag == v[i]->tag) {
+                            (void)tp_cancel_deferred(S.eng, S.waiting_ack[k].ticket);
+                            S.waiting_ack.erase(S.waiting_ack.begin() + (long)k);
+                        } else {
                             ++k;
-                    v.erase(v.begin() + i);
+                        }
+                    v.erase(v.begin() + (long)i);
                 } else {
                     ++i;
                 }

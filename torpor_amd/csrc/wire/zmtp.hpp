@@ -18,7 +18,9 @@
 #include <sys/un.h>
 #include <unistd.h>
 
+#include <chrono>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 #include <memory>
@@ -88,6 +90,8 @@ inline std::string ready_command(SockType t) {
     return out;
 }
 
+constexpr uint64_t kMaxFrame = 1ull << 31;
+
 // One peer connection: incremental parser + blocking writer.
 class Conn {
 public:
@@ -103,6 +107,7 @@ public:
     Conn& operator=(const Conn&) = delete;
 
     int fd() const { return fd_; }
+    uint64_t tag = 0;  // set by the owner: a name for this connection that is never reused
     bool failed() const { return failed_; }
     bool ready() const { return stage_ == 2; }
     const std::string& peer_type() const { return peer_type_; }
@@ -136,8 +141,21 @@ public:
     }
 
 private:
+    // The writer blocks, but not for ever: a peer that does not drain its socket for send_budget_ms()
+    // in all while one message is written is dropped, so that one stalled reader cannot hold up a
+    // single-threaded server and every other peer with it.
+    static int send_budget_ms() {
+        static const int ms = [] {
+            const char* e = std::getenv("TORPOR_SEND_TIMEOUT_MS");
+            const long v = (e && *e) ? std::strtol(e, nullptr, 10) : 0;
+            return (int)(v > 0 && v < 3600000 ? v : 3000);
+        }();
+        return ms;
+    }
     bool send_raw(const std::string& data) {
         size_t off = 0;
+        if (failed_) return false;
+        const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(send_budget_ms());
         while (off < data.size()) {
             const ssize_t n = ::send(fd_, data.data() + off, data.size() - off, MSG_NOSIGNAL);
             if (n > 0) {
@@ -145,8 +163,14 @@ private:
                 continue;
             }
             if (n < 0 && (errno == EAGAIN || errno == EWOULDBLOCK)) {
+                const auto left = std::chrono::duration_cast<std::chrono::milliseconds>(
+                                      deadline - std::chrono::steady_clock::now()).count();
+                if (left <= 0) {
+                    failed_ = true;
+                    return false;
+                }
                 struct pollfd p = {fd_, POLLOUT, 0};
-                ::poll(&p, 1, 1000);
+                ::poll(&p, 1, (int)(left < 1000 ? left : 1000));
                 continue;
             }
             if (n < 0 && errno == EINTR) continue;
@@ -180,7 +204,9 @@ private:
             } else {
                 len = (uint8_t)rbuf_[pos + 1];
             }
-            if (len > (1ull << 34)) {
+            // No legitimate message is larger than a protobuf message can be (2 GiB); the largest the
+            // clients send is one weight tensor per upload.
+            if (len > kMaxFrame) {
                 failed_ = true;
                 break;
             }

@@ -99,6 +99,29 @@ class Server:
             raise TorporError(r, "tp_take_deferred_ack")
         return (ack.value, resp.value) if r == 1 else None
 
+    def signal_ticket(self, req_type, function, payload=""):
+        """Returns (ack, resp, deferred, ticket); ticket is 0 unless the signal was queued."""
+        ack, resp, dfr, tk = C.c_int32(), C.c_int32(), C.c_int32(), C.c_uint64()
+        _chk(self._l.tp_signal_ticket(self._h, req_type, str(function).encode(), str(payload).encode(),
+                                      C.byref(ack), C.byref(resp), C.byref(dfr), C.byref(tk)), "tp_signal_ticket")
+        return ack.value, resp.value, bool(dfr.value), tk.value
+
+    def take_deferred_ack_ticket(self):
+        ack, resp, tk = C.c_int32(), C.c_int32(), C.c_uint64()
+        r = self._l.tp_take_deferred_ack_ticket(self._h, C.byref(ack), C.byref(resp), C.byref(tk))
+        if r < 0:
+            raise TorporError(r, "tp_take_deferred_ack_ticket")
+        return (ack.value, resp.value, tk.value) if r == 1 else None
+
+    def cancel_deferred(self, ticket):
+        r = self._l.tp_cancel_deferred(self._h, int(ticket))
+        if r < 0:
+            raise TorporError(r, "tp_cancel_deferred")
+        return r
+
+    def check_address(self, fid, va, nbytes):
+        return self._l.tp_check_address(self._h, fid, int(va), int(nbytes))
+
     def poll(self):
         r = self._l.tp_poll(self._h)
         if r < 0:
