@@ -15,6 +15,10 @@ dominant kernel over timed warm requests, "swap" holds the swap-in GB/s (bytes t
 link; compressible tensors travel in a lossless 27-bit format) against the measured pinned-host ->
 HBM link peak, and "cpu_baseline" is the PyTorch CPU forward of the same
 seeded model timed on this box's host cores (oracle/models.py, a reported baseline only).
+"link_roofline" prices the cold start against the host link: the bytes the request has to wait for
+divided by the measured (and the nominal) link rate.  workloads["multitenant-64"] is a short leg of the
+64-model configuration (BASELINE.json configs[4]) under its own 24 GiB cap and under a cap that binds.
+`--ablate` adds the reference's pipeline ablation (evaluation/figure7/Figure7_README.md:12-33).
 """
 import argparse
 import gc
@@ -134,6 +138,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         gathers = st["host_gathers"]
         swap_gbps.append(st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))   # bytes that crossed the link
         link_bytes = st["bytes"]
+        deferred_bytes = st["deferred_bytes"]
     server.stream_synchronize(fid)
     t_total = time.perf_counter() - t_begin
     out = fn.postprocess([v.copy() for v in views])
@@ -164,6 +169,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
         link_bytes=link_bytes,   # below weight_bytes when tensors travel in the packed format
+        deferred_link_bytes=deferred_bytes,   # of those: index-looked-up tables, which travel last; the request does not wait for them
         weights_gbps_p50=info["image_bytes"] / 1e9 / (pctl(swap_ms, 0.5) * 1e-3),   # weight bytes in place per second
         copy_streams=streams, host_gathers=gathers, steps_total_s=t_total,
     )
@@ -171,37 +177,81 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
 
 
 def measured_traffic(workload, kernel):
-    """HBM bytes per launch of `kernel` in `workload`, from the committed rocprofv3 --pmc summary
-    (FETCH_SIZE and WRITE_SIZE runs of this same script, scaled by the copy-kernel calibration
-    stated in that file); None when no summary covers this workload / kernel."""
-    path = os.path.join(ROOT, "profiles", workload.replace("-", "_") + "_pmc_traffic.md")
+    """(HBM bytes per launch of `kernel` in `workload`, file) from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE runs of this same script, scaled by the copy-kernel calibration stated in
+    that file); (None, None) when no summary covers this workload / kernel.  It is a figure read from that
+    file, not a counter of this run: counters need the profiler."""
+    rel = os.path.join("profiles", workload.replace("-", "_") + "_pmc_traffic.md")
     try:
-        text = open(path).read()
+        text = open(os.path.join(ROOT, rel)).read()
     except OSError:
-        return None
+        return None, None
     m = re.search(r"^traffic_bytes_per_launch\[" + re.escape(kernel) + r"\]:\s*(\d+)", text, re.M)
-    return int(m.group(1)) if m else None
+    return (int(m.group(1)), rel) if m else (None, None)
+
+
+def by_symbol(kstats):
+    """{kernel symbol: summed stats + {shape: stats}} from the per-shape records of the engine
+    (names are `symbol[shape]` for GEMM and convolution launches)."""
+    out = {}
+    for name, st in kstats.items():
+        sym, _, shape = name.partition("[")
+        e = out.setdefault(sym, dict(launches=0, total_us=0.0, flops=0.0, bytes=0.0, shapes={}))
+        for k in ("launches", "total_us", "flops", "bytes"):
+            e[k] += st[k]
+        if shape:
+            e["shapes"][shape.rstrip("]")] = st
+    return out
 
 
 def roofline_from(kstats, empty_us, workload):
-    """Dominant kernel = largest summed duration; achieved = algorithmic work / time."""
+    """Dominant kernel = the symbol with the largest summed duration; achieved = algorithmic work / time,
+    per launch durations from HIP events around every launch on the compute stream, minus the duration of
+    an empty event bracket."""
     if not kstats:
         return None
-    name, st = max(kstats.items(), key=lambda kv: kv[1]["total_us"])
-    traffic = measured_traffic(workload, name)
+    syms = by_symbol(kstats)
+    name, st = max(syms.items(), key=lambda kv: kv[1]["total_us"])
+    traffic, traffic_file = measured_traffic(workload, name)
     n = st["launches"]
     t_us = max(st["total_us"] - n * empty_us, 1e-3)
     avg_us = t_us / n
-    if st["flops"] > 0:
-        ach = st["flops"] / (t_us * 1e-6) / 1e12
-        return dict(kernel=name, bound="mfma", achieved=ach, peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s",
-                    frac=ach / PEAK_FP32_MFMA_TFLOPS, traffic=traffic, launches=n, avg_launch_us=avg_us,
-                    event_overhead_us=empty_us, flop_per_launch=st["flops"] / n, bytes_per_launch=st["bytes"] / n,
-                    hbm_gbps=st["bytes"] / (t_us * 1e-6) / 1e9)
-    ach = st["bytes"] / (t_us * 1e-6) / 1e9
-    return dict(kernel=name, bound="hbm", achieved=ach, peak=PEAK_HBM_GBPS, unit="GB/s", frac=ach / PEAK_HBM_GBPS,
-                traffic=traffic, launches=n, avg_launch_us=avg_us, event_overhead_us=empty_us,
-                bytes_per_launch=st["bytes"] / n)
+    mfma = st["flops"] > 0
+    ach = st["flops"] / (t_us * 1e-6) / 1e12 if mfma else st["bytes"] / (t_us * 1e-6) / 1e9
+    peak = PEAK_FP32_MFMA_TFLOPS if mfma else PEAK_HBM_GBPS
+    shapes = {}
+    for shape, ss in sorted(st["shapes"].items(), key=lambda kv: -kv[1]["total_us"]):
+        tt = max(ss["total_us"] - ss["launches"] * empty_us, 1e-3)
+        a = ss["flops"] / (tt * 1e-6) / 1e12 if mfma else ss["bytes"] / (tt * 1e-6) / 1e9
+        shapes[shape] = dict(launches=ss["launches"], avg_launch_us=tt / ss["launches"], achieved=a, frac=a / peak)
+    r = dict(kernel=name, bound="mfma" if mfma else "hbm", achieved=ach, peak=peak, unit="TFLOP/s" if mfma else "GB/s",
+             frac=ach / peak, traffic=traffic,
+             traffic_source=(traffic_file + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command; read "
+                             "from that file, not counted in this run)") if traffic_file else None,
+             launches=n, avg_launch_us=avg_us, event_overhead_us=empty_us, bytes_per_launch=st["bytes"] / n,
+             by_shape=shapes)
+    if mfma:
+        r.update(flop_per_launch=st["flops"] / n, hbm_gbps=st["bytes"] / (t_us * 1e-6) / 1e9)
+    return r
+
+
+def link_roofline(res, link_gbps):
+    """The cold start against the host link.  A request cannot answer before the bytes it needs have
+    crossed the link: floor = (link bytes - tables that travel last) / link rate."""
+    waited = res["link_bytes"] - res["deferred_link_bytes"]
+    floor_meas = waited / (link_gbps * 1e9) * 1e3
+    floor_nom = waited / (PCIE_GEN5_X16_GBPS * 1e9) * 1e3
+    return dict(bound="host link", bytes_waited_for=waited, link_bytes=res["link_bytes"], weight_bytes=res["weight_bytes"],
+                cold_ms_p50=res["cold_ms_p50"], floor_ms_at_measured_link=floor_meas,
+                frac_of_measured_link_floor=floor_meas / res["cold_ms_p50"],
+                floor_ms_at_nominal_64=floor_nom, frac_of_nominal_floor=floor_nom / res["cold_ms_p50"],
+                full_image_floor_ms_at_measured_link=res["weight_bytes"] / (link_gbps * 1e9) * 1e3,
+                # cold <= 1.3 x warm would need at most this many bytes over the measured link:
+                bytes_for_1p3x_warm=1.3 * res["warm_ms_p50"] * 1e-3 * link_gbps * 1e9,
+                # ... which is this many bits per 32-bit weight word the request waits for (the transfer
+                # format sends 32 * link_bytes / weight_bytes of them today)
+                bits_per_weight_word_for_1p3x_warm=32.0 * res["link_bytes"] / res["weight_bytes"] *
+                                                   (1.3 * res["warm_ms_p50"] * 1e-3 * link_gbps * 1e9) / max(waited, 1))
 
 
 def cpu_baseline(name, weights, inputs, first):
@@ -245,6 +295,49 @@ def cpu_baseline(name, weights, inputs, first):
                 min_ms=min(times), logits_rel_err_vs_gpu=err)
 
 
+def ablation(names, steps, warmup):
+    """Cold p50 (ms) per workload under the reference's pipeline ablation (evaluation/figure7/Figure7_README.md:
+    12-33: BUFFER_SIZE = 2 MiB default, 1 = a group per tensor, 1.6 GB = no pipelining) and with this build's two
+    own transfer features switched off.  Every variant is a fresh engine, since these are engine settings."""
+    from torpor_amd.server import Server
+
+    variants = {
+        "default": {},
+        "group_per_tensor (BUFFER_SIZE=1)": dict(chunk_bytes=1, chunk_max_bytes=1),
+        "one_group (no pipelining)": dict(chunk_bytes=2 << 30, chunk_max_bytes=2 << 30),
+        "fixed_2MiB_groups (the reference's default)": dict(chunk_bytes=2 << 20, chunk_max_bytes=2 << 20),
+        "weights_sent_as_they_are (TORPOR_PACK=0)": dict(pack=False),
+        "lookups_wait_for_their_table (TORPOR_HOST_GATHER=0)": dict(host_gather=False),
+    }
+    out = {}
+    for vname, kw in variants.items():
+        row = {}
+        for fid, name in enumerate(names):
+            with Server(mem_limit_bytes=8 << 30, pool_bytes=9 << 30, **kw) as server:
+                fn, inputs, _ = make_function(server, fid, name)
+                first = fn.register(inputs)
+                packed, outbuf, views = fn.pack(inputs, pinned=True)
+                cold = []
+                for i in range(warmup + steps):
+                    fn.unload()
+                    t0 = time.perf_counter()
+                    ack, _, dfr = server.signal(1, fid, "")
+                    assert ack == 0 and not dfr
+                    server.replay(fid, packed, outbuf)
+                    if i >= warmup:
+                        cold.append((time.perf_counter() - t0) * 1e3)
+                    st = server.swap_stats(fid)
+                out_now = fn.postprocess([v.copy() for v in views])
+                for a, b in zip(first, out_now):
+                    if not np.array_equal(a, b):
+                        raise SystemExit(f"ablation {vname} / {name}: output differs from the registration run")
+                row[name] = dict(cold_ms_p50=pctl(cold, 0.5), groups=st["chunks"], link_bytes=st["bytes"],
+                                 swap_gbps=st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
+                del fn
+        out[vname] = row
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -254,6 +347,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--chunk-max-bytes", type=int, default=0)
+    ap.add_argument("--no-multitenant", action="store_true", help="skip the 64-model leg")
+    ap.add_argument("--multitenant-seconds", type=float, default=10.0)
+    ap.add_argument("--multitenant-caps-gb", type=float, nargs="+", default=[24.0, 8.0])
+    ap.add_argument("--ablate", action="store_true",
+                    help="also measure cold p50 per config with per-tensor groups, one whole-image group, weights "
+                         "sent as they are, and lookups that wait for their table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build serves from one GPU (one executor, one pool, one LRU per GPU); "
@@ -279,6 +378,7 @@ def main():
                                   tflops=(v["flops"] / max(v["total_us"] - v["launches"] * empty_us, 1e-3) / 1e6),
                                   gbps=(v["bytes"] / max(v["total_us"] - v["launches"] * empty_us, 1e-3) / 1e3))
                           for k, v in sorted(kstats.items(), key=lambda kv: -kv[1]["total_us"])}
+        res["link_roofline"] = link_roofline(res, link)
         if name == primary:
             keep = ctx
         else:
@@ -314,6 +414,17 @@ def main():
         "rooflines": roof,
     }
     server.close()
+    if args.workload == "all" and not args.no_multitenant:
+        from torpor_amd import multitenant as mt
+        runs = {}
+        for cap in args.multitenant_caps_gb:
+            runs[f"cap_{cap:g}GiB"] = mt.run_cap(cap, args.multitenant_seconds, 200.0)
+        line["workloads"]["multitenant-64"] = dict(
+            config="32x ResNet-50 + 16x BERT-base s128 + 16x ResNet-152, seeds 0..63, batch 1, open-loop Poisson "
+                   f"200 req/s, Zipf(1.1) popularity, {args.multitenant_seconds:g} s per cap; latency = completion - arrival",
+            runs=runs)
+    if args.ablate:
+        line["ablation"] = ablation(names, max(args.steps // 2, 5), max(args.warmup, 8))
     print(json.dumps(line))
 
 

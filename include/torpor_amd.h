@@ -107,7 +107,8 @@ typedef struct tp_config {
     int32_t device;             /* HIP device ordinal */
     uint64_t mem_limit_bytes;   /* LRU budget; 0: env MEM_LIMIT_IN_GB or 24 GiB (controller.hpp:83-93) */
     uint64_t pool_bytes;        /* HBM arena; 0: mem_limit + pool headroom (memory_manager.hpp:42-44) */
-    uint64_t chunk_bytes;       /* first swap-in gate group; 0: env BUFFER_SIZE or 2 MiB (memory_manager.hpp:22,169-173) */
+    uint64_t chunk_bytes;       /* first swap-in gate group; 0: env BUFFER_SIZE or 2 MiB (memory_manager.hpp:22,169-173);
+                                   below 256 (the reference's BUFFER_SIZE=1 ablation): one group per tensor */
     uint64_t chunk_max_bytes;   /* groups double up to this size; 0: 8 MiB; set = chunk_bytes for fixed groups */
     uint64_t workspace_bytes;   /* split-K scratch; 0: 64 MiB */
     int32_t flags;              /* TP_FLAG_* */
@@ -158,6 +159,14 @@ typedef struct tp_pool_stats {
     uint64_t live_extents, free_extents;
     uint64_t lru_budget, lru_used, lru_models;
     uint64_t evictions, swap_ins;
+    /* victims taken because no contiguous extent fitted although the budget test had passed (the reference
+     * exits there, block_manager.hpp:345-351); they are included in `evictions` */
+    uint64_t fragmentation_evictions;
+    /* pinned host memory held outside the pool: weight images, their transfer images (the second, smaller
+     * copy that crosses the link), request staging and result buffers */
+    uint64_t host_image_bytes, host_transfer_bytes, host_staging_bytes;
+    /* device memory outside the pool and its budget: staging area of packed transfers, kernel workspace */
+    uint64_t device_staging_bytes, device_workspace_bytes;
 } tp_pool_stats;
 
 typedef struct tp_model_info {
@@ -185,6 +194,8 @@ typedef struct tp_swap_stats {
     uint32_t gate_waits; /* compute-stream waits issued during the last request */
     uint32_t copy_streams; /* streams the last swap-in alternated over */
     uint32_t host_gathers; /* lookups of the last request that read their table in place from the host store */
+    uint64_t deferred_bytes; /* of `bytes`: transfer groups that hold nothing but tables looked up by index; they
+                                travel last and a request does not wait for them */
 } tp_swap_stats;
 
 /* ------------------------------------------------------------------ lifecycle
@@ -332,7 +343,8 @@ int tp_time_op(tp_server* s, int32_t client, int32_t op_index, int32_t iters, do
  * overhead), measured at end, to be subtracted per launch.  No counterpart in the reference,
  * which logs host-side timestamps only (memory_manager.hpp:425-431, cuda_server.hpp:294-295). */
 typedef struct tp_kernel_stat {
-    char name[64];
+    char name[64];   /* kernel variant; GEMM and convolution launches carry their shape: name[MxNxK] or
+                        name[NxHxWxCin>Cout kKHxKW sS] */
     uint64_t launches;
     double total_us; /* sum of bracketed durations */
     double flops;    /* algorithmic floating-point operations of those launches */

@@ -262,3 +262,28 @@ def test_executor_log_reports_every_swap_in(tmp_path, monkeypatch):
         assert int(m.group(1)) == st["bytes"] and int(m.group(2)) == st["chunks"] and int(m.group(3)) == st["copy_streams"]
         assert abs(int(m.group(4)) - st["copy_ms"] * 1e3) <= 2
     assert sum("Request of model 0 completed" in ln and "(swapped in)" in ln for ln in lines) == 3
+
+
+def test_device_image_equals_host_image_wherever_it_lands():
+    """Functions of different architectures take turns on the same pool memory: after every swap-in the
+    device image equals the host image byte for byte, the alignment gaps between tensors included (they hold
+    zeros in the host copy, and whatever the previous tenant left in the pool memory a swap-in lands in)."""
+    from torpor_amd.functions import mobilenet
+    with Server(mem_limit_bytes=260 << 20, pool_bytes=400 << 20) as s:
+        rng = np.random.default_rng(3)
+        a, xa, ya = _mk(s, 0, seed=1)
+        cfg = dict(bert.CONFIGS["bert-base"], layers=2)
+        b = bert.Bert(s, 1, "bert-base", batch=1, seq=32, seed=2, cfg=cfg, vocab=60000)   # 230 MB: the pair cannot both stay
+        ids = rng.integers(0, 60000, (1, 32))
+        yb = b.register([ids])
+        c = mobilenet.MobileNetV2(s, 2, batch=1, weights=mobilenet.init_weights(seed=3))
+        xc = rng.standard_normal((1, 3, 224, 224)).astype(np.float32)
+        (yc,) = c.register([xc])
+        # 0xFF everywhere the models do not write: activations of a poisoning function
+        for turn in range(3):
+            for fn, x, want in ((a, [xa], [ya]), (b, [ids], yb), (c, [xc], [yc])):
+                got = fn.invoke(x)
+                for g, w in zip(got, want):
+                    assert np.array_equal(g, w)
+                assert np.array_equal(s.readback_weights(fn.fid), s.host_weights(fn.fid)), (turn, fn.fid)
+        assert s.pool_stats()["evictions"] >= 4

@@ -92,6 +92,68 @@ def test_pool_random_invariants():
     assert q["used"] == 0 and q["largest_free"] == cap and q["free_extents"] == 1
 
 
+def test_pool_at_288_gb_with_ten_thousand_live_extents():
+    """The arena of a whole MI355X (288 GB) full of small models: invariants hold, best fit agrees with a
+    brute-force scan of the holes, and an allocation stays a tree search (the bound below is generous for a
+    call through ctypes: a linear scan of ~10^4 holes would not meet it in the steady state)."""
+    import time
+    rng = random.Random(7)
+    cap = 288 * 10 ** 9
+    p = Pool(cap)
+    cap = p.query()["capacity"]
+    live = {}
+    while True:                                  # fill it: 2 .. 20 MiB extents
+        n = rng.randint(1, 10) * SLAB
+        off = p.alloc(n)
+        if off == NOFIT:
+            break
+        live[off] = n
+    assert len(live) > 20000
+    for off in rng.sample(sorted(live), len(live) // 2):   # punch ~12 000 holes
+        assert p.release(off) == 0
+        del live[off]
+    q = p.query()
+    assert q["live"] == len(live) >= 10000 and q["used"] == sum(live.values())
+    assert q["free_extents"] > 5000
+
+    def holes():
+        out, pos = [], 0
+        for off in sorted(live):
+            if off > pos:
+                out.append((pos, off - pos))
+            pos = off + live[off]
+        if pos < cap:
+            out.append((pos, cap - pos))
+        return out
+    for _ in range(40):                          # best fit == brute force: smallest hole that fits, lowest address
+        n = rng.randint(1, 30) * SLAB
+        fit = [(ln, o) for o, ln in holes() if ln >= n]
+        off = p.alloc(n)
+        if not fit:
+            assert off == NOFIT
+            continue
+        assert off == min(fit)[1]
+        live[off] = n
+    assert p.query()["largest_free"] == max(ln for _, ln in holes())
+    ops = 20000
+    offs = sorted(live)
+    t0 = time.perf_counter()
+    for i in range(ops):                         # steady state: release one, allocate one
+        off = offs[(i * 7919) % len(offs)]
+        if off in live:
+            assert p.release(off) == 0
+            n = live.pop(off)
+            o2 = p.alloc(n)
+            assert o2 != NOFIT
+            live[o2] = n
+    per_op_us = (time.perf_counter() - t0) / ops * 1e6
+    assert per_op_us < 50.0, per_op_us
+    srt = sorted(live.items())
+    assert all(a[0] + a[1] <= b[0] for a, b in zip(srt, srt[1:])) and srt[-1][0] + srt[-1][1] <= cap
+    assert p.query()["used"] == sum(live.values())
+    assert p.alloc(cap + SLAB) == NOFIT and p.alloc((1 << 64) - 1) == NOFIT
+
+
 def test_pool_layout_is_deterministic():
     seq = [(1, 5 * SLAB), (1, SLAB), (0, 0), (1, 2 * SLAB), (1, 7 * SLAB), (0, 1), (1, 3 * SLAB)]
     outs = []

@@ -77,7 +77,9 @@ class ConvDesc(C.Structure):
 class PoolStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "capacity", "used", "largest_free", "live_extents", "free_extents",
-        "lru_budget", "lru_used", "lru_models", "evictions", "swap_ins")]
+        "lru_budget", "lru_used", "lru_models", "evictions", "swap_ins", "fragmentation_evictions",
+        "host_image_bytes", "host_transfer_bytes", "host_staging_bytes", "device_staging_bytes",
+        "device_workspace_bytes")]
 
 
 class ModelInfo(C.Structure):
@@ -89,7 +91,7 @@ class ModelInfo(C.Structure):
 class SwapStats(C.Structure):
     _fields_ = [("bytes", C.c_uint64), ("copy_ms", C.c_double), ("alloc_us", C.c_double),
                 ("evict_us", C.c_double), ("chunks", C.c_uint32), ("gate_waits", C.c_uint32),
-                ("copy_streams", C.c_uint32), ("host_gathers", C.c_uint32)]
+                ("copy_streams", C.c_uint32), ("host_gathers", C.c_uint32), ("deferred_bytes", C.c_uint64)]
 
 
 class KernelStat(C.Structure):

@@ -121,7 +121,8 @@ int Engine::init() {
     // here any positive value up to the device size is accepted.
     if (cfg_.mem_limit_bytes == 0) cfg_.mem_limit_bytes = env_u64("MEM_LIMIT_IN_GB", 24) << 30;
     if (cfg_.chunk_bytes == 0) cfg_.chunk_bytes = env_u64("BUFFER_SIZE", 2ull << 20);  // memory_manager.hpp:22
-    if (cfg_.chunk_bytes < kTensorAlign) cfg_.chunk_bytes = kTensorAlign;              // BUFFER_SIZE=1 ablation
+    per_tensor_groups_ = cfg_.chunk_bytes < kTensorAlign;                              // BUFFER_SIZE=1 ablation
+    if (cfg_.chunk_bytes < kTensorAlign) cfg_.chunk_bytes = kTensorAlign;
     chunk_max_auto_ = cfg_.chunk_max_bytes == 0;
     if (cfg_.chunk_max_bytes == 0) cfg_.chunk_max_bytes = 8ull << 20;
     if (cfg_.chunk_max_bytes < cfg_.chunk_bytes) cfg_.chunk_max_bytes = cfg_.chunk_bytes;
@@ -638,6 +639,7 @@ int Engine::unpack_on_device(const uint8_t* payload, uint64_t n_words, int32_t b
     a.piece[0].bytes = 0;
     a.piece[0].w_from = w_from;
     a.piece[0].w_to = w_to;
+    a.piece[0].w_zero_to = 0;
     a.piece[0].ext = d_ext;
     a.piece[0].tab = reinterpret_cast<const uint32_t*>(d_tab);
     a.piece[0].base = base;
@@ -1014,13 +1016,22 @@ int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hi
             pc.bytes = 0;
             pc.w_from = (from - p.image_off) / 4;
             pc.w_to = (to - p.image_off) / 4;
+            // The image keeps every tensor 256 B aligned and the host copy holds zeros in the gaps; the
+            // pool memory a swap-in lands in holds whatever its previous tenant left.  The run that
+            // delivers a tensor's last word clears the gap behind it, so that the device image equals the
+            // host image byte for byte wherever it is placed.
+            pc.w_zero_to = (to == p.image_off + p.size) ? align_up(p.size, kTensorAlign) / 4 : 0;
+            if (pc.w_zero_to == pc.w_to) pc.w_zero_to = 0;
             pc.ext = xfer_stage_ + p.ext_off;
             pc.tab = reinterpret_cast<const uint32_t*>(xfer_stage_ + p.tab_off);
         } else {
             pc.src = xfer_stage_ + p.t_off + (from - p.image_off);
             pc.dst = m.w_dev + from;
-            pc.bytes = to - from;
+            // a run that ends the tensor takes the zeros behind it along (the transfer image holds zeros
+            // up to the next tensor's region, which starts no earlier than the aligned end)
+            pc.bytes = (to == p.image_off + p.size ? align_up(p.image_off + p.size, kTensorAlign) : to) - from;
             pc.w_from = pc.w_to = 0;
+            pc.w_zero_to = 0;
             pc.ext = nullptr;
             pc.tab = nullptr;
         }
@@ -1072,6 +1083,20 @@ void Engine::build_chunks(Model& m) {
     choose_copy_plan(m);
     m.chunk_end.clear();
     uint64_t sz = cfg_.chunk_bytes, pos = 0;
+    if (per_tensor_groups_) {
+        // memory_manager.hpp:399-409 with BUFFER_SIZE=1: a group closes behind every tensor
+        std::vector<uint64_t> ends;
+        ends.reserve(m.params.size());
+        for (const Param& p : m.params) ends.push_back(align_up(p.image_off + p.size, kTensorAlign));
+        std::sort(ends.begin(), ends.end());
+        for (uint64_t e : ends)
+            if (e > pos) {
+                m.chunk_end.push_back(e);
+                pos = e;
+            }
+        if (pos < m.image_bytes) m.chunk_end.push_back(m.image_bytes);
+        pos = m.image_bytes;
+    }
     while (pos < m.image_bytes) {
         uint64_t end = pos + align_up(sz, kTensorAlign);
         if (end > m.image_bytes) end = m.image_bytes;
@@ -1309,6 +1334,7 @@ int Engine::swap_in(Model& m) {
         lru_.force_evict(victim);
         Model* v = find(std::atoi(victim.c_str()));
         if (v) evict_model(*v);
+        ++frag_evictions_;
     }
     m.w_dev = arena_ + m.w_pool_off;
     m.a_dev = arena_ + m.a_pool_off;
@@ -1323,6 +1349,11 @@ int Engine::swap_in(Model& m) {
     m.transfer_logged = false;
     m.stats.alloc_us = us_since(t0);
     m.stats.bytes = m.timg ? m.timg_bytes : m.image_bytes;
+    m.stats.deferred_bytes = 0;
+    if (m.defer_from != UINT32_MAX && m.defer_from > 0 && m.defer_from < m.chunk_end.size()) {
+        const uint64_t from = m.chunk_end[m.defer_from - 1];
+        m.stats.deferred_bytes = m.timg ? m.timg_bytes - xfer_off(m, from) : m.image_bytes - from;
+    }
     m.stats.chunks = (uint32_t)m.chunk_end.size();
     m.stats.copy_streams = (uint32_t)m.ncopy;
     ++swap_ins_;
@@ -2049,9 +2080,28 @@ int Engine::exec_compute(Model& m, const Op& op, bool launch) {
     HIPCHK(hipEventRecord(a, compute_));
     const int r = exec_compute_impl(m, op, true);
     HIPCHK(hipEventRecord(b, compute_));
-    prof_records_.push_back({tpk::last_kernel_name(), a, b, flops, bytes});
+    // GEMM and convolution launches are accounted per shape: the same kernel runs at very different
+    // fractions of the matrix peak on different shapes
+    std::string label = tpk::last_kernel_name();
+    char shape[48] = "";
+    if (op.kind == OPK_GEMM) {
+        if (op.i[8] * op.i[9] > 1)
+            std::snprintf(shape, sizeof shape, "[%lldx%lldx%lld b%lld]", (long long)op.i[0], (long long)op.i[1],
+                          (long long)op.i[2], (long long)(op.i[8] * op.i[9]));
+        else
+            std::snprintf(shape, sizeof shape, "[%lldx%lldx%lld]", (long long)op.i[0], (long long)op.i[1], (long long)op.i[2]);
+    } else if (op.kind == OPK_CONV) {
+        std::snprintf(shape, sizeof shape, "[%lldx%lldx%lldx%lld>%lld k%lldx%lld s%lld]", (long long)op.i[0], (long long)op.i[1],
+                      (long long)op.i[2], (long long)op.i[3], (long long)op.i[4], (long long)op.i[5], (long long)op.i[6],
+                      (long long)op.i[7]);
+    }
+    label += shape;
+    prof_records_.push_back({prof_label(label), a, b, flops, bytes});
     return r;
 }
+
+// Labels live as long as the engine: records and statistics hold pointers to them.
+const char* Engine::prof_label(const std::string& s) { return prof_labels_.insert(s).first->c_str(); }
 
 int Engine::profile_begin() {
     std::lock_guard<std::mutex> lk(mu_);
@@ -2338,6 +2388,16 @@ int Engine::pool_stats(tp_pool_stats* out) {
     out->lru_models = lru_.size();
     out->evictions = evictions_;
     out->swap_ins = swap_ins_;
+    out->fragmentation_evictions = frag_evictions_;
+    out->host_image_bytes = out->host_transfer_bytes = 0;
+    for (auto& kv : models_) {
+        if (kv.second->host_image) out->host_image_bytes += kv.second->image_bytes;
+        if (kv.second->timg) out->host_transfer_bytes += kv.second->timg_bytes;
+    }
+    out->host_staging_bytes = h2d_cap_ + d2h_cap_;
+    for (auto& kv : user_pinned_) out->host_staging_bytes += kv.second;
+    out->device_staging_bytes = xfer_stage_cap_;
+    out->device_workspace_bytes = host_only() ? 0 : cfg_.workspace_bytes;
     return 0;
 }
 

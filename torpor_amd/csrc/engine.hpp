@@ -21,6 +21,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <set>
 #include <string>
 #include <thread>
 #include <unordered_map>
@@ -328,6 +329,7 @@ private:
     bool pack_ = true;
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
+    bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor
     int d2h_kernel_ = 0;
     bool host_gather_ = true;  // lookups may read a table in place from the host store during a swap-in
     int graph_min_ops_ = 0;  // 0: warm replays launch op by op; n: capture compute runs of at least n ops
@@ -352,7 +354,7 @@ private:
     uint64_t d2h_cap_ = 0, d2h_pos_ = 0;
     std::vector<PendingD2H> pending_d2h_;
 
-    uint64_t evictions_ = 0, swap_ins_ = 0;
+    uint64_t evictions_ = 0, swap_ins_ = 0, frag_evictions_ = 0;
 
     struct ProfRecord {
         const char* name;
@@ -364,6 +366,8 @@ private:
     size_t prof_next_ = 0;
     std::vector<ProfRecord> prof_records_;
     std::vector<tp_kernel_stat> prof_stats_;
+    std::set<std::string> prof_labels_;
+    const char* prof_label(const std::string& s);
 
     ExecLog log_;
     uint64_t req_range_ = 0;  // open "request" range of the marker trace, 0 = none

@@ -117,11 +117,14 @@ int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t s);
 // the tensor's payload and dst the tensor's place in the image; words [w_from, w_to) are expanded
 // (w_from a multiple of 64; w_to a multiple of 64 or the tensor's word count), reading the codes of
 // the same 2048-word block before w_from as well, which an earlier transfer group has delivered.
+// w_zero_to > w_to (a multiple of 64, less than 64 words past w_to): the words [w_to, w_zero_to) -- the
+// alignment gap behind the tensor's last word -- are written as zeros, as they are in the host image.
 struct UnpackPiece {
     const uint8_t* src;
     uint8_t* dst;
     uint64_t bytes;
     uint64_t w_from, w_to;
+    uint64_t w_zero_to;   // 0 = nothing to clear behind w_to
     const uint8_t* ext;   // the tensor's extension stream
     const uint32_t* tab;  // the tensor's block table
     int32_t base;

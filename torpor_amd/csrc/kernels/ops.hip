@@ -829,7 +829,17 @@ __global__ __launch_bounds__(256) void unpack_kernel(const UnpackArgs a) {
     __syncthreads();
     uint32_t rank = x - cnt;
     for (int w = 0; w < wave; ++w) rank += wave_total[w];
-    if (!have || word0 < pc.w_from) return;
+    if (!have) {
+        // behind the tensor's last word: the alignment gap of the image reads as zeros
+        if (word0 < pc.w_zero_to) {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            u32x4* z = reinterpret_cast<u32x4*>(reinterpret_cast<uint32_t*>(pc.dst) + word0);
+            z[0] = u32x4{0u, 0u, 0u, 0u};
+            z[1] = u32x4{0u, 0u, 0u, 0u};
+        }
+        return;
+    }
+    if (word0 < pc.w_from) return;
     const uint8_t* __restrict__ ext = pc.ext + pc.tab[bi] + rank;
     uint32_t w[8];
 #pragma unroll
@@ -847,6 +857,8 @@ __global__ __launch_bounds__(256) void unpack_kernel(const UnpackArgs a) {
     } else {  // last group of a tensor whose word count is not a multiple of 8
         const uint64_t words = pc.w_to - word0;
         for (uint64_t j = 0; j < words; ++j) out[j] = w[j];
+        if (pc.w_zero_to > pc.w_to)
+            for (uint64_t j = words; j < 8; ++j) out[j] = 0u;
     }
 }
 int launch_unpack(UnpackArgs& a, hipStream_t s) {
@@ -860,6 +872,8 @@ int launch_unpack(UnpackArgs& a, hipStream_t s) {
             blocks += (pc.bytes + kUnpackBlockBytes - 1) / kUnpackBlockBytes;
         } else {
             if (pc.base > 255 || !pc.tab || pc.w_to < pc.w_from || (pc.w_from & 63)) return K_EINVAL;
+            if (pc.w_zero_to && (pc.w_zero_to < pc.w_to || pc.w_zero_to - pc.w_to >= 64 || (pc.w_zero_to & 63)))
+                return K_EINVAL;
             if (pc.w_to > pc.w_from) blocks += (pc.w_to + 2047) / 2048 - pc.w_from / 2048;
         }
         if (blocks > 0x7FFFFFFFull) return K_EINVAL;

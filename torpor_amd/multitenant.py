@@ -1,0 +1,151 @@
+"""Multi-tenant serving of one GPU: a fleet of registered functions, a seeded request trace, and the loop
+that serves it.  The arrival process is that of the reference's load generator
+(scripts/sender_fix_rate.py:46-56): exponential gaps at a fixed mean rate, here with Zipf popularity over
+the functions.  Used by bench.py, bench_multitenant.py and the GPU tests of the 64-model configuration."""
+import sys
+import time
+
+import numpy as np
+
+# 32 ResNet-50 + 16 BERT-base (sequence 128) + 16 ResNet-152, seeds 0..63, batch 1
+FLEET_64 = (32, 16, 16)
+
+
+def fleet_plan(n_r50, n_bert, n_r152):
+    return [("resnet50", "resnet")] * n_r50 + [("bert-base", "bert")] * n_bert + [("resnet152", "resnet")] * n_r152
+
+
+def function_inputs(fid, family):
+    """The seeded request of function `fid` (the same one a CPU re-computation of its answer uses)."""
+    import torch
+    g = torch.Generator().manual_seed(1000 + fid)
+    if family == "resnet":
+        return [torch.randn(1, 3, 224, 224, generator=g).numpy()]
+    return [torch.randint(0, 30522, (1, 128), generator=g).numpy()]
+
+
+def build_fleet(server, n_r50=32, n_bert=16, n_r152=16, levels=None, keep_weights=()):
+    """Registers the functions (ids 0..n-1, weights seeded by the id); `levels` maps family name ->
+    model level of the ExecuteAfterLoad payload (0 light, 1 median, 2 heavy; default: the functions'
+    own default).  `keep_weights`: ids whose host-side weight dictionaries are kept for re-computation."""
+    from torpor_amd.functions import bert, resnet
+
+    fleet = []
+    for fid, (arch, family) in enumerate(fleet_plan(n_r50, n_bert, n_r152)):
+        kw = {}
+        if levels is not None and arch in levels:
+            kw["level"] = levels[arch]
+        if family == "resnet":
+            fn = resnet.ResNet(server, fid, arch, batch=1, seed=fid, **kw)
+        else:
+            fn = bert.Bert(server, fid, arch, batch=1, seq=128, seed=fid, **kw)
+        inputs = function_inputs(fid, family)
+        weights = fn._weights if fid in keep_weights else None   # as init_weights made them (the oracle twins load these)
+        first = fn.register(inputs)
+        fn._weights = None          # the server holds the authoritative copy now
+        packed, outbuf, views = fn.pack(inputs)
+        fleet.append(dict(fn=fn, fid=fid, arch=arch, family=family, inputs=inputs, weights=weights, packed=packed,
+                          outbuf=outbuf, views=views, first=[a.copy() for a in first]))
+    return fleet
+
+
+def zipf_probs(n, s=1.1):
+    p = 1.0 / np.arange(1, n + 1) ** s
+    return p / p.sum()
+
+
+def make_trace(n_functions, n_requests, rate, seed=0, zipf_s=1.1):
+    """(arrival times in seconds, function id per request).  Popularity rank -> function id is a fixed
+    shuffle, so that the hot functions are a mix of the model families."""
+    rng = np.random.default_rng(seed)
+    arrivals = np.cumsum(rng.exponential(1.0 / rate, n_requests))
+    order = rng.permutation(n_functions)
+    picks = order[rng.choice(n_functions, size=n_requests, p=zipf_probs(n_functions, zipf_s))]
+    return arrivals, picks
+
+
+def pct(xs, q):
+    if not len(xs):
+        return None
+    xs = np.sort(np.asarray(xs))
+    return float(xs[min(len(xs) - 1, int(round(q * (len(xs) - 1))))])
+
+
+def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after_request=None, note_every_s=30.0):
+    """Serves the trace in arrival order on the single executor.  open_loop: a request is not issued before
+    its arrival time and latency = completion - arrival (queueing included); otherwise requests run back to
+    back and latency is the service time.  Every `check_every`-th answer is compared bit for bit with the
+    function's registration run.  after_request(i, fid, hit) is called after each request."""
+    n_req = len(picks)
+    st0 = server.pool_stats()
+    lat_hit, lat_miss, by_arch, swap_bytes, swap_ms = [], [], {}, 0, 0.0
+    t0 = time.perf_counter()
+    next_note = note_every_s
+    for i in range(n_req):
+        now = time.perf_counter() - t0
+        if now >= next_note:        # a line now and then, so that a long run is seen to be alive
+            print(f"[{now:6.0f} s] {i} of {n_req} requests served", file=sys.stderr, flush=True)
+            next_note += note_every_s
+        if open_loop and now < arrivals[i]:
+            while time.perf_counter() - t0 < arrivals[i]:
+                pass
+        f = fleet[picks[i]]
+        fid = f["fid"]
+        hit = server.resident(fid)
+        t_req = time.perf_counter()
+        ack, _, dfr = server.signal(1, fid, "")
+        assert ack == 0 and not dfr
+        server.replay(fid, f["packed"], f["outbuf"])
+        done = time.perf_counter()
+        lat = ((done - t0 - arrivals[i]) if open_loop else (done - t_req)) * 1e3
+        (lat_hit if hit else lat_miss).append(lat)
+        by_arch.setdefault((f["arch"], hit), []).append(lat)
+        if not hit:
+            s = server.swap_stats(fid)
+            swap_bytes += s["bytes"]
+            swap_ms += s["copy_ms"]
+        if check_every and i % check_every == 0:
+            out = f["fn"].postprocess(f["views"])
+            for a, b in zip(f["first"], out):
+                if not np.array_equal(a, b):
+                    raise AssertionError(f"function {fid}: answer changed after swapping")
+        if after_request is not None:
+            after_request(i, fid, hit)
+    wall = time.perf_counter() - t0
+    st1 = server.pool_stats()
+    all_lat = lat_hit + lat_miss
+    return dict(
+        requests=n_req, wall_s=wall, achieved_rps=n_req / wall,
+        hit_ratio=len(lat_hit) / max(n_req, 1), evictions=st1["evictions"] - st0["evictions"],
+        fragmentation_evictions=st1["fragmentation_evictions"] - st0["fragmentation_evictions"],
+        swap_ins=st1["swap_ins"] - st0["swap_ins"],
+        latency_ms=dict(p50=pct(all_lat, 0.5), p99=pct(all_lat, 0.99), mean=float(np.mean(all_lat)) if all_lat else None),
+        hit_ms=dict(p50=pct(lat_hit, 0.5), p99=pct(lat_hit, 0.99), n=len(lat_hit)),
+        miss_ms=dict(p50=pct(lat_miss, 0.5), p99=pct(lat_miss, 0.99), n=len(lat_miss)),
+        per_model_ms={f"{a}/{'hit' if h else 'miss'}": dict(p50=pct(v, 0.5), p99=pct(v, 0.99), n=len(v))
+                      for (a, h), v in sorted(by_arch.items())},
+        swap_gbps=(swap_bytes / 1e9) / (swap_ms * 1e-3) if swap_ms else None,
+        pool_used_gib=st1["used"] / 2 ** 30, lru_models=st1["lru_models"],
+        pinned_host_gib=(st1["host_image_bytes"] + st1["host_transfer_bytes"] + st1["host_staging_bytes"]) / 2 ** 30,
+        device_outside_pool_gib=(st1["device_staging_bytes"] + st1["device_workspace_bytes"]) / 2 ** 30,
+    )
+
+
+def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2.0, **server_kw):
+    """One engine with an LRU budget of `cap_gib`, the fleet registered, the open-loop trace served."""
+    from torpor_amd.server import Server
+
+    limit = int(cap_gib * 2 ** 30)
+    with Server(mem_limit_bytes=limit, pool_bytes=limit + int(pool_headroom_gib * 2 ** 30), **server_kw) as server:
+        link = server.measure_h2d(256 << 20, 5)
+        t0 = time.perf_counter()
+        fleet = build_fleet(server, *models)
+        reg_s = time.perf_counter() - t0
+        charged = sum(server.model_info(f["fid"])["total_bytes"] for f in fleet)
+        weights = sum(server.model_info(f["fid"])["image_bytes"] for f in fleet)
+        arrivals, picks = make_trace(len(fleet), int(seconds * rate), rate, seed)
+        r = serve(server, fleet, arrivals, picks)
+        r.update(cap_gib=cap_gib, cap_binds=charged >= limit, registration_s=reg_s, offered_rps=rate,
+                 charged_total_gib=charged / 2 ** 30, weights_total_gb=weights / 1e9, link_peak_gbps=link)
+        del fleet
+    return r
