@@ -2,6 +2,9 @@ import os
 import sys
 
 import pytest
+import torch  # noqa: F401  (first: PyTorch ships its own HIP runtime, and in a process that uses both that one
+#               has to be loaded before the engine's library initialises the system's; the other order
+#               leaves torch.cuda without a device)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:

@@ -3,6 +3,7 @@ tp_gemm on the same inputs: bit-identical, on two calls in a row, the second wit
 that the second call runs over the partial sums the first one left in the shared scratch array."""
 import numpy as np
 import pytest
+import torch  # before anything initialises the system's HIP runtime: see tests/conftest.py
 
 from tests.harness import OpSession
 from torpor_amd import _lib
@@ -37,8 +38,6 @@ def _no_alloc(torch, X, W, b, M, N, K, act, stream):
 
 
 def test_no_alloc_gemm_matches_tp_gemm_twice_in_a_row():
-    import torch
-
     torch.cuda.set_device(0)
     stream = torch.cuda.Stream()
     rng = np.random.default_rng(11)
@@ -76,8 +75,6 @@ def test_no_alloc_gemm_refuses_what_does_not_fit_or_is_malformed():
     import os
     import subprocess
     import sys
-
-    import torch
 
     torch.cuda.set_device(0)
     x = torch.zeros((8, 8), device="cuda")

@@ -622,8 +622,9 @@ int Engine::unpack_on_device(const uint8_t* payload, uint64_t n_words, int32_t b
     if (active_ >= 0) return TP_EBUSY;  // the workspace belongs to the running request
     const uint64_t pb = align_up(packed_bytes(n_words), 256), eb = align_up(n_ext + 1, 256),
                    tb = align_up(packed_blocks(n_words) * 4, 256), wb = align_up(n_words * 4 + 4, 256);
-    if (cfg_.workspace_bytes < 8192 || pb + eb + tb + wb > cfg_.workspace_bytes - 4096) return TP_EINVAL;
-    uint8_t* d_payload = reinterpret_cast<uint8_t*>(workspace_) + 4096;
+    // behind the zero page and the ticket counters at the head of the workspace
+    if (cfg_.workspace_bytes < 16384 || pb + eb + tb + wb > cfg_.workspace_bytes - 8192) return TP_EINVAL;
+    uint8_t* d_payload = reinterpret_cast<uint8_t*>(workspace_) + 8192;
     uint8_t* d_ext = d_payload + pb;
     uint8_t* d_tab = d_ext + eb;
     uint8_t* d_words = d_tab + tb;
@@ -650,7 +651,7 @@ int Engine::unpack_on_device(const uint8_t* payload, uint64_t n_words, int32_t b
     HIPCHK(hipMemcpy(words, d_words, n_words * 4, hipMemcpyDeviceToHost));
     uint32_t guard = 0;  // the word past the end must be untouched (the last group is written word by word)
     HIPCHK(hipMemcpy(&guard, d_words + n_words * 4, 4, hipMemcpyDeviceToHost));
-    HIPCHK(hipMemset(reinterpret_cast<uint8_t*>(workspace_) + 4096, 0, pb + eb + tb + wb));
+    HIPCHK(hipMemset(reinterpret_cast<uint8_t*>(workspace_) + 8192, 0, pb + eb + tb + wb));
     return guard == 0xA5A5A5A5u ? 0 : TP_EFAULT;
 }
 
@@ -1703,10 +1704,12 @@ static tpk::EpilogueArgs ep_from(const Op& op, void* const* q, int pbase, int fb
 //  LAUNCH p/i/f per op id (see torpor_amd.h)
 int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
     void* q[12] = {nullptr};
-    // the first 256 bytes of the scratch allocation stay zero for good (padding source of the
-    // 3x3 convolution); split-K partial sums live behind them
-    // no device workspace in host-only mode (nothing is launched there)
-    const tpk::Workspace ws = workspace_ ? tpk::Workspace{workspace_ + 64, (size_t)cfg_.workspace_bytes - 256, workspace_}
+    // The scratch allocation: 256 bytes that stay zero for good (padding source of the 3x3
+    // convolution), the ticket counters of split K ranges (zero between launches), then the partial
+    // sums.  No device workspace in host-only mode (nothing is launched there).
+    constexpr size_t kHead = 256 + tpk::kSplitTickets * sizeof(unsigned);
+    const tpk::Workspace ws = workspace_ ? tpk::Workspace{workspace_ + kHead / 4, (size_t)cfg_.workspace_bytes - kHead, workspace_,
+                                                           reinterpret_cast<unsigned*>(workspace_ + 64)}
                                         : tpk::Workspace{};
     // Every operand is translated together with the byte span the kernel will touch, so an op
     // whose shapes do not fit its buffers is refused on the host instead of faulting the GPU.

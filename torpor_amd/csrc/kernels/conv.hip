@@ -20,7 +20,8 @@ void set_last_kernel(const char* n);
 int num_cu();
 Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
 int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, const Epilogue& e, hipStream_t s);
-int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, long* kper_out);
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out);
+unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
 
 struct ConvDev {
     const float* x;
@@ -33,6 +34,7 @@ struct ConvDev {
     int splits;
     long kper;  // K (generic) or channels (3x3 fast) per split
     float* ws;
+    unsigned* tickets;  // non-null: a split is summed inside the launch (finish_split)
     const float* zeros;
     int tiles_m, tiles_n;
     Epilogue ep;
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     constexpr int T = KH * KW;
     static_assert(C::BK == 8 * T, "K-block = 8 channels x taps");
     static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
-    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, red_floats<C>() + stage_floats<C>())];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, red_floats<C>() + stage_floats<C>() + 4)];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
     const int wm = wsp / C::WGN, wn = wsp % C::WGN;
@@ -169,7 +171,15 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     }
     if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
-    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wsp, lane,
+                                 reinterpret_cast<unsigned*>(lds + red_floats<C>() + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.Cout;
+        }
+    }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial,
                   lds + red_floats<C>() + wsp * STAGE_BLOCK);
 }
@@ -181,7 +191,7 @@ using ConvGenCfg = TileCfg<64, 64, 16, 2, 2>;
 
 __global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(const ConvDev p) {
     using C = ConvGenCfg;
-    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>() + 4)];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -247,7 +257,15 @@ __global__ __launch_bounds__(ConvGenCfg::THREADS, 2) void conv_generic_kernel(co
         __syncthreads();
     }
     float* partial = nullptr;
-    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.Cout;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wave, lane,
+                                 reinterpret_cast<unsigned*>(lds + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.Cout;
+        }
+    }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
@@ -484,6 +502,7 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     p.M = M;
     p.K = (long)a.Cin * a.KH * a.KW;
     p.ws = ws.ptr;
+    p.tickets = nullptr;  // set below once the tile grid is known
     p.zeros = ws.zeros;
     EpilogueArgs ea = a.ep;
     if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;
@@ -506,8 +525,9 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         p.tiles_m = (int)((M + 63) / 64);
         p.tiles_n = (a.Cout + 63) / 64;
         long kper_k = p.K;
-        p.splits = choose_splits((long)p.tiles_m * p.tiles_n, p.K, 8 * T, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
+        p.splits = choose_splits((long)p.tiles_m * p.tiles_n, p.K, 8 * T, 64 * 64, ws.ptr ? ws.bytes : 0, &kper_k);
         p.kper = kper_k / T;
+        p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
         switch (other_taps) {
             case 1: hipLaunchKernelGGL((conv_taps_kernel<TileCfg<64, 64, 56, 2, 2>, 1, 7>), grid, dim3(256), 0, s, p); break;
@@ -540,8 +560,9 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         // split over channel blocks of 8 (one K-block each)
         long kper_k = p.K;
         p.splits = 1;
-        if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, M, a.Cout, ws.ptr ? ws.bytes : 0, &kper_k);
+        if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k);
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
+        p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
         switch (cfg) {
             case 0:
@@ -573,14 +594,15 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         p.tiles_m = (int)((M + 63) / 64);
         p.tiles_n = (a.Cout + 63) / 64;
         const long tiles = (long)p.tiles_m * p.tiles_n;
-        p.splits = choose_splits(tiles, p.K, 16, M, a.Cout, ws.ptr ? ws.bytes : 0, &p.kper);
+        p.splits = choose_splits(tiles, p.K, 16, 64 * 64, ws.ptr ? ws.bytes : 0, &p.kper);
+        p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);
         hipLaunchKernelGGL(conv_generic_kernel, grid, dim3(256), 0, s, p);
         set_last_kernel("conv_generic_64x64");
     }
     int err = (int)hipGetLastError();
     if (err) return err;
-    if (p.splits > 1) return launch_splitk_reduce(ws.ptr, p.splits, M, a.Cout, a.y, p.ep, s);
+    if (p.splits > 1 && !p.tickets) return launch_splitk_reduce(ws.ptr, p.splits, M, a.Cout, a.y, p.ep, s);
     return 0;
 }
 

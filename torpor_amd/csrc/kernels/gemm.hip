@@ -41,6 +41,7 @@ struct GemmDev {
     int splits;
     long kper;
     float* ws;
+    unsigned* tickets;  // non-null: the split is summed inside the launch (finish_split)
     int tiles_m, tiles_n;
     int xr, xc;  // the 8 XCDs form an xr x xc grid over the tile grid (xr*xc == 8), 0 = linear mapping
     Epilogue ep;
@@ -93,7 +94,7 @@ template <class C, bool YKC>
 __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_fast_kernel(const GemmDev p) {
     // two LDS stages: while the MFMAs read one, the next K-block is written to the other, so
     // the loop needs a single barrier per K-block
-    __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, stage_floats<C>())];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, stage_floats<C>() + 4)];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / C::WGN, wn = wave % C::WGN;
     int tm, tn, t;
@@ -228,7 +229,15 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
         __syncthreads();
     }
     float* partial = nullptr;
-    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wave, lane,
+                                 reinterpret_cast<unsigned*>(lds + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.N;
+        }
+    }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
@@ -243,7 +252,7 @@ template <class C, bool YKC, int STAGES>
 #endif
 __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(const GemmDev p) {
     constexpr int RED_FLOATS = red_floats<C>();  // K-slice reduction area, then the epilogue staging blocks
-    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>())];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
     const int wm = wsp / C::WGN, wn = wsp % C::WGN;
@@ -374,7 +383,15 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     }
     if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
-    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wsp, lane,
+                                 reinterpret_cast<unsigned*>(lds + RED_FLOATS + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.N;
+        }
+    }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK);
 }
 
@@ -383,7 +400,7 @@ using GenCfg = TileCfg<64, 64, 16, 2, 2>;
 
 __global__ __launch_bounds__(GenCfg::THREADS, 2) void gemm_generic_kernel(const GemmDev p) {
     using C = GenCfg;
-    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>())];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(C::LDS_FLOATS, stage_floats<C>() + 4)];
     float* As = lds;
     float* Bs = lds + C::BM * C::LDK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -451,7 +468,15 @@ __global__ __launch_bounds__(GenCfg::THREADS, 2) void gemm_generic_kernel(const 
         __syncthreads();
     }
     float* partial = nullptr;
-    if (p.splits > 1) partial = p.ws + (long)split * p.M * p.N;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wave, lane,
+                                 reinterpret_cast<unsigned*>(lds + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.N;
+        }
+    }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + wave * STAGE_BLOCK);
 }
 
@@ -622,18 +647,33 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Pick the split-K factor: fill the chip when the tile count alone cannot.
-int choose_splits(long tiles, long K, int bk, long M, long N, size_t ws_bytes, long* kper_out) {
+// The ticket counters of a workspace, if the in-launch summation of split K ranges is to be used for a
+// grid of `tiles` output tiles split `splits` ways.  Measured on MI355X: with up to 8 slots the workgroup
+// that finishes a tile last sums them as fast as a reduction launch would or faster (ResNet-152 batch 8,
+// 3x3 convolutions of 100 tiles x 6: 29.1 against 30.2 us, and the cold request, whose launches queue behind
+// the swap-in's copies, 4.11 against 4.23 ms); with 16 to 32 slots its serial read of them loses to the
+// reduction kernel's whole-chip pass (1x1000x2048, 32 slots: 13.6 against 11.3 us).
+// TORPOR_SPLITK_FUSED=0 forces the two-launch form, =2 the in-launch form for any split count.
+unsigned* split_tickets(const Workspace& ws, long tiles, int splits) {
+    static const int mode = getenv("TORPOR_SPLITK_FUSED") ? atoi(getenv("TORPOR_SPLITK_FUSED")) : 1;
+    if (mode == 0 || tiles > kSplitTickets || splits < 2) return nullptr;
+    return (mode == 2 || splits <= 8) ? ws.tickets : nullptr;
+}
+
+// One split's partial sums are `tiles` whole output tiles of tile_floats each (the in-launch summation
+// keeps them per tile and per wavefront; the two-launch form needs no more than that).
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out) {
     int splits = 1;
     const long kblocks = (K + bk - 1) / bk;
+    const size_t per = (size_t)tiles * (size_t)tile_floats * sizeof(float);
     static const int forced = getenv("TORPOR_SPLITS") ? atoi(getenv("TORPOR_SPLITS")) : 0;
-    if (forced > 0 && kblocks >= 2L * forced && (size_t)forced * (size_t)M * (size_t)N * sizeof(float) <= ws_bytes) {
+    if (forced > 0 && kblocks >= 2L * forced && (size_t)forced * per <= ws_bytes) {
         splits = forced;
     } else if (tiles < g_num_cu && kblocks >= 8) {
         long want = (2L * g_num_cu + tiles - 1) / tiles;
         long maxs = kblocks / 4;  // keep at least 4 K-blocks per split
         if (want > maxs) want = maxs;
         if (want > 32) want = 32;
-        const size_t per = (size_t)M * (size_t)N * sizeof(float);
         while (want > 1 && (size_t)want * per > ws_bytes) --want;
         if (want > 1) splits = (int)want;
     }
@@ -672,13 +712,13 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
         g.tiles_n = (int)((a.N + g.bn - 1) / g.bn);
         const long tiles = (long)g.tiles_m * g.tiles_n * batch;
         g.kper = ((a.K + 31) / 32) * 32;
-        if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, a.M, a.N, ws_bytes, &g.kper);
+        if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, (long)g.bm * g.bn, ws_bytes, &g.kper);
     } else {
         g.tiles_m = (int)((a.M + 63) / 64);
         g.tiles_n = (int)((a.N + 63) / 64);
         const long tiles = (long)g.tiles_m * g.tiles_n * batch;
         g.kper = ((a.K + 15) / 16) * 16;
-        if (batch == 1) g.splits = choose_splits(tiles, a.K, 16, a.M, a.N, ws_bytes, &g.kper);
+        if (batch == 1) g.splits = choose_splits(tiles, a.K, 16, 64 * 64, ws_bytes, &g.kper);
     }
     return g;
 }
@@ -695,7 +735,7 @@ static bool gemm_args_ok(const GemmArgs& a) {
 long gemm_workspace_need(const GemmArgs& a) {
     if (!gemm_args_ok(a)) return K_EINVAL;
     const GemmPlan g = plan_gemm(a, ~(size_t)0);
-    return g.splits > 1 ? (long)g.splits * a.M * a.N * (long)sizeof(float) : 0;
+    return g.splits > 1 ? (long)g.splits * g.tiles_m * g.tiles_n * g.bm * g.bn * (long)sizeof(float) : 0;
 }
 
 int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
@@ -729,6 +769,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     p.sw = a.sw;
     p.ws = ws.ptr;
     p.ep = make_epilogue(a.ep, a.ldc);
+    p.tickets = split_tickets(ws, (long)g.tiles_m * g.tiles_n, g.splits);
 
     p.tiles_m = g.tiles_m;
     p.tiles_n = g.tiles_n;
@@ -777,7 +818,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     }
     int err = (int)hipGetLastError();
     if (err) return err;
-    if (p.splits > 1) return launch_splitk_reduce(ws.ptr, p.splits, a.M, a.N, a.C, p.ep, s);
+    if (p.splits > 1 && !p.tickets) return launch_splitk_reduce(ws.ptr, p.splits, a.M, a.N, a.C, p.ep, s);
     return 0;
 }
 

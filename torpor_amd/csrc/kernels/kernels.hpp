@@ -60,7 +60,11 @@ struct Workspace {
     float* ptr = nullptr;  // split-K partial sums
     size_t bytes = 0;
     const float* zeros = nullptr;  // >= 64 zero bytes, 16 B aligned: source for padded convolution taps
+    // kSplitTickets counters, zero between launches: with them a K range split over workgroups is summed
+    // by the workgroup that finishes a tile last, inside the same launch; without, by a second launch
+    unsigned* tickets = nullptr;
 };
+constexpr int kSplitTickets = 1024;
 
 void kernels_init(int device);  // caches CU count
 int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s);

@@ -202,6 +202,75 @@ __device__ __forceinline__ bool reduce_k_slices(f32x16 (&acc)[C::TM][C::TN], flo
     return true;
 }
 
+// A K range split over `splits` workgroups, summed inside the launch.  Every workgroup of a tile writes
+// its accumulators, register by register and lane-major (so each store instruction covers 256 contiguous
+// bytes), to slot `split` of the tile's block in `part`, then draws a ticket; the workgroup that draws the
+// last one reads all slots back in slot order -- a fixed order of summation, whichever workgroup it is --
+// and returns true with the complete sums in acc; the others return false and are done.
+//
+// The 8 XCDs have private L2s that are not coherent with each other for ordinary accesses, and an
+// agent-scope fence writes back / invalidates a whole L2.  So partial sums and tickets are moved with
+// relaxed agent-scope atomic accesses instead (write-through stores, loads that bypass the L2, a
+// read-modify-write at the memory side): coherent per access, nothing to flush.  The wait for the stores
+// before the ticket is explicit, since a workgroup barrier alone does not wait for global stores.
+// tickets[tile] is zero at entry and zero again when the last workgroup leaves.
+// Call it from every wavefront that holds sums (the K-slice-0 wavefronts) after the K loop's last
+// barrier; `flag` is one word of LDS that nobody uses meanwhile.
+template <class C>
+__device__ __forceinline__ bool finish_split(f32x16 (&acc)[C::TM][C::TN], float* __restrict__ part,
+                                             unsigned* __restrict__ tickets, int splits, int tile, int split, int wsp,
+                                             int lane, unsigned* flag) {
+    constexpr int PER_WAVE = C::TM * C::TN * 16 * 64;
+    constexpr long TILE_FLOATS = (long)C::WGM * C::WGN * PER_WAVE;
+    float* mine = part + ((long)tile * splits + split) * TILE_FLOATS + wsp * PER_WAVE + lane;
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                __hip_atomic_store(mine + ((i * C::TN + j) * 16 + v) * 64, acc[i][j][v], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's partial sums have reached memory
+    __syncthreads();
+    if (threadIdx.x == 0)
+        *flag = __hip_atomic_fetch_add(tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*flag != (unsigned)(splits - 1)) return false;
+    if (threadIdx.x == 0) __hip_atomic_store(tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float* src = part + (long)tile * splits * TILE_FLOATS + wsp * PER_WAVE + lane;
+    // four slots are fetched together (their loads are all in flight before the first is used) and
+    // then added in slot order
+    constexpr int NR = C::TM * C::TN * 16;
+    constexpr int ZU = NR <= 16 ? 4 : 2;
+#pragma unroll 1
+    for (int z = 0; z < splits; z += ZU) {
+        float x[ZU][NR];
+#pragma unroll
+        for (int u = 0; u < ZU; ++u) {
+            const int zz = z + u < splits ? z + u : splits - 1;  // past the end: re-read the last slot, unused
+#pragma unroll
+            for (int r = 0; r < NR; ++r)
+                x[u][r] = __hip_atomic_load(src + (long)zz * TILE_FLOATS + r * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < ZU; ++u) {
+            if (z + u < splits) {
+#pragma unroll
+                for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const float y = x[u][(i * C::TN + j) * 16 + v];
+                            acc[i][j][v] = (z + u == 0) ? y : acc[i][j][v] + y;
+                        }
+            }
+        }
+    }
+    return true;
+}
+
 __device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // Vector form of the accumulator write-out for the common case: row-major output with 16-byte

@@ -5,8 +5,10 @@
 // in device memory that the library's code object carries, one copy per GPU.
 //
 // Every call on a GPU shares that GPU's array: two calls that overlap on one GPU (different
-// streams or threads) race on it.  The array keeps the previous call's partial sums; nothing in it
-// has to start at zero, because a split GEMM writes every partial sum it later reads.
+// streams or threads) race on it.  The array keeps the previous call's partial sums: a split GEMM
+// writes every partial sum it later reads.  Its first 4 KiB are the ticket counters by which the
+// workgroups of a split tile find out which of them finishes last; they start at zero (the array is
+// zero-initialised with the code object) and the last workgroup of every tile sets its counter back.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -104,7 +106,10 @@ extern "C" int tp_gemm_noalloc(const tp_gemm_desc* d, void* stream) {
     // that both entry points keep computing the same bits.
     const long need = tpk::gemm_workspace_need(g);
     if (need < 0) return (int)need;
-    if ((size_t)need > kScratchBytes) return TP_ESCRATCH;
-    const tpk::Workspace ws{ptr, kScratchBytes, nullptr};
+    constexpr size_t kTicketBytes = tpk::kSplitTickets * sizeof(unsigned);
+    if ((size_t)need > kScratchBytes - kTicketBytes) return TP_ESCRATCH;
+    // head of the array: the ticket counters of split K ranges.  They are zero when the code object is
+    // loaded and every launch leaves them zero, so nothing has to be cleared between calls.
+    const tpk::Workspace ws{ptr + kTicketBytes / 4, kScratchBytes - kTicketBytes, nullptr, reinterpret_cast<unsigned*>(ptr)};
     return tpk::launch_gemm(g, ws, static_cast<hipStream_t>(stream));
 }
