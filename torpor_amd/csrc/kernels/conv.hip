@@ -40,6 +40,34 @@ struct ConvDev {
     Epilogue ep;
 };
 
+__device__ __forceinline__ void fetch_now(const ConvDev& p) {
+    fetch_now(p.x);
+    fetch_now(p.w);
+    fetch_now(p.y);
+    fetch_now(p.H);
+    fetch_now(p.W);
+    fetch_now(p.Cin);
+    fetch_now(p.Cout);
+    fetch_now(p.Ho);
+    fetch_now(p.Wo);
+    fetch_now(p.sh);
+    fetch_now(p.sw);
+    fetch_now(p.ph);
+    fetch_now(p.pw);
+    fetch_now(p.xs_n);
+    fetch_now(p.xs_h);
+    fetch_now(p.xs_w);
+    fetch_now(p.M);
+    fetch_now(p.splits);
+    fetch_now(p.kper);
+    fetch_now(p.ws);
+    fetch_now(p.tickets);
+    fetch_now(p.zeros);
+    fetch_now(p.tiles_m);
+    fetch_now(p.tiles_n);
+    fetch_now(p.ep);
+}
+
 __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
     const int q = n >> 3, rem = n & 7;
     const int xcd = bid & 7, local = bid >> 3;
@@ -63,6 +91,7 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
 // matrix work overlap and an iteration has one barrier instead of two.
 template <class C, int KH, int KW, int STAGES = 2>
 __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_taps_kernel(const ConvDev p) {
+    fetch_now(p);
     constexpr int T = KH * KW;
     static_assert(C::BK == 8 * T, "K-block = 8 channels x taps");
     static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
@@ -111,6 +140,8 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     zero_acc<C>(acc);
     f32x4 ra[NVA];
     f32x4 rw[T];
+    ColConsts<C::TN> cc;  // bias / batch-norm vectors of this wavefront's columns: requested now, used at the end
+    if (wk == 0) cols_issue<C>(cc, p.ep, p.y, n0, wn, lane, (long)p.Cout);
 
     auto load_regs = [&](int c0) {
         if (c0 > cend - 8) c0 = cend - 8;  // look-ahead past the end re-reads the last block
@@ -146,6 +177,7 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     };
 
     load_regs(cbeg);
+    if (wk == 0) cols_fold<C>(cc, p.ep);
     if (STAGES == 2) {
         store_lds(0);
         load_regs(cbeg + 8);
@@ -181,7 +213,7 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
         }
     }
     store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, (long)p.Cout, p.y, p.ep, partial,
-                  lds + red_floats<C>() + wsp * STAGE_BLOCK);
+                  lds + red_floats<C>() + wsp * STAGE_BLOCK, &cc);
 }
 
 // Any kernel size / stride / padding / input layout; K ordered (c, kh, kw) as

@@ -15,6 +15,12 @@
 
 #include <cstdlib>
 
+// Cycle stamps for kernel-phase measurements: an experiment harness that includes this file defines
+// TP_CLK before it; in the library the hooks are empty.
+#ifndef TP_CLK
+#define TP_CLK(n)
+#endif
+
 namespace tpk {
 
 static int g_num_cu = 256;
@@ -44,6 +50,11 @@ struct GemmDev {
     unsigned* tickets;  // non-null: the split is summed inside the launch (finish_split)
     int tiles_m, tiles_n;
     int xr, xc;  // the 8 XCDs form an xr x xc grid over the tile grid (xr*xc == 8), 0 = linear mapping
+    // the rectangle of each XCD (first tile row / column, width, height), worked out on the host: in the
+    // kernel the same arithmetic is four 64-bit divisions, about two thousand cycles before the first load
+    struct Rect {
+        unsigned short r0, c0, w, h;
+    } rect[8];
     Epilogue ep;
 };
 
@@ -68,17 +79,37 @@ __device__ __forceinline__ bool tile_of(const GemmDev& p, int bid, int* tm, int*
         *tn = *t - *tm * p.tiles_n;
         return true;
     }
-    const int xcd = bid & 7, local = bid >> 3;
-    const int br = xcd / p.xc, bc = xcd - br * p.xc;
-    const int r0 = (int)((long)p.tiles_m * br / p.xr), r1 = (int)((long)p.tiles_m * (br + 1) / p.xr);
-    const int c0 = (int)((long)p.tiles_n * bc / p.xc), c1 = (int)((long)p.tiles_n * (bc + 1) / p.xc);
-    const int w = c1 - c0, h = r1 - r0;
+    const int xcd = bid & 7;
+    const unsigned local = (unsigned)bid >> 3;
+    const unsigned w = p.rect[xcd].w, h = p.rect[xcd].h;
     if (local >= w * h) return false;
-    const int lr = local / w;
-    *tm = r0 + lr;
-    *tn = c0 + (local - lr * w);
+    const unsigned lr = local / w;
+    *tm = (int)(p.rect[xcd].r0 + lr);
+    *tn = (int)(p.rect[xcd].c0 + (local - lr * w));
     *t = *tm * p.tiles_n + *tn;
     return true;
+}
+
+__device__ __forceinline__ void fetch_now(const GemmDev& p) {
+    fetch_now(p.X);
+    fetch_now(p.Y);
+    fetch_now(p.C);
+    fetch_now(p.M);
+    fetch_now(p.N);
+    fetch_now(p.K);
+    fetch_now(p.xs_r);
+    fetch_now(p.ys_c);
+    fetch_now(p.ys_k);
+    fetch_now(p.nb1);
+    fetch_now(p.gather);
+    fetch_now(p.splits);
+    fetch_now(p.kper);
+    fetch_now(p.ws);
+    fetch_now(p.tickets);
+    fetch_now(p.tiles_m);
+    fetch_now(p.tiles_n);
+    fetch_now(p.xr);
+    fetch_now(p.ep);
 }
 
 __device__ __forceinline__ long gather_row(const GemmDev& p, long grow) {
@@ -92,6 +123,7 @@ __device__ __forceinline__ long gather_row(const GemmDev& p, long grow) {
 
 template <class C, bool YKC>
 __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm_fast_kernel(const GemmDev p) {
+    fetch_now(p);
     // two LDS stages: while the MFMAs read one, the next K-block is written to the other, so
     // the loop needs a single barrier per K-block
     __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, stage_floats<C>() + 4)];
@@ -251,8 +283,10 @@ template <class C, bool YKC, int STAGES>
 #define TP_CLEAN_OCC (C::TM * C::TN >= 4 ? 1 : 2)
 #endif
 __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(const GemmDev p) {
+    fetch_now(p);
     constexpr int RED_FLOATS = red_floats<C>();  // K-slice reduction area, then the epilogue staging blocks
     __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
+    TP_CLK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
     const int wm = wsp / C::WGN, wn = wsp % C::WGN;
@@ -271,6 +305,8 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     const long kbeg = (long)split * p.kper;
     const long kend = (kbeg + p.kper < p.K) ? kbeg + p.kper : p.K;
     const long klast = kend - C::BK;
+    ColConsts<C::TN> cc;  // bias / batch-norm vectors of this wavefront's columns: requested now, used at the end
+    if (wk == 0) cols_issue<C>(cc, p.ep, Cc, n0, wn, lane, p.N);
 
     constexpr int KV = C::BK / 4;
     constexpr int CV = C::BN / 4;
@@ -337,12 +373,14 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         }
     };
 
+    TP_CLK(1);
     const float* As0 = lds;
     const long kpairs = kbeg + (kend - kbeg) / (2 * C::BK) * (2 * C::BK);  // end of the whole pairs of K-blocks
     if (STAGES == 2) {
         const float* As1 = lds + C::LDS_FLOATS;
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
+        if (wk == 0) cols_fold<C>(cc, p.ep);
         store_lds(ra0, rb0, 0);
         __syncthreads();
         for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
@@ -362,6 +400,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         // workgroups stay resident and hide each other's barrier and memory latency
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
+        if (wk == 0) cols_fold<C>(cc, p.ep);
         for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
             store_lds(ra0, rb0, 0);
             __syncthreads();
@@ -381,6 +420,140 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             __syncthreads();
         }
     }
+    TP_CLK(2);
+    if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
+    TP_CLK(3);
+    float* partial = nullptr;
+    if (p.splits > 1) {
+        if (p.tickets) {
+            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wsp, lane,
+                                 reinterpret_cast<unsigned*>(lds + RED_FLOATS + stage_floats<C>())))
+                return;
+        } else {
+            partial = p.ws + (long)split * p.M * p.N;
+        }
+    }
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK, &cc);
+    TP_CLK(4);
+}
+
+// The branch-free kernel for grids that leave a CU with one or two workgroups: there nothing hides the
+// memory latency of a K-block but the workgroup's own look-ahead, and two K-blocks ahead (a few hundred
+// cycles of matrix work) is far less than a round trip to memory.  D register sets keep D K-blocks in
+// flight per workgroup; block b travels through set b % D and LDS stage b & 1, one barrier per block.
+// Same preconditions as gemm_clean_kernel (whole K-blocks, clamped edges); any number of K-blocks.
+template <class C, bool YKC, int D>
+__global__ __launch_bounds__(C::THREADS, 1) void gemm_deep_kernel(const GemmDev p) {
+    fetch_now(p);
+    static_assert(D >= 2 && D % 2 == 0, "the LDS stage of a block must follow from its register set");
+    constexpr int RED_FLOATS = red_floats<C>();
+    __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
+    const int wm = wsp / C::WGN, wn = wsp % C::WGN;
+    int tm, tn, t;
+    if (!tile_of(p, blockIdx.x, &tm, &tn, &t)) return;
+    const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
+    int split = 0, batch = blockIdx.z;
+    if (p.splits > 1) {
+        split = blockIdx.z;
+        batch = 0;
+    }
+    const int b0 = batch / p.nb1, b1 = batch - b0 * p.nb1;
+    const float* __restrict__ X = p.X + b0 * p.xb0 + b1 * p.xb1;
+    const float* __restrict__ Y = p.Y + b0 * p.yb0 + b1 * p.yb1;
+    float* __restrict__ Cc = p.C + b0 * p.cb0 + b1 * p.cb1;
+    const long kbeg = (long)split * p.kper;
+    const long kend = (kbeg + p.kper < p.K) ? kbeg + p.kper : p.K;
+    const int nb = (int)((kend - kbeg) / C::BK);  // whole K-blocks of this workgroup
+    ColConsts<C::TN> cc;
+    if (wk == 0) cols_issue<C>(cc, p.ep, Cc, n0, wn, lane, p.N);
+
+    constexpr int KV = C::BK / 4;
+    constexpr int CV = C::BN / 4;
+    constexpr int NVA = C::BM * KV / C::THREADS;
+    constexpr int NVB = (YKC ? C::BN * KV : C::BK * CV) / C::THREADS;
+    static_assert(C::BM * KV % C::THREADS == 0 && C::BN * KV % C::THREADS == 0 && C::BK * CV % C::THREADS == 0,
+                  "tile must split evenly over the workgroup");
+    const float* pa[NVA];
+    const float* pb[NVB];
+    int sa[NVA], sb[NVB];
+#pragma unroll
+    for (int i = 0; i < NVA; ++i) {
+        const int idx = i * C::THREADS + tid;
+        const int row = idx / KV, kq = idx - row * KV;
+        long grow = m0 + row;
+        if (grow > p.M - 1) grow = p.M - 1;
+        pa[i] = X + gather_row(p, grow) * p.xs_r + kq * 4 + kbeg;
+        sa[i] = row * C::LDK + kq * 4;
+    }
+    const long ystep = YKC ? 1 : p.ys_k;
+#pragma unroll
+    for (int i = 0; i < NVB; ++i) {
+        const int idx = i * C::THREADS + tid;
+        if (YKC) {
+            const int col = idx / KV, kq = idx - col * KV;
+            long gcol = n0 + col;
+            if (gcol > p.N - 1) gcol = p.N - 1;
+            pb[i] = Y + gcol * p.ys_c + kq * 4 + kbeg;
+            sb[i] = col * C::LDK + kq * 4;
+        } else {
+            const int kk = idx / CV, cq = idx - kk * CV;
+            long gcol = n0 + cq * 4;
+            if (gcol > p.N - 4) gcol = p.N - 4;
+            pb[i] = Y + (kk + kbeg) * p.ys_k + gcol;
+            sb[i] = (cq * 4) * C::LDK + kk;
+        }
+    }
+
+    f32x16 acc[C::TM][C::TN];
+    zero_acc<C>(acc);
+    f32x4 ra[D][NVA], rb[D][NVB];
+    auto load_regs = [&](int set, int b) {  // K-block b of this workgroup into register set `set`
+        const long k = (long)b * C::BK;
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) ra[set][i] = *reinterpret_cast<const f32x4*>(pa[i] + k);
+#pragma unroll
+        for (int i = 0; i < NVB; ++i) rb[set][i] = *reinterpret_cast<const f32x4*>(pb[i] + k * ystep);
+    };
+    auto store_lds = [&](int set, int stage) {
+        float* As = lds + stage * C::LDS_FLOATS;
+        float* Bs = As + C::BM * C::LDK;
+#pragma unroll
+        for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[set][i];
+#pragma unroll
+        for (int i = 0; i < NVB; ++i) {
+            if (YKC) {
+                *reinterpret_cast<f32x4*>(Bs + sb[i]) = rb[set][i];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) Bs[sb[i] + j * C::LDK] = rb[set][i][j];
+            }
+        }
+    };
+    // one K-block: refill the set that block b left, multiply block b, move block b + 1 into the other stage
+    auto phase = [&](int d, int b) {
+        if (b + D < nb) load_regs(d, b + D);
+        const float* As = lds + (d & 1) * C::LDS_FLOATS;
+        mma_block<C>(As, As + C::BM * C::LDK, acc, wm, wn, lane, wk);
+        if (b + 1 < nb) store_lds((d + 1) % D, (d + 1) & 1);
+        __syncthreads();
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (d < nb) load_regs(d, d);
+    if (wk == 0) cols_fold<C>(cc, p.ep);
+    store_lds(0, 0);
+    __syncthreads();
+    int b = 0;
+    for (; b + D <= nb; b += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) phase(d, b + d);
+    }
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (b + d < nb) phase(d, b + d);
+
     if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
     float* partial = nullptr;
     if (p.splits > 1) {
@@ -392,7 +565,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             partial = p.ws + (long)split * p.M * p.N;
         }
     }
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK);
+    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK, &cc);
 }
 
 // Any strides, any alignment.  64x64x16 tile, scalar loads.
@@ -543,11 +716,21 @@ static int plan_xcd_grid(GemmDev& p, long M, long N) {
         }
     }
     if (p.xr == 0) return p.tiles_m * p.tiles_n;  // fewer tiles than a split needs: linear mapping
+    if (p.tiles_m > 65535 || p.tiles_n > 65535) {  // beyond the rectangle table's range: linear mapping
+        p.xr = p.xc = 0;
+        return p.tiles_m * p.tiles_n;
+    }
     int biggest = 0;
     for (int br = 0; br < p.xr; ++br)
         for (int bc = 0; bc < p.xc; ++bc) {
-            const int h = (int)((long)p.tiles_m * (br + 1) / p.xr) - (int)((long)p.tiles_m * br / p.xr);
-            const int w = (int)((long)p.tiles_n * (bc + 1) / p.xc) - (int)((long)p.tiles_n * bc / p.xc);
+            const int r0 = (int)((long)p.tiles_m * br / p.xr), r1 = (int)((long)p.tiles_m * (br + 1) / p.xr);
+            const int c0 = (int)((long)p.tiles_n * bc / p.xc), c1 = (int)((long)p.tiles_n * (bc + 1) / p.xc);
+            const int h = r1 - r0, w = c1 - c0;
+            GemmDev::Rect& q = p.rect[br * p.xc + bc];
+            q.r0 = (unsigned short)r0;
+            q.c0 = (unsigned short)c0;
+            q.w = (unsigned short)w;
+            q.h = (unsigned short)h;
             if (h * w > biggest) biggest = h * w;
         }
     return 8 * biggest;
@@ -605,6 +788,15 @@ static int launch_clean_only(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t
     else
         hipLaunchKernelGGL((gemm_clean_kernel<C, false, 2>), grid, dim3(C::THREADS), 0, s, p);
     return 2;
+}
+
+// The deep look-ahead kernel (gemm_deep_kernel) for grids of at most two workgroups per CU.
+template <class C>
+static void launch_deep(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t s) {
+    if (y_kc)
+        hipLaunchKernelGGL((gemm_deep_kernel<C, true, 6>), grid, dim3(C::THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((gemm_deep_kernel<C, false, 6>), grid, dim3(C::THREADS), 0, s, p);
 }
 
 // Tile shape.  Measured on MI355X over the served shapes (BERT-large 1536 x {1024,4096} x
@@ -787,19 +979,32 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
-        static const char* const names[5][2][3] = {
-            {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2"},
-             {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2"}},
-            {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2"},
-             {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2"}},
-            {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2"},
-             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}},
-            {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2"},
-             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}},
-            {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2"},
-             {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2"}}};
+        static const char* const names[5][2][4] = {
+            {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2", ""},
+             {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2", ""}},
+            {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2", ""},
+             {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2", ""}},
+            {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2", "gemm_fast_64x64_cc_d6"},
+             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2", "gemm_fast_64x64_kc_d6"}},
+            {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2", "gemm_fast_64x32_cc_d6"},
+             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2", "gemm_fast_64x32_kc_d6"}},
+            {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2", "gemm_fast_32x32_cc_d6"},
+             {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2", "gemm_fast_32x32_kc_d6"}}};
+        // _d6: six K-blocks in flight per workgroup, for grids that leave a CU at most two workgroups
+        // (TORPOR_GEMM_DEEP=0 switches it off, =n moves the bound to n workgroups per CU)
+        static const int deep_per_cu = getenv("TORPOR_GEMM_DEEP") ? atoi(getenv("TORPOR_GEMM_DEEP")) : 2;
+        const long wgs = (long)p.tiles_m * p.tiles_n * grid.z;
+        const bool deep = clean && cfg >= 2 && deep_per_cu > 0 && wgs <= (long)deep_per_cu * g_num_cu;
         int variant;
-        if (cfg == 0)
+        if (deep) {
+            if (cfg == 2)
+                launch_deep<CfgM>(p, y_kc, grid, s);
+            else if (cfg == 3)
+                launch_deep<CfgS>(p, y_kc, grid, s);
+            else
+                launch_deep<CfgT>(p, y_kc, grid, s);
+            variant = 3;
+        } else if (cfg == 0)
             variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
         else if (cfg == 1)
             variant = launch_fast<CfgW>(p, y_kc, clean, grid, s);

@@ -20,6 +20,16 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum Act : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_TANH = 3, ACT_RELU6 = 4, ACT_SILU = 5, ACT_SIGMOID = 6 };
 
+// Kernel arguments live in memory and the compiler fetches each one where it is first used; in a
+// prologue full of dependent branches that is a chain of a dozen scalar-load round trips of a few
+// hundred cycles each before the first operand load goes out.  fetch_now pins a value into a scalar
+// register at the point of the call, so a run of calls at the top of a kernel turns the chain into
+// one batch of loads and one wait.
+template <class T>
+__device__ __forceinline__ void fetch_now(const T& v) {
+    asm volatile("" ::"s"(v));
+}
+
 // out = act( bn( alpha*acc + beta*C_old + bias[n] ) + residual )
 struct Epilogue {
     float alpha;
@@ -40,6 +50,22 @@ struct Epilogue {
     long howo;
     long ncols;
 };
+
+__device__ __forceinline__ void fetch_now(const Epilogue& e) {
+    fetch_now(e.alpha);
+    fetch_now(e.beta);
+    fetch_now(e.bias);
+    fetch_now(e.bn_scale);
+    fetch_now(e.bn_bias);
+    fetch_now(e.bn_mean);
+    fetch_now(e.bn_var);
+    fetch_now(e.bn_eps);
+    fetch_now(e.residual);
+    fetch_now(e.ldr);
+    fetch_now(e.act);
+    fetch_now(e.ldc);
+    fetch_now(e.out_nchw);
+}
 
 __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == ACT_RELU) return v > 0.f ? v : 0.f;
@@ -273,83 +299,146 @@ __device__ __forceinline__ bool finish_split(f32x16 (&acc)[C::TM][C::TN], float*
 
 __device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Activation with the kind fixed at compile time: the write-out loops are instantiated per kind and
+// entered through one switch, instead of testing the kind for every element (a taken branch costs a
+// wavefront that is alone on its SIMD tens of cycles, and there were six per element).
+template <int ACT>
+__device__ __forceinline__ float act_fixed(float v) {
+    if (ACT == ACT_RELU) return v > 0.f ? v : 0.f;
+    if (ACT == ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    if (ACT == ACT_TANH) return tanhf(v);
+    if (ACT == ACT_RELU6) return fminf(fmaxf(v, 0.f), 6.f);
+    if (ACT == ACT_SILU) return v / (1.0f + expf(-v));
+    if (ACT == ACT_SIGMOID) return 1.0f / (1.0f + expf(-v));
+    return v;
+}
+
+// The per-column constants of a wavefront's TN column blocks for the vector write-out, folded to
+// x * cs + ct.  A kernel issues the loads when it starts (cols_issue) and folds them once its first
+// operand loads are on their way (cols_fold), so that their latency is not paid at the end, where
+// nothing else is left to hide it.  ok = the wavefront qualifies for the vector write-out.
+template <int TN>
+struct ColConsts {
+    f32x4 cs[TN], ct[TN];   // after cols_issue: ct = bias, cs = gamma
+    f32x4 vr[TN], mu[TN], bb[TN];
+    bool ok = false, bn = false;
+};
+
+template <class C>
+__device__ __forceinline__ bool vec_store_ok(const Epilogue& e, const float* Cout, long n0, int wn, long N) {
+    return n0 + (wn + 1) * C::WTN <= N && !e.out_nchw && e.beta == 0.f && (e.ldc & 3) == 0 && aligned16_dev(Cout) &&
+           (!e.bias || aligned16_dev(e.bias)) &&
+           (!e.bn_scale || (aligned16_dev(e.bn_scale) && aligned16_dev(e.bn_var) && aligned16_dev(e.bn_mean) &&
+                            aligned16_dev(e.bn_bias))) &&
+           (!e.residual || ((e.ldr & 3) == 0 && aligned16_dev(e.residual)));
+}
+
+template <class C>
+__device__ __forceinline__ void cols_issue(ColConsts<C::TN>& cc, const Epilogue& e, const float* Cout, long n0, int wn,
+                                           int lane, long N) {
+    cc.ok = vec_store_ok<C>(e, Cout, n0, wn, N);
+    cc.bn = e.bn_scale != nullptr;
+    if (!cc.ok) return;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+        const long col = n0 + wn * C::WTN + j * 32 + (lane & 7) * 4;
+        cc.ct[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        cc.cs[j] = f32x4{1.f, 1.f, 1.f, 1.f};
+        if (e.bias) cc.ct[j] = *reinterpret_cast<const f32x4*>(e.bias + col);
+        if (cc.bn) {
+            cc.cs[j] = *reinterpret_cast<const f32x4*>(e.bn_scale + col);
+            cc.vr[j] = *reinterpret_cast<const f32x4*>(e.bn_var + col);
+            cc.mu[j] = *reinterpret_cast<const f32x4*>(e.bn_mean + col);
+            cc.bb[j] = *reinterpret_cast<const f32x4*>(e.bn_bias + col);
+        }
+    }
+}
+
+template <class C>
+__device__ __forceinline__ void cols_fold(ColConsts<C::TN>& cc, const Epilogue& e) {
+    if (!cc.ok || !cc.bn) return;
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {  // same arithmetic as epilogue_column
+            const float inv = 1.0f / sqrtf(cc.vr[j][c] + e.bn_eps);
+            const float gg = cc.cs[j][c] * inv;
+            const float b = cc.ct[j][c];
+            cc.cs[j][c] = gg;
+            cc.ct[j][c] = (b - cc.mu[j][c]) * gg + cc.bb[j][c];
+        }
+}
+
 // Vector form of the accumulator write-out for the common case: row-major output with 16-byte
 // aligned rows, no beta term, whole 32-column blocks in range.  Each 32x32 block goes through the
 // wavefront's LDS staging block and comes back transposed to "four consecutive columns per
 // lane", so one step writes eight rows with 128-bit stores (4 steps per block instead of 16 with
-// 32-bit stores).  The loop body has no conditional load: a load under a branch makes the
-// compiler wait for every outstanding memory operation at the join, stores of the previous step
-// included, which serialised the old loop on the store round trip.  RES: add a residual tensor
+// 32-bit stores).  The four steps are straight-line code with the activation fixed at compile time:
+// no load sits under a branch (that makes the compiler wait for every outstanding memory operation
+// at the join, stores included) and no branch is taken per element.  RES: add a residual tensor
 // (rows clamped for the load, the store is predicated).  RAW: split-K partial sums, no epilogue.
-template <class C, bool RES, bool RAW>
-__device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
-                                               long M, float* __restrict__ out, long pitch, const Epilogue& e,
-                                               float* __restrict__ stage) {
+template <class C, bool RES, bool RAW, int ACT>
+__device__ __forceinline__ void store_tile_rows(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
+                                                long M, float* __restrict__ out, long pitch, const Epilogue& e,
+                                                float* __restrict__ stage, const ColConsts<C::TN>& cc) {
     const int r = lane & 31;
     const int h = lane >> 5;
     const int cq = (lane & 7) * 4;  // this lane's four columns within the block
     const int rq = lane >> 3;       // and its row within each group of eight
-    const bool colvec = !RAW && (!e.bias || aligned16_dev(e.bias)) &&
-                        (!e.bn_scale || (aligned16_dev(e.bn_scale) && aligned16_dev(e.bn_var) && aligned16_dev(e.bn_mean) &&
-                                         aligned16_dev(e.bn_bias)));
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) {
         const long col = n0 + wn * C::WTN + j * 32 + cq;
-        float cs[4] = {1.f, 1.f, 1.f, 1.f}, ct[4] = {0.f, 0.f, 0.f, 0.f};
-        if (!RAW) {
-            if (colvec) {
-                // the constants of the four columns as vectors: one round trip for the bias and one for the
-                // four batch-norm arrays, instead of one per scalar load under its own branch
-                f32x4 b = {0.f, 0.f, 0.f, 0.f};
-                if (e.bias) b = *reinterpret_cast<const f32x4*>(e.bias + col);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) ct[c] = b[c];
-                if (e.bn_scale) {
-                    const f32x4 g = *reinterpret_cast<const f32x4*>(e.bn_scale + col);
-                    const f32x4 vr = *reinterpret_cast<const f32x4*>(e.bn_var + col);
-                    const f32x4 mu = *reinterpret_cast<const f32x4*>(e.bn_mean + col);
-                    const f32x4 bb = *reinterpret_cast<const f32x4*>(e.bn_bias + col);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {  // same arithmetic as epilogue_column
-                        const float inv = 1.0f / sqrtf(vr[c] + e.bn_eps);
-                        const float gg = g[c] * inv;
-                        cs[c] = gg;
-                        ct[c] = (b[c] - mu[c]) * gg + bb[c];
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) epilogue_column(e, col + c, cs[c], ct[c]);
-            }
-        }
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) stage[((v >> 2) * 8 + h * 4 + (v & 3)) * 32 + r] = acc[i][j][v];
             wave_lds_sync();
             const long row0 = m0 + wm * C::WTM + i * 32 + rq;
-#pragma unroll 1
+            f32x4 x[4], res[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                x[it] = *reinterpret_cast<const f32x4*>(stage + (it * 8 + rq) * 32 + cq);
+                if (RES) {
+                    const long row = row0 + it * 8;
+                    const long rr = row < M ? row : M - 1;
+                    res[it] = *reinterpret_cast<const f32x4*>(e.residual + rr * e.ldr + col);
+                }
+            }
+#pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const long row = row0 + it * 8;
-                f32x4 x = *reinterpret_cast<const f32x4*>(stage + (it * 8 + rq) * 32 + cq);
-                f32x4 res;
-                if (RES) {
-                    const long rr = row < M ? row : M - 1;
-                    res = *reinterpret_cast<const f32x4*>(e.residual + rr * e.ldr + col);
-                }
                 if (!RAW) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        float y = x[c] * e.alpha;
-                        y = y * cs[c] + ct[c];
-                        if (RES) y += res[c];
-                        x[c] = apply_act(y, e.act);
+                        float y = x[it][c] * e.alpha;
+                        y = y * cc.cs[j][c] + cc.ct[j][c];
+                        if (RES) y += res[it][c];
+                        x[it][c] = act_fixed<ACT>(y);
                     }
                 }
-                if (row < M) *reinterpret_cast<f32x4*>(out + row * pitch + col) = x;
+                if (row < M) *reinterpret_cast<f32x4*>(out + row * pitch + col) = x[it];
             }
             wave_lds_sync();
         }
+    }
+}
+
+template <class C, bool RES, bool RAW>
+__device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
+                                               long M, float* __restrict__ out, long pitch, const Epilogue& e,
+                                               float* __restrict__ stage, const ColConsts<C::TN>& cc) {
+    if (RAW) {
+        store_tile_rows<C, false, true, ACT_NONE>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc);
+        return;
+    }
+    switch (e.act) {
+        case ACT_RELU: store_tile_rows<C, RES, false, ACT_RELU>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        case ACT_GELU: store_tile_rows<C, RES, false, ACT_GELU>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        case ACT_TANH: store_tile_rows<C, RES, false, ACT_TANH>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        case ACT_RELU6: store_tile_rows<C, RES, false, ACT_RELU6>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        case ACT_SILU: store_tile_rows<C, RES, false, ACT_SILU>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        case ACT_SIGMOID: store_tile_rows<C, RES, false, ACT_SIGMOID>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
+        default: store_tile_rows<C, RES, false, ACT_NONE>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
     }
 }
 
@@ -366,24 +455,29 @@ __device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int 
 template <class C>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
                                            long M, long N, float* __restrict__ Cout, const Epilogue& e,
-                                           float* __restrict__ partial, float* __restrict__ stage) {
+                                           float* __restrict__ partial, float* __restrict__ stage,
+                                           const ColConsts<C::TN>* pre = nullptr) {
     const int r = lane & 31;
     const int h = lane >> 5;
     if (n0 + (wn + 1) * C::WTN <= N) {  // the same for every lane of the wavefront
         if (partial) {
             if ((N & 3) == 0 && aligned16_dev(partial)) {
-                store_tile_vec<C, false, true>(acc, wm, wn, lane, m0, n0, M, partial, N, e, stage);
+                ColConsts<C::TN> none;
+                store_tile_vec<C, false, true>(acc, wm, wn, lane, m0, n0, M, partial, N, e, stage, none);
                 return;
             }
-        } else if (!e.out_nchw && e.beta == 0.f && (e.ldc & 3) == 0 && aligned16_dev(Cout)) {
-            if (!e.residual) {
-                store_tile_vec<C, false, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage);
-                return;
+        } else if (pre ? pre->ok : vec_store_ok<C>(e, Cout, n0, wn, N)) {
+            ColConsts<C::TN> own;
+            if (!pre) {  // the kernel did not fetch them ahead: fetch and fold here
+                cols_issue<C>(own, e, Cout, n0, wn, lane, N);
+                cols_fold<C>(own, e);
+                pre = &own;
             }
-            if ((e.ldr & 3) == 0 && aligned16_dev(e.residual)) {
-                store_tile_vec<C, true, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage);
-                return;
-            }
+            if (!e.residual)
+                store_tile_vec<C, false, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage, *pre);
+            else
+                store_tile_vec<C, true, false>(acc, wm, wn, lane, m0, n0, M, Cout, e.ldc, e, stage, *pre);
+            return;
         }
     }
 #pragma unroll
