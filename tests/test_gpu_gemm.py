@@ -21,9 +21,9 @@ def _rand(rng, *shape):
     (1536, 1024, 1024, "gemm_fast_64x32_kc"),   # BERT-large projection: 384 64x64 tiles = 1.5 per CU -> 64x32
     (1536, 1024, 4096, "gemm_fast_64x32_kc"),   # BERT-large FFN down-projection
     (4096, 2048, 160, "gemm_fast_64x64_kc"),    # K % 64 != 0: predicated kernel
-    (1, 1000, 2048, "gemm_fast_64x64_kc"),      # ResNet classifier, batch 1 (split-K)
+    (1, 1000, 2048, "gemm_fast_32x32_kc"),      # ResNet classifier, batch 1: 32 small tiles, K split over 8 workgroups each
     (1568, 256, 1024, "gemm_fast_32x32_kc"),    # ResNet-152 batch 8 layer3 1x1: 100 64x64 tiles -> 32x32, K split in the workgroup
-    (49, 512, 2048, "gemm_fast_64x64_kc"),      # ragged M
+    (49, 512, 2048, "gemm_fast_32x32_kc"),      # ragged M (ResNet-50 batch 1, 7x7 pixels)
     (100, 37, 52, "gemm_fast_64x64_kc"),        # ragged N, K % 32 != 0
     (33, 65, 7, "gemm_generic_64x64"),          # K % 4 != 0 -> scalar path
 ])

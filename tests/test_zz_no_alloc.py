@@ -41,8 +41,9 @@ def test_no_alloc_gemm_matches_tp_gemm_twice_in_a_row():
     torch.cuda.set_device(0)
     stream = torch.cuda.Stream()
     rng = np.random.default_rng(11)
-    # both shapes split K over workgroups (fewer 64x64 tiles than CUs, long K): the scratch array is used
-    shapes = [(128, 768, 3072, ACT_RELU), (1, 1000, 2048, 0), (64, 256, 1024, 0)]
+    # every shape splits K over workgroups (few output tiles, long K): the scratch array is used -- by 32x32
+    # tiles whose slots are summed inside the launch, and (K not a multiple of 128) by 64x64 tiles
+    shapes = [(128, 768, 3072, ACT_RELU), (96, 200, 1056, 0), (1, 1000, 2048, 0), (64, 256, 1024, 0)]
     cases = []
     for M, N, K, act in shapes:
         X = rng.standard_normal((M, K)).astype(np.float32)
@@ -51,7 +52,7 @@ def test_no_alloc_gemm_matches_tp_gemm_twice_in_a_row():
         cases.append((X, W, b, M, N, K, act))
     with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
         want = [_through_engine(s, *c) for c in cases]
-    assert any("64x64" in k for _, k in want), [k for _, k in want]   # a split-over-workgroups kernel ran
+    assert any("64x64" in k for _, k in want) and any("32x32" in k for _, k in want), [k for _, k in want]
     for c, (ref, kernel) in zip(cases, want):   # largest first: later calls see stale partial sums
         print("case", c[3:], kernel, flush=True)
         got = _no_alloc(torch, *c, stream)

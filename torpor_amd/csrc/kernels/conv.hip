@@ -20,7 +20,7 @@ void set_last_kernel(const char* n);
 int num_cu();
 Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
 int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, const Epilogue& e, hipStream_t s);
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out);
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32);
 unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
 
 struct ConvDev {
@@ -584,6 +584,16 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         int cfg = tl >= 2L * num_cu() ? 0 : 1;
         if (cfg == 1 && t64 >= num_cu() / 2 && t64 < num_cu()) cfg = 2;
         if (cfg == 1 && t64 < num_cu() / 4 && t32 >= num_cu() / 2 && a.Cin <= 128) cfg = 3;
+        // Few 64x64 tiles (batch 1): 32x32 tiles with nine K slices, split over channel blocks as well
+        // when even those leave CUs idle -- up to eight slots, summed inside the launch.  Its workgroups
+        // are short-lived, where a 64x64 tile with a deep split pays a long serial chain per wavefront
+        // and a reduction launch.  TORPOR_CONV3_SMALL=0 restores the old rule, =n moves the bound to
+        // t64 < n.
+        static const int small_bound = getenv("TORPOR_CONV3_SMALL") ? atoi(getenv("TORPOR_CONV3_SMALL")) : num_cu() / 4;
+        // (only where the launch is bound by latency, not by matrix work: ResNet-152 batch 8, 392 pixels x 512
+        // channels, 1.85 GFLOP, runs 56 us this way against 30 us as 64x64 tiles)
+        const bool small = cfg == 1 && t64 < small_bound && 2.0 * (double)M * a.Cout * (double)p.K < 6.0e8;
+        if (small) cfg = 3;
         if (forced >= 0 && forced <= 4) cfg = forced;
         const int bm = cfg == 0 ? 128 : cfg <= 2 ? 64 : 32;
         p.tiles_m = (int)((M + bm - 1) / bm);
@@ -593,6 +603,7 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         long kper_k = p.K;
         p.splits = 1;
         if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k);
+        if (cfg == 3) p.splits = choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, 8);
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);

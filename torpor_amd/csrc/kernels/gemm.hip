@@ -437,137 +437,6 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     TP_CLK(4);
 }
 
-// The branch-free kernel for grids that leave a CU with one or two workgroups: there nothing hides the
-// memory latency of a K-block but the workgroup's own look-ahead, and two K-blocks ahead (a few hundred
-// cycles of matrix work) is far less than a round trip to memory.  D register sets keep D K-blocks in
-// flight per workgroup; block b travels through set b % D and LDS stage b & 1, one barrier per block.
-// Same preconditions as gemm_clean_kernel (whole K-blocks, clamped edges); any number of K-blocks.
-template <class C, bool YKC, int D>
-__global__ __launch_bounds__(C::THREADS, 1) void gemm_deep_kernel(const GemmDev p) {
-    fetch_now(p);
-    static_assert(D >= 2 && D % 2 == 0, "the LDS stage of a block must follow from its register set");
-    constexpr int RED_FLOATS = red_floats<C>();
-    __shared__ __attribute__((aligned(16))) float lds[cmax(2 * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
-    const int wm = wsp / C::WGN, wn = wsp % C::WGN;
-    int tm, tn, t;
-    if (!tile_of(p, blockIdx.x, &tm, &tn, &t)) return;
-    const long m0 = (long)tm * C::BM, n0 = (long)tn * C::BN;
-    int split = 0, batch = blockIdx.z;
-    if (p.splits > 1) {
-        split = blockIdx.z;
-        batch = 0;
-    }
-    const int b0 = batch / p.nb1, b1 = batch - b0 * p.nb1;
-    const float* __restrict__ X = p.X + b0 * p.xb0 + b1 * p.xb1;
-    const float* __restrict__ Y = p.Y + b0 * p.yb0 + b1 * p.yb1;
-    float* __restrict__ Cc = p.C + b0 * p.cb0 + b1 * p.cb1;
-    const long kbeg = (long)split * p.kper;
-    const long kend = (kbeg + p.kper < p.K) ? kbeg + p.kper : p.K;
-    const int nb = (int)((kend - kbeg) / C::BK);  // whole K-blocks of this workgroup
-    ColConsts<C::TN> cc;
-    if (wk == 0) cols_issue<C>(cc, p.ep, Cc, n0, wn, lane, p.N);
-
-    constexpr int KV = C::BK / 4;
-    constexpr int CV = C::BN / 4;
-    constexpr int NVA = C::BM * KV / C::THREADS;
-    constexpr int NVB = (YKC ? C::BN * KV : C::BK * CV) / C::THREADS;
-    static_assert(C::BM * KV % C::THREADS == 0 && C::BN * KV % C::THREADS == 0 && C::BK * CV % C::THREADS == 0,
-                  "tile must split evenly over the workgroup");
-    const float* pa[NVA];
-    const float* pb[NVB];
-    int sa[NVA], sb[NVB];
-#pragma unroll
-    for (int i = 0; i < NVA; ++i) {
-        const int idx = i * C::THREADS + tid;
-        const int row = idx / KV, kq = idx - row * KV;
-        long grow = m0 + row;
-        if (grow > p.M - 1) grow = p.M - 1;
-        pa[i] = X + gather_row(p, grow) * p.xs_r + kq * 4 + kbeg;
-        sa[i] = row * C::LDK + kq * 4;
-    }
-    const long ystep = YKC ? 1 : p.ys_k;
-#pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-        const int idx = i * C::THREADS + tid;
-        if (YKC) {
-            const int col = idx / KV, kq = idx - col * KV;
-            long gcol = n0 + col;
-            if (gcol > p.N - 1) gcol = p.N - 1;
-            pb[i] = Y + gcol * p.ys_c + kq * 4 + kbeg;
-            sb[i] = col * C::LDK + kq * 4;
-        } else {
-            const int kk = idx / CV, cq = idx - kk * CV;
-            long gcol = n0 + cq * 4;
-            if (gcol > p.N - 4) gcol = p.N - 4;
-            pb[i] = Y + (kk + kbeg) * p.ys_k + gcol;
-            sb[i] = (cq * 4) * C::LDK + kk;
-        }
-    }
-
-    f32x16 acc[C::TM][C::TN];
-    zero_acc<C>(acc);
-    f32x4 ra[D][NVA], rb[D][NVB];
-    auto load_regs = [&](int set, int b) {  // K-block b of this workgroup into register set `set`
-        const long k = (long)b * C::BK;
-#pragma unroll
-        for (int i = 0; i < NVA; ++i) ra[set][i] = *reinterpret_cast<const f32x4*>(pa[i] + k);
-#pragma unroll
-        for (int i = 0; i < NVB; ++i) rb[set][i] = *reinterpret_cast<const f32x4*>(pb[i] + k * ystep);
-    };
-    auto store_lds = [&](int set, int stage) {
-        float* As = lds + stage * C::LDS_FLOATS;
-        float* Bs = As + C::BM * C::LDK;
-#pragma unroll
-        for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[set][i];
-#pragma unroll
-        for (int i = 0; i < NVB; ++i) {
-            if (YKC) {
-                *reinterpret_cast<f32x4*>(Bs + sb[i]) = rb[set][i];
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) Bs[sb[i] + j * C::LDK] = rb[set][i][j];
-            }
-        }
-    };
-    // one K-block: refill the set that block b left, multiply block b, move block b + 1 into the other stage
-    auto phase = [&](int d, int b) {
-        if (b + D < nb) load_regs(d, b + D);
-        const float* As = lds + (d & 1) * C::LDS_FLOATS;
-        mma_block<C>(As, As + C::BM * C::LDK, acc, wm, wn, lane, wk);
-        if (b + 1 < nb) store_lds((d + 1) % D, (d + 1) & 1);
-        __syncthreads();
-    };
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-        if (d < nb) load_regs(d, d);
-    if (wk == 0) cols_fold<C>(cc, p.ep);
-    store_lds(0, 0);
-    __syncthreads();
-    int b = 0;
-    for (; b + D <= nb; b += D) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) phase(d, b + d);
-    }
-#pragma unroll
-    for (int d = 0; d < D - 1; ++d)
-        if (b + d < nb) phase(d, b + d);
-
-    if (!reduce_k_slices<C>(acc, lds, wk, wsp, lane)) return;
-    float* partial = nullptr;
-    if (p.splits > 1) {
-        if (p.tickets) {
-            if (!finish_split<C>(acc, p.ws, p.tickets, p.splits, t, split, wsp, lane,
-                                 reinterpret_cast<unsigned*>(lds + RED_FLOATS + stage_floats<C>())))
-                return;
-        } else {
-            partial = p.ws + (long)split * p.M * p.N;
-        }
-    }
-    store_tile<C>(acc, wm, wn, lane, m0, n0, p.M, p.N, Cc, p.ep, partial, lds + RED_FLOATS + wsp * STAGE_BLOCK, &cc);
-}
-
 // Any strides, any alignment.  64x64x16 tile, scalar loads.
 using GenCfg = TileCfg<64, 64, 16, 2, 2>;
 
@@ -790,15 +659,6 @@ static int launch_clean_only(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t
     return 2;
 }
 
-// The deep look-ahead kernel (gemm_deep_kernel) for grids of at most two workgroups per CU.
-template <class C>
-static void launch_deep(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t s) {
-    if (y_kc)
-        hipLaunchKernelGGL((gemm_deep_kernel<C, true, 6>), grid, dim3(C::THREADS), 0, s, p);
-    else
-        hipLaunchKernelGGL((gemm_deep_kernel<C, false, 6>), grid, dim3(C::THREADS), 0, s, p);
-}
-
 // Tile shape.  Measured on MI355X over the served shapes (BERT-large 1536 x {1024,4096} x
 // {1024,4096}, ResNet 1x1 convolutions from 25088x256x64 to 392x2048x512), the 64x64 tile is
 // the fastest everywhere: it keeps the most workgroups resident per CU, and for fp32 MFMA
@@ -825,14 +685,17 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
         const double r32 = 0.5 * (double)((t32 + g_num_cu - 1) / g_num_cu);
         if (r32 <= 0.8 * r64) return 3;
     }
-    // Fewer 64x64 tiles than CUs: rather than splitting K across workgroups (partial sums through
-    // memory plus a reduction launch), quarter the tile and split K inside the workgroup.
+    // Fewer 64x64 tiles than CUs: quarter the tile and split each K-block over its four wavefronts
+    // (1568x256x1024: 22.4 -> 16.0 us against a split over workgroups).  A long K with few of these small
+    // tiles is split over workgroups as well (plan_gemm): up to eight slots are summed inside the launch, and
+    // a workgroup of this shape is short-lived -- 128x768x3072 runs 96 tiles x 6 slots instead of 24 tiles of
+    // 64x64 x 16 slots and a reduction launch.  TORPOR_GEMM_SMALL=0 restores the old rule for comparison.
+    static const bool small_split = getenv("TORPOR_GEMM_SMALL") == nullptr || atoi(getenv("TORPOR_GEMM_SMALL")) != 0;
     const long t3232 = ((M + 31) / 32) * ((N + 31) / 32) * batch;
-    // (with less than one small tile per CU a long K still wants the split over workgroups:
-    // 128x768x3072 runs 19 us that way, 23 us as 96 tiles of 32x32)
-    if (batch == 1 && K >= 256 && K % 128 == 0 && t64 < g_num_cu && t3232 >= 3 * g_num_cu / 8 &&
-        (t3232 >= g_num_cu || K <= 1024))
-        return 4;
+    if (batch == 1 && K >= 256 && K % 128 == 0 && t64 < g_num_cu) {
+        if (small_split) return 4;
+        if (t3232 >= 3 * g_num_cu / 8 && (t3232 >= g_num_cu || K <= 1024)) return 4;
+    }
     return 2;
 }
 
@@ -854,7 +717,7 @@ unsigned* split_tickets(const Workspace& ws, long tiles, int splits) {
 
 // One split's partial sums are `tiles` whole output tiles of tile_floats each (the in-launch summation
 // keeps them per tile and per wavefront; the two-launch form needs no more than that).
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out) {
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32) {
     int splits = 1;
     const long kblocks = (K + bk - 1) / bk;
     const size_t per = (size_t)tiles * (size_t)tile_floats * sizeof(float);
@@ -865,7 +728,7 @@ int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes,
         long want = (2L * g_num_cu + tiles - 1) / tiles;
         long maxs = kblocks / 4;  // keep at least 4 K-blocks per split
         if (want > maxs) want = maxs;
-        if (want > 32) want = 32;
+        if (want > max_splits) want = max_splits;
         while (want > 1 && (size_t)want * per > ws_bytes) --want;
         if (want > 1) splits = (int)want;
     }
@@ -905,6 +768,9 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
         const long tiles = (long)g.tiles_m * g.tiles_n * batch;
         g.kper = ((a.K + 31) / 32) * 32;
         if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, (long)g.bm * g.bn, ws_bytes, &g.kper);
+        // (with more than half a tile per CU the split does not pay: 196x1024x512, 224 tiles, 8.5 against 7.4 us)
+        if (batch == 1 && cfg == 4 && tiles <= g_num_cu / 2)
+            g.splits = choose_splits(tiles, a.K, 64, 32 * 32, ws_bytes, &g.kper, /*max_splits=*/8);
     } else {
         g.tiles_m = (int)((a.M + 63) / 64);
         g.tiles_n = (int)((a.N + 63) / 64);
@@ -979,32 +845,19 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
-        static const char* const names[5][2][4] = {
-            {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2", ""},
-             {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2", ""}},
-            {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2", ""},
-             {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2", ""}},
-            {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2", "gemm_fast_64x64_cc_d6"},
-             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2", "gemm_fast_64x64_kc_d6"}},
-            {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2", "gemm_fast_64x32_cc_d6"},
-             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2", "gemm_fast_64x32_kc_d6"}},
-            {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2", "gemm_fast_32x32_cc_d6"},
-             {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2", "gemm_fast_32x32_kc_d6"}}};
-        // _d6: six K-blocks in flight per workgroup, for grids that leave a CU at most two workgroups
-        // (TORPOR_GEMM_DEEP=0 switches it off, =n moves the bound to n workgroups per CU)
-        static const int deep_per_cu = getenv("TORPOR_GEMM_DEEP") ? atoi(getenv("TORPOR_GEMM_DEEP")) : 2;
-        const long wgs = (long)p.tiles_m * p.tiles_n * grid.z;
-        const bool deep = clean && cfg >= 2 && deep_per_cu > 0 && wgs <= (long)deep_per_cu * g_num_cu;
+        static const char* const names[5][2][3] = {
+            {{"gemm_fast_128x128_cc", "gemm_fast_128x128_cc_s1", "gemm_fast_128x128_cc_s2"},
+             {"gemm_fast_128x128_kc", "gemm_fast_128x128_kc_s1", "gemm_fast_128x128_kc_s2"}},
+            {{"gemm_fast_128x64_cc", "gemm_fast_128x64_cc_s1", "gemm_fast_128x64_cc_s2"},
+             {"gemm_fast_128x64_kc", "gemm_fast_128x64_kc_s1", "gemm_fast_128x64_kc_s2"}},
+            {{"gemm_fast_64x64_cc", "gemm_fast_64x64_cc_s1", "gemm_fast_64x64_cc_s2"},
+             {"gemm_fast_64x64_kc", "gemm_fast_64x64_kc_s1", "gemm_fast_64x64_kc_s2"}},
+            {{"gemm_fast_64x32_cc", "gemm_fast_64x32_cc_s1", "gemm_fast_64x32_cc_s2"},
+             {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}},
+            {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2"},
+             {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2"}}};
         int variant;
-        if (deep) {
-            if (cfg == 2)
-                launch_deep<CfgM>(p, y_kc, grid, s);
-            else if (cfg == 3)
-                launch_deep<CfgS>(p, y_kc, grid, s);
-            else
-                launch_deep<CfgT>(p, y_kc, grid, s);
-            variant = 3;
-        } else if (cfg == 0)
+        if (cfg == 0)
             variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
         else if (cfg == 1)
             variant = launch_fast<CfgW>(p, y_kc, clean, grid, s);
