@@ -56,16 +56,26 @@ EXTRA_WORKLOADS = {
     "efficientnet-b0-b1": ("efficientnet", "efficientnet_b0", 1, None),
     "inception-v3-b1": ("inception", "inception_v3", 1, None),
     "bert-large-qa-b1-s512": ("bert-qa", "bert-large", 1, 512),   # the reference endpoint's own call
+    "vgg16-b1": ("vgg", "vgg16", 1, None),
+    "squeezenet1_1-b1": ("squeezenet", "squeezenet1_1", 1, None),
 }
 
 
 def make_function(server, fid, name, seed=0):
     import torch
-    from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet
+    from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet, squeezenet, vgg
 
     family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     g = torch.Generator().manual_seed(0)
-    if family == "densenet":
+    if family == "vgg":
+        weights = vgg.init_weights(seed=seed)
+        fn = vgg.VGG16(server, fid, batch=batch, weights=weights)
+        inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
+    elif family == "squeezenet":
+        weights = squeezenet.init_weights(seed=seed)
+        fn = squeezenet.SqueezeNet11(server, fid, batch=batch, weights=weights)
+        inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
+    elif family == "densenet":
         weights = densenet.init_weights(arch, seed=seed)
         fn = densenet.DenseNet(server, fid, arch, batch=batch, weights=weights)
         inputs = [torch.randn(batch, 3, 224, 224, generator=g).numpy()]
@@ -263,8 +273,9 @@ def cpu_baseline(name, weights, inputs, first):
     family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
     cores = int(os.environ.get("OMP_NUM_THREADS") or torch.get_num_threads())
     torch.set_num_threads(cores)
-    if family in ("resnet", "densenet", "mobilenet", "efficientnet", "inception"):
+    if family in ("resnet", "densenet", "mobilenet", "efficientnet", "inception", "vgg", "squeezenet"):
         net = {"resnet": lambda: om.ResNet(arch), "densenet": lambda: om.DenseNet(arch),
+               "vgg": lambda: om.VGG16(), "squeezenet": lambda: om.SqueezeNet11(),
                "mobilenet": lambda: om.MobileNetV2(), "efficientnet": lambda: om.EfficientNetB0(),
                "inception": lambda: om.InceptionV3()}[family]()
         model = om.load_numpy_state(net, weights)

@@ -45,7 +45,12 @@ typedef struct tp_server tp_server;
 #define TP_ENOTACTIVE (-72)    /* client id is not the active function */
 #define TP_EUNSUPPORTED (-38)  /* shape / option not implemented */
 #define TP_EFAULT (-14)        /* virtual address does not translate */
+#define TP_ERANGE (-34)        /* function id above TP_MAX_FUNCTION_ID */
 #define TP_ESCRATCH (-75)      /* the call needs more scratch memory than tp_gemm_noalloc's fixed buffer holds */
+
+/* Function ids are decimal strings, as in the reference (stoi(func), cuda_server.hpp:221-224), in
+ * 0 .. TP_MAX_FUNCTION_ID: the id is part of every virtual address handed to the function. */
+#define TP_MAX_FUNCTION_ID 65535
 
 /* ---- signal.proto enums (proto/signal.proto:5-30) ---- */
 #define TP_REQ_EXECUTE_AFTER_LOAD 0 /* register model */

@@ -448,6 +448,64 @@ class InceptionV3(nn.Module):
         return self.fc(x.mean((2, 3)))
 
 
+VGG16_CFG = (64, 64, "M", 128, 128, "M", 256, 256, 256, "M", 512, 512, 512, "M", 512, 512, 512, "M")
+
+
+class VGG16(nn.Module):
+    """VGG-16 (configuration D of Simonyan & Zisserman 2014) with torchvision's module names:
+    3x3 convolutions with bias + ReLU, 2x2 max-pooling, three fully connected layers on the
+    channel-major flattening of the 512 x 7 x 7 map.  Served by the reference (tests/endpoint.py:26-27)."""
+
+    def __init__(self, num_classes=1000):
+        super().__init__()
+        layers, cin = [], 3
+        for v in VGG16_CFG:
+            if v == "M":
+                layers.append(nn.MaxPool2d(2, 2))
+            else:
+                layers += [nn.Conv2d(cin, v, 3, padding=1), nn.ReLU(inplace=True)]
+                cin = v
+        self.features = nn.Sequential(*layers)
+        self.classifier = nn.Sequential(nn.Linear(512 * 7 * 7, 4096), nn.ReLU(True), nn.Dropout(),
+                                        nn.Linear(4096, 4096), nn.ReLU(True), nn.Dropout(), nn.Linear(4096, num_classes))
+
+    def forward(self, x):
+        x = F.adaptive_avg_pool2d(self.features(x), 7)
+        return self.classifier(torch.flatten(x, 1))
+
+
+class _Fire(nn.Module):
+    def __init__(self, cin, squeeze, e1, e3):
+        super().__init__()
+        self.squeeze = nn.Conv2d(cin, squeeze, 1)
+        self.expand1x1 = nn.Conv2d(squeeze, e1, 1)
+        self.expand3x3 = nn.Conv2d(squeeze, e3, 3, padding=1)
+
+    def forward(self, x):
+        x = F.relu(self.squeeze(x))
+        return torch.cat([F.relu(self.expand1x1(x)), F.relu(self.expand3x3(x))], 1)
+
+
+class SqueezeNet11(nn.Module):
+    """SqueezeNet 1.1 (Iandola et al. 2016, the lighter revision) with torchvision's module names: a 3x3
+    stride-2 stem, eight fire modules (1x1 squeeze, then 1x1 and 3x3 expansions side by side), three
+    3x3 stride-2 max-poolings that keep a partial last window (ceil mode), a 1x1 classifier convolution
+    and a global average.  Served by the reference (tests/endpoint.py:20-21)."""
+
+    def __init__(self, num_classes=1000):
+        super().__init__()
+        self.features = nn.Sequential(
+            nn.Conv2d(3, 64, 3, stride=2), nn.ReLU(inplace=True), nn.MaxPool2d(3, 2, ceil_mode=True),
+            _Fire(64, 16, 64, 64), _Fire(128, 16, 64, 64), nn.MaxPool2d(3, 2, ceil_mode=True),
+            _Fire(128, 32, 128, 128), _Fire(256, 32, 128, 128), nn.MaxPool2d(3, 2, ceil_mode=True),
+            _Fire(256, 48, 192, 192), _Fire(384, 48, 192, 192), _Fire(384, 64, 256, 256), _Fire(512, 64, 256, 256))
+        self.classifier = nn.Sequential(nn.Dropout(), nn.Conv2d(512, num_classes, 1), nn.ReLU(inplace=True),
+                                        nn.AdaptiveAvgPool2d(1))
+
+    def forward(self, x):
+        return torch.flatten(self.classifier(self.features(x)), 1)
+
+
 def load_numpy_state(module, weights):
     """Strictly load a {name: np.ndarray} dict (BN `num_batches_tracked` buffers excepted)."""
     sd = {k: torch.from_numpy(v.copy()) for k, v in weights.items()}

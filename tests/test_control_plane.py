@@ -333,6 +333,9 @@ def test_default_topology_is_an_eight_gpu_all_to_all_node():
 
 
 # ------------------------------------------------------------ the engine's own victims vs the oracle
+_ACT_VA = {}   # function id -> address of its activation block
+
+
 def _tiny_function(s, fid, level, weight_mib):
     """Registers a function of `weight_mib` MiB of weights and one 1 KiB activation through the C-ABI of a
     host-only engine (no device): the LRU charges round_up(weights) + round_up(activations) slabs."""
@@ -349,6 +352,7 @@ def _tiny_function(s, fid, level, weight_mib):
         s.stream_synchronize(fid)
     except Exception:              # host-only: no data to deliver (-19)
         pass
+    _ACT_VA[fid] = a
     return s.model_info(fid)["total_bytes"]
 
 
@@ -442,8 +446,7 @@ def _finish(s, fid):
     """Ends the running request of `fid` the way a function does: one asynchronous device-to-host copy of
     its activation (the completion marker, cuda_server.hpp:1044) and the stream synchronisation."""
     from torpor_amd._lib import TorporError
-    va = (0x7A << 56) | (fid << 44) | (1 << 43)   # the function's first activation block
-    s.d2h_async(fid, np.empty(256, np.float32), va)
+    s.d2h_async(fid, np.empty(256, np.float32), _ACT_VA[fid])
     try:
         s.stream_synchronize(fid)
     except TorporError:

@@ -7,7 +7,7 @@ import torch
 
 from oracle import models as om
 from tests.harness import assert_close
-from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet
+from torpor_amd.functions import bert, densenet, efficientnet, inception, mobilenet, resnet, squeezenet, vgg
 
 pytestmark = pytest.mark.gpu
 LOGIT_RTOL = 1e-3   # north-star bar: rel 1e-3 (fp32) on logits
@@ -154,7 +154,7 @@ def test_resnet101(gpu_server):
     fn.unload()
 
 
-@pytest.mark.parametrize("arch,image,batch", [("densenet121", 64, 2), ("densenet169", 224, 1)])
+@pytest.mark.parametrize("arch,image,batch", [("densenet121", 64, 2), ("densenet169", 224, 1), ("densenet201", 224, 1)])
 def test_densenet(gpu_server, arch, image, batch):
     """DenseNet (served by the reference, tests/endpoint.py:20-23): dense blocks built in place in one
     wide buffer (pitched batch-norm input, convolution output into a channel slice)."""
@@ -219,6 +219,73 @@ def test_inception_v3(gpu_server, image, batch):
         want = model(torch.from_numpy(x)).numpy()
     e = assert_close(logits, want, LOGIT_RTOL, "inception_v3 logits")
     print(f"inception_v3 b{batch} {image}px: rel err {e:.2e}")
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+def test_bert_large_question_answering_at_the_endpoints_size(gpu_server):
+    """The reference endpoint's own BERT call at full size (tests/endpoint.py:36-40,52-57): BERT-large with
+    the span head, batch 1, 512 tokens, token type ids."""
+    arch, B, S = "bert-large", 1, 512
+    weights = bert.init_weights(arch, seed=3, qa_head=True)
+    g = torch.Generator().manual_seed(21)
+    ids = torch.randint(0, 30522, (B, S), generator=g).numpy()
+    tt = torch.randint(0, 2, (B, S), generator=g).numpy()
+    fn = bert.Bert(gpu_server, 17, arch, batch=B, seq=S, weights=weights, token_types=True)
+    start, end = fn.register([ids, tt])
+    model = om.load_numpy_state(om.Bert(qa_head=True, **bert.CONFIGS[arch]), weights)
+    with torch.no_grad():
+        want_s, want_e = model(torch.from_numpy(ids), torch.from_numpy(tt))
+    assert start.shape == (B, S) and end.shape == (B, S)
+    e1 = assert_close(start, want_s.numpy(), LOGIT_RTOL, "span start logits")
+    e2 = assert_close(end, want_e.numpy(), LOGIT_RTOL, "span end logits")
+    print(f"bert-large QA b{B} s{S}: rel err start {e1:.2e} end {e2:.2e}")
+    _check_swap_identity(gpu_server, fn, fn.weights())
+    _cycle(gpu_server, fn, [ids, tt], [start, end])
+    fn.unload()
+
+
+def test_vgg16(gpu_server):
+    """VGG-16 (tests/endpoint.py:26-27): 3x3 convolutions with bias, 2x2 max-pooling, 411 MB first fully
+    connected layer on the channel-major flattening."""
+    weights = vgg.init_weights(seed=18)
+    rng = np.random.default_rng(19)
+    for k in weights:   # non-zero biases, so that a dropped bias cannot pass
+        if k.endswith(".bias"):
+            weights[k] = (rng.standard_normal(weights[k].shape) * 0.05).astype(np.float32)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(20)).numpy()
+    fn = vgg.VGG16(gpu_server, 18, batch=1, weights=weights)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.VGG16(), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, "vgg16 logits")
+    print(f"vgg16 b1: rel err {e:.2e}")
+    assert gpu_server.model_info(18)["param_bytes"] == 4 * 138357544
+    _check_swap_identity(gpu_server, fn, weights)
+    _cycle(gpu_server, fn, [x], [logits])
+    fn.unload()
+
+
+@pytest.mark.parametrize("image,batch", [(96, 2), (224, 1)])
+def test_squeezenet11(gpu_server, image, batch):
+    """SqueezeNet 1.1 (tests/endpoint.py:20-21): fire modules whose two expansions write into the halves
+    of one buffer."""
+    weights = squeezenet.init_weights(seed=22)
+    rng = np.random.default_rng(23)
+    for k in weights:
+        if k.endswith(".bias"):
+            weights[k] = (rng.standard_normal(weights[k].shape) * 0.05).astype(np.float32)
+    weights["classifier.1.weight"] = (weights["classifier.1.weight"] * 5).astype(np.float32)   # logits of a visible size
+    x = torch.randn(batch, 3, image, image, generator=torch.Generator().manual_seed(24)).numpy()
+    fn = squeezenet.SqueezeNet11(gpu_server, 19, batch=batch, weights=weights, image=image)
+    (logits,) = fn.register([x])
+    model = om.load_numpy_state(om.SqueezeNet11(), weights)
+    with torch.no_grad():
+        want = model(torch.from_numpy(x)).numpy()
+    e = assert_close(logits, want, LOGIT_RTOL, "squeezenet1_1 logits")
+    print(f"squeezenet1_1 b{batch} {image}px: rel err {e:.2e}")
     _check_swap_identity(gpu_server, fn, weights)
     _cycle(gpu_server, fn, [x], [logits])
     fn.unload()

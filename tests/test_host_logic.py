@@ -503,6 +503,10 @@ def test_error_paths(host_server):
     assert s.signal(11, 1, "")[0] == ACK_INAVAIL                     # Replay signal is refused
     with pytest.raises(TorporError):
         s.signal(REQ_EXECUTE, "abc", "")                             # function must be a decimal id
+    with pytest.raises(TorporError) as e:
+        s.signal(REQ_EXECUTE_AFTER_LOAD, 65536, "1")                 # ids are 0 .. 65535
+    assert e.value.code == -34 and "range" in str(e.value)
+    assert s.signal(REQ_EXECUTE, 65535, "")[0] == ACK_INAVAIL        # in range, never registered
     with pytest.raises(TorporError):
         s.malloc(0, 16)                                              # no active function
     # registration: ops before the end of the upload phase are refused; uploads outside a block too
@@ -621,3 +625,12 @@ def test_deferred_acks_carry_tickets_and_can_be_cancelled():
         assert s.cancel_deferred(t4[3]) == 2        # ack dropped, the started request completed at once
         assert s.take_deferred_ack_ticket() is None
         assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)   # the executor is free again
+
+
+def test_function_ids_up_to_65535_register_and_run():
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20) as s:
+        fn = _register(s, 65535, seed=1)
+        assert s.model_info(65535)["registered"] == 1 and s.resident(65535)
+        assert (fn.w["conv1.weight"] >> 40) & 0xFFFF == 65535       # the id travels in every address
+        assert s.signal(REQ_UNLOAD, 65535, "")[0] == ACK_OK and not s.resident(65535)
+        assert s.signal(REQ_LOAD, 65535, "")[0] == ACK_OK and s.resident(65535)

@@ -260,3 +260,57 @@ def test_inception_v3_counts():
     assert widths == [256, 288, 288, 768, 768, 768, 768, 768, 1280, 2048, 2048] and x.shape[2:] == (8, 8)
     from torpor_amd.functions import inception as pinc
     om.load_numpy_state(om.InceptionV3(), pinc.init_weights())
+
+
+def test_vgg16_counts_and_flattening():
+    """138,357,544 parameters and 15.47 G multiply-accumulates per 224x224 image (published for
+    configuration D); 13 convolutions of 3x3 with bias, 5 poolings, and fully connected layers on the
+    channel-major flattening of the 512 x 7 x 7 map; the product-side weight generator loads strictly."""
+    model = om.VGG16().eval()
+    assert sum(p.numel() for p in model.parameters()) == 138357544
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000) and round(m / 1e9, 2) == 15.47
+    convs = [c for c in model.modules() if isinstance(c, torch.nn.Conv2d)]
+    assert len(convs) == 13 and all(c.kernel_size == (3, 3) and c.bias is not None for c in convs)
+    assert sum(1 for c in model.modules() if isinstance(c, torch.nn.MaxPool2d)) == 5
+    # flattening: feature (c, h, w) feeds classifier input c * 49 + h * 7 + w
+    with torch.no_grad():
+        for p in model.parameters():
+            p.zero_()
+        model.classifier[0].weight[5, 3 * 49 + 2 * 7 + 4] = 1.0
+        f = torch.zeros(1, 512, 7, 7)
+        f[0, 3, 2, 4] = 2.5
+        h = model.classifier[0](torch.flatten(f, 1))
+    assert h[0, 5] == 2.5 and h.abs().sum() == 2.5
+    from torpor_amd.functions import vgg as pvgg
+    om.load_numpy_state(om.VGG16(), pvgg.init_weights())
+
+
+def test_squeezenet11_counts_and_fire_module():
+    """1,235,496 parameters and 0.35 G multiply-accumulates per 224x224 image (published for revision 1.1),
+    eight fire modules; a fire module is relu(squeeze) followed by relu(1x1) and relu(3x3) side by side."""
+    model = om.SqueezeNet11().eval()
+    assert sum(p.numel() for p in model.parameters()) == 1235496
+    m, y = _macs(model, torch.zeros(1, 3, 224, 224))
+    assert y.shape == (1, 1000) and round(m / 1e9, 2) == 0.35
+    fires = [f for f in model.modules() if isinstance(f, om._Fire)]
+    assert len(fires) == 8
+    assert [f.squeeze.out_channels for f in fires] == [16, 16, 32, 32, 48, 48, 64, 64]
+    torch.manual_seed(2)
+    f = om._Fire(12, 4, 6, 10).eval()
+    x = torch.randn(2, 12, 7, 5)
+    with torch.no_grad():
+        s_ = F.relu(F.conv2d(x, f.squeeze.weight, f.squeeze.bias))
+        want = torch.cat([F.relu(F.conv2d(s_, f.expand1x1.weight, f.expand1x1.bias)),
+                          F.relu(F.conv2d(s_, f.expand3x3.weight, f.expand3x3.bias, padding=1))], 1)
+        assert torch.allclose(f(x), want, atol=1e-6)
+    # map sizes at 224: 111 after the stem, 55 / 27 / 13 after the three ceil-mode poolings
+    sizes, t = [], torch.zeros(1, 3, 224, 224)
+    with torch.no_grad():
+        for layer in model.features:
+            t = layer(t)
+            if isinstance(layer, (torch.nn.Conv2d, torch.nn.MaxPool2d)):
+                sizes.append(t.shape[-1])
+    assert sizes == [111, 55, 27, 13]
+    from torpor_amd.functions import squeezenet as psq
+    om.load_numpy_state(om.SqueezeNet11(), psq.init_weights())

@@ -39,6 +39,7 @@ const char* tp_strerror(int code) {
         case TP_ENOTACTIVE: return "client is not the active function";
         case TP_EUNSUPPORTED: return "not supported";
         case TP_EFAULT: return "virtual address does not translate";
+        case TP_ERANGE: return "function id out of range (0..65535)";
         case TP_ESCRATCH: return "needs more scratch memory than the fixed buffer of the no-allocation entry point";
         default: break;
     }

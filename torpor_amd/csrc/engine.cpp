@@ -1610,7 +1610,8 @@ int Engine::signal(int type, const char* function, const char* payload, int* ack
     if (deferred) *deferred = 0;
     if (ticket) *ticket = 0;
     int id = -1;
-    if (!parse_int(function, &id) || id < 0 || id > kMaxClient) return TP_EINVAL;  // cuda_server.hpp:221 stoi(func)
+    if (!parse_int(function, &id) || id < 0) return TP_EINVAL;  // cuda_server.hpp:221 stoi(func)
+    if (id > kMaxClient) return TP_ERANGE;  // the id is part of every address handed to the function
     poll_timeout_locked();
     const bool busy = exec_status_ != ES_AVAIL;
     switch (type) {

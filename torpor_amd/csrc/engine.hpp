@@ -38,11 +38,14 @@ namespace tp {
 constexpr uint64_t kTensorAlign = 256;
 constexpr uint64_t kVaTag = 0x7Aull << 56;
 constexpr uint64_t kVaTagMask = 0xFFull << 56;
-constexpr int kVaClientShift = 44;
-constexpr uint64_t kVaClientMask = 0xFFFull;
-constexpr uint64_t kVaActBit = 1ull << 43;
-constexpr uint64_t kVaOffMask = (1ull << 43) - 1;
-constexpr int kMaxClient = 4095;
+// tag (8 bits) | function id (16 bits) | region bit | offset (39 bits: 512 GiB per region, above the
+// 288 GB of the part).  The reference takes any integer as a function id (cuda_server.hpp:221-224);
+// here ids above kMaxClient are refused with TP_ERANGE.
+constexpr int kVaClientShift = 40;
+constexpr uint64_t kVaClientMask = 0xFFFFull;
+constexpr uint64_t kVaActBit = 1ull << 39;
+constexpr uint64_t kVaOffMask = (1ull << 39) - 1;
+constexpr int kMaxClient = 65535;
 
 enum OpKind : int { OPK_GEMM = 1, OPK_CONV, OPK_BN, OPK_LAUNCH, OPK_H2D, OPK_D2H, OPK_D2D, OPK_MEMSET };
 
