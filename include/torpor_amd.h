@@ -201,6 +201,13 @@ typedef struct tp_swap_stats {
     uint32_t host_gathers; /* lookups of the last request that read their table in place from the host store */
     uint64_t deferred_bytes; /* of `bytes`: transfer groups that hold nothing but tables looked up by index; they
                                 travel last and a request does not wait for them */
+    /* host side of the last swap-in: time the copy thread took to hand every group to the streams, and its
+     * slowest single runtime call (group index; kind 0 = copy, 1 = event record, 2 = stream wait, 3 = expansion
+     * launch).  A swap-in is paced by the link unless a call here stalls. */
+    double issue_ms;
+    double max_call_us;
+    uint32_t max_call_group;
+    uint32_t max_call_kind;
 } tp_swap_stats;
 
 /* ------------------------------------------------------------------ lifecycle

@@ -91,7 +91,9 @@ class ModelInfo(C.Structure):
 class SwapStats(C.Structure):
     _fields_ = [("bytes", C.c_uint64), ("copy_ms", C.c_double), ("alloc_us", C.c_double),
                 ("evict_us", C.c_double), ("chunks", C.c_uint32), ("gate_waits", C.c_uint32),
-                ("copy_streams", C.c_uint32), ("host_gathers", C.c_uint32), ("deferred_bytes", C.c_uint64)]
+                ("copy_streams", C.c_uint32), ("host_gathers", C.c_uint32), ("deferred_bytes", C.c_uint64),
+                ("issue_ms", C.c_double), ("max_call_us", C.c_double), ("max_call_group", C.c_uint32),
+                ("max_call_kind", C.c_uint32)]
 
 
 class KernelStat(C.Structure):

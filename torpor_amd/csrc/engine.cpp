@@ -196,6 +196,38 @@ int Engine::init() {
             HIPCHK(hipStreamSynchronize(copy_));
             HIPCHK(hipStreamSynchronize(copy2_));
             HIPCHK(hipStreamSynchronize(decode_));
+            // One swap-in in the first few dozen of a process used to take 6.5 ms longer: a single
+            // hipMemcpyAsync call of one of its first groups blocked that long on the host (timed per call,
+            // tp_swap_stats.max_call_*), whatever the model.  It is a one-time set-up inside the runtime that
+            // a copy triggers when it is submitted while the copy engines used so far are busy; two streams
+            // taking turns reach that state only now and then.  Copies in flight on several more streams at
+            // once reach it here: 3 of 8 fresh processes showed the stall within 160 swap-ins without this
+            // burst, none of 8 with it.  (TORPOR_INIT_STREAMS=0 leaves it out.)
+            const int extra = (int)env_u64("TORPOR_INIT_STREAMS", 6);
+            if (extra > 0) {
+                std::vector<hipStream_t> tmp((size_t)extra, nullptr);
+                for (auto& t : tmp) (void)hipStreamCreateWithFlags(&t, hipStreamNonBlocking);
+                const uint64_t piece = (n / (uint64_t)(extra + 2)) & ~uint64_t(255);
+                for (int rep = 0; rep < 4 && piece; ++rep) {
+                    int k = 0;
+                    (void)hipMemcpyAsync(ws + half + piece * k, h2d_stage_ + piece * k, piece, hipMemcpyHostToDevice, copy_);
+                    ++k;
+                    (void)hipMemcpyAsync(ws + half + piece * k, h2d_stage_ + piece * k, piece, hipMemcpyHostToDevice, copy2_);
+                    ++k;
+                    for (auto& t : tmp)
+                        if (t) {
+                            (void)hipMemcpyAsync(ws + half + piece * k, h2d_stage_ + piece * k, piece, hipMemcpyHostToDevice, t);
+                            ++k;
+                        }
+                }
+                (void)hipStreamSynchronize(copy_);
+                (void)hipStreamSynchronize(copy2_);
+                for (auto& t : tmp)
+                    if (t) {
+                        (void)hipStreamSynchronize(t);
+                        (void)hipStreamDestroy(t);
+                    }
+            }
             HIPCHK(hipMemset(ws + half, 0, 2 * n));  // the workspace is handed to the kernels zeroed
         }
     }
@@ -979,6 +1011,26 @@ uint64_t Engine::xfer_off(const Model& m, uint64_t d) const {
     return p.t_off + (p.pack_base >= 0 ? rel / 256 * kPackUnitBytes : rel);
 }
 
+// The copy thread times every runtime call of a swap-in's hand-over and keeps the slowest: the link paces
+// a swap-in unless one of these calls stalls on the host (tp_swap_stats.max_call_*).
+namespace {
+thread_local Model* t_timed = nullptr;
+enum : uint32_t { CALL_COPY = 0, CALL_RECORD = 1, CALL_WAIT = 2, CALL_EXPAND = 3 };
+template <class F>
+inline auto timed_call(uint32_t group, uint32_t kind, F&& f) -> decltype(f()) {
+    if (!t_timed) return f();
+    const auto t0 = Clock::now();
+    const auto r = f();
+    const double us = us_since(t0);
+    if (us > t_timed->max_call_us) {
+        t_timed->max_call_us = us;
+        t_timed->max_call_group = group;
+        t_timed->max_call_kind = kind;
+    }
+    return r;
+}
+}  // namespace
+
 // One transfer group of a packed swap-in: DMA into the staging area, then, on the expansion stream,
 // every tensor run of the group into its place, the out-of-window words patched, the group published.
 int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs, bool do_dma,
@@ -988,12 +1040,14 @@ int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hi
         const uint64_t te = end >= m.image_bytes ? m.timg_bytes : xfer_off(m, end);
         if (te < tb || te > xfer_stage_cap_) return TP_EFAULT;
         hipError_t e = hipSuccess;
-        if (te > tb) e = hipMemcpyAsync(xfer_stage_ + tb, m.timg + tb, te - tb, hipMemcpyHostToDevice, cs);
-        if (e == hipSuccess) e = hipEventRecord(m.dma_ev[i], cs);
+        if (te > tb)
+            e = timed_call((uint32_t)i, CALL_COPY,
+                           [&] { return hipMemcpyAsync(xfer_stage_ + tb, m.timg + tb, te - tb, hipMemcpyHostToDevice, cs); });
+        if (e == hipSuccess) e = timed_call((uint32_t)i, CALL_RECORD, [&] { return hipEventRecord(m.dma_ev[i], cs); });
         if (e != hipSuccess) return (int)e;
     }
     if (!do_expand) return 0;
-    hipError_t e = hipStreamWaitEvent(decode_, m.dma_ev[i], 0);
+    hipError_t e = timed_call((uint32_t)i, CALL_WAIT, [&] { return hipStreamWaitEvent(decode_, m.dma_ev[i], 0); });
     if (e != hipSuccess) return (int)e;
     size_t lo = 0, hi = m.image_order.size();
     while (lo < hi) {
@@ -1037,13 +1091,13 @@ int Engine::copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hi
             pc.tab = nullptr;
         }
         if (a.n == tpk::kUnpackMaxPieces) {
-            r = tpk::launch_unpack(a, decode_);
+            r = timed_call((uint32_t)i, CALL_EXPAND, [&] { return tpk::launch_unpack(a, decode_); });
             a.n = 0;
         }
     }
-    if (!r && a.n) r = tpk::launch_unpack(a, decode_);
+    if (!r && a.n) r = timed_call((uint32_t)i, CALL_EXPAND, [&] { return tpk::launch_unpack(a, decode_); });
     if (r) return r;
-    return (int)hipEventRecord(m.chunk_ev[i], decode_);
+    return (int)timed_call((uint32_t)i, CALL_RECORD, [&] { return hipEventRecord(m.chunk_ev[i], decode_); });
 }
 
 // One copy stream or two.  Measured on MI355X: a single stream loses ~15 us of DMA set-up per
@@ -1219,6 +1273,10 @@ void Engine::copy_main() {
         // publish each group.  Publishing is an event record, not a host synchronisation.
         int err = 0;
         TraceRange trace("swap-in: issue copies of model", m->id);
+        const auto t_issue = Clock::now();
+        m->max_call_us = 0;
+        m->max_call_group = m->max_call_kind = 0;
+        t_timed = m;  // every runtime call of the hand-over is timed (timed_call)
         if (!m->cancel.load()) {
             if (m->timg && stage_used_) {  // the staging area is shared: the previous expansion must be done with it
                 (void)hipStreamWaitEvent(copy_, stage_free_ev_, 0);
@@ -1237,8 +1295,10 @@ void Engine::copy_main() {
                 if (m->ncopy == 2 && (i == m->defer_from || i == m->defer_from + 1) && i >= 2)
                     (void)hipStreamWaitEvent(cs, (m->timg ? m->dma_ev : m->chunk_ev)[i == m->defer_from ? i - 1 : i - 2], 0);
                 if (m->timg) return copy_chunk_packed(*m, i, beg, end, cs, /*dma=*/true, /*expand=*/false);
-                hipError_t e = hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
-                if (e == hipSuccess) e = hipEventRecord(m->chunk_ev[i], cs);
+                hipError_t e = timed_call((uint32_t)i, CALL_COPY, [&] {
+                    return hipMemcpyAsync(m->w_dev + beg, m->host_image + beg, end - beg, hipMemcpyHostToDevice, cs);
+                });
+                if (e == hipSuccess) e = timed_call((uint32_t)i, CALL_RECORD, [&] { return hipEventRecord(m->chunk_ev[i], cs); });
                 return (int)e;
             };
             auto publish = [&](size_t i, uint64_t beg, uint64_t end) -> int {
@@ -1282,6 +1342,8 @@ void Engine::copy_main() {
                 (void)hipEventRecord(m->t1, copy_);
             }
         }
+        t_timed = nullptr;
+        m->issue_ms = us_since(t_issue) / 1000.0;
         if (err) m->copy_error.store(err);
         m->copy_state.store(CS_ISSUED, std::memory_order_release);
     }
@@ -2418,6 +2480,12 @@ int Engine::swap_stats(int client, tp_swap_stats* out) {
             float ms = 0.f;
             if (hipEventElapsedTime(&ms, m->t0, m->t1) == hipSuccess) m->stats.copy_ms = ms;
         }
+    }
+    if (m->copy_state.load(std::memory_order_acquire) == CS_ISSUED) {
+        m->stats.issue_ms = m->issue_ms;
+        m->stats.max_call_us = m->max_call_us;
+        m->stats.max_call_group = m->max_call_group;
+        m->stats.max_call_kind = m->max_call_kind;
     }
     *out = m->stats;
     return 0;

@@ -156,6 +156,9 @@ struct Model {
     std::atomic<int> copy_state{CS_IDLE};
     std::atomic<bool> cancel{false};
     std::atomic<int> copy_error{0};
+    // written by the copy thread before it publishes CS_ISSUED, read by the engine after that
+    double issue_ms = 0, max_call_us = 0;
+    uint32_t max_call_group = 0, max_call_kind = 0;
     uint32_t gated_upto = 0;
     uint64_t touch_seq = 0;   // Engine::work_seq_ at this model's last data-plane call
     uint32_t defer_from = UINT32_MAX;  // first transfer group made of deferred tables only

@@ -76,7 +76,10 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
     its arrival time and latency = completion - arrival (queueing included); otherwise requests run back to
     back and latency is the service time.  Every `check_every`-th answer is compared bit for bit with the
     function's registration run.  after_request(i, fid, hit) is called after each request."""
+    import gc
     n_req = len(picks)
+    gc.collect()
+    gc.disable()   # a collection of the interpreter inside a request (tens of milliseconds) is not the path's
     st0 = server.pool_stats()
     lat_hit, lat_miss, by_arch, swap_bytes, swap_ms = [], [], {}, 0, 0.0
     t0 = time.perf_counter()
@@ -112,6 +115,7 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
         if after_request is not None:
             after_request(i, fid, hit)
     wall = time.perf_counter() - t0
+    gc.enable()
     st1 = server.pool_stats()
     all_lat = lat_hit + lat_miss
     return dict(
