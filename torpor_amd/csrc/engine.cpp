@@ -2401,8 +2401,13 @@ int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uin
         if (r) break;
         if (op.kind == OPK_D2H) completed = true;
     }
+    const double issue_us = us_since(t_start);
     int sr = do_stream_sync(m);
     if (!ret) ret = sr;
+    static const bool dbg_timing = std::getenv("TORPOR_REPLAY_TIMING") != nullptr;
+    if (dbg_timing)
+        std::fprintf(stderr, "replay of %d (%s, %d ops): issued in %.1f us, done after %.1f us\n", m->id,
+                     warm ? "warm" : "cold", n_ops, issue_us, us_since(t_start));
     if (warm && !ret && !profiling_) {
         const double us = us_since(t_start);
         if (m->warm_us <= 0 || us < m->warm_us) m->warm_us = us;

@@ -20,7 +20,7 @@ void set_last_kernel(const char* n);
 int num_cu();
 Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
 int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, const Epilogue& e, hipStream_t s);
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32);
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true);
 unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
 
 struct ConvDev {
@@ -602,8 +602,9 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         // split over channel blocks of 8 (one K-block each)
         long kper_k = p.K;
         p.splits = 1;
-        if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k);
-        if (cfg == 3) p.splits = choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, 8);
+        static const bool pairs = getenv("TORPOR_CONV_PAIRS") != nullptr;
+        if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k, 32, pairs);
+        if (cfg == 3) p.splits = choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, 8, pairs);
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);

@@ -717,7 +717,7 @@ unsigned* split_tickets(const Workspace& ws, long tiles, int splits) {
 
 // One split's partial sums are `tiles` whole output tiles of tile_floats each (the in-launch summation
 // keeps them per tile and per wavefront; the two-launch form needs no more than that).
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32) {
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true) {
     int splits = 1;
     const long kblocks = (K + bk - 1) / bk;
     const size_t per = (size_t)tiles * (size_t)tile_floats * sizeof(float);
@@ -731,9 +731,28 @@ int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes,
         if (want > max_splits) want = max_splits;
         while (want > 1 && (size_t)want * per > ws_bytes) --want;
         if (want > 1) splits = (int)want;
+        if (!pairs && want > 1) {
+            // Kernels that take any number of K-blocks per split: weigh the candidates by what the
+            // fullest CU has to work through.  With s splits of b = ceil(kblocks / s) blocks the
+            // tiles * s workgroups land ceil(tiles * s / CUs) deep on some CU; a CU that holds a single
+            // workgroup hides no latency (about 1.3x per block), and every slot costs its tile's last
+            // workgroup a quarter of a block to read back.  8x14x14x256>256 (100 tiles, 32 blocks): 5
+            // splits of 7 (two deep, 14 blocks) run 29.0 us, the 6 of 6 (three deep, 18) 30.9 us.
+            double best = 1e30;
+            for (long s = 2; s <= want + 2 && s <= maxs && s <= max_splits && (size_t)s * per <= ws_bytes; ++s) {
+                const long b = (kblocks + s - 1) / s;
+                const long s_eff = (kblocks + b - 1) / b;
+                const long deep = (tiles * s_eff + g_num_cu - 1) / g_num_cu;
+                const double cost = (double)deep * (double)b * (deep == 1 ? 1.3 : 1.0) + 0.25 * (double)s_eff;
+                if (cost < best) {
+                    best = cost;
+                    splits = (int)s_eff;
+                }
+            }
+        }
     }
     long per_blocks = (kblocks + splits - 1) / splits;
-    if (splits > 1 && (per_blocks & 1)) ++per_blocks;  // whole pairs of K-blocks per split
+    if (pairs && splits > 1 && (per_blocks & 1)) ++per_blocks;  // whole pairs of K-blocks per split
     splits = (int)((kblocks + per_blocks - 1) / per_blocks);
     *kper_out = per_blocks * bk;
     return splits;
