@@ -420,6 +420,7 @@ def main():
         "warm_ms_p50": p["warm_ms_p50"],
         "cold_over_warm": p["cold_over_warm"],
         "roofline": roof[primary],
+        "link_roofline": p.get("link_roofline"),
         "cpu_baseline": cpu,
         "workloads": results,
         "rooflines": roof,
