@@ -306,46 +306,67 @@ def cpu_baseline(name, weights, inputs, first):
                 min_ms=min(times), logits_rel_err_vs_gpu=err)
 
 
+ABLATION_VARIANTS = {
+    "default": {},
+    "group_per_tensor (BUFFER_SIZE=1)": dict(chunk_bytes=1, chunk_max_bytes=1),
+    "one_group (no pipelining)": dict(chunk_bytes=2 << 30, chunk_max_bytes=2 << 30),
+    "fixed_2MiB_groups (the reference's default)": dict(chunk_bytes=2 << 20, chunk_max_bytes=2 << 20),
+    "weights_sent_as_they_are (TORPOR_PACK=0)": dict(pack=False),
+    "lookups_wait_for_their_table (TORPOR_HOST_GATHER=0)": dict(host_gather=False),
+}
+
+
+def ablation_variant(vname, names, steps, warmup):
+    """One variant of the ablation: one engine with that setting, the workloads one after the other on it, as in
+    the main leg.  Cold p50 (ms), transfer groups, link bytes and swap-in GB/s per workload."""
+    from torpor_amd.server import Server
+
+    row = {}
+    with Server(mem_limit_bytes=24 << 30, pool_bytes=25 << 30, **ABLATION_VARIANTS[vname]) as server:
+        server.measure_h2d(256 << 20, 10)
+        for fid, name in enumerate(names):
+            fn, inputs, _ = make_function(server, fid, name)
+            first = fn.register(inputs)
+            packed, outbuf, views = fn.pack(inputs, pinned=True)
+            cold = []
+            for i in range(warmup + steps):
+                fn.unload()
+                t0 = time.perf_counter()
+                ack, _, dfr = server.signal(1, fid, "")
+                assert ack == 0 and not dfr
+                server.replay(fid, packed, outbuf)
+                if i >= warmup:
+                    cold.append((time.perf_counter() - t0) * 1e3)
+                st = server.swap_stats(fid)
+            out_now = fn.postprocess([v.copy() for v in views])
+            for a, b in zip(first, out_now):
+                if not np.array_equal(a, b):
+                    raise SystemExit(f"ablation {vname} / {name}: output differs from the registration run")
+            row[name] = dict(cold_ms_p50=pctl(cold, 0.5), groups=st["chunks"], link_bytes=st["bytes"],
+                             swap_gbps=st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
+            fn.unload()
+            del fn
+    return row
+
+
 def ablation(names, steps, warmup):
     """Cold p50 (ms) per workload under the reference's pipeline ablation (evaluation/figure7/Figure7_README.md:
     12-33: BUFFER_SIZE = 2 MiB default, 1 = a group per tensor, 1.6 GB = no pipelining) and with this build's two
-    own transfer features switched off.  Every variant is a fresh engine, since these are engine settings."""
-    from torpor_amd.server import Server
+    own transfer features switched off.  These are engine settings, so every variant is an engine of its own --
+    and a process of its own: the second and later engines of one process were measured with swap-ins of the small
+    models at 40 instead of 55 GB/s (an engine's teardown frees tens of GiB of device memory, and copies that
+    follow large frees run slower; a serving process has one engine and never frees device memory on the request
+    path), which would be charged to the variant."""
+    import subprocess
 
-    variants = {
-        "default": {},
-        "group_per_tensor (BUFFER_SIZE=1)": dict(chunk_bytes=1, chunk_max_bytes=1),
-        "one_group (no pipelining)": dict(chunk_bytes=2 << 30, chunk_max_bytes=2 << 30),
-        "fixed_2MiB_groups (the reference's default)": dict(chunk_bytes=2 << 20, chunk_max_bytes=2 << 20),
-        "weights_sent_as_they_are (TORPOR_PACK=0)": dict(pack=False),
-        "lookups_wait_for_their_table (TORPOR_HOST_GATHER=0)": dict(host_gather=False),
-    }
     out = {}
-    for vname, kw in variants.items():
-        row = {}
-        for fid, name in enumerate(names):
-            with Server(mem_limit_bytes=8 << 30, pool_bytes=9 << 30, **kw) as server:
-                fn, inputs, _ = make_function(server, fid, name)
-                first = fn.register(inputs)
-                packed, outbuf, views = fn.pack(inputs, pinned=True)
-                cold = []
-                for i in range(warmup + steps):
-                    fn.unload()
-                    t0 = time.perf_counter()
-                    ack, _, dfr = server.signal(1, fid, "")
-                    assert ack == 0 and not dfr
-                    server.replay(fid, packed, outbuf)
-                    if i >= warmup:
-                        cold.append((time.perf_counter() - t0) * 1e3)
-                    st = server.swap_stats(fid)
-                out_now = fn.postprocess([v.copy() for v in views])
-                for a, b in zip(first, out_now):
-                    if not np.array_equal(a, b):
-                        raise SystemExit(f"ablation {vname} / {name}: output differs from the registration run")
-                row[name] = dict(cold_ms_p50=pctl(cold, 0.5), groups=st["chunks"], link_bytes=st["bytes"],
-                                 swap_gbps=st["bytes"] / 1e9 / (st["copy_ms"] * 1e-3))
-                del fn
-        out[vname] = row
+    for vname in ABLATION_VARIANTS:
+        cmd = [sys.executable, os.path.abspath(__file__), "--ablation-variant", vname, "--steps", str(steps),
+               "--warmup", str(warmup), "--workload", "all" if len(names) > 1 else names[0]]
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=900)
+        if r.returncode != 0:
+            raise SystemExit(f"bench.py: ablation variant {vname!r} failed:\n{r.stderr[-2000:]}")
+        out[vname] = json.loads(r.stdout.strip().splitlines()[-1])
     return out
 
 
@@ -364,7 +385,12 @@ def main():
     ap.add_argument("--ablate", action="store_true",
                     help="also measure cold p50 per config with per-tensor groups, one whole-image group, weights "
                          "sent as they are, and lookups that wait for their table")
+    ap.add_argument("--ablation-variant", default=None, help=argparse.SUPPRESS)   # child of --ablate
     args = ap.parse_args()
+    if args.ablation_variant is not None:
+        names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+        print(json.dumps(ablation_variant(args.ablation_variant, names, args.steps, args.warmup)))
+        return
     if args.gpus != 1:
         print("bench.py: this build serves from one GPU (one executor, one pool, one LRU per GPU); "
               "--gpus N with N > 1 is not supported", file=sys.stderr)
