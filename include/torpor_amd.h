@@ -154,7 +154,9 @@ typedef struct tp_conv_desc {
     int32_t x_layout, y_layout; /* TP_LAYOUT_* */
     /* NHWC only: elements between consecutive pixels of x / y, 0 = cin / cout.  A larger pitch reads the first
      * cin channels of a wider tensor, or writes a channel slice of one (concatenation without a copy).
-     * groups: 0 / 1, or cin == cout == groups (depthwise, NHWC, w is [C][1][KH][KW]). */
+     * groups: 0 / 1; cin == cout == groups (depthwise, NHWC, w is [C][1][KH][KW]); or any divisor of cin and cout
+     * (cudnnSetConvolutionGroupCount, cuda_server.hpp:671; NHWC in and out, w is [cout][cin/groups][KH][KW], one
+     * launch per group). */
     int64_t x_pitch, y_pitch;
     tp_epilogue ep;
 } tp_conv_desc;

@@ -100,8 +100,8 @@ def test_conv_rejects_bad_shapes(gpu_server):
             t.s.conv(t.fid, xv, t.w[0], yv, 1, 8, 8, 8, 8, 3, 3, stride=1, pad=1)
         with pytest.raises(TorporError):   # claims more filters than uploaded
             t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 16, 3, 3, stride=1, pad=1)
-        with pytest.raises(TorporError):   # grouped convolution is not implemented
-            t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1, groups=2)
+        with pytest.raises(TorporError):   # a group count that does not divide the channels
+            t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1, groups=3)
         with pytest.raises(TorporError):
             t.s.stream_synchronize(t.fid)
         t.s.conv(t.fid, xv, t.w[0], yv, 1, 6, 6, 8, 8, 3, 3, stride=1, pad=1)
@@ -158,14 +158,54 @@ def test_depthwise(gpu_server, C, k, stride, HW):
         t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=C,
                  bn=tuple(t.w[1:5]), bn_eps=1e-5, act=ACT_RELU6)
         fused = t.read(yv, (N, Ho, Ho, C))
-        with pytest.raises(TorporError):   # grouped but not depthwise
-            t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=2)
+        with pytest.raises(TorporError):   # a group count that does not divide the channels
+            t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, C, C, k, k, stride=stride, pad=pad, groups=7)
         with pytest.raises(TorporError):
             t.s.stream_synchronize(t.fid)
     want = ref.depthwise_conv2d(x, w, (stride, stride), (pad, pad))
     assert_close(plain, want, RTOL, "depthwise")
     z = ref.bn(want, g, b, mu, var, 1e-5, C, nhwc=True)
     assert_close(fused, ref.activation(z, "relu6"), 5e-5, "depthwise+bn+relu6")
+
+
+@pytest.mark.parametrize("Cin,Cout,groups,k,stride,HW", [(64, 128, 4, 3, 1, 14), (32, 32, 2, 1, 1, 9), (24, 36, 3, 3, 2, 11),
+                                                         (6, 10, 2, 5, 1, 8), (128, 128, 32, 3, 1, 7)])
+def test_grouped_convolution(gpu_server, Cin, Cout, groups, k, stride, HW):
+    """cudnnSetConvolutionGroupCount (cuda_server.hpp:671) with groups that are not the channel count (ResNeXt-style):
+    against torch's float64 grouped convolution, and against the fp64 oracle applied group by group; with the
+    fused bias + residual + relu epilogue on top."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(Cin + Cout + groups)
+    N, pad = 2, k // 2
+    x = _rand(rng, N, HW, HW, Cin)
+    w = _rand(rng, Cout, Cin // groups, k, k)
+    bias = _rand(rng, Cout)
+    Ho = (HW + 2 * pad - k) // stride + 1
+    res = _rand(rng, N, Ho, Ho, Cout)
+    with OpSession(gpu_server, [w, bias]) as t:
+        xv = t.act(x)
+        rv = t.act(res)
+        yv = t.empty(N * Ho * Ho * Cout * 4)
+        t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, Cin, Cout, k, k, stride=stride, pad=pad, groups=groups)
+        plain = t.read(yv, (N, Ho, Ho, Cout))
+        t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, Cin, Cout, k, k, stride=stride, pad=pad, groups=groups,
+                 bias=t.w[1], residual=rv, act=ACT_RELU)
+        fused = t.read(yv, (N, Ho, Ho, Cout))
+        with pytest.raises(TorporError):   # grouped and not depthwise needs NHWC on both sides
+            t.s.conv(t.fid, xv, t.w[0], yv, N, HW, HW, Cin, Cout, k, k, stride=stride, pad=pad, groups=groups,
+                     x_layout=NCHW)
+        with pytest.raises(TorporError):
+            t.s.stream_synchronize(t.fid)
+    want64 = F.conv2d(torch.from_numpy(x).double().permute(0, 3, 1, 2), torch.from_numpy(w).double(), stride=stride,
+                      padding=pad, groups=groups).permute(0, 2, 3, 1).numpy()
+    assert_close(plain, want64.astype(np.float32), RTOL, "grouped conv vs torch float64")
+    cig, cog = Cin // groups, Cout // groups
+    per_group = [ref.conv2d(np.ascontiguousarray(x[..., g * cig:(g + 1) * cig]), np.ascontiguousarray(w[g * cog:(g + 1) * cog]),
+                            (stride, stride), (pad, pad), x_nhwc=True, y_nhwc=True) for g in range(groups)]
+    want = np.concatenate(per_group, axis=-1)
+    assert_close(plain, want, RTOL, "grouped conv vs the oracle, group by group")
+    assert_close(fused, np.maximum(want + bias + res, 0).astype(np.float32), 5e-5, "grouped conv + bias + residual + relu")
 
 
 @pytest.mark.parametrize("k", [1, 3])

@@ -1875,7 +1875,9 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             const i128 groups = (op.ni > 17 && I[17] > 0) ? I[17] : 1;
             const bool x_nhwc = I[11] != 0, y_nhwc = I[12] != 0;
             if ((xpitch && (!x_nhwc || xpitch < Cin)) || (ypitch && (!y_nhwc || ypitch < Cout))) return TP_EINVAL;
-            if (groups != 1 && (groups != Cin || Cin != Cout)) return TP_EUNSUPPORTED;
+            if (groups != 1 && (Cin % groups != 0 || Cout % groups != 0)) return TP_EINVAL;
+            // grouped but not depthwise: one launch per group over channel slices, NHWC only
+            if (groups != 1 && (groups != Cin || Cin != Cout) && (!x_nhwc || !y_nhwc)) return TP_EUNSUPPORTED;
             const i128 ys = ypitch ? (N * Ho * Wo - 1) * ypitch + Cout : N * Ho * Wo * Cout;
             const i128 xs = xpitch ? (N * H * W - 1) * xpitch + Cin : N * H * W * Cin;
             if ((r = R(0, false, xs)) || (r = R(1, false, Cout * (Cin / groups) * KH * KW)) || (r = R(2, false, ys)))

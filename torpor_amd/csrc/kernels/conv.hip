@@ -473,7 +473,45 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         return K_EINVAL;
     const long xp = a.x_pitch ? a.x_pitch : a.Cin;   // floats between pixels (NHWC)
     const long yp = a.y_pitch ? a.y_pitch : a.Cout;
-    if (a.groups != 1) return launch_depthwise(a, Ho, Wo, xp, yp, s);
+    if (a.groups != 1 && a.groups == a.Cin && a.Cin == a.Cout) {
+        const int r = launch_depthwise(a, Ho, Wo, xp, yp, s);
+        if (r != K_EUNSUPPORTED) return r;  // else: as a grouped convolution, below
+    }
+    if (a.groups != 1) {
+        // General grouped convolution (cudnnSetConvolutionGroupCount, cuda_server.hpp:671): group g maps input
+        // channels [g*Cin/G, (g+1)*Cin/G) to output channels [g*Cout/G, (g+1)*Cout/G) with its own block of
+        // the [Cout][Cin/G][KH][KW] filter.  In NHWC each group is a convolution over a channel slice of x
+        // written into a channel slice of y, which the kernels serve through their pixel pitches; one launch
+        // per group.
+        if (a.groups < 1 || a.Cin % a.groups || a.Cout % a.groups) return K_EINVAL;
+        if (!a.x_nhwc || !a.y_nhwc) return K_EUNSUPPORTED;
+        const int cig = a.Cin / a.groups, cog = a.Cout / a.groups;
+        for (int g = 0; g < a.groups; ++g) {
+            ConvArgs b = a;
+            b.groups = 1;
+            b.Cin = cig;
+            b.Cout = cog;
+            b.x = a.x + (long)g * cig;
+            b.y = a.y + (long)g * cog;
+            b.w = a.w + (long)g * cog * cig * a.KH * a.KW;
+            b.x_pitch = xp;
+            b.y_pitch = yp;
+            if (b.ep.bias) b.ep.bias += (long)g * cog;
+            if (b.ep.bn_scale) {
+                b.ep.bn_scale += (long)g * cog;
+                b.ep.bn_bias += (long)g * cog;
+                b.ep.bn_mean += (long)g * cog;
+                b.ep.bn_var += (long)g * cog;
+            }
+            if (b.ep.residual) {
+                if (b.ep.ldr == 0) b.ep.ldr = a.Cout;
+                b.ep.residual += (long)g * cog;
+            }
+            const int r = launch_conv2d(b, ws, s);
+            if (r) return r;
+        }
+        return 0;
+    }
 
     // 1x1 over NHWC is a dense GEMM, with a row gather when strided.
     if (a.KH == 1 && a.KW == 1 && a.ph == 0 && a.pw == 0 && a.x_nhwc && a.y_nhwc) {
