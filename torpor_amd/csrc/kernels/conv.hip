@@ -20,7 +20,8 @@ void set_last_kernel(const char* n);
 int num_cu();
 Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
 int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, const Epilogue& e, hipStream_t s);
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true);
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true,
+                  int balance = -1);
 unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
 
 struct ConvDev {
@@ -642,7 +643,15 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         p.splits = 1;
         static const bool pairs = getenv("TORPOR_CONV_PAIRS") != nullptr;
         if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k, 32, pairs);
-        if (cfg == 3) p.splits = choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, 8, pairs);
+        if (cfg == 3) {
+            // Nine-wavefront workgroups do not share a CU well: two of them on one CU take 2.4x as long per
+            // K-block as one alone, so the split stops where every workgroup still has a CU to itself
+            // (1x14x14x256>256, 56 tiles: 4 slots 9.8 us, 8 slots 11.4 us; 1x56x56x64>64, 196 tiles: unsplit
+            // 7.1 us, 2 slots 10.1 us).  TORPOR_CONV_PAIRS=1 keeps the earlier rule (two workgroups per CU).
+            int cap = pairs ? 8 : (int)(num_cu() / tiles);
+            if (cap > 8) cap = 8;
+            p.splits = cap >= 2 ? choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, cap, true, 0) : 1;
+        }
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits);

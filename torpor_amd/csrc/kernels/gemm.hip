@@ -717,7 +717,8 @@ unsigned* split_tickets(const Workspace& ws, long tiles, int splits) {
 
 // One split's partial sums are `tiles` whole output tiles of tile_floats each (the in-launch summation
 // keeps them per tile and per wavefront; the two-launch form needs no more than that).
-int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true) {
+int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true,
+                  int balance = -1) {
     int splits = 1;
     const long kblocks = (K + bk - 1) / bk;
     const size_t per = (size_t)tiles * (size_t)tile_floats * sizeof(float);
@@ -731,7 +732,7 @@ int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes,
         if (want > max_splits) want = max_splits;
         while (want > 1 && (size_t)want * per > ws_bytes) --want;
         if (want > 1) splits = (int)want;
-        if (!pairs && want > 1) {
+        if ((balance < 0 ? !pairs : balance != 0) && want > 1) {
             // Kernels that take any number of K-blocks per split: weigh the candidates by what the
             // fullest CU has to work through.  With s splits of b = ceil(kblocks / s) blocks the
             // tiles * s workgroups land ceil(tiles * s / CUs) deep on some CU; a CU that holds a single
@@ -740,7 +741,8 @@ int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes,
             // splits of 7 (two deep, 14 blocks) run 29.0 us, the 6 of 6 (three deep, 18) 30.9 us.
             double best = 1e30;
             for (long s = 2; s <= want + 2 && s <= maxs && s <= max_splits && (size_t)s * per <= ws_bytes; ++s) {
-                const long b = (kblocks + s - 1) / s;
+                long b = (kblocks + s - 1) / s;
+                if (pairs && (b & 1)) ++b;
                 const long s_eff = (kblocks + b - 1) / b;
                 const long deep = (tiles * s_eff + g_num_cu - 1) / g_num_cu;
                 const double cost = (double)deep * (double)b * (deep == 1 ? 1.3 : 1.0) + 0.25 * (double)s_eff;
@@ -757,6 +759,11 @@ int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes,
     *kper_out = per_blocks * bk;
     return splits;
 }
+
+// 32x32 GEMM tiles: the split is weighed by the depth of the fullest CU as well (128x768x3072, 96 tiles of 48
+// K-blocks: 8 slots of 6 blocks, three deep, 11.6 us; the 6 slots of 8 that "two workgroups per CU" gives, also three
+// deep, 13.0 us).  TORPOR_GEMM_BALANCE=0 restores the plain rule.
+static const int g_small_balance = getenv("TORPOR_GEMM_BALANCE") ? atoi(getenv("TORPOR_GEMM_BALANCE")) : 1;
 
 // What launch_gemm decides from the shape alone: kernel family, tile and split of K over workgroups.
 struct GemmPlan {
@@ -789,7 +796,7 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
         if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, (long)g.bm * g.bn, ws_bytes, &g.kper);
         // (with more than half a tile per CU the split does not pay: 196x1024x512, 224 tiles, 8.5 against 7.4 us)
         if (batch == 1 && cfg == 4 && tiles <= g_num_cu / 2)
-            g.splits = choose_splits(tiles, a.K, 64, 32 * 32, ws_bytes, &g.kper, /*max_splits=*/8);
+            g.splits = choose_splits(tiles, a.K, 64, 32 * 32, ws_bytes, &g.kper, /*max_splits=*/8, true, g_small_balance);
     } else {
         g.tiles_m = (int)((a.M + 63) / 64);
         g.tiles_n = (int)((a.N + 63) / 64);
