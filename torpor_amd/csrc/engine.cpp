@@ -1152,18 +1152,35 @@ void Engine::build_chunks(Model& m) {
         if (pos < m.image_bytes) m.chunk_end.push_back(m.image_bytes);
         pos = m.image_bytes;
     }
+    // Where the part of the image ends that a request streams through (tables looked up by index lie behind it).
+    uint64_t table_off = UINT64_MAX;
+    for (const Param& p : m.params)
+        if (p.gathered) table_off = std::min(table_off, p.image_off);
+    const uint64_t streamed_end = (host_gather_ && table_off != UINT64_MAX) ? table_off : m.image_bytes;
+    // The last layers cannot start before their group has landed whole, so the time the last group spends on
+    // the link is added to a cold request that the link paces.  With two copy streams (the link-bound models)
+    // the groups therefore shrink again towards the end of the streamed part: none is larger than half of what
+    // is left, down to the first group's size (BERT-base batch 1 cold 5.35 -> 5.30 ms, BERT-large 18.95 ->
+    // 18.89 ms).  With one stream every extra copy costs link time and the request ends 0.07 ms after the last
+    // byte anyway (ResNet-152 batch 8: 3.98 -> 4.01 ms tapered), so those keep full groups.  TORPOR_TAPER=0 /
+    // =2: never / always.
+    static const uint64_t taper_mode = env_u64("TORPOR_TAPER", 1);
+    const bool taper = taper_mode == 2 || (taper_mode == 1 && m.ncopy == 2);
+    const uint64_t cmin = align_up(std::max<uint64_t>(cfg_.chunk_bytes, kTensorAlign), kTensorAlign);
     while (pos < m.image_bytes) {
-        uint64_t end = pos + align_up(sz, kTensorAlign);
-        if (end > m.image_bytes) end = m.image_bytes;
+        uint64_t g = align_up(sz, kTensorAlign);
+        uint64_t limit = m.image_bytes;
+        if (taper && !per_tensor_groups_ && pos < streamed_end) {
+            g = std::min(g, std::max(cmin, align_up((streamed_end - pos) / 2, kTensorAlign)));
+            limit = streamed_end;
+        }
+        uint64_t end = (g > limit - pos) ? limit : pos + g;
         m.chunk_end.push_back(end);
         pos = end;
         if (sz < m.chunk_max) sz = std::min(sz * 2, m.chunk_max);
     }
     // first group that holds nothing but tables looked up by index (they are last in the image)
     m.defer_from = UINT32_MAX;
-    uint64_t table_off = UINT64_MAX;
-    for (const Param& p : m.params)
-        if (p.gathered) table_off = std::min(table_off, p.image_off);
     if (host_gather_ && table_off != UINT64_MAX)
         for (size_t i = 0; i < m.chunk_end.size(); ++i)
             if ((i ? m.chunk_end[i - 1] : 0) >= table_off) {
