@@ -114,7 +114,8 @@ typedef struct tp_config {
     uint64_t pool_bytes;        /* HBM arena; 0: mem_limit + pool headroom (memory_manager.hpp:42-44) */
     uint64_t chunk_bytes;       /* first swap-in gate group; 0: env BUFFER_SIZE or 2 MiB (memory_manager.hpp:22,169-173);
                                    below 256 (the reference's BUFFER_SIZE=1 ablation): one group per tensor */
-    uint64_t chunk_max_bytes;   /* groups double up to this size; 0: 8 MiB; set = chunk_bytes for fixed groups */
+    uint64_t chunk_max_bytes;   /* groups double up to this size; 0: chosen per model (16 MiB with two copy streams,
+                                 * 32 MiB with one); set = chunk_bytes for fixed groups */
     uint64_t workspace_bytes;   /* split-K scratch; 0: 64 MiB */
     int32_t flags;              /* TP_FLAG_* */
     int32_t request_timeout_ms; /* 0: 5000 (cuda_server.hpp:29) */

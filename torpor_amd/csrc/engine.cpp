@@ -1129,6 +1129,11 @@ void Engine::choose_copy_plan(Model& m) {
     if (copy_streams_cfg_ == 1 || copy_streams_cfg_ == 2) m.ncopy = copy_streams_cfg_;
     m.chunk_max = cfg_.chunk_max_bytes;
     if (chunk_max_auto_ && m.ncopy == 1) m.chunk_max = std::max<uint64_t>(cfg_.chunk_max_bytes, 32ull << 20);
+    // Two streams: 16 MiB.  Groups of 8 MiB left a whole swap-in of BERT-large in one of two modes from one
+    // process to the next (56.1 or 55.2 GB/s, cold 18.84 or 19.09 ms); with 16 MiB all of 5 fresh processes ran
+    // 56.3 GB/s and 18.66-18.69 ms.  The size in the middle of the image costs a link-bound request nothing,
+    // since the groups shrink again towards the end (build_chunks); 32 MiB was no faster and worse for ResNet-50.
+    if (chunk_max_auto_ && m.ncopy == 2) m.chunk_max = std::max<uint64_t>(cfg_.chunk_max_bytes, 16ull << 20);
 }
 
 // Transfer groups: the first is chunk_bytes, each next one doubles up to chunk_max_bytes, so the
