@@ -67,6 +67,8 @@ typedef struct tp_server tp_server;
 #define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
 #define TP_FLAG_NO_HOST_GATHER 4 /* embedding lookups always wait for their table's transfer group, as env TORPOR_HOST_GATHER=0 */
 #define TP_FLAG_NO_PACK 8 /* weights cross the link as they are instead of in the packed transfer format, as env TORPOR_PACK=0 */
+#define TP_FLAG_KEEP_HOST_IMAGE 16 /* keep the raw weight image in pinned host memory beside the packed transfer image (by default the
+                                   * transfer image, checked to decode back bit for bit, is the host store), as env TORPOR_SLIM_HOST=0 */
 
 /* ---- activation / epilogue ---- */
 #define TP_ACT_NONE 0
@@ -170,8 +172,9 @@ typedef struct tp_pool_stats {
     /* victims taken because no contiguous extent fitted although the budget test had passed (the reference
      * exits there, block_manager.hpp:345-351); they are included in `evictions` */
     uint64_t fragmentation_evictions;
-    /* pinned host memory held outside the pool: weight images, their transfer images (the second, smaller
-     * copy that crosses the link), request staging and result buffers */
+    /* pinned host memory: raw weight images (whole, for models that travel as they are; only the tables looked
+     * up by index for models whose packed transfer image is their host store), transfer images, request
+     * staging and result buffers */
     uint64_t host_image_bytes, host_transfer_bytes, host_staging_bytes;
     /* device memory outside the pool and its budget: staging area of packed transfers, kernel workspace */
     uint64_t device_staging_bytes, device_workspace_bytes;
@@ -338,7 +341,9 @@ int tp_get_pool_stats(tp_server* s, tp_pool_stats* out);
 int tp_get_swap_stats(tp_server* s, int32_t client, tp_swap_stats* out);
 /* Copies the device-resident weight image (waits for an in-flight swap-in). */
 int tp_readback_weights(tp_server* s, int32_t client, void* dst, uint64_t bytes);
-/* The authoritative host copy of the same image, same layout. */
+/* The authoritative host copy of the same image, same layout.  For a model whose host store is its packed
+ * transfer image the image is decoded into a buffer of the engine's; *ptr stays valid until the next call for
+ * the same function (or its re-registration / the server's destruction). */
 int tp_host_weights(tp_server* s, int32_t client, const void** ptr, uint64_t* bytes);
 /* Image offset of a weight virtual address (first-access-order layout). */
 int tp_weight_offset(tp_server* s, int32_t client, uint64_t vaddr, uint64_t* image_off);

@@ -129,6 +129,51 @@ def test_embedding_table_travels_last_and_is_read_in_place_meanwhile(host_gather
         fn.unload()
 
 
+def _assert_host_store_holds_the_upload(s, fn, host):
+    """Every uploaded tensor sits unmodified at its offset of the host copy of the image."""
+    for name, arr in fn.weights().items():
+        raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+        off = s.weight_offset(fn.fid, fn.w[name])
+        assert np.array_equal(host[off:off + raw.size], raw), name
+
+
+@pytest.mark.parametrize("keep", [False, True])
+def test_host_store_is_the_transfer_image_plus_the_tables(keep, monkeypatch):
+    """By default a packed model's raw image is released once its transfer image has been decoded back to it
+    on the host: pinned memory holds the transfer image and a raw copy of the tables that lookups read in place
+    during a swap-in.  tp_host_weights then decodes on demand, and what it returns is the upload, byte for
+    byte; cold requests still read table rows from host memory and answer as at registration."""
+    monkeypatch.delenv("TORPOR_SLIM_HOST", raising=False)
+    monkeypatch.delenv("TORPOR_PACK", raising=False)
+    monkeypatch.delenv("TORPOR_HOST_GATHER", raising=False)
+    cfg = dict(layers=2, hidden=512, heads=8, ffn=1024)
+    weights = bert.init_weights(seed=22, vocab=30522, max_pos=128, cfg=cfg)   # word table: 62 MB of 71
+    ids = np.random.default_rng(5).integers(0, 30522, (2, 64))
+    with Server(mem_limit_bytes=1 << 30, keep_host_image=keep) as s:
+        fn = bert.Bert(s, 3, batch=2, seq=64, weights=weights, cfg=cfg)
+        first = fn.register([ids])
+        info = s.model_info(3)
+        image = info["image_bytes"]
+        st = s.pool_stats()
+        table = weights["embeddings.word_embeddings.weight"].nbytes
+        assert 0.82 * image < st["host_transfer_bytes"] < 0.91 * image
+        if keep:
+            assert st["host_image_bytes"] == image
+        else:
+            assert table <= st["host_image_bytes"] < table + (1 << 20)   # the table (plus alignment), nothing else
+        host = s.host_weights(3)
+        _assert_host_store_holds_the_upload(s, fn, host)
+        for _ in range(3):
+            fn.unload()
+            cold = fn.invoke([ids])
+            assert s.swap_stats(3)["host_gathers"] == 1
+            for a, b in zip(first, cold):
+                assert np.array_equal(a, b)
+            assert np.array_equal(s.readback_weights(3), host)
+        assert np.array_equal(s.host_weights(3), host)
+        fn.unload()
+
+
 @pytest.mark.parametrize("pack", [True, False])
 def test_packed_transfer_is_lossless_for_any_bits(pack, monkeypatch):
     """Weights cross the link in the packed format and are expanded on the device.  Doctored tensors
@@ -156,6 +201,11 @@ def test_packed_transfer_is_lossless_for_any_bits(pack, monkeypatch):
         host = s.host_weights(2).copy()
         image = s.model_info(2)["image_bytes"]
         assert np.array_equal(s.readback_weights(2), host)
+        _assert_host_store_holds_the_upload(s, fn, host)
+        st = s.pool_stats()
+        # packed: the transfer image is the host store (the raw image was released after decoding back to it)
+        assert st["host_image_bytes"] == (0 if pack else image)
+        assert (0.82 * image < st["host_transfer_bytes"] < 0.91 * image) if pack else st["host_transfer_bytes"] == 0
         for _ in range(3):
             fn.unload()
             cold = fn.invoke([x])

@@ -135,6 +135,14 @@ struct Model {
     // [block table][extension stream][payload].  Null when the image travels as it is.
     uint8_t* timg = nullptr;
     uint64_t timg_bytes = 0;
+    // Once the transfer image exists and has been decoded back to the image bit for bit, the image itself is
+    // given up (host_image == nullptr): the host store of such a model is its transfer image, plus a raw copy
+    // of the tables looked up by index -- image bytes [gather_off, image_bytes) -- that lookups read in place
+    // during a swap-in.  host_view is where tp_host_weights decodes the image to when asked.
+    uint8_t* gather_image = nullptr;
+    uint8_t* gather_dev = nullptr;
+    uint64_t gather_off = 0, gather_bytes = 0;
+    std::vector<uint8_t> host_view;
     std::vector<uint32_t> image_order; // params[] indices by image_off
     std::vector<hipEvent_t> dma_ev;    // transfer group arrived in the staging area (packed transfers)
     int next_rank = 0;
@@ -266,6 +274,9 @@ private:
     int resolve(Model& m, uint64_t va, uint64_t span, bool optional, void** out, bool gather = false);
     bool landed(Model& m, uint32_t idx);
     int build_transfer(Model& m);
+    int slim_host_store(Model& m);
+    bool decode_transfer(const Model& m, uint8_t* image_out, const uint8_t* expect);
+    void free_host_store(Model& m);
     uint64_t xfer_off(const Model& m, uint64_t image_off) const;
     void free_transfer(Model& m);
     int copy_chunk_packed(Model& m, size_t i, uint64_t beg, uint64_t end, hipStream_t cs, bool do_dma, bool do_expand);
@@ -333,6 +344,7 @@ private:
     hipEvent_t stage_free_ev_ = nullptr;  // the last expansion that read the staging area
     bool stage_used_ = false;
     bool pack_ = true;
+    bool slim_host_ = true;  // give up the raw image of a model whose transfer image decodes back to it
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
     bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor

@@ -23,6 +23,7 @@ FLAG_HOST_ONLY = 1
 FLAG_EVICT_LRU = 2   # plain LRU instead of the two-class policy (as env EVICT_POLICY=LRU)
 FLAG_NO_PACK = 8   # weights cross the link as they are
 FLAG_NO_HOST_GATHER = 4   # embedding lookups wait for their table instead of reading it from host memory
+FLAG_KEEP_HOST_IMAGE = 16   # keep the raw weight image in pinned memory beside the packed transfer image
 
 
 def _chk(code, what):
@@ -49,7 +50,8 @@ def gemm_noalloc(x, y, c, m, n, k, xs_r, ys_c, ldc, xs_k=1, ys_k=1, nb0=1, nb1=1
 
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
-                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True, pack=True):
+                 device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True, pack=True,
+                 keep_host_image=False):
         self._l = _lib.lib()
         cfg = _lib.Config()
         cfg.struct_size = C.sizeof(_lib.Config)
@@ -60,7 +62,8 @@ class Server:
         cfg.chunk_max_bytes = chunk_max_bytes
         cfg.workspace_bytes = workspace_bytes
         cfg.flags = (FLAG_HOST_ONLY if host_only else 0) | (FLAG_EVICT_LRU if evict_lru else 0) | \
-            (0 if host_gather else FLAG_NO_HOST_GATHER) | (0 if pack else FLAG_NO_PACK)
+            (0 if host_gather else FLAG_NO_HOST_GATHER) | (0 if pack else FLAG_NO_PACK) | \
+            (FLAG_KEEP_HOST_IMAGE if keep_host_image else 0)
         cfg.request_timeout_ms = request_timeout_ms
         cfg.copy_streams = copy_streams
         h = C.c_void_p()
