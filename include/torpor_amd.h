@@ -342,8 +342,8 @@ int tp_get_swap_stats(tp_server* s, int32_t client, tp_swap_stats* out);
 /* Copies the device-resident weight image (waits for an in-flight swap-in). */
 int tp_readback_weights(tp_server* s, int32_t client, void* dst, uint64_t bytes);
 /* The authoritative host copy of the same image, same layout.  For a model whose host store is its packed
- * transfer image the image is decoded into a buffer of the engine's; *ptr stays valid until the next call for
- * the same function (or its re-registration / the server's destruction). */
+ * transfer image the image is decoded into a buffer of the engine's; *ptr stays valid until the next
+ * tp_host_weights call on this server (or the server's destruction). */
 int tp_host_weights(tp_server* s, int32_t client, const void** ptr, uint64_t* bytes);
 /* Image offset of a weight virtual address (first-access-order layout). */
 int tp_weight_offset(tp_server* s, int32_t client, uint64_t vaddr, uint64_t* image_off);

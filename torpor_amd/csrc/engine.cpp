@@ -880,7 +880,6 @@ void Engine::free_host_store(Model& m) {
     host_free(m.gather_image);
     m.host_image = m.host_image_dev = m.timg = m.gather_image = m.gather_dev = nullptr;
     m.timg_bytes = m.gather_off = m.gather_bytes = 0;
-    std::vector<uint8_t>().swap(m.host_view);
 }
 
 void Engine::free_transfer(Model& m) {
@@ -2660,11 +2659,11 @@ int Engine::host_weights(int client, const void** ptr, uint64_t* bytes) {
         return 0;
     }
     if (!m->timg) return TP_ESTATE;
-    // the host store is the transfer image: decode it (the view stays valid until the next call for this model)
+    // the host store is the transfer image: decode it into the engine's one view buffer
     if (ptr) {
-        m->host_view.assign(m->image_bytes, 0);
-        if (!decode_transfer(*m, m->host_view.data(), nullptr)) return TP_ESTATE;  // cannot happen: it decoded at registration
-        *ptr = m->host_view.data();
+        host_view_.assign(m->image_bytes, 0);
+        if (!decode_transfer(*m, host_view_.data(), nullptr)) return TP_ESTATE;  // cannot happen: it decoded at registration
+        *ptr = host_view_.data();
     }
     if (bytes) *bytes = m->image_bytes;
     return 0;

@@ -138,11 +138,10 @@ struct Model {
     // Once the transfer image exists and has been decoded back to the image bit for bit, the image itself is
     // given up (host_image == nullptr): the host store of such a model is its transfer image, plus a raw copy
     // of the tables looked up by index -- image bytes [gather_off, image_bytes) -- that lookups read in place
-    // during a swap-in.  host_view is where tp_host_weights decodes the image to when asked.
+    // during a swap-in.
     uint8_t* gather_image = nullptr;
     uint8_t* gather_dev = nullptr;
     uint64_t gather_off = 0, gather_bytes = 0;
-    std::vector<uint8_t> host_view;
     std::vector<uint32_t> image_order; // params[] indices by image_off
     std::vector<hipEvent_t> dma_ev;    // transfer group arrived in the staging area (packed transfers)
     int next_rank = 0;
@@ -345,6 +344,7 @@ private:
     bool stage_used_ = false;
     bool pack_ = true;
     bool slim_host_ = true;  // give up the raw image of a model whose transfer image decodes back to it
+    std::vector<uint8_t> host_view_;  // where tp_host_weights decodes such a model's image to (one at a time)
     int copy_streams_cfg_ = 0;
     bool chunk_max_auto_ = true;
     bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor
