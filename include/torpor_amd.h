@@ -150,20 +150,6 @@ typedef struct tp_gemm_desc {
     tp_epilogue ep;
 } tp_gemm_desc;
 
-/* A LayerNorm between two GEMMs without a launch of its own (tp_gemm_ln; unbatched GEMMs).  The GEMM that
- * produces the LayerNorm's input stores row statistics beside its output (stats_out); the GEMM that consumes the
- * LayerNorm's output normalises its X operand while loading it (a_*) and writes the normalised rows out as well.
- * Shapes for which the kernels have no such variant run the same arithmetic with launches of their own. */
-typedef struct tp_gemm_ln_desc {
-    uint64_t stats_out; /* 0, or [m][n/32][2] floats: per row of C and block of 32 columns, mean and sum of squared
-                         * deviations of the block (n a multiple of 32, ep.act == TP_ACT_NONE) */
-    uint64_t a_stats;   /* 0, or the statistics [m][k/32][2] a previous tp_gemm_ln stored for the rows of X */
-    uint64_t a_gamma;   /* [k] */
-    uint64_t a_beta;    /* [k] */
-    uint64_t a_out;     /* [m][k]: receives (x - mean) / sqrt(var + a_eps) * gamma + beta, the operand actually multiplied */
-    float a_eps;
-} tp_gemm_ln_desc;
-
 typedef struct tp_conv_desc {
     uint64_t x, w, y; /* w is [Cout][Cin][KH][KW] */
     int32_t n, h, w_in, cin, cout, kh, kw;
@@ -303,9 +289,6 @@ int tp_sgemm_strided_batched(tp_server* s, int32_t client, int32_t transa, int32
                              int32_t count);
 /* Row-major GEMM with fused epilogue and two-level batching (the HIP-native form of the two above). */
 int tp_gemm(tp_server* s, int32_t client, const tp_gemm_desc* d);
-/* tp_gemm with a LayerNorm folded into it on either side (no counterpart in the reference, which forwards the
- * LayerNorm of cuda_server.hpp:1226-1310 as a launch of its own between the two cublasSgemm calls). */
-int tp_gemm_ln(tp_server* s, int32_t client, const tp_gemm_desc* d, const tp_gemm_ln_desc* ln);
 /* cudnnConvolutionForwardService (cuda_server.hpp:708-735), shapes inline instead of descriptor
  * handles (cuda_server.hpp:579-706), optional fused epilogue. */
 int tp_conv_forward(tp_server* s, int32_t client, const tp_conv_desc* d);

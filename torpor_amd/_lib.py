@@ -61,11 +61,6 @@ class GemmDesc(C.Structure):
     ]
 
 
-class GemmLnDesc(C.Structure):
-    _fields_ = [("stats_out", C.c_uint64), ("a_stats", C.c_uint64), ("a_gamma", C.c_uint64), ("a_beta", C.c_uint64),
-                ("a_out", C.c_uint64), ("a_eps", C.c_float)]
-
-
 class ConvDesc(C.Structure):
     _fields_ = [
         ("x", C.c_uint64), ("w", C.c_uint64), ("y", C.c_uint64),
@@ -138,7 +133,6 @@ SYMBOLS = {
     "tp_sgemm_strided_batched": (C.c_int, [_P, _I32, _I32, _I32, _I32, _I32, _I32, C.c_float, _U64, _I32, _I64,
                                            _U64, _I32, _I64, C.c_float, _U64, _I32, _I64, _I32]),
     "tp_gemm": (C.c_int, [_P, _I32, C.POINTER(GemmDesc)]),
-    "tp_gemm_ln": (C.c_int, [_P, _I32, C.POINTER(GemmDesc), C.POINTER(GemmLnDesc)]),
     "tp_gemm_noalloc": (C.c_int, [C.POINTER(GemmDesc), _P]),
     "tp_conv_forward": (C.c_int, [_P, _I32, C.POINTER(ConvDesc)]),
     "tp_bn_inference": (C.c_int, [_P, _I32, _U64, _U64, _U64, _U64, _U64, _U64, C.c_double, _I64, _I32, _I64,

@@ -216,33 +216,6 @@ int tp_gemm(tp_server* s, int32_t client, const tp_gemm_desc* d) {
     TP_GUARD_END
 }
 
-int tp_gemm_ln(tp_server* s, int32_t client, const tp_gemm_desc* d, const tp_gemm_ln_desc* ln) {
-    TP_GUARD_BEGIN
-    ENG(s);
-    if (!d || !ln) return TP_EINVAL;
-    if (ln->a_stats && (!ln->a_gamma || !ln->a_beta || !ln->a_out)) return TP_EINVAL;
-    tp::Op op;
-    op.kind = tp::OPK_GEMM;
-    op.p[0] = d->x;
-    op.p[1] = d->y;
-    op.p[2] = d->c;
-    const int64_t iv[16] = {d->m,   d->n,   d->k,   d->xs_r, d->xs_k, d->ys_c, d->ys_k, d->ldc,
-                            d->nb0, d->nb1, d->xb0, d->xb1,  d->yb0,  d->yb1,  d->cb0,  d->cb1};
-    for (int k = 0; k < 16; ++k) op.i[k] = iv[k];
-    fill_epilogue(op, d->ep, 3, 16);
-    op.p[9] = ln->stats_out;
-    op.p[10] = ln->a_stats;
-    op.p[11] = ln->a_gamma;
-    op.p[12] = ln->a_beta;
-    op.p[13] = ln->a_out;
-    op.f[3] = ln->a_eps;
-    op.np = 14;
-    op.ni = 18;
-    op.nf = 4;
-    return E.op_compute(client, op);
-    TP_GUARD_END
-}
-
 // Column-major C(m x n) = alpha*op(A)*op(B) + beta*C is the row-major product
 // C'[j][i] = sum_k X(j,k) * Y(i,k) with X(j,k) = op(B)(k,j) and Y(i,k) = op(A)(i,k).
 static int sgemm_common(tp_server* s, int32_t client, int transa, int transb, int m, int n, int k, float alpha,

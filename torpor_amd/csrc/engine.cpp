@@ -1894,13 +1894,13 @@ static tpk::EpilogueArgs ep_from(const Op& op, void* const* q, int pbase, int fb
 }
 
 // Layout of Op for the compute kinds (filled by the C-ABI layer):
-//  GEMM  p: x y c bias bns bnb bnm bnv res [ln_stats_out ln_a_stats ln_a_gamma ln_a_beta ln_a_out]
-//        i: m n k xs_r xs_k ys_c ys_k ldc nb0 nb1 xb0 xb1 yb0 yb1 cb0 cb1 ldr act   f: alpha beta eps [ln_a_eps]
+//  GEMM  p: x y c bias bns bnb bnm bnv res   i: m n k xs_r xs_k ys_c ys_k ldc nb0 nb1 xb0 xb1 yb0 yb1 cb0 cb1 ldr act
+//        f: alpha beta eps
 //  CONV  p: x w y bias bns bnb bnm bnv res   i: n h w cin cout kh kw sh sw ph pw xl yl ldr act   f: alpha beta eps
 //  BN    p: x y g b mean var                 i: rows C hw layout relu   f: eps
 //  LAUNCH p/i/f per op id (see torpor_amd.h)
 int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
-    void* q[16] = {nullptr};
+    void* q[12] = {nullptr};
     // The scratch allocation: 256 bytes that stay zero for good (padding source of the 3x3
     // convolution), the ticket counters of split K ranges (zero between launches), then the partial
     // sums.  No device workspace in host-only mode (nothing is launched there).
@@ -1995,25 +1995,6 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             g.cb1 = (long)I[15];
             g.ep = ep_from(op, q, 3, 0, 16);
             g.ep.ldr = (long)ldr;
-            if (op.np > 9 && (op.p[9] || op.p[10])) {  // a LayerNorm folded into this GEMM (tp_gemm_ln)
-                if (nb0 * nb1 != 1) return TP_EUNSUPPORTED;
-                if (op.p[9]) {  // statistics of the output rows, [M][N/32][2]
-                    if (N % 32 != 0 || I[17] != 0) return TP_EINVAL;
-                    if ((r = R(9, false, M * (N / 32) * 2))) return r;
-                    g.ln.stats_out = static_cast<float*>(q[9]);
-                }
-                if (op.p[10]) {  // X normalised on load from statistics [M][K/32][2]; gamma, beta [K]; rows also to a_out [M][K]
-                    if (K < 32 || K % 32 != 0 || I[3] != K || I[4] != 1) return TP_EINVAL;
-                    if ((r = R(10, false, M * (K / 32) * 2)) || (r = R(11, false, K)) || (r = R(12, false, K)) ||
-                        (r = R(13, false, M * K)))
-                        return r;
-                    g.ln.a_stats = static_cast<const float*>(q[10]);
-                    g.ln.a_gamma = static_cast<const float*>(q[11]);
-                    g.ln.a_beta = static_cast<const float*>(q[12]);
-                    g.ln.a_out = static_cast<float*>(q[13]);
-                    g.ln.a_eps = op.f[3];
-                }
-            }
             if (!launch) return 0;
             return tpk::launch_gemm(g, ws, compute_);
         }

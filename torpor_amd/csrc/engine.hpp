@@ -54,7 +54,7 @@ struct Op {
     int kind = 0;
     int op_id = 0;
     int np = 0, ni = 0, nf = 0;
-    uint64_t p[16] = {0};
+    uint64_t p[12] = {0};
     int64_t i[20] = {0};
     float f[4] = {0};
 };

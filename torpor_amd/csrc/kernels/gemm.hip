@@ -56,16 +56,6 @@ struct GemmDev {
         unsigned short r0, c0, w, h;
     } rect[8];
     Epilogue ep;
-    // LayerNorm applied to the X operand on its way into LDS (a_stats non-null: on).  a_stats holds, per row of
-    // X and per block of 32 of its K columns, (mean, sum of squared deviations) as a preceding GEMM's write-out
-    // stored them (Epilogue::ln_stats); gamma / beta are [K]; the workgroups of tile column 0 also write the
-    // normalised rows to a_out ([M][K], dense), where later launches find them.
-    const float* a_stats;
-    const float* a_gamma;
-    const float* a_beta;
-    float* a_out;
-    float a_eps;
-    int a_nblk;
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id; remap so that
@@ -120,12 +110,6 @@ __device__ __forceinline__ void fetch_now(const GemmDev& p) {
     fetch_now(p.tiles_n);
     fetch_now(p.xr);
     fetch_now(p.ep);
-    fetch_now(p.a_stats);
-    fetch_now(p.a_gamma);
-    fetch_now(p.a_beta);
-    fetch_now(p.a_out);
-    fetch_now(p.a_eps);
-    fetch_now(p.a_nblk);
 }
 
 __device__ __forceinline__ long gather_row(const GemmDev& p, long grow) {
@@ -294,15 +278,14 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
 // (their products are computed and thrown away at the store) and the look-ahead loads past the
 // end of K are clamped to the last K-block, so the loop body has no predication and no control
 // flow: loads, LDS traffic and MFMAs can be interleaved freely by the scheduler.
-template <class C, bool YKC, int STAGES, bool LNA = false>
+template <class C, bool YKC, int STAGES>
 #ifndef TP_CLEAN_OCC
 #define TP_CLEAN_OCC (C::TM * C::TN >= 4 ? 1 : 2)
 #endif
 __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(const GemmDev p) {
     fetch_now(p);
     constexpr int RED_FLOATS = red_floats<C>();  // K-slice reduction area, then the epilogue staging blocks
-    constexpr int MAIN_FLOATS = cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4);
-    __shared__ __attribute__((aligned(16))) float lds[MAIN_FLOATS + (LNA ? 2 * C::BM : 0)];
+    __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
     TP_CLK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
@@ -363,56 +346,9 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     }
     const long ystep = YKC ? 1 : p.ys_k;
 
-    // LayerNorm of the X operand: mean and 1/sigma of this tile's rows from the per-block statistics a preceding
-    // launch left (blocks of 32 columns, equal weight: the means average, the squared deviations add up together
-    // with 32 x the squared distance of each block mean from the row mean), THREADS / BM threads per row.
-    float mu[NVA], rs[NVA];
-    const int kqa = tid % KV;  // the same k quad for every vector this thread moves (THREADS % KV == 0)
-    if constexpr (LNA) {
-        static_assert(C::THREADS % C::BM == 0 && C::THREADS % KV == 0, "row / k assignment of the LayerNorm prologue");
-        constexpr int TPR = C::THREADS / C::BM;
-        float* rowstat = lds + MAIN_FLOATS;
-        const int srow = tid / TPR, part = tid - srow * TPR;
-        long grow = m0 + srow;
-        if (grow > p.M - 1) grow = p.M - 1;
-        const float2* sp = reinterpret_cast<const float2*>(p.a_stats) + grow * p.a_nblk;
-        float s1 = 0.f;
-        for (int b = part; b < p.a_nblk; b += TPR) s1 += sp[b].x;
-#pragma unroll
-        for (int o = 1; o < TPR; o <<= 1) s1 += __shfl_xor(s1, o);
-        const float mean = s1 / (float)p.a_nblk;
-        float s2 = 0.f;
-        for (int b = part; b < p.a_nblk; b += TPR) {
-            const float2 v = sp[b];
-            const float d = v.x - mean;
-            s2 += v.y + 32.0f * d * d;
-        }
-#pragma unroll
-        for (int o = 1; o < TPR; o <<= 1) s2 += __shfl_xor(s2, o);
-        if (part == 0) {
-            rowstat[2 * srow] = mean;
-            rowstat[2 * srow + 1] = 1.0f / sqrtf(s2 / (32.0f * (float)p.a_nblk) + p.a_eps);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < NVA; ++i) {
-            const int row = (i * C::THREADS + tid) / KV;
-            mu[i] = rowstat[2 * row];
-            rs[i] = rowstat[2 * row + 1];
-        }
-    }
-    const bool ln_write = LNA && tn == 0 && p.a_out != nullptr;
-
     f32x16 acc[C::TM][C::TN];
     zero_acc<C>(acc);
     f32x4 ra0[NVA], rb0[NVB], ra1[NVA], rb1[NVB];
-    // gamma / beta of the K-block that goes to LDS next (LNA only): K-blocks are stored in order, and the pair
-    // for the following block is requested right after each store, half an iteration before it is needed
-    f32x4 rg, rt;
-    if constexpr (LNA) {
-        rg = *reinterpret_cast<const f32x4*>(p.a_gamma + kbeg + kqa * 4);
-        rt = *reinterpret_cast<const f32x4*>(p.a_beta + kbeg + kqa * 4);
-    }
 
     auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0) {
         const long k = k0 < klast ? k0 : klast;
@@ -421,25 +357,9 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
 #pragma unroll
         for (int i = 0; i < NVB; ++i) rb[i] = *reinterpret_cast<const f32x4*>(pb[i] + k * ystep);
     };
-    // kblk: first K index of the block these registers hold (the look-ahead past the end re-reads the last
-    // block; such a block is stored to LDS but neither multiplied nor written out)
-    auto store_lds = [&](f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage, long kblk) {
+    auto store_lds = [&](const f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage) {
         float* As = lds + stage * C::LDS_FLOATS;
         float* Bs = As + C::BM * C::LDK;
-        if constexpr (LNA) {
-#pragma unroll
-            for (int i = 0; i < NVA; ++i) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) ra[i][c] = (ra[i][c] - mu[i]) * rs[i] * rg[c] + rt[c];
-                if (ln_write && kblk < kend) {
-                    const long grow = m0 + (i * C::THREADS + tid) / KV;
-                    if (grow < p.M) *reinterpret_cast<f32x4*>(p.a_out + grow * p.K + kblk + kqa * 4) = ra[i];
-                }
-            }
-            const long kn = kblk + C::BK < klast ? kblk + C::BK : klast;
-            rg = *reinterpret_cast<const f32x4*>(p.a_gamma + kn + kqa * 4);
-            rt = *reinterpret_cast<const f32x4*>(p.a_beta + kn + kqa * 4);
-        }
 #pragma unroll
         for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[i];
 #pragma unroll
@@ -461,16 +381,16 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
         if (wk == 0) cols_fold<C>(cc, p.ep);
-        store_lds(ra0, rb0, 0, kbeg);
+        store_lds(ra0, rb0, 0);
         __syncthreads();
         for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
             load_regs(ra0, rb0, k0 + 2 * C::BK);
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
-            store_lds(ra1, rb1, 1, k0 + C::BK);
+            store_lds(ra1, rb1, 1);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
             mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);
-            store_lds(ra0, rb0, 0, k0 + 2 * C::BK);
+            store_lds(ra0, rb0, 0);
             __syncthreads();
         }
         // an odd last K-block is in stage 0 by now (kept out of the loop: a branch there costs 10 %)
@@ -482,19 +402,19 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         load_regs(ra1, rb1, kbeg + C::BK);
         if (wk == 0) cols_fold<C>(cc, p.ep);
         for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
-            store_lds(ra0, rb0, 0, k0);
+            store_lds(ra0, rb0, 0);
             __syncthreads();
             load_regs(ra0, rb0, k0 + 2 * C::BK);
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
-            store_lds(ra1, rb1, 0, k0 + C::BK);
+            store_lds(ra1, rb1, 0);
             __syncthreads();
             load_regs(ra1, rb1, k0 + 3 * C::BK);
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
         }
         if (kpairs < kend) {  // odd last K-block: it is in the first register set
-            store_lds(ra0, rb0, 0, kpairs);
+            store_lds(ra0, rb0, 0);
             __syncthreads();
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
@@ -632,8 +552,6 @@ Epilogue make_epilogue(const EpilogueArgs& a, long ldc) {
     e.out_nchw = 0;
     e.howo = 1;
     e.ncols = 0;
-    e.ln_stats = nullptr;
-    e.ln_nblk = 0;
     return e;
 }
 
@@ -702,15 +620,6 @@ static int launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipSt
     const long tiles = (long)p.tiles_m * p.tiles_n * grid.z;
     static const int dbg_st = getenv("TORPOR_GEMM_STAGES") ? atoi(getenv("TORPOR_GEMM_STAGES")) : 0;
     const bool one_stage = dbg_st ? dbg_st == 1 : tiles >= 5L * g_num_cu;
-    if (clean && y_kc && p.a_stats) {  // LayerNorm on the X operand (the caller has checked that this tile has the variant)
-        if constexpr (C::TM * C::TN == 1) {
-            if (one_stage)
-                hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1, true>), grid, dim3(C::THREADS), 0, s, p);
-            else
-                hipLaunchKernelGGL((gemm_clean_kernel<C, true, 2, true>), grid, dim3(C::THREADS), 0, s, p);
-        }
-        return one_stage ? 1 : 2;
-    }
     if (clean && one_stage) {
         if (y_kc)
             hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
@@ -736,10 +645,6 @@ static int launch_fast(const GemmDev& p, bool y_kc, bool clean, dim3 grid, hipSt
 template <class C>
 static int launch_clean_only(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t s) {
     static const int dbg_st = getenv("TORPOR_GEMM_STAGES") ? atoi(getenv("TORPOR_GEMM_STAGES")) : 0;
-    if (y_kc && p.a_stats) {
-        hipLaunchKernelGGL((gemm_clean_kernel<C, true, 2, true>), grid, dim3(C::THREADS), 0, s, p);
-        return 2;
-    }
     if (dbg_st == 1) {
         if (y_kc)
             hipLaunchKernelGGL((gemm_clean_kernel<C, true, 1>), grid, dim3(C::THREADS), 0, s, p);
@@ -917,67 +822,10 @@ long gemm_workspace_need(const GemmArgs& a) {
     return g.splits > 1 ? (long)g.splits * g.tiles_m * g.tiles_n * g.bm * g.bn * (long)sizeof(float) : 0;
 }
 
-// Fallback for Epilogue::ln_stats when the write-out of the chosen kernel cannot produce them: the same
-// per-block statistics from the finished output, one thread per (row, block of 32 columns).
-__global__ __launch_bounds__(256) void row_block_stats_kernel(const float* __restrict__ C, long ldc, long M, int nblk,
-                                                              float* __restrict__ stats) {
-    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= M * nblk) return;
-    const long row = i / nblk;
-    const int b = (int)(i - row * nblk);
-    const float* x = C + row * ldc + b * 32;
-    float sum = 0.f;
-    for (int c = 0; c < 32; ++c) sum += x[c];
-    const float mean = sum * (1.0f / 32.0f);
-    float m2 = 0.f;
-    for (int c = 0; c < 32; ++c) m2 += (x[c] - mean) * (x[c] - mean);
-    stats[i * 2] = mean;
-    stats[i * 2 + 1] = m2;
-}
-
 int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     if (!gemm_args_ok(a)) return K_EINVAL;
     const int batch = a.nb0 * a.nb1;
     const GemmPlan g = plan_gemm(a, ws.ptr ? ws.bytes : 0);
-    const bool want_lna = a.ln.a_stats != nullptr, want_stats = a.ln.stats_out != nullptr;
-    if (want_lna || want_stats) {
-        if (batch != 1 || a.gather) return K_EUNSUPPORTED;
-        if (want_stats && (a.N % 32 != 0 || a.ep.act != 0)) return K_EINVAL;
-        if (want_lna && (!a.ln.a_gamma || !a.ln.a_beta || !a.ln.a_out || a.K % 32 != 0 || a.K < 32 || a.xs_r != a.K ||
-                         a.xs_k != 1))
-            return K_EINVAL;
-    }
-    // whole K-blocks (the condition of the branch-free kernels, as below)
-    const long kq_plan = g.cfg >= 3 ? 64 : 32;
-    const bool clean_plan = getenv("TORPOR_GEMM_NOCLEAN") == nullptr && g.fast && a.K >= kq_plan && a.K % kq_plan == 0 &&
-                            (g.splits == 1 || g.kper % 64 == 0) && (g.y_kc || (a.N % 4 == 0 && a.N >= 4));
-    if (want_lna && !(clean_plan && g.y_kc && g.cfg >= 2 && aligned16(a.ln.a_gamma) && aligned16(a.ln.a_beta) &&
-                      aligned16(a.ln.a_out) && aligned16(a.ln.a_stats))) {
-        // no kernel variant for this shape: a LayerNorm launch of its own, then the GEMM on its output
-        int r = launch_layernorm(a.X, nullptr, a.ln.a_gamma, a.ln.a_beta, a.ln.a_out, a.M, (int)a.K, a.ln.a_eps, s);
-        if (r) return r;
-        GemmArgs b = a;
-        b.X = a.ln.a_out;
-        b.ln.a_stats = nullptr;
-        return launch_gemm(b, ws, s);
-    }
-    if (want_stats) {
-        const bool fused_finish = g.splits == 1 || split_tickets(ws, (long)g.tiles_m * g.tiles_n, g.splits) != nullptr;
-        const bool vec = a.ep.beta == 0.f && (a.ldc & 3) == 0 && aligned16(a.C) && (!a.ep.bias || aligned16(a.ep.bias)) &&
-                         (!a.ep.bn_scale || (aligned16(a.ep.bn_scale) && aligned16(a.ep.bn_var) && aligned16(a.ep.bn_mean) &&
-                                             aligned16(a.ep.bn_bias))) &&
-                         (!a.ep.residual || (((a.ep.ldr ? a.ep.ldr : a.ldc) & 3) == 0 && aligned16(a.ep.residual)));
-        if (!(g.fast && fused_finish && vec && a.N % g.bn == 0 && aligned16(a.ln.stats_out))) {
-            GemmArgs b = a;
-            b.ln.stats_out = nullptr;
-            int r = launch_gemm(b, ws, s);
-            if (r) return r;
-            const long n = a.M * (a.N / 32);
-            hipLaunchKernelGGL(row_block_stats_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.C, a.ldc, a.M,
-                               (int)(a.N / 32), a.ln.stats_out);
-            return (int)hipGetLastError();
-        }
-    }
     GemmDev p;
     p.X = a.X;
     p.Y = a.Y;
@@ -1005,14 +853,6 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     p.sw = a.sw;
     p.ws = ws.ptr;
     p.ep = make_epilogue(a.ep, a.ldc);
-    p.ep.ln_stats = a.ln.stats_out;
-    p.ep.ln_nblk = (int)(a.N / 32);
-    p.a_stats = a.ln.a_stats;
-    p.a_gamma = a.ln.a_gamma;
-    p.a_beta = a.ln.a_beta;
-    p.a_out = a.ln.a_out;
-    p.a_eps = a.ln.a_eps;
-    p.a_nblk = (int)(a.K / 32);
     p.tickets = split_tickets(ws, (long)g.tiles_m * g.tiles_n, g.splits);
 
     p.tiles_m = g.tiles_m;

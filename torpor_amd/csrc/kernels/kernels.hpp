@@ -39,21 +39,6 @@ struct GemmArgs {
     // (n*Ho + ho)*Wo + wo reads X row ((n*H + ho*sh)*W + wo*sw).
     int gather = 0, Ho = 0, Wo = 0, H = 0, W = 0, sh = 1, sw = 1;
     EpilogueArgs ep;
-    // A LayerNorm between two GEMMs without a launch of its own (unbatched, row-major GEMMs only).
-    // stats_out: this GEMM also stores, per row of C and per block of 32 columns, the block's mean and its sum
-    //   of squared deviations, [M][N/32][2] floats (N a multiple of 32, no activation).
-    // a_stats (with a_gamma, a_beta [K], a_eps, a_out [M][K]): X is normalised row by row on its way into the
-    //   multiplication -- (x - mean) / sqrt(var + eps) * gamma + beta with mean and var from the statistics
-    //   [M][K/32][2] that the GEMM which produced X stored -- and the normalised rows are written to a_out as
-    //   well; X must be dense (xs_r == K, xs_k == 1), K a multiple of 32.
-    struct LnFuse {
-        float* stats_out = nullptr;
-        const float* a_stats = nullptr;
-        const float* a_gamma = nullptr;
-        const float* a_beta = nullptr;
-        float* a_out = nullptr;
-        float a_eps = 1e-5f;
-    } ln;
 };
 
 struct ConvArgs {

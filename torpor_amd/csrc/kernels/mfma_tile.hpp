@@ -49,11 +49,6 @@ struct Epilogue {
     int out_nchw;
     long howo;
     long ncols;
-    // Row statistics for a LayerNorm that a following GEMM applies to this output while loading it (non-null:
-    // on): for every row and every block of 32 columns, the block's mean and its sum of squared deviations
-    // from that mean, at ln_stats[(row * ln_nblk + block) * 2 .. +1].  Written by the vector write-out only.
-    float* ln_stats;
-    int ln_nblk;
 };
 
 __device__ __forceinline__ void fetch_now(const Epilogue& e) {
@@ -70,8 +65,6 @@ __device__ __forceinline__ void fetch_now(const Epilogue& e) {
     fetch_now(e.act);
     fetch_now(e.ldc);
     fetch_now(e.out_nchw);
-    fetch_now(e.ln_stats);
-    fetch_now(e.ln_nblk);
 }
 
 __device__ __forceinline__ float apply_act(float v, int act) {
@@ -384,7 +377,7 @@ __device__ __forceinline__ void cols_fold(ColConsts<C::TN>& cc, const Epilogue& 
 // no load sits under a branch (that makes the compiler wait for every outstanding memory operation
 // at the join, stores included) and no branch is taken per element.  RES: add a residual tensor
 // (rows clamped for the load, the store is predicated).  RAW: split-K partial sums, no epilogue.
-template <class C, bool RES, bool RAW, int ACT, bool STATS = false>
+template <class C, bool RES, bool RAW, int ACT>
 __device__ __forceinline__ void store_tile_rows(f32x16 (&acc)[C::TM][C::TN], int wm, int wn, int lane, long m0, long n0,
                                                 long M, float* __restrict__ out, long pitch, const Epilogue& e,
                                                 float* __restrict__ stage, const ColConsts<C::TN>& cc) {
@@ -423,24 +416,6 @@ __device__ __forceinline__ void store_tile_rows(f32x16 (&acc)[C::TM][C::TN], int
                         x[it][c] = act_fixed<ACT>(y);
                     }
                 }
-                if (STATS) {
-                    // the eight lanes that share this row hold its 32 columns of the block, four each
-                    float sum = (x[it][0] + x[it][1]) + (x[it][2] + x[it][3]);
-                    sum += __shfl_xor(sum, 1);
-                    sum += __shfl_xor(sum, 2);
-                    sum += __shfl_xor(sum, 4);
-                    const float mean = sum * (1.0f / 32.0f);
-                    const float d0 = x[it][0] - mean, d1 = x[it][1] - mean, d2 = x[it][2] - mean, d3 = x[it][3] - mean;
-                    float m2 = (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
-                    m2 += __shfl_xor(m2, 1);
-                    m2 += __shfl_xor(m2, 2);
-                    m2 += __shfl_xor(m2, 4);
-                    if ((lane & 7) == 0 && row < M) {
-                        float* sp = e.ln_stats + (row * e.ln_nblk + (col >> 5)) * 2;
-                        sp[0] = mean;
-                        sp[1] = m2;
-                    }
-                }
                 if (row < M) *reinterpret_cast<f32x4*>(out + row * pitch + col) = x[it];
             }
             wave_lds_sync();
@@ -463,12 +438,7 @@ __device__ __forceinline__ void store_tile_vec(f32x16 (&acc)[C::TM][C::TN], int 
         case ACT_RELU6: store_tile_rows<C, RES, false, ACT_RELU6>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
         case ACT_SILU: store_tile_rows<C, RES, false, ACT_SILU>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
         case ACT_SIGMOID: store_tile_rows<C, RES, false, ACT_SIGMOID>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
-        default:
-            if (e.ln_stats)
-                store_tile_rows<C, RES, false, ACT_NONE, true>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc);
-            else
-                store_tile_rows<C, RES, false, ACT_NONE>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc);
-            break;
+        default: store_tile_rows<C, RES, false, ACT_NONE>(acc, wm, wn, lane, m0, n0, M, out, pitch, e, stage, cc); break;
     }
 }
 

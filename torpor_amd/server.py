@@ -174,21 +174,12 @@ class Server:
         ep.bn_eps, ep.residual, ep.ldr, ep.act = bn_eps, residual, ldr, act
 
     def gemm(self, fid, x, y, c, m, n, k, xs_r, ys_c, ldc, xs_k=1, ys_k=1, nb0=1, nb1=1,
-             xb0=0, xb1=0, yb0=0, yb1=0, cb0=0, cb1=0, ln_stats_out=0, ln_a=None, **ep):
-        """ln_stats_out: address that receives the row statistics of C for a LayerNorm applied by the next GEMM;
-        ln_a = (stats, gamma, beta, out, eps): LayerNorm of the X operand on load, normalised rows also to out."""
+             xb0=0, xb1=0, yb0=0, yb1=0, cb0=0, cb1=0, **ep):
         d = _lib.GemmDesc()
         d.x, d.y, d.c, d.m, d.n, d.k = x, y, c, m, n, k
         d.xs_r, d.xs_k, d.ys_c, d.ys_k, d.ldc = xs_r, xs_k, ys_c, ys_k, ldc
         d.nb0, d.nb1, d.xb0, d.xb1, d.yb0, d.yb1, d.cb0, d.cb1 = nb0, nb1, xb0, xb1, yb0, yb1, cb0, cb1
         self._epilogue(d.ep, **ep)
-        if ln_stats_out or ln_a:
-            ln = _lib.GemmLnDesc()
-            ln.stats_out = ln_stats_out
-            if ln_a:
-                ln.a_stats, ln.a_gamma, ln.a_beta, ln.a_out, ln.a_eps = ln_a
-            _chk(self._l.tp_gemm_ln(self._h, fid, C.byref(d), C.byref(ln)), "tp_gemm_ln")
-            return
         _chk(self._l.tp_gemm(self._h, fid, C.byref(d)), "tp_gemm")
 
     def sgemm(self, fid, transa, transb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc):
