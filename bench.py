@@ -457,6 +457,9 @@ def main():
         runs = {}
         for cap in args.multitenant_caps_gb:
             runs[f"cap_{cap:g}GiB"] = mt.run_cap(cap, args.multitenant_seconds, 200.0)
+        # the binding cap once more, with the models of requests that already wait prefetched (Load requests)
+        tight = min(args.multitenant_caps_gb)
+        runs[f"cap_{tight:g}GiB_lookahead1"] = mt.run_cap(tight, args.multitenant_seconds, 200.0, lookahead=1)
         line["workloads"]["multitenant-64"] = dict(
             config="32x ResNet-50 + 16x BERT-base s128 + 16x ResNet-152, seeds 0..63, batch 1, open-loop Poisson "
                    f"200 req/s, Zipf(1.1) popularity, {args.multitenant_seconds:g} s per cap; latency = completion - arrival",

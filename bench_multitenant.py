@@ -14,7 +14,10 @@ include/server/model_repo.hpp:139-140).  The 64 models total about 14 GiB charge
 24 GiB cap of the config does not force evictions; the run is therefore repeated with a binding
 cap (default 8 GiB) and both are reported.
 
-Prints one JSON line.  Usage: python bench_multitenant.py [--seconds 60] [--rate 200] [--caps-gb 24 8]
+--lookahead N: when a request starts, the models of up to N requests already waiting behind it are
+prefetched with Load requests (their swap-ins then overlap this request's compute).
+
+Prints one JSON line.  Usage: python bench_multitenant.py [--seconds 60] [--rate 200] [--caps-gb 24 8] [--lookahead 1]
 """
 import argparse
 import json
@@ -32,11 +35,13 @@ def main():
     ap.add_argument("--rate", type=float, default=200.0)
     ap.add_argument("--caps-gb", type=float, nargs="+", default=[24.0, 8.0])
     ap.add_argument("--models", type=int, nargs=3, default=[32, 16, 16], metavar=("R50", "BERT", "R152"))
+    ap.add_argument("--lookahead", type=int, default=0)
     args = ap.parse_args()
 
     from torpor_amd import multitenant as mt
 
-    runs = {f"cap_{cap:g}GiB": mt.run_cap(cap, args.seconds, args.rate, models=tuple(args.models)) for cap in args.caps_gb}
+    runs = {f"cap_{cap:g}GiB": mt.run_cap(cap, args.seconds, args.rate, models=tuple(args.models), lookahead=args.lookahead)
+            for cap in args.caps_gb}
     primary = runs[next(iter(runs))]
     print(json.dumps({
         "metric": "multi-tenant request latency p50 (ms), 64 models on 1 GPU, Poisson arrivals, Zipf(1.1) popularity",

@@ -122,3 +122,32 @@ def test_64_models_under_a_binding_cap_two_class_policy_with_levels():
 def test_64_models_under_a_binding_cap_plain_lru():
     r = _run(8.0, two_class=False)
     assert r["evictions"] > 50 and 0.3 < r["hit_ratio"] < 1.0
+
+
+def test_prefetching_the_models_of_waiting_requests_changes_no_answer():
+    """Load requests (controller.hpp:208-215) for the models of requests already waiting, issued while the current
+    request runs: every answer still equals the function's registration run bit for bit, the budget holds after
+    every request, and what is resident at the end reads back byte for byte."""
+    limit = int(1.5 * 2 ** 30)
+    with Server(mem_limit_bytes=limit, pool_bytes=2 * limit) as s:
+        fleet = mt.build_fleet(s, 8, 4, 4)
+        assert sum(s.model_info(f["fid"])["total_bytes"] for f in fleet) > 2 * limit      # the cap binds
+        # arrivals faster than the executor serves them, so that requests do wait behind one another
+        arrivals, picks = mt.make_trace(len(fleet), 600, 3000.0, seed=3)
+        over = []
+
+        def after(i, fid, hit):
+            st = s.pool_stats()
+            if st["lru_used"] > limit:
+                over.append((i, st["lru_used"]))
+
+        r0 = mt.serve(s, fleet, arrivals, picks, check_every=1, after_request=after, lookahead=0)
+        r2 = mt.serve(s, fleet, arrivals, picks, check_every=1, after_request=after, lookahead=2)
+        assert not over, over[:3]
+        assert r0["prefetches"] == 0 and r2["prefetches"] > 20, (r0["prefetches"], r2["prefetches"])
+        assert r2["hit_ratio"] > r0["hit_ratio"]
+        assert r2["fragmentation_evictions"] == 0
+        resident = [f["fid"] for f in fleet if s.resident(f["fid"])]
+        assert resident
+        for fid in resident:
+            assert np.array_equal(s.readback_weights(fid), s.host_weights(fid)), fid

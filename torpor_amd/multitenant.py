@@ -71,17 +71,26 @@ def pct(xs, q):
     return float(xs[min(len(xs) - 1, int(round(q * (len(xs) - 1))))])
 
 
-def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after_request=None, note_every_s=30.0):
+def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after_request=None, note_every_s=30.0,
+          lookahead=0):
     """Serves the trace in arrival order on the single executor.  open_loop: a request is not issued before
     its arrival time and latency = completion - arrival (queueing included); otherwise requests run back to
     back and latency is the service time.  Every `check_every`-th answer is compared bit for bit with the
-    function's registration run.  after_request(i, fid, hit) is called after each request."""
+    function's registration run.  after_request(i, fid, hit) is called after each request.
+
+    lookahead > 0 (open loop only): once a request has been started, the models of up to that many requests
+    that are already waiting behind it are asked for with a Load request (the reference's prefetch signal,
+    include/server/controller.hpp:208-215), so that their swap-ins queue behind this request's copies and
+    run while it computes.  A request whose model arrived that way counts as a hit."""
     import gc
+
+    from .server import REQ_LOAD
     n_req = len(picks)
     gc.collect()
     gc.disable()   # a collection of the interpreter inside a request (tens of milliseconds) is not the path's
     st0 = server.pool_stats()
     lat_hit, lat_miss, by_arch, swap_bytes, swap_ms = [], [], {}, 0, 0.0
+    prefetches = 0
     t0 = time.perf_counter()
     next_note = note_every_s
     for i in range(n_req):
@@ -98,6 +107,14 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
         t_req = time.perf_counter()
         ack, _, dfr = server.signal(1, fid, "")
         assert ack == 0 and not dfr
+        if lookahead and open_loop:
+            now = time.perf_counter() - t0
+            for j in range(i + 1, min(i + 1 + lookahead, n_req)):
+                if arrivals[j] > now:
+                    break
+                nxt = fleet[picks[j]]["fid"]
+                if nxt != fid and not server.resident(nxt):
+                    prefetches += server.signal(REQ_LOAD, nxt, "")[0] == 0
         server.replay(fid, f["packed"], f["outbuf"])
         done = time.perf_counter()
         lat = ((done - t0 - arrivals[i]) if open_loop else (done - t_req)) * 1e3
@@ -122,7 +139,7 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
         requests=n_req, wall_s=wall, achieved_rps=n_req / wall,
         hit_ratio=len(lat_hit) / max(n_req, 1), evictions=st1["evictions"] - st0["evictions"],
         fragmentation_evictions=st1["fragmentation_evictions"] - st0["fragmentation_evictions"],
-        swap_ins=st1["swap_ins"] - st0["swap_ins"],
+        swap_ins=st1["swap_ins"] - st0["swap_ins"], lookahead=lookahead, prefetches=int(prefetches),
         latency_ms=dict(p50=pct(all_lat, 0.5), p99=pct(all_lat, 0.99), mean=float(np.mean(all_lat)) if all_lat else None),
         hit_ms=dict(p50=pct(lat_hit, 0.5), p99=pct(lat_hit, 0.99), n=len(lat_hit)),
         miss_ms=dict(p50=pct(lat_miss, 0.5), p99=pct(lat_miss, 0.99), n=len(lat_miss)),
@@ -135,7 +152,7 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
     )
 
 
-def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2.0, **server_kw):
+def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2.0, lookahead=0, **server_kw):
     """One engine with an LRU budget of `cap_gib`, the fleet registered, the open-loop trace served."""
     from torpor_amd.server import Server
 
@@ -148,7 +165,7 @@ def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2
         charged = sum(server.model_info(f["fid"])["total_bytes"] for f in fleet)
         weights = sum(server.model_info(f["fid"])["image_bytes"] for f in fleet)
         arrivals, picks = make_trace(len(fleet), int(seconds * rate), rate, seed)
-        r = serve(server, fleet, arrivals, picks)
+        r = serve(server, fleet, arrivals, picks, lookahead=lookahead)
         r.update(cap_gib=cap_gib, cap_binds=charged >= limit, registration_s=reg_s, offered_rps=rate,
                  charged_total_gib=charged / 2 ** 30, weights_total_gb=weights / 1e9, link_peak_gbps=link)
         del fleet
