@@ -387,6 +387,8 @@ def main():
                          "sent as they are, and lookups that wait for their table")
     ap.add_argument("--ablation-variant", default=None, help=argparse.SUPPRESS)   # child of --ablate
     args = ap.parse_args()
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # a fresh checkout is compiled first; a built tree is used as it is
     if args.ablation_variant is not None:
         names = list(WORKLOADS) if args.workload == "all" else [args.workload]
         print(json.dumps(ablation_variant(args.ablation_variant, names, args.steps, args.warmup)))

@@ -13,6 +13,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # builds only in a tree without the library; a built one is loaded as it is
 
 
 @pytest.fixture(scope="module")
