@@ -250,3 +250,40 @@ def test_senders():
     assert syn.shape == (203, 31) and syn.dtype == np.int64 and 8 < syn.mean() < 12 and syn.min() >= 0
     ka = R.keepalive_p99([(1.0, 0), (1.0, 1), (1.0, 0), (5.0, 0), (1.0, 1)])
     assert ka[0] == pytest.approx(np.percentile([2.0, 5.0], 99)) and ka[1] == pytest.approx(7.0)
+
+
+class HintBackend(FakeBackend):
+    def execute(self, f, n, prefetch=None):
+        self.log.append((f, n, prefetch))
+        self.clock.t += self.service[f]
+
+
+@pytest.mark.parametrize("policy", ["fifo", "sa"])
+def test_prefetch_names_the_function_the_queue_hands_out_next(policy):
+    """With prefetch on, every dispatch names the function of the request that the policy hands out next (never the
+    one being served, nothing when nobody else waits), and the order of service is what it is without prefetch."""
+    def run(prefetch):
+        clock = Clock()
+        backend = (HintBackend if prefetch else FakeBackend)(clock, {f: 0.010 for f in range(4)})
+        r = R.Router(backend, 0.98, 0.1, 1, policy, clock=clock, prefetch=prefetch)
+        for f in range(4):
+            r.launch(f, 1)
+        rng = random.Random(5)
+        for i in range(60):
+            r.submit(rng.randrange(4), arrival=0.001 * i)
+        while r.pump():
+            pass
+        return r, backend.log
+
+    r1, hinted = run(True)
+    _, plain = run(False)
+    assert [(f, n) for f, n, _ in hinted] == plain
+    for i, (f, _, nxt) in enumerate(hinted):
+        assert nxt != f
+        later = [g for g, _, _ in hinted[i + 1:] if g != f]
+        if policy == "fifo":
+            assert nxt == (later[0] if later else None), i      # FIFO: the first later request of another function
+        elif nxt is not None:
+            assert nxt in later, i
+    assert r1.prefetch_hints == sum(1 for _, _, nxt in hinted if nxt is not None) > 20
+    assert r1.summary()["prefetch_hints"] == r1.prefetch_hints

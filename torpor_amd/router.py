@@ -97,6 +97,13 @@ class FifoPolicy:
             arrivals.append(self.queue.popleft()[1])
         return f, arrivals
 
+    def peek(self, running):
+        """The function of the first waiting request that is not `running`'s (what follows the batch just taken)."""
+        for f, _ in self.queue:
+            if f != running:
+                return f
+        return None
+
     def update(self):
         return self.stats.slo_ratio(self.slo)
 
@@ -164,6 +171,11 @@ class SloAwarePolicy:
                     return q, i
         return None, None
 
+    def peek(self, running):
+        """The function next_batch would take now (`running` has been marked unavailable by the caller)."""
+        q, i = self._first_available()
+        return None if q is None or q[i][0] == running else q[i][0]
+
     def next_batch(self, limit):
         q, i = self._first_available()
         if q is None:
@@ -230,8 +242,12 @@ class Router:
     UPDATE_PERIOD_S = 2.0               # router.py:495
 
     def __init__(self, backend, slo_percentile=0.98, deadline_s=0.1, batch_limit=1, policy="sa", clock=time.monotonic,
-                 deadlines=None, batch_limits=None):
+                 deadlines=None, batch_limits=None, prefetch=False):
         self.backend = backend
+        # prefetch: when a batch is dispatched, the function whose request the queue would hand out next is named
+        # to the backend, which asks the server to load its model (the Load signal) while this batch runs
+        self.prefetch = prefetch
+        self.prefetch_hints = 0
         self.slo = slo_percentile
         self.deadline_s = deadline_s
         self.deadlines = dict(deadlines or {})          # per-function overrides (router.py:18: 0.2 s for BERT)
@@ -290,7 +306,12 @@ class Router:
         f, arrivals = got
         self.stats.avail[f] = False
         try:
-            self.backend.execute(f, len(arrivals))
+            nxt = self.policy.peek(f) if self.prefetch else None
+            if nxt is not None:
+                self.prefetch_hints += 1
+                self.backend.execute(f, len(arrivals), prefetch=nxt)
+            else:
+                self.backend.execute(f, len(arrivals))
         except Exception:
             self.unhealthy.add(f)       # router.py:104-106: a function that fails is taken out of service
             self.stats.avail[f] = True
@@ -318,7 +339,8 @@ class Router:
                     requests_within_deadline=(sum(s[0] for s in self.stats.stat.values()) /
                                               max(1, sum(s[1] for s in self.stats.stat.values()))),
                     worst_function_hit_rate=min(per_func.values()) if per_func else None,
-                    alpha=getattr(self.policy, "alpha", None), batches=dict(self.batches), queued=self.queued())
+                    alpha=getattr(self.policy, "alpha", None), batches=dict(self.batches), queued=self.queued(),
+                    prefetch_hints=self.prefetch_hints)
 
 
 def serve_arrivals(router, arrivals, clock=time.monotonic, drain=True):
@@ -428,7 +450,7 @@ class FunctionBackend:
         fn, _, _, views = self.fn[func_id]
         return fn.postprocess(views)
 
-    def execute(self, func_id, n):
+    def execute(self, func_id, n, prefetch=None):
         fn, packed, outbuf, _ = self.fn[func_id]
         batch = getattr(fn, "batch", n)
         if 0 < n < batch:               # fewer requests than the registered batch: run at that size
@@ -437,6 +459,9 @@ class FunctionBackend:
         ack, _, deferred = self.conn[func_id].signal(1, func_id, "")
         if ack != 0 or deferred:
             raise RuntimeError(f"execute {func_id}: ack={ack} deferred={deferred}")
+        if prefetch is not None and prefetch != func_id and prefetch in self.conn:
+            # its copies queue behind this request's on the server's copy thread and run while this one computes
+            self.conn[prefetch].signal(2, prefetch, "")
         self.conn[func_id].replay(func_id, packed, outbuf)
         self.last[func_id] = None
 
@@ -498,6 +523,8 @@ def main(argv=None):
                     help="serve through a running torpor_server whose sockets are in DIR (one connection per function) "
                          "instead of an in-process server")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--prefetch", action="store_true",
+                    help="while a batch runs, ask the server to load the model of the request the queue hands out next")
     a = ap.parse_args(argv)
 
     from .server import Server
@@ -513,7 +540,7 @@ def main(argv=None):
     def serve(server_or_factory, stats):
         backend = FunctionBackend(server_or_factory, lambda s, fid, lv: build_function(s, fid, lv, a.m, a.b), ones_inputs)
         router = Router(backend, a.t / 100, a.d / 1000, a.b, a.p, deadlines={f: 2 * a.d / 1000 for f in qa},
-                        batch_limits={f: 1 for f in qa})
+                        batch_limits={f: 1 for f in qa}, prefetch=a.prefetch)
         for f in range(a.f):
             router.launch(f, mixed_model_level(f) if a.m == "mixed" else 1)
         for f in range(a.f):
