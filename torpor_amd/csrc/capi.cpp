@@ -221,7 +221,7 @@ int tp_gemm(tp_server* s, int32_t client, const tp_gemm_desc* d) {
 static int sgemm_common(tp_server* s, int32_t client, int transa, int transb, int m, int n, int k, float alpha,
                         uint64_t a, int lda, int64_t stride_a, uint64_t b, int ldb, int64_t stride_b, float beta,
                         uint64_t c, int ldc, int64_t stride_c, int count) {
-    ENG(s);
+    if (!s || !s->engine) return TP_EINVAL;
     if (m < 0 || n < 0 || k < 0 || count < 1) return TP_EINVAL;
     if (m == 0 || n == 0) return 0;
     tp_gemm_desc d;
