@@ -267,9 +267,10 @@ def test_attention(gpu_server, B, A, S, packed, masked):
     assert_close(got, ref.attention(q, k, v, mask, scale), 2e-5, "attention")
 
 
-def test_embedding(gpu_server):
+@pytest.mark.parametrize("H", [96, 1024, 37])     # one float4 pass, several, and a width the float4 path cannot take
+def test_embedding(gpu_server, H):
     rng = np.random.default_rng(2)
-    V, P, T, H, B, S = 100, 40, 2, 96, 3, 17
+    V, P, T, B, S = 100, 40, 2, 3, 17
     word, pos, typ = _rand(rng, V, H), _rand(rng, P, H), _rand(rng, T, H)
     ids = rng.integers(0, V, (B, S)).astype(np.int64)
     tids = rng.integers(0, T, (B, S)).astype(np.int64)
@@ -282,3 +283,7 @@ def test_embedding(gpu_server):
         got0 = t.read(yv, (B * S, H))
     assert_close(got, ref.embedding(ids, tids, word, pos, typ, S), 1e-6, "embedding")
     assert_close(got0, ref.embedding(ids, None, word, pos, typ, S), 1e-6, "embedding type 0")
+    # the vector and the scalar path add in the same order, (word + position) + type in float32
+    p_rows = pos[np.arange(B * S) % S]
+    assert np.array_equal(got, (word[ids.ravel()] + p_rows) + typ[tids.ravel()])
+    assert np.array_equal(got0, (word[ids.ravel()] + p_rows) + typ[0])

@@ -727,6 +727,24 @@ __global__ __launch_bounds__(256) void embedding_kernel(const int64_t* __restric
     if (ty >= n_types) ty = n_types - 1;
     const float* tr = type ? type + ty * width : nullptr;
     float* yr = y + tok * width;
+    // rows that start on 16 bytes go four floats at a time (the sums are the same: (word + pos) + type)
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(pr) |
+                           reinterpret_cast<uintptr_t>(tr) | reinterpret_cast<uintptr_t>(yr);
+    if ((width & 3) == 0 && (bits & 15) == 0) {
+        for (int c = lane * 4; c < width; c += 256) {
+            float4 v = *reinterpret_cast<const float4*>(wr + c);
+            if (pr) {
+                const float4 q = *reinterpret_cast<const float4*>(pr + c);
+                v.x += q.x, v.y += q.y, v.z += q.z, v.w += q.w;
+            }
+            if (tr) {
+                const float4 q = *reinterpret_cast<const float4*>(tr + c);
+                v.x += q.x, v.y += q.y, v.z += q.z, v.w += q.w;
+            }
+            *reinterpret_cast<float4*>(yr + c) = v;
+        }
+        return;
+    }
     for (int c = lane; c < width; c += 64) {
         float v = wr[c];
         if (pr) v += pr[c];
