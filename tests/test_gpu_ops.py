@@ -160,17 +160,19 @@ def test_new_activations_window_average_and_strided_views(gpu_server):
             t.s.stream_synchronize(t.fid)
 
 
+@pytest.mark.parametrize("C", [24, 10])          # NHWC: four channels per thread, and a count that path cannot take
 @pytest.mark.parametrize("layout", [NHWC, NCHW])
-def test_pooling(gpu_server, layout):
+def test_pooling(gpu_server, layout, C):
     rng = np.random.default_rng(9)
-    N, H, W, C = 2, 15, 14, 24
+    N, H, W = 2, 15, 14
     x = _rand(rng, N, H, W, C) if layout == NHWC else _rand(rng, N, C, H, W)
     with OpSession(gpu_server, [np.zeros(4, np.float32)]) as t:
         xv = t.act(x)
-        want = ref.maxpool(x, 3, 2, 1, nhwc=(layout == NHWC))
-        yv = t.empty(want.nbytes)
-        t.s.launch(t.fid, OP_MAXPOOL, [xv, yv], [N, H, W, C, 3, 2, 1, layout])
-        np.testing.assert_array_equal(t.read(yv, want.shape), want)
+        for k, stride, pad in ((3, 2, 1), (2, 2, 0), (3, 1, 1), (3, 2, 0)):
+            want = ref.maxpool(x, k, stride, pad, nhwc=(layout == NHWC))
+            yv = t.empty(want.nbytes)
+            t.s.launch(t.fid, OP_MAXPOOL, [xv, yv], [N, H, W, C, k, stride, pad, layout])
+            np.testing.assert_array_equal(t.read(yv, want.shape), want, err_msg=str((k, stride, pad)))
         av = t.empty(N * C * 4)
         t.s.launch(t.fid, OP_AVGPOOL, [xv, av], [N, H * W, C, layout])
         assert_close(t.read(av, (N, C)), ref.avgpool(x, nhwc=(layout == NHWC)), 2e-6, "avgpool")

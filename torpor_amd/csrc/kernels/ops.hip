@@ -356,6 +356,33 @@ __global__ __launch_bounds__(256) void maxpool_kernel(const float* __restrict__ 
         y[nhwc ? (i / C) * y_pitch + c : i] = m;
     }
 }
+// NHWC with C % 4 == 0 and 16-byte aligned rows: a thread takes four channels of one output pixel, so the
+// window is k*k 128-bit loads and the index arithmetic is done once per four results, in 32 bits.
+__global__ __launch_bounds__(256) void maxpool_nhwc4_kernel(const float* __restrict__ x, float* __restrict__ y, int H,
+                                                            int W, int C4, int Ho, int Wo, int k, int stride, int pad,
+                                                            long y_pitch, unsigned total) {
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const unsigned c4 = i % (unsigned)C4;
+        unsigned t = i / (unsigned)C4;
+        const unsigned pix = t;  // (n * Ho + ho) * Wo + wo
+        const int wo = (int)(t % (unsigned)Wo);
+        t /= (unsigned)Wo;
+        const int ho = (int)(t % (unsigned)Ho);
+        const long n = t / (unsigned)Ho;
+        float4 m = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        for (int kh = 0; kh < k; ++kh) {
+            const int hi = ho * stride - pad + kh;
+            if (hi < 0 || hi >= H) continue;
+            for (int kw = 0; kw < k; ++kw) {
+                const int wi = wo * stride - pad + kw;
+                if (wi < 0 || wi >= W) continue;
+                const float4 v = *reinterpret_cast<const float4*>(x + (((n * H + hi) * W + wi) * C4 + c4) * 4);
+                m.x = fmaxf(m.x, v.x), m.y = fmaxf(m.y, v.y), m.z = fmaxf(m.z, v.z), m.w = fmaxf(m.w, v.w);
+            }
+        }
+        *reinterpret_cast<float4*>(y + (long)pix * y_pitch + c4 * 4) = m;
+    }
+}
 int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k, int stride, int pad, int nhwc,
                      long y_pitch, hipStream_t s) {
     if (!x || !y || N <= 0 || H <= 0 || W <= 0 || C <= 0 || k <= 0 || stride <= 0 || pad < 0 || pad * 2 > k)
@@ -365,6 +392,13 @@ int launch_maxpool2d(const float* x, float* y, int N, int H, int W, int C, int k
     const int Ho = (H + 2 * pad - k) / stride + 1, Wo = (W + 2 * pad - k) / stride + 1;
     if (Ho <= 0 || Wo <= 0) return K_EINVAL;
     const long total = (long)N * Ho * Wo * C;
+    const bool vec4 = nhwc && (C & 3) == 0 && (y_pitch & 3) == 0 && total / 4 < (1L << 31) &&
+                      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (vec4) {
+        hipLaunchKernelGGL(maxpool_nhwc4_kernel, dim3(grid_for(total / 4, 256)), dim3(256), 0, s, x, y, H, W, C / 4, Ho,
+                           Wo, k, stride, pad, y_pitch, (unsigned)(total / 4));
+        return (int)hipGetLastError();
+    }
     hipLaunchKernelGGL(maxpool_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, x, y, N, H, W, C, Ho, Wo, k,
                        stride, pad, nhwc, y_pitch);
     return (int)hipGetLastError();
