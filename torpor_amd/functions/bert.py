@@ -121,9 +121,9 @@ class Bert(Function):
                     xs_r=inp if xs_r is None else xs_r, ys_c=inp, ldc=out, bias=self.w[name + ".bias"], act=act)
         return y
 
-    def _ln(self, x, res, tok, name):
+    def _ln(self, x, res, tok, name, dst=None):
         H = self.cfg["hidden"]
-        y = self.alloc(tok * H * 4)
+        y = self.alloc(tok * H * 4) if dst is None else dst
         self.s.launch(self.fid, OP_LAYERNORM,
                       [x.va, res.va if res is not None else 0, self.w[name + ".weight"], self.w[name + ".bias"], y.va],
                       [tok, H], [LN_EPS])
@@ -178,7 +178,10 @@ class Bert(Function):
             inter = self._linear(h1, tok, H, F, p + ".intermediate.dense", act=ACT_GELU)
             out = self._linear(inter, tok, F, H, p + ".output.dense")
             self.release(inter)
-            h = self._ln(out, h1, tok, p + ".output.LayerNorm")
+            # One result buffer = [last hidden state | pooled], because the first D2H copy of a request is its
+            # completion marker (reference cuda_server.hpp:1044): the last LayerNorm writes straight into it.
+            result = self.alloc((tok * H + B * H) * 4) if (i == L - 1 and not self.qa_head) else None
+            h = self._ln(out, h1, tok, p + ".output.LayerNorm", dst=result)
             self.release(out)
             self.release(h1)
         if self.qa_head:
@@ -186,15 +189,15 @@ class Bert(Function):
             out = self._linear(h, tok, H, 2, "qa_outputs")
             self.release(h)
             return [(out, (tok * 2,), np.float32)]
-        # One result buffer = [last hidden state | pooled], because the first D2H copy of a request
-        # is its completion marker (reference cuda_server.hpp:1044).
-        out = self.alloc((tok * H + B * H) * 4)
-        self.s.d2d(self.fid, out.va, h.va, tok * H * 4)
+        if L == 0:      # no encoder layer: the embedding output is the last hidden state
+            result = self.alloc((tok * H + B * H) * 4)
+            self.s.d2d(self.fid, result.va, h.va, tok * H * 4)
+            self.release(h)
+            h = result
         # pooler: tanh(W . h[:, 0] + b); row b of X is token b*S
-        self.s.gemm(self.fid, h.va, self.w["pooler.dense.weight"], out.va + tok * H * 4, B, H, H,
+        self.s.gemm(self.fid, h.va, self.w["pooler.dense.weight"], h.va + tok * H * 4, B, H, H,
                     xs_r=S * H, ys_c=H, ldc=H, bias=self.w["pooler.dense.bias"], act=ACT_TANH)
-        self.release(h)
-        return [(out, (tok * H + B * H,), np.float32)]
+        return [(h, (tok * H + B * H,), np.float32)]
 
     def postprocess(self, host):
         (flat,) = host
