@@ -23,7 +23,8 @@ CASES = [
     (2, 28, 28, 128, 128, 3, 2, 1, NHWC, NHWC, "conv3x3_fast"),   # 3x3 stride 2
     (1, 7, 7, 512, 512, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # tiny map, split-K
     (8, 28, 28, 128, 128, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),   # batch 8
-    (1, 64, 64, 3, 64, 7, 2, 3, NCHW, NHWC, "conv_generic"),      # stem: NCHW in, NHWC out
+    (1, 64, 64, 3, 64, 7, 2, 3, NCHW, NHWC, "conv_stem7x7"),      # stem: NCHW in, NHWC out
+    (1, 64, 64, 3, 48, 7, 2, 3, NCHW, NHWC, "conv_generic"),      # a stem whose channel count the stem kernel does not take
     (1, 13, 11, 5, 7, 3, 1, 1, NCHW, NCHW, "conv_generic"),       # odd sizes, NCHW both
     (1, 9, 9, 12, 20, 5, 2, 2, NHWC, NCHW, "conv_generic"),       # 5x5, mixed layouts
     (1, 10, 10, 12, 16, 3, 1, 0, NHWC, NHWC, "conv_generic"),     # Cin % 8 != 0
@@ -67,6 +68,42 @@ def test_conv_bn_residual_relu(gpu_server, k, Cin, Cout, HW):
     z = ref.conv2d(x, w, (1, 1), (pad, pad), x_nhwc=True, y_nhwc=True)
     z = ref.bn(z, g, b, mu, var, 1e-5, Cout, nhwc=True).astype(np.float64) + res
     assert_close(got, np.maximum(z, 0), 5e-5, "conv+bn+res+relu")
+
+
+@pytest.mark.parametrize("N,H,W,Cout,xl,yl", [
+    (1, 224, 224, 64, NCHW, NHWC),      # the served shape
+    (2, 30, 29, 64, NCHW, NHWC),        # odd output height (15): the second row of the last pair does not exist
+    (1, 70, 75, 128, NCHW, NHWC),       # two channel blocks; 38 output columns: a full block and a ragged one
+    (2, 33, 64, 64, NHWC, NHWC),        # channels-last input
+    (1, 40, 36, 64, NCHW, NCHW),        # NCHW output (the element-wise write-out)
+])
+def test_stem_convolution(gpu_server, N, H, W, Cout, xl, yl):
+    """7x7 stride 2 padding 3 from 3 channels (cudnnConvolutionForward of the ResNet / DenseNet stem,
+    cuda_server.hpp:708-735) with the batch-norm + ReLU that follows it fused, against the direct-loop oracle."""
+    rng = np.random.default_rng(H * 7 + W + Cout)
+    x_nchw = _rand(rng, N, 3, H, W)
+    w = _rand(rng, Cout, 3, 7, 7) * np.float32(1.0 / np.sqrt(147))
+    g, b, mu = _rand(rng, Cout), _rand(rng, Cout), _rand(rng, Cout)
+    var = rng.uniform(0.5, 2.0, Cout).astype(np.float32)
+    x = x_nchw if xl == NCHW else np.ascontiguousarray(x_nchw.transpose(0, 2, 3, 1))
+    Ho, Wo = (H + 6 - 7) // 2 + 1, (W + 6 - 7) // 2 + 1
+    shape = (N, Ho, Wo, Cout) if yl == NHWC else (N, Cout, Ho, Wo)
+    with OpSession(gpu_server, [w, g, b, mu, var]) as t:
+        xv = t.act(x)
+        guard = np.full(shape, 7.0, np.float32)
+        yv = t.act(np.concatenate([guard.ravel(), np.full(64, 7.0, np.float32)]))   # 64 floats behind y must stay
+        t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, 3, Cout, 7, 7, stride=2, pad=3, x_layout=xl, y_layout=yl)
+        assert t.s.last_kernel().startswith("conv_stem7x7"), t.s.last_kernel()
+        plain = t.read(yv, shape)
+        tail = t.read(yv + guard.nbytes, (64,))
+        t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, 3, Cout, 7, 7, stride=2, pad=3, x_layout=xl, y_layout=yl,
+                 bn=tuple(t.w[1:5]), bn_eps=1e-5, act=ACT_RELU)
+        fused = t.read(yv, shape)
+    z = ref.conv2d(x, w, (2, 2), (3, 3), x_nhwc=(xl == NHWC), y_nhwc=(yl == NHWC))
+    assert_close(plain, z, RTOL, "stem")
+    assert np.all(tail == 7.0), "stem wrote past the end of its output"
+    zb = ref.bn(z, g, b, mu, var, 1e-5, Cout, hw=Ho * Wo, nhwc=(yl == NHWC))
+    assert_close(fused, np.maximum(zb, 0), 5e-5, "stem+bn+relu")
 
 
 def test_conv_identities(gpu_server):

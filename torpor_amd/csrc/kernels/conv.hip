@@ -461,6 +461,125 @@ static int launch_depthwise(const ConvArgs& a, int Ho, int Wo, long xp, long yp,
 
 static inline bool aligned16c(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// ---------------------------------------------------------------- 7x7 stride-2 stem (3 input channels)
+// The first layer of the ResNets and DenseNets: 7x7, stride 2, padding 3, 3 -> Cout channels (Cout % 64 == 0).
+// With 3 input channels the taps kernels' channel blocks do not apply and the general kernel spends its time on
+// gather addresses (1x224x224: 16 us).  Here a workgroup owns 2 output rows x 32 output columns x 64 output
+// channels: the input patch they read (3 channels x 10 rows x 69 columns) and the 64 filters, as they lie in
+// memory, are put into LDS once, and every MFMA operand is then one LDS word at a compile-time offset from a
+// per-lane base.
+//
+// K order.  v_mfma_f32_32x32x2_f32 takes k = 0 from lanes 0-31 and k = 1 from lanes 32-63.  The 7 filter rows are
+// split 4 + 3 between the lane halves: step (c, j, kw) multiplies filter row kh = 4*half + j, so the two halves read
+// patch and filter 4 rows apart -- constants that fold into the lanes' base addresses -- and 3 * 4 * 7 = 84 steps
+// cover the 147 products.  Filter row 7 does not exist: in the 21 steps with j = 3 the upper half's filter operand
+// is replaced by zero (what it reads instead is the next channel's first row, or the 8 floats of padding behind
+// the last filter).
+struct StemCfg {  // what store_tile needs to know: one 32x32 accumulator per wavefront, 2 x 2 wavefronts
+    static constexpr int BM = 64, BN = 64, WGM = 2, WGN = 2, WGK = 1, THREADS = 256;
+    static constexpr int WTM = 32, WTN = 32, TM = 1, TN = 1;
+};
+constexpr int kStemRows = 10, kStemCols = 69, kStemPitch = 72;  // patch rows 2*ty + kh (kh 0..7), columns 2*tx + kw
+constexpr int kStemPatch = 3 * kStemRows * kStemPitch;          // floats
+constexpr int kStemFilters = 64 * 147;
+constexpr int kStemLds = kStemPatch + kStemFilters + 8;
+static_assert(kStemFilters + 8 >= 4 * STAGE_BLOCK, "the filter area doubles as the write-out staging blocks");
+
+__global__ __launch_bounds__(256, 2) void conv_stem7_kernel(const ConvDev p) {
+    __shared__ __attribute__((aligned(16))) float lds[kStemLds];
+    float* P = lds;
+    float* Wt = lds + kStemPatch;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r = lane & 31, h = lane >> 5;
+    // workgroup -> (image, pair of output rows, block of 32 output columns, block of 64 output channels)
+    const int tiles_x = (p.Wo + 31) >> 5, tiles_y = (p.Ho + 1) >> 1;
+    int t = (int)blockIdx.x;
+    const int tx0 = t % tiles_x;
+    t /= tiles_x;
+    const int ty0 = t % tiles_y;
+    const int n = t / tiles_y;
+    const int ho0 = ty0 * 2, wo0 = tx0 * 32;
+    const int n0 = (int)blockIdx.y * 64;
+    const int hi0 = ho0 * 2 - 3, wi0 = wo0 * 2 - 3;
+
+    ColConsts<1> cc;
+    cols_issue<StemCfg>(cc, p.ep, p.y, n0, wn, lane, (long)p.Cout);
+
+    // the 64 filters: 64 * 147 contiguous floats, copied as they are (16-byte aligned: checked by the launcher)
+    const f32x4* wsrc = reinterpret_cast<const f32x4*>(p.w + (long)n0 * 147);
+    constexpr int NW4 = kStemFilters / 4;  // 2352
+    f32x4 wv[(NW4 + 255) / 256];
+#pragma unroll
+    for (int it = 0; it < (NW4 + 255) / 256; ++it) {
+        const int i = it * 256 + tid;
+        wv[it] = wsrc[i < NW4 ? i : NW4 - 1];
+    }
+    // the input patch, zero outside the image (the padding): a wavefront per (channel, row) line of 69 columns
+    const float* xn = p.x + (long)n * p.xs_n;
+    float pv[8][2];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const int line = wave + 4 * q;  // 0..31, 30 lines exist
+        const int c = line / kStemRows, row = line - c * kStemRows;
+        const int hi = hi0 + row;
+        const bool line_ok = line < 3 * kStemRows && hi >= 0 && hi < p.H;
+        const float* src = xn + (long)(line_ok ? c : 0) * p.xs_c + (long)(line_ok ? hi : 0) * p.xs_h;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int col = lane + 64 * u;
+            const int wi = wi0 + col;
+            const bool ok = line_ok && col < kStemCols && wi >= 0 && wi < p.W;
+            const float v = src[(long)(ok ? wi : 0) * p.xs_w];  // always a valid address: element (n, c, 0 or hi, 0 or wi)
+            pv[q][u] = ok ? v : 0.f;
+        }
+    }
+    cols_fold<StemCfg>(cc, p.ep);
+#pragma unroll
+    for (int it = 0; it < (NW4 + 255) / 256; ++it) {
+        const int i = it * 256 + tid;
+        if (i < NW4) *reinterpret_cast<f32x4*>(Wt + 4 * i) = wv[it];
+    }
+    if (tid < 8) Wt[kStemFilters + tid] = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const int line = wave + 4 * q;
+        if (line < 3 * kStemRows) {
+            P[line * kStemPitch + lane] = pv[q][0];
+            if (lane + 64 < kStemPitch) P[line * kStemPitch + lane + 64] = pv[q][1];
+        }
+    }
+    __syncthreads();
+
+    f32x16 acc[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[0][0][v] = 0.f;
+    const float* ap = P + (2 * wm + 4 * h) * kStemPitch + 2 * r;
+    const float* bp = Wt + (wn * 32 + r) * 147 + h * 28;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int kw = 0; kw < 7; ++kw) {
+                float b = bp[c * 49 + j * 7 + kw];
+                if (j == 3) b = h ? 0.f : b;  // filter row 7
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[(c * kStemRows + j) * kStemPitch + kw], b, acc[0][0],
+                                                                 0, 0, 0);
+            }
+    __syncthreads();  // the operands are no longer read: the filter area becomes the write-out staging blocks
+
+    // rows of this wavefront's block = 32 consecutive pixels of output row ho0 + wm; those past the end of the
+    // row (or a row past the image) are cut off through the row bound
+    const int ho = ho0 + wm;
+    const long m0 = ((long)n * p.Ho + ho) * p.Wo + wo0;
+    int valid = p.Wo - wo0;
+    if (valid > 32) valid = 32;
+    if (ho >= p.Ho) valid = 0;
+    store_tile<StemCfg>(acc, 0, wn, lane, m0, (long)n0, m0 + valid, (long)p.Cout, p.y, p.ep, nullptr,
+                        Wt + wave * STAGE_BLOCK, &cc);
+}
+
 int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     if (!a.x || !a.w || !a.y) return K_EINVAL;
     if (a.N <= 0 || a.H <= 0 || a.W <= 0 || a.Cin <= 0 || a.Cout <= 0 || a.KH <= 0 || a.KW <= 0) return K_EINVAL;
@@ -589,6 +708,11 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     const bool fast3 = a.KH == 3 && a.KW == 3 && taps_ok;
     const int other_taps = !taps_ok ? 0 : (a.KH == 1 && a.KW == 7) ? 1 : (a.KH == 7 && a.KW == 1) ? 2
                            : (a.KH == 1 && a.KW == 3) ? 3 : (a.KH == 3 && a.KW == 1) ? 4 : 0;
+    // TORPOR_CONV_STEM=0: the general kernel for the 7x7 stem, as before
+    static const bool stem_on = getenv("TORPOR_CONV_STEM") == nullptr || atoi(getenv("TORPOR_CONV_STEM")) != 0;
+    const bool stem7 = stem_on && a.KH == 7 && a.KW == 7 && a.sh == 2 && a.sw == 2 && a.ph == 3 && a.pw == 3 &&
+                       a.Cin == 3 && a.Cout % 64 == 0 && a.Cout / 64 <= 65535 && aligned16c(a.w) &&
+                       (long)a.N * ((Ho + 1) / 2) * ((Wo + 31) / 32) < (1L << 31);
     if (other_taps) {
         // the asymmetric shapes (Inception): one 64x64 tile shape, split over channel blocks.  (5x5 stays on
         // the general kernel: a 200-wide K-block leaves one workgroup per CU and measured 2x slower.)
@@ -681,6 +805,11 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
                 set_last_kernel("conv3x3_fast_32x32_k3");
                 break;
         }
+    } else if (stem7) {
+        const long wgs = (long)a.N * ((Ho + 1) / 2) * ((Wo + 31) / 32);
+        p.splits = 1;
+        hipLaunchKernelGGL(conv_stem7_kernel, dim3((unsigned)wgs, (unsigned)(a.Cout / 64)), dim3(256), 0, s, p);
+        set_last_kernel("conv_stem7x7_s2");
     } else {
         p.tiles_m = (int)((M + 63) / 64);
         p.tiles_n = (a.Cout + 63) / 64;
