@@ -370,6 +370,33 @@ def ablation(names, steps, warmup):
     return out
 
 
+CAL_COPY_BYTES = 64 << 20
+
+
+def counter_calibration_copy(server, fid=65000, repeats=3):
+    """Plain device-to-device copies of known size (64 MiB read and 64 MiB written each, far beyond the L2s) by
+    the library's `copy_kernel`: what the FETCH_SIZE / WRITE_SIZE counters of a profiled run of this command are
+    scaled by.  A scratch function of its own, registered, run once and unloaded; a few milliseconds."""
+    import numpy as np
+
+    from torpor_amd.server import OP_FILL, REQ_EXECUTE_AFTER_LOAD, REQ_UNLOAD
+    ack, _, deferred = server.signal(REQ_EXECUTE_AFTER_LOAD, fid, "1")
+    assert ack == 0 and not deferred
+    w = np.zeros(4, np.float32)
+    server.h2d(fid, server.malloc(fid, w.nbytes), w)
+    server.device_synchronize(fid)                      # end of the loading phase
+    src, dst = server.malloc(fid, CAL_COPY_BYTES), server.malloc(fid, CAL_COPY_BYTES)
+    server.memset(fid, src, 0, CAL_COPY_BYTES)
+    for _ in range(repeats):
+        server.d2d(fid, dst, src, CAL_COPY_BYTES)
+    done = server.malloc(fid, 4)                        # the request ends with its device-to-host copy
+    server.launch(fid, OP_FILL, [done], [1], [0.0])
+    out = np.empty(1, np.float32)                       # alive until the synchronisation has delivered it
+    server.d2h_async(fid, out, done)
+    server.stream_synchronize(fid)
+    server.signal(REQ_UNLOAD, fid, "")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -408,6 +435,7 @@ def main():
     server = Server(mem_limit_bytes=24 << 30, pool_bytes=25 << 30, chunk_bytes=args.chunk_bytes,
                     chunk_max_bytes=args.chunk_max_bytes)
     link = server.measure_h2d(256 << 20, 10)
+    counter_calibration_copy(server)
     results, roof, keep = {}, {}, {}
     for fid, name in enumerate(names):
         res, kstats, empty_us, ctx = run_workload(server, fid, name, args.steps, args.warmup, link)
