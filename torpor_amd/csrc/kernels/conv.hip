@@ -9,7 +9,7 @@
 // residual / activation.
 //
 //   1x1, NHWC, Cin%4==0, pad 0      -> the dense GEMM kernel with a row gather
-//   3x3, 1x7, 7x1, 1x3, 3x1; NHWC, Cin%8==0 -> conv_taps_kernel (K-block = 8 channels x taps)
+//   3x3, 1x7, 7x1, 1x3, 3x1; NHWC, Cin%8==0 -> conv_taps_kernel (K-block = 8 or 16 channels x taps)
 //   everything else (7x7 stem, NCHW) -> conv_generic_kernel (scalar gathers)
 #include "kernels.hpp"
 #include "mfma_tile.hpp"
@@ -76,10 +76,11 @@ __device__ __forceinline__ int remap_xcd_c(int bid, int n) {
 }
 
 // KH x KW taps (T = KH*KW; 3x3, and the 1x7 / 7x1 / 1x3 / 3x1 shapes of Inception), NHWC,
-// Cin % 8 == 0.  K-block = 8 input channels x T taps, ordered k_local = tap*8 + c in LDS.
-// Activation side: for (pixel, tap) the 8 channels are 32 contiguous bytes of
-// the NHWC input (two dwordx4 loads by two neighbouring threads).  Weight side:
-// for one output channel the 8 x T block is 8T contiguous floats of the
+// Cin % 8 == 0.  K-block = CB input channels x T taps (CB = BK / T: 8, or 16 for the nine-wavefront
+// 3x3 tile), ordered k_local = tap*CB + c in LDS.
+// Activation side: for (pixel, tap) the CB channels are 4*CB contiguous bytes of
+// the NHWC input (CB/4 dwordx4 loads by neighbouring threads).  Weight side:
+// for one output channel the CB x T block is CB*T contiguous floats of the
 // [Cout][Cin][KH][KW] tensor; each thread loads 4T of them (4 channels x T taps)
 // with dwordx4 and transposes in registers to the tap-major LDS order.
 //
@@ -94,8 +95,10 @@ template <class C, int KH, int KW, int STAGES = 2>
 __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_taps_kernel(const ConvDev p) {
     fetch_now(p);
     constexpr int T = KH * KW;
-    static_assert(C::BK == 8 * T, "K-block = 8 channels x taps");
-    static_assert(C::BN * 2 <= C::THREADS, "two threads fetch the weights of one output channel");
+    constexpr int CB = C::BK / T;  // input channels per K-block
+    constexpr int Q = CB / 4;      // 128-bit pieces of a pixel's channel block
+    static_assert(C::BK == CB * T && (CB == 8 || CB == 16), "K-block = 8 or 16 channels x taps");
+    static_assert(C::BN * Q <= C::THREADS, "Q threads fetch the weights of one output channel");
     __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, red_floats<C>() + stage_floats<C>() + 4)];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
@@ -110,15 +113,15 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     // Branch-free operand fetch: rows past the last pixel are clamped to it (computed, then
     // dropped at the store) and taps that fall into the padding read from a page of zeros with
     // a zero channel step, so every load in the loop is unconditional.
-    constexpr int NVA = (C::BM * 2 * T + C::THREADS - 1) / C::THREADS;
+    constexpr int NVA = (C::BM * Q * T + C::THREADS - 1) / C::THREADS;
     const float* pa[NVA];
     int stepA[NVA];
 #pragma unroll
     for (int i = 0; i < NVA; ++i) {
         int idx = i * C::THREADS + tid;
-        if (idx > C::BM * 2 * T - 1) idx = C::BM * 2 * T - 1;
-        const int row = idx / (2 * T), t2 = idx - row * (2 * T);
-        const int tap = t2 >> 1, cq = t2 & 1;
+        if (idx > C::BM * Q * T - 1) idx = C::BM * Q * T - 1;
+        const int row = idx / (Q * T), t2 = idx - row * (Q * T);
+        const int tap = t2 / Q, cq = t2 % Q;
         long grow = m0 + row;
         if (grow > p.M - 1) grow = p.M - 1;
         const int wo = (int)(grow % p.Wo);
@@ -131,8 +134,8 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
         pa[i] = inside ? p.x + n * p.xs_n + (long)hi * p.xs_h + (long)wi * p.xs_w + cq * 4 : p.zeros;
         stepA[i] = inside ? 1 : 0;
     }
-    // weight assignment: thread -> (col = tid/2, cq = tid%2)
-    const int wcol = tid >> 1, wcq = tid & 1;
+    // weight assignment: thread -> (col = tid / Q, cq = tid % Q)
+    const int wcol = tid / Q, wcq = tid % Q;
     long wc = n0 + wcol;
     if (wc > p.Cout - 1) wc = p.Cout - 1;
     const float* __restrict__ wbase = p.w + (wc * (long)p.Cin + wcq * 4) * T;
@@ -145,10 +148,10 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     if (wk == 0) cols_issue<C>(cc, p.ep, p.y, n0, wn, lane, (long)p.Cout);
 
     auto load_regs = [&](int c0) {
-        if (c0 > cend - 8) c0 = cend - 8;  // look-ahead past the end re-reads the last block
+        if (c0 > cend - CB) c0 = cend - CB;  // look-ahead past the end re-reads the last block
 #pragma unroll
         for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + c0 * stepA[i]);
-        if (tid < C::BN * 2) {
+        if (tid < C::BN * Q) {
 #pragma unroll
             for (int j = 0; j < T; ++j) rw[j] = *reinterpret_cast<const f32x4*>(wbase + (long)c0 * T + j * 4);
         }
@@ -159,10 +162,10 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
 #pragma unroll
         for (int i = 0; i < NVA; ++i) {
             const int idx = i * C::THREADS + tid;
-            const int row = idx / (2 * T), t2 = idx - row * (2 * T);
-            if (idx < C::BM * 2 * T) *reinterpret_cast<f32x4*>(As + row * C::LDK + t2 * 4) = ra[i];
+            const int row = idx / (Q * T), t2 = idx - row * (Q * T);
+            if (idx < C::BM * Q * T) *reinterpret_cast<f32x4*>(As + row * C::LDK + t2 * 4) = ra[i];
         }
-        if (tid < C::BN * 2) {
+        if (tid < C::BN * Q) {
             // rw holds w[c][tap] for c = 0..3 (this thread's channel quad), flat index c*T + tap
 #pragma unroll
             for (int tap = 0; tap < T; ++tap) {
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
                     const int f = c * T + tap;
                     v[c] = rw[f >> 2][f & 3];
                 }
-                *reinterpret_cast<f32x4*>(Bs + wcol * C::LDK + tap * 8 + wcq * 4) = v;
+                *reinterpret_cast<f32x4*>(Bs + wcol * C::LDK + tap * CB + wcq * 4) = v;
             }
         }
     };
@@ -181,23 +184,23 @@ __global__ __launch_bounds__(C::THREADS, (C::THREADS > 512 ? 1 : 2)) void conv_t
     if (wk == 0) cols_fold<C>(cc, p.ep);
     if (STAGES == 2) {
         store_lds(0);
-        load_regs(cbeg + 8);
+        load_regs(cbeg + CB);
         __syncthreads();
         int cur = 0;
-        for (int c0 = cbeg; c0 < cend; c0 += 8) {
+        for (int c0 = cbeg; c0 < cend; c0 += CB) {
             // the other stage was last read before the barrier that ended the previous iteration
             store_lds(cur ^ 1);
-            load_regs(c0 + 16);
+            load_regs(c0 + 2 * CB);
             const float* As = lds + cur * C::LDS_FLOATS;
             mma_block<C>(As, As + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
             cur ^= 1;
         }
     } else {
-        for (int c0 = cbeg; c0 < cend; c0 += 8) {
+        for (int c0 = cbeg; c0 < cend; c0 += CB) {
             store_lds(0);
             __syncthreads();
-            load_regs(c0 + 8);
+            load_regs(c0 + CB);
             mma_block<C>(lds, lds + C::BM * C::LDK, acc, wm, wn, lane, wk);
             __syncthreads();
         }
@@ -307,6 +310,7 @@ using Conv3M = TileCfg<64, 64, 72, 2, 2>;
 using Conv3S = TileCfg<64, 64, 72, 2, 2, 3>;  // 12 wavefronts: 2x2 over the tile, 3 K slices
 using Conv3T = TileCfg<32, 32, 72, 1, 1, 9>;  // 9 wavefronts, one k-group each
 using Conv3U = TileCfg<32, 32, 72, 1, 1, 3>;  // 3 wavefronts
+using Conv3T16 = TileCfg<32, 32, 144, 1, 1, 9>;  // as Conv3T with 16 input channels per K-block
 
 // Depthwise convolution (groups == Cin == Cout), NHWC, weights [C][1][KH][KW]: HBM-bound, one
 // thread per output pixel and channel quad, taps accumulated in registers, same fused epilogue
@@ -765,6 +769,7 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         // split over channel blocks of 8 (one K-block each)
         long kper_k = p.K;
         p.splits = 1;
+        bool cb16 = false;
         static const bool pairs = getenv("TORPOR_CONV_PAIRS") != nullptr;
         if (cfg <= 1) p.splits = choose_splits(tiles, p.K, 72, (long)bm * bm, ws.ptr ? ws.bytes : 0, &kper_k, 32, pairs);
         if (cfg == 3) {
@@ -774,7 +779,11 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
             // 7.1 us, 2 slots 10.1 us).  TORPOR_CONV_PAIRS=1 keeps the earlier rule (two workgroups per CU).
             int cap = pairs ? 8 : (int)(num_cu() / tiles);
             if (cap > 8) cap = 8;
-            p.splits = cap >= 2 ? choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, cap, true, 0) : 1;
+            // K-blocks of 16 input channels where the channel count allows: a wavefront then issues 8 MFMAs between
+            // two barriers instead of 4 (ResNet-50 batch 1: 10.6 -> 9.9 us per launch; TORPOR_CONV3_CB16=0: always 8)
+            static const bool cb16_on = getenv("TORPOR_CONV3_CB16") == nullptr || atoi(getenv("TORPOR_CONV3_CB16")) != 0;
+            cb16 = cb16_on && a.Cin % 16 == 0;
+            p.splits = cap >= 2 ? choose_splits(tiles, p.K, cb16 ? 144 : 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, cap, true, 0) : 1;
         }
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
@@ -797,8 +806,13 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
                 set_last_kernel("conv3x3_fast_64x64_k3");
                 break;
             case 3:
-                hipLaunchKernelGGL((conv_taps_kernel<Conv3T, 3, 3, 1>), grid, dim3(Conv3T::THREADS), 0, s, p);
-                set_last_kernel("conv3x3_fast_32x32_k9");
+                if (cb16) {
+                    hipLaunchKernelGGL((conv_taps_kernel<Conv3T16, 3, 3, 1>), grid, dim3(Conv3T16::THREADS), 0, s, p);
+                    set_last_kernel("conv3x3_fast_32x32_k9");
+                } else {
+                    hipLaunchKernelGGL((conv_taps_kernel<Conv3T, 3, 3, 1>), grid, dim3(Conv3T::THREADS), 0, s, p);
+                    set_last_kernel("conv3x3_fast_32x32_k9");
+                }
                 break;
             default:
                 hipLaunchKernelGGL((conv_taps_kernel<Conv3U, 3, 3, 1>), grid, dim3(Conv3U::THREADS), 0, s, p);
