@@ -271,7 +271,7 @@ def cpu_baseline(name, weights, inputs, first):
     from torpor_amd.functions import bert
 
     family, arch, batch, seq = {**WORKLOADS, **EXTRA_WORKLOADS}[name]
-    cores = int(os.environ.get("OMP_NUM_THREADS") or torch.get_num_threads())
+    cores = host_cores()
     torch.set_num_threads(cores)
     if family in ("resnet", "densenet", "mobilenet", "efficientnet", "inception", "vgg", "squeezenet"):
         net = {"resnet": lambda: om.ResNet(arch), "densenet": lambda: om.DenseNet(arch),
@@ -301,9 +301,32 @@ def cpu_baseline(name, weights, inputs, first):
     for a, b in zip(first, out):
         b = b.numpy()
         err = max(err, float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)))
-    return dict(value=statistics.median(times), unit="ms", cores=cores, kind="port",
+    return dict(value=statistics.median(times), unit="ms", cores=cores, kind="port", cpu=cpu_model_name(),
+                os_cpu_count=os.cpu_count(),
                 sample=f"10 timed forwards after 3 warm-ups of {name} (oracle/models.py, torch CPU fp32)",
                 min_ms=min(times), logits_rel_err_vs_gpu=err)
+
+
+def host_cores():
+    """Host threads for the CPU leg: every core this process may run on (the scheduler's affinity mask where
+    the platform has one, else os.cpu_count()), unless OMP_NUM_THREADS names the box's share explicitly."""
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit() and int(env) > 0:
+        return int(env)
+    try:
+        return len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        return os.cpu_count() or 1
+
+
+def cpu_model_name():
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name"):
+                return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 ABLATION_VARIANTS = {
@@ -397,6 +420,101 @@ def counter_calibration_copy(server, fid=65000, repeats=3):
     server.signal(REQ_UNLOAD, fid, "")
 
 
+COMPACT_LIMIT_BYTES = 6000   # the final stdout line stays below this; everything else goes to the detail file
+
+
+def sig(x, digits=4):
+    """Floats to `digits` significant figures (the line is read by programs and people, not re-used in arithmetic)."""
+    if isinstance(x, bool) or not isinstance(x, float):
+        return x
+    if x != x or x in (float("inf"), float("-inf")):
+        return None
+    return float(f"{x:.{digits}g}")
+
+
+def trim(obj, digits=4):
+    if isinstance(obj, dict):
+        return {k: trim(v, digits) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [trim(v, digits) for v in obj]
+    if isinstance(obj, (np.floating,)):
+        return sig(float(obj), digits)
+    if isinstance(obj, (np.integer,)):
+        return int(obj)
+    return sig(obj, digits)
+
+
+def compact_roofline(r):
+    """The roofline object without its per-shape table and prose."""
+    if not r:
+        return None
+    keep = ("kernel", "bound", "achieved", "peak", "unit", "frac", "traffic", "launches", "avg_launch_us",
+            "flop_per_launch", "bytes_per_launch", "timing")
+    out = {k: r[k] for k in keep if k in r}
+    if r.get("traffic") and r.get("bytes_per_launch"):
+        out["traffic_over_algorithmic"] = r["traffic"] / r["bytes_per_launch"]
+    return out
+
+
+def compact_line(line, detail_path=None):
+    """The one JSON line a driver parses: the headline, its roofline / link roofline / CPU baseline, one short
+    record per workload and a few numbers per multi-tenant run.  Per-shape tables, per-kernel lists, per-model
+    percentiles and the ablation live in the detail file."""
+    out = {k: line[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config", "swap",
+                                "warm_ms_p50", "cold_over_warm") if k in line}
+    out["roofline"] = compact_roofline(line.get("roofline"))
+    lr = line.get("link_roofline") or {}
+    out["link_roofline"] = {k: lr[k] for k in ("bound", "bytes_waited_for", "floor_ms_at_measured_link",
+                                               "frac_of_measured_link_floor", "floor_ms_at_nominal_64") if k in lr} or None
+    cpu = line.get("cpu_baseline")
+    out["cpu_baseline"] = ({k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample", "cpu", "os_cpu_count",
+                                                "logits_rel_err_vs_gpu") if k in cpu} if cpu else None)
+    wl = {}
+    for name, res in (line.get("workloads") or {}).items():
+        if name == "multitenant-64":
+            continue
+        roof = (line.get("rooflines") or {}).get(name) or {}
+        lrw = res.get("link_roofline") or {}
+        wl[name] = dict(cold_ms_p50=res["cold_ms_p50"], warm_ms_p50=res["warm_ms_p50"],
+                        cold_over_warm=res["cold_over_warm"], swap_gbps=res["swap_gbps_p50"],
+                        frac_of_link=res["swap_frac_of_link"], cold_over_link_floor=(
+                            1.0 / lrw["frac_of_measured_link_floor"] if lrw.get("frac_of_measured_link_floor") else None),
+                        launches=res.get("ops"), kernel=roof.get("kernel"), frac=roof.get("frac"),
+                        avg_launch_us=roof.get("avg_launch_us"))
+    out["workloads"] = wl
+    mt = ((line.get("workloads") or {}).get("multitenant-64") or {}).get("runs") or {}
+    if mt:
+        out["multitenant"] = {
+            run: dict(seconds=r.get("wall_s"), dispatch=r.get("dispatch"), hit_ratio=r["hit_ratio"],
+                      p50_ms=r["latency_ms"]["p50"], p99_ms=r["latency_ms"]["p99"], hit_p50_ms=r["hit_ms"]["p50"],
+                      hit_p99_ms=r["hit_ms"]["p99"], miss_p50_ms=r["miss_ms"]["p50"], swap_gbps=r.get("swap_gbps"))
+            for run, r in mt.items()}
+    if detail_path:
+        out["detail"] = detail_path
+    out = trim(out)
+    # never let the line outgrow what the driver reads: drop the optional blocks, largest first
+    for victim in ("multitenant", "workloads", "link_roofline"):
+        if len(json.dumps(out, separators=(",", ":"))) <= COMPACT_LIMIT_BYTES:
+            break
+        out.pop(victim, None)
+    return out
+
+
+def write_detail(line, path=None):
+    """Everything measured, as indented JSON beside the other run outputs; returns the path written (relative to the
+    repository) or None when the directory cannot be written."""
+    path = path or os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(trim(line, 6), f, indent=1)
+    except OSError as e:
+        print(f"bench.py: detail file not written: {e}", file=sys.stderr)
+        return None
+    return os.path.relpath(path, ROOT)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -413,6 +531,7 @@ def main():
                     help="also measure cold p50 per config with per-tensor groups, one whole-image group, weights "
                          "sent as they are, and lookups that wait for their table")
     ap.add_argument("--ablation-variant", default=None, help=argparse.SUPPRESS)   # child of --ablate
+    ap.add_argument("--detail", default=None, help="where the full results go (default gpurun_out/bench_detail.json)")
     args = ap.parse_args()
     import __graft_entry__
     __graft_entry__.ensure_built()      # a fresh checkout is compiled first; a built tree is used as it is
@@ -496,7 +615,8 @@ def main():
             runs=runs)
     if args.ablate:
         line["ablation"] = ablation(names, max(args.steps // 2, 5), max(args.warmup, 8))
-    print(json.dumps(line))
+    detail_path = write_detail(line, args.detail)
+    print(json.dumps(compact_line(line, detail_path), separators=(",", ":")))
 
 
 if __name__ == "__main__":
