@@ -67,6 +67,8 @@ typedef struct tp_server tp_server;
 #define TP_FLAG_EVICT_LRU 2 /* plain LRU eviction, as env EVICT_POLICY=LRU (controller.hpp:103-109); default: two-class */
 #define TP_FLAG_NO_HOST_GATHER 4 /* embedding lookups always wait for their table's transfer group, as env TORPOR_HOST_GATHER=0 */
 #define TP_FLAG_NO_PACK 8 /* weights cross the link as they are instead of in the packed transfer format, as env TORPOR_PACK=0 */
+#define TP_FLAG_POOL_FIXED 32 /* pool policy of FixedSizeBlockManager, as env BLOCK_MANAGER=Fixed (memory_manager.hpp:46-52,
+                               * block_manager.hpp:188-258): released extents are kept per exact size and reused, newest first */
 #define TP_FLAG_KEEP_HOST_IMAGE 16 /* keep the raw weight image in pinned host memory beside the packed transfer image (by default the
                                    * transfer image, checked to decode back bit for bit, is the host store), as env TORPOR_SLIM_HOST=0 */
 
@@ -178,6 +180,8 @@ typedef struct tp_pool_stats {
     uint64_t host_image_bytes, host_transfer_bytes, host_staging_bytes;
     /* device memory outside the pool and its budget: staging area of packed transfers, kernel workspace */
     uint64_t device_staging_bytes, device_workspace_bytes;
+    /* TP_FLAG_POOL_FIXED: released extents waiting in the per-size idle lists (not part of `used`) */
+    uint64_t pool_cached_bytes, pool_idle_extents;
 } tp_pool_stats;
 
 typedef struct tp_model_info {
@@ -336,6 +340,16 @@ int tp_host_free(tp_server* s, void* ptr);
 
 /* ------------------------------------------------------------------ introspection (tests, bench) */
 int tp_model_resident(tp_server* s, int32_t client); /* 1/0, negative on error */
+/* 1 when the function is resident and every transfer group of its last swap-in is in place, 0 while a swap-in is
+ * still on its way or the function is swapped out (asked of the device without waiting).  The reference keeps this
+ * per tensor in ParamLocMap (memory_manager.hpp:33,590) and never exposes it. */
+int tp_model_loaded(tp_server* s, int32_t client);
+/* What a scheduler above the boundary needs in order to place a request of a swapped-out function: how long the
+ * swap-in occupies the host link before the request can complete (bytes the request waits for / the link rate the
+ * engine measured), and the forward pass on its own (timed at registration, the best warm request since).  The
+ * reference's router and simulator work from per-model constants instead (scripts/router.py:17,
+ * misc/tools/node_simu.py:99-117). */
+int tp_get_load_estimate(tp_server* s, int32_t client, double* swap_ms, double* forward_ms);
 int tp_get_model_info(tp_server* s, int32_t client, tp_model_info* out);
 int tp_get_pool_stats(tp_server* s, tp_pool_stats* out);
 int tp_get_swap_stats(tp_server* s, int32_t client, tp_swap_stats* out);
@@ -383,7 +397,14 @@ int tp_profile_read(tp_server* s, int32_t index, tp_kernel_stat* out);
  * tp_lru:  LRUEvictor (evictor.hpp:190-264).  check_and_add writes the victims, oldest first and
  *          newline-separated, into `victims` (truncated to `cap` bytes incl. the terminator). */
 typedef struct tp_pool tp_pool;
+#define TP_POOL_BEST_FIT 0   /* default */
+#define TP_POOL_FIXED_SIZE 1 /* FixedSizeBlockManager (block_manager.hpp:188-258): per-size idle lists, newest first;
+                              * idle extents are given back, largest size first, when a new size does not fit */
 tp_pool* tp_pool_create(uint64_t capacity_bytes);
+tp_pool* tp_pool_create_policy(uint64_t capacity_bytes, int32_t policy);
+/* fixed-size policy: bytes and count of idle extents; tp_pool_trim gives them all back and returns the count */
+int tp_pool_cached(tp_pool* p, uint64_t* cached_bytes, uint64_t* idle_extents);
+int tp_pool_trim(tp_pool* p);
 void tp_pool_destroy(tp_pool* p);
 uint64_t tp_pool_alloc(tp_pool* p, uint64_t bytes);
 int tp_pool_release(tp_pool* p, uint64_t offset);

@@ -11,6 +11,10 @@
               interference-aware scheduling decisions over executor states, residency and the
               PCIe-sibling and peer-link tables (defaults: the reference's 4-GPU tables,
               controller.hpp:117-118).
+  FixedBlocksRef  include/server/block_manager.hpp:188-258 (FixedSizeBlockManager): a byte budget over
+              raw device allocations, idle lists per exact size (taken from the back), and idle blocks
+              freed largest size first (the map is ordered by std::greater, common/include/types.hpp:31)
+              when the budget does not cover a new size.  Blocks are numbered instead of addressed.
   signal_*    proto3 wire bytes of proto/signal.proto:5-30, written from the protobuf encoding
               spec (varint field keys, length-delimited strings, default values omitted).
 
@@ -21,7 +25,8 @@ when one GPU holds it) on random multi-GPU traces, and on hand-worked traces; Sc
 hand-worked cases over the reference's 4-GPU tables and against exhaustive properties (never a
 busy GPU, a resident idle GPU always wins, the sibling-status minimum); the codec against the known-answer byte strings derived by hand from
 the proto3 spec and against the installed `google.protobuf` runtime with a descriptor built in
-code (tests/test_wire.py).
+code (tests/test_wire.py); FixedBlocksRef on a hand-worked trace read off the reference's code and by
+conservation (budget + bytes of live and idle blocks is constant, tests/test_host_logic.py).
 """
 from collections import OrderedDict
 
@@ -60,6 +65,45 @@ class LruRef:
 
     def unlock(self, func):
         self.locked.discard(func)
+
+
+class FixedBlocksRef:
+    def __init__(self, budget):
+        self.budget = budget
+        self.idle = {}            # size -> [block ids], released last at the back
+        self.next_block = 0
+        self.over_budget = 0      # block_manager.hpp:222-234: allocated although the budget was spent
+
+    def acquire(self, size):
+        """Returns (block, reused, freed): the block handed out, whether it came from the idle list of
+        its size, and the idle blocks freed to make room, in order."""
+        lst = self.idle.get(size)
+        if lst:                                            # block_manager.hpp:193-198
+            return lst.pop(), True, []
+        freed = []
+        if self.budget < size:                             # block_manager.hpp:205-221
+            for sz in sorted(self.idle, reverse=True):     # std::map<..., std::greater<>>: largest first
+                blocks = self.idle[sz]
+                while blocks:
+                    freed.append((blocks.pop(), sz))
+                    self.budget += sz
+                    if self.budget >= size:
+                        break
+                if self.budget >= size:
+                    break
+        if self.budget >= size:
+            self.budget -= size
+        else:
+            self.over_budget += 1
+        block = self.next_block
+        self.next_block += 1
+        return block, False, freed
+
+    def evict(self, block, size):                          # block_manager.hpp:243-252, free_flag == false
+        self.idle.setdefault(size, []).append(block)
+
+    def idle_bytes(self):
+        return sum(sz * len(b) for sz, b in self.idle.items())
 
 
 class IaRef:

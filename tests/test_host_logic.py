@@ -9,7 +9,7 @@ import re
 import numpy as np
 import pytest
 
-from oracle.host_ref import LruRef
+from oracle.host_ref import FixedBlocksRef, LruRef
 from torpor_amd import _lib
 from torpor_amd._lib import TorporError
 from torpor_amd.functions import resnet
@@ -23,9 +23,18 @@ NOFIT = (1 << 64) - 1
 
 # ---------------------------------------------------------------------------------- pool
 class Pool:
-    def __init__(self, cap):
+    def __init__(self, cap, policy=None):
         self.l = _lib.lib()
-        self.p = self.l.tp_pool_create(cap)
+        self.p = self.l.tp_pool_create(cap) if policy is None else self.l.tp_pool_create_policy(cap, policy)
+        assert self.p
+
+    def cached(self):
+        b, n = C.c_uint64(), C.c_uint64()
+        assert self.l.tp_pool_cached(self.p, C.byref(b), C.byref(n)) == 0
+        return b.value, n.value
+
+    def trim(self):
+        return self.l.tp_pool_trim(self.p)
 
     def alloc(self, n):
         return self.l.tp_pool_alloc(self.p, n)
@@ -90,6 +99,121 @@ def test_pool_random_invariants():
         assert p.release(off) == 0
     q = p.query()
     assert q["used"] == 0 and q["largest_free"] == cap and q["free_extents"] == 1
+
+
+POOL_FIXED = 1
+
+
+def test_fixed_blocks_restatement_on_a_hand_worked_trace():
+    """Read off block_manager.hpp:188-258 by hand: budget 10; sizes in arbitrary units."""
+    r = FixedBlocksRef(10)
+    a, reused, freed = r.acquire(4)
+    assert (a, reused, freed, r.budget) == (0, False, [], 6)
+    b, _, _ = r.acquire(4)
+    c, _, _ = r.acquire(2)
+    assert (b, c, r.budget) == (1, 2, 0)
+    r.evict(a, 4)
+    r.evict(b, 4)
+    r.evict(c, 2)
+    assert r.acquire(4) == (b, True, [])                       # same size: the one released last, no budget change
+    assert r.budget == 0
+    # a size nobody has released: idle blocks are freed largest size first (the 4 before the 2) until it fits
+    d, reused, freed = r.acquire(3)
+    assert (reused, freed, r.budget) == (False, [(a, 4)], 1)
+    e, reused, freed = r.acquire(3)                            # 1 + 2 covers it: the idle 2 goes
+    assert (reused, freed, r.budget, r.over_budget) == (False, [(c, 2)], 0, 0)
+    f, reused, freed = r.acquire(5)                            # nothing left to free: allocated beyond the budget
+    assert (reused, freed, r.over_budget) == (False, [], 1)
+    assert len({a, b, c, d, e, f}) == 6
+
+
+def test_fixed_size_pool_matches_the_restatement_and_keeps_the_pool_invariants():
+    """The fixed-size policy of the pool against FixedBlocksRef on random traces of a few recurring sizes
+    (models come in a few sizes): a request served from the idle list gets the extent released last at
+    that size in both; when a new size needs room, the idle extents given back are the restatement's, in
+    its order, until the request fits (the pool may need more of them than the byte budget alone says,
+    because its extents must be contiguous - never fewer); and the best-fit invariants hold throughout:
+    no overlap, inside the arena, used = sum of live extents."""
+    rng = random.Random(11)
+    cap = 96 * SLAB
+    sizes = [1 * SLAB, 3 * SLAB, 7 * SLAB, 12 * SLAB, 20 * SLAB]
+    for trial in range(6):
+        p = Pool(cap, POOL_FIXED)
+        ref = FixedBlocksRef(cap)
+        live = {}          # offset -> (size, ref block)
+        where = {}         # ref block -> offset of the extent that stands for it
+        reuses = trims = 0
+        for step in range(1500):
+            if live and (rng.random() < 0.5 or sum(s for s, _ in live.values()) > 0.8 * cap):
+                off = rng.choice(sorted(live))
+                sz, blk = live.pop(off)
+                assert p.release(off) == 0
+                ref.evict(blk, sz)
+                continue
+            sz = rng.choice(sizes)
+            idle_before = {s: list(b) for s, b in ref.idle.items()}
+            cached_before, n_before = p.cached()
+            assert cached_before == ref.idle_bytes() and n_before == sum(len(b) for b in ref.idle.values())
+            off = p.alloc(sz - rng.randint(0, SLAB - 1))        # any byte count that rounds to this size
+            if idle_before.get(sz):
+                blk, reused, freed = ref.acquire(sz)
+                assert reused and off == where[blk], "the extent released last at this size is reused"
+                live[off] = (sz, blk)
+                reuses += 1
+                continue
+            # a new size: the order in which idle extents would go, largest size first, newest first
+            order = [(b, s) for s in sorted(idle_before, reverse=True) for b in reversed(idle_before[s])]
+            cached_after, n_after = p.cached()
+            k = n_before - n_after
+            assert cached_before - cached_after == sum(s for _, s in order[:k])
+            # bring the restatement to the same state: it frees by bytes, the pool until a contiguous fit
+            ref.budget = max(ref.budget, 0)
+            for b, s in order[:k]:
+                ref.idle[s].remove(b)
+                ref.budget += s
+                del where[b]
+            trims += k
+            if off == NOFIT:
+                assert k == len(order), "refused only after every idle extent has been given back"
+                assert p.query()["largest_free"] < sz
+                continue
+            blk = ref.next_block
+            ref.next_block += 1
+            ref.budget -= sz
+            where[blk] = off
+            live[off] = (sz, blk)
+            assert off % SLAB == 0 and off + sz <= cap
+            spans = sorted([(o, o + s) for o, (s, _) in live.items()] + [(where[b], where[b] + s) for s, bl in ref.idle.items() for b in bl])
+            for (a0, a1), (b0, b1) in zip(spans, spans[1:]):
+                assert a1 <= b0, "live and idle extents never overlap"
+            q = p.query()
+            assert q["used"] == sum(s for s, _ in live.values()) and q["live"] == len(live)
+        assert reuses > 200 and trims > 5
+        for off in list(live):
+            assert p.release(off) == 0
+        n_idle = p.cached()[1]
+        assert p.trim() == n_idle and p.cached() == (0, 0)
+        q = p.query()
+        assert q["used"] == 0 and q["largest_free"] == cap and q["free_extents"] == 1
+
+
+def test_host_only_engine_with_the_fixed_size_pool_reuses_a_models_extents(monkeypatch):
+    """BLOCK_MANAGER=Fixed (memory_manager.hpp:46-52): a model swapped out and in again lands where it was,
+    and the idle extents are visible in the pool statistics."""
+    monkeypatch.setenv("BLOCK_MANAGER", "Fixed")
+    with Server(mem_limit_bytes=1 << 30, pool_bytes=1 << 30, host_only=True) as s:
+        _register(s, 0)
+        _register(s, 1, seed=1)
+        before = (s.model_info(0)["weight_off"], s.model_info(0)["act_off"])
+        st0 = s.pool_stats()      # the per-allocation extents of the tracked runs wait in the idle lists already
+        assert s.signal(REQ_UNLOAD, 0)[0] == ACK_OK
+        st = s.pool_stats()
+        assert st["pool_idle_extents"] == st0["pool_idle_extents"] + 2
+        assert st["pool_cached_bytes"] == st0["pool_cached_bytes"] + s.model_info(0)["total_bytes"]
+        assert st["used"] == st0["used"] - s.model_info(0)["total_bytes"]
+        assert s.signal(REQ_LOAD, 0)[0] == ACK_OK
+        assert (s.model_info(0)["weight_off"], s.model_info(0)["act_off"]) == before
+        assert s.pool_stats()["pool_idle_extents"] == st0["pool_idle_extents"]
 
 
 def test_pool_at_288_gb_with_ten_thousand_live_extents():

@@ -79,7 +79,7 @@ class PoolStats(C.Structure):
         "capacity", "used", "largest_free", "live_extents", "free_extents",
         "lru_budget", "lru_used", "lru_models", "evictions", "swap_ins", "fragmentation_evictions",
         "host_image_bytes", "host_transfer_bytes", "host_staging_bytes", "device_staging_bytes",
-        "device_workspace_bytes")]
+        "device_workspace_bytes", "pool_cached_bytes", "pool_idle_extents")]
 
 
 class ModelInfo(C.Structure):
@@ -143,6 +143,8 @@ SYMBOLS = {
                             C.POINTER(C.c_float), _I32]),
     "tp_replay": (C.c_int, [_P, _I32, _P, _U64, _P, _U64]),
     "tp_model_resident": (C.c_int, [_P, _I32]),
+    "tp_model_loaded": (C.c_int, [_P, _I32]),
+    "tp_get_load_estimate": (C.c_int, [_P, _I32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "tp_get_model_info": (C.c_int, [_P, _I32, C.POINTER(ModelInfo)]),
     "tp_get_pool_stats": (C.c_int, [_P, C.POINTER(PoolStats)]),
     "tp_get_swap_stats": (C.c_int, [_P, _I32, C.POINTER(SwapStats)]),
@@ -156,6 +158,9 @@ SYMBOLS = {
     "tp_profile_end": (C.c_int, [_P]),
     "tp_profile_read": (C.c_int, [_P, _I32, C.POINTER(KernelStat)]),
     "tp_pool_create": (_P, [_U64]),
+    "tp_pool_create_policy": (_P, [_U64, _I32]),
+    "tp_pool_cached": (C.c_int, [_P, C.POINTER(_U64), C.POINTER(_U64)]),
+    "tp_pool_trim": (C.c_int, [_P]),
     "tp_pool_destroy": (None, [_P]),
     "tp_pool_alloc": (_U64, [_P, _U64]),
     "tp_pool_release": (C.c_int, [_P, _U64]),

@@ -396,6 +396,18 @@ int tp_model_resident(tp_server* s, int32_t client) {
     return E.model_resident(client);
     TP_GUARD_END
 }
+int tp_model_loaded(tp_server* s, int32_t client) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.model_loaded(client);
+    TP_GUARD_END
+}
+int tp_get_load_estimate(tp_server* s, int32_t client, double* swap_ms, double* forward_ms) {
+    TP_GUARD_BEGIN
+    ENG(s);
+    return E.load_estimate(client, swap_ms, forward_ms);
+    TP_GUARD_END
+}
 int tp_get_model_info(tp_server* s, int32_t client, tp_model_info* out) {
     TP_GUARD_BEGIN
     ENG(s);
@@ -480,6 +492,28 @@ tp_pool* tp_pool_create(uint64_t capacity_bytes) {
     } catch (...) {
         return nullptr;
     }
+}
+tp_pool* tp_pool_create_policy(uint64_t capacity_bytes, int32_t policy) {
+    if (policy != TP_POOL_BEST_FIT && policy != TP_POOL_FIXED_SIZE) return nullptr;
+    try {
+        auto* p = new tp_pool;
+        p->pool.reset(capacity_bytes, policy);
+        return p;
+    } catch (...) {
+        return nullptr;
+    }
+}
+int tp_pool_cached(tp_pool* p, uint64_t* cached_bytes, uint64_t* idle_extents) {
+    if (!p) return TP_EINVAL;
+    if (cached_bytes) *cached_bytes = p->pool.cached_bytes();
+    if (idle_extents) *idle_extents = p->pool.idle_extents();
+    return 0;
+}
+int tp_pool_trim(tp_pool* p) {
+    TP_GUARD_BEGIN
+    if (!p) return TP_EINVAL;
+    return (int)p->pool.trim();
+    TP_GUARD_END
 }
 void tp_pool_destroy(tp_pool* p) { delete p; }
 uint64_t tp_pool_alloc(tp_pool* p, uint64_t bytes) {

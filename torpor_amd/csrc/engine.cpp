@@ -136,7 +136,11 @@ int Engine::init() {
         lru_.two_class = !((cfg_.flags & TP_FLAG_EVICT_LRU) || (pol && std::string(pol) == "LRU"));
     }
     lru_.set_budget(cfg_.mem_limit_bytes);
-    pool_.reset(cfg_.pool_bytes);
+    {
+        const char* bm = std::getenv("BLOCK_MANAGER");  // memory_manager.hpp:46-52
+        const bool fixed = (cfg_.flags & TP_FLAG_POOL_FIXED) || (bm && std::string(bm) == "Fixed");
+        pool_.reset(cfg_.pool_bytes, fixed ? SlabPool::kFixedSize : SlabPool::kBestFit);
+    }
     log_.open(cfg_.device);
     log_.write(ExecLog::INFO, "Executor %d started: budget %llu MiB, pool %llu MiB, first transfer group %llu KiB, %s eviction",
                cfg_.device, (unsigned long long)(cfg_.mem_limit_bytes >> 20), (unsigned long long)(pool_.capacity() >> 20),
@@ -189,14 +193,44 @@ int Engine::init() {
         const uint64_t half = cfg_.workspace_bytes / 2;
         const uint64_t n = std::min<uint64_t>(std::min<uint64_t>(half / 2, h2d_cap_ / 2), 8ull << 20) & ~uint64_t(255);
         if (n) {
-            for (int rep = 0; rep < 24; ++rep) {
+            // The second half of the burst is timed: both streams taking turns, as a swap-in of a link-bound
+            // model drives them, is the rate the swap-in plans are made with until tp_measure_h2d is asked
+            // for the single-copy figure.
+            hipEvent_t ev_a = nullptr, ev_b = nullptr, ev_2 = nullptr;
+            (void)hipEventCreate(&ev_a);
+            (void)hipEventCreate(&ev_b);
+            (void)hipEventCreateWithFlags(&ev_2, hipEventDisableTiming);
+            constexpr int kBurst = 24, kTimedFrom = 12;
+            for (int rep = 0; rep < kBurst; ++rep) {
+                if (rep == kTimedFrom && ev_a && ev_2) {
+                    (void)hipEventRecord(ev_2, copy2_);
+                    (void)hipStreamWaitEvent(copy_, ev_2, 0);  // both streams start the timed half together
+                    (void)hipEventRecord(ev_a, copy_);
+                    (void)hipStreamWaitEvent(copy2_, ev_a, 0);
+                }
                 HIPCHK(hipMemcpyAsync(ws + half, h2d_stage_, n, hipMemcpyHostToDevice, copy_));
                 HIPCHK(hipMemcpyAsync(ws + half + n, h2d_stage_ + n, n, hipMemcpyHostToDevice, copy2_));
+            }
+            if (ev_a && ev_b && ev_2) {
+                (void)hipEventRecord(ev_2, copy2_);
+                (void)hipStreamWaitEvent(copy_, ev_2, 0);
+                (void)hipEventRecord(ev_b, copy_);
             }
             (void)tpk::launch_copy(ws + half, ws + half + n, 4096, decode_);
             HIPCHK(hipStreamSynchronize(copy_));
             HIPCHK(hipStreamSynchronize(copy2_));
             HIPCHK(hipStreamSynchronize(decode_));
+            float burst_ms = 0.f;
+            if (ev_a && ev_b && hipEventElapsedTime(&burst_ms, ev_a, ev_b) == hipSuccess && burst_ms > 0.f) {
+                const double gbps = 2.0 * (kBurst - kTimedFrom) * (double)n / (burst_ms * 1e-3) / 1e9 / 0.99;
+                if (gbps > 1.0 && gbps < 1000.0) link_gbps_ = gbps;
+            } else {
+                (void)hipGetLastError();
+            }
+            if (ev_a) (void)hipEventDestroy(ev_a);
+            if (ev_b) (void)hipEventDestroy(ev_b);
+            if (ev_2) (void)hipEventDestroy(ev_2);
+            log_.write(ExecLog::INFO, "Host link measured at %.1f GB/s", link_gbps_);
             // One swap-in in the first few dozen of a process used to take 6.5 ms longer: a single
             // hipMemcpyAsync call of one of its first groups blocked that long on the host (timed per call,
             // tp_swap_stats.max_call_*), whatever the model.  It is a one-time set-up inside the runtime that
@@ -248,16 +282,10 @@ Engine::~Engine() {
         (void)hipDeviceSynchronize();
     }
     for (auto& kv : models_) {
-        Model& m = *kv.second;
-        free_host_store(m);
-        if (!host_only()) {
-            for (auto ev : m.dma_ev) (void)hipEventDestroy(ev);
-            for (auto ev : m.chunk_ev) (void)hipEventDestroy(ev);
-            if (m.t0) (void)hipEventDestroy(m.t0);
-            if (m.t1) (void)hipEventDestroy(m.t1);
-            drop_graph(m);
-        }
+        kv.second->copy_state.store(CS_IDLE);  // the copy thread is gone: a job it never took is not waited for
+        destroy_model(*kv.second);
     }
+    models_.clear();
     for (auto& kv : user_pinned_) host_free(reinterpret_cast<void*>(kv.first));
     user_pinned_.clear();
     if (!host_only()) {
@@ -905,7 +933,7 @@ int Engine::build_transfer(Model& m) {
     // A model whose forward pass outlasts its swap-in hides the copy behind compute as it is; the
     // expansion kernels would only compete with its own (measured on MobileNetV2, EfficientNet-B0,
     // DenseNet-169/201: cold equal or up to 0.04 ms slower with the format than without).
-    if (m.warm_us > 0 && (double)m.image_bytes / 54.0e3 < 0.8 * m.warm_us) return 0;
+    if (m.warm_us > 0 && (double)m.image_bytes / stream_rate_bytes_per_us(1, 32ull << 20) < 0.8 * m.warm_us) return 0;
     std::vector<int32_t> base(m.params.size(), -1);
     std::vector<uint64_t> n_ext(m.params.size(), 0), tab_off(m.params.size(), 0), ext_off(m.params.size(), 0);
     std::vector<uint64_t> t_off(m.params.size(), 0);
@@ -1224,15 +1252,19 @@ void Engine::choose_copy_plan(Model& m) {
         double flops, bytes;
         const char* name;
         op_work(op, &flops, &bytes, &name);
-        est += std::max(6.0, std::max(flops / 5.0e7, bytes / 2.0e6));  // 50 TFLOP/s, 2 TB/s, 6 us floor
+        // only used before the first timed forward pass exists (an engine without a device): 50 TFLOP/s, 2 TB/s, 6 us floor
+        est += std::max(6.0, std::max(flops / 5.0e7, bytes / 2.0e6));
         kernels += (op.kind == OPK_GEMM || op.kind == OPK_CONV) ? 1.5 : 1.0;
     }
     if (compute_us <= 0) compute_us = est;
     const double bytes = (double)(m.timg ? m.timg_bytes : m.image_bytes);  // what crosses the link
-    const double t1 = std::max(bytes / 54.0e3, compute_us + kernels * 1.2);
+    // Rates follow the link this engine measured (init, tp_measure_h2d), not a figure of the box they were
+    // tuned on: two streams hide each copy's fixed cost and deliver about 99 % of it; one stream pays the fixed
+    // cost once per group (its groups grow to 32 MiB).
+    const double t1 = std::max(bytes / stream_rate_bytes_per_us(1, 32ull << 20), compute_us + kernels * 1.2);
     // (measured on ResNet-152 batch 8: kernels that share the device with two copy streams run
     // about 15 % longer, on top of the per-launch cost)
-    const double t2 = std::max(bytes / 56.5e3, compute_us * 1.15 + kernels * 2.4);
+    const double t2 = std::max(bytes / stream_rate_bytes_per_us(2, 16ull << 20), compute_us * 1.15 + kernels * 2.4);
     m.ncopy = (t2 <= t1) ? 2 : 1;
     if (copy_streams_cfg_ == 1 || copy_streams_cfg_ == 2) m.ncopy = copy_streams_cfg_;
     m.chunk_max = cfg_.chunk_max_bytes;
@@ -1242,6 +1274,17 @@ void Engine::choose_copy_plan(Model& m) {
     // 56.3 GB/s and 18.66-18.69 ms.  The size in the middle of the image costs a link-bound request nothing,
     // since the groups shrink again towards the end (build_chunks); 32 MiB was no faster and worse for ResNet-50.
     if (chunk_max_auto_ && m.ncopy == 2) m.chunk_max = std::max<uint64_t>(cfg_.chunk_max_bytes, 16ull << 20);
+}
+
+// Sustained swap-in rate, in bytes per microsecond, of `streams` copy streams moving groups of `group`
+// bytes over the measured link.  Every hipMemcpyAsync carries a fixed cost (kCopyFixedUs, measured: 51 GB/s
+// at 8 MiB and 55 GB/s at 32 MiB groups on one stream of a 57 GB/s link); one stream pays it per group,
+// two streams overlap it with the other stream's transfer and lose about 1 %.
+double Engine::stream_rate_bytes_per_us(int streams, uint64_t group) const {
+    const double link = link_gbps_ * 1.0e3;  // bytes per microsecond
+    if (streams >= 2) return 0.99 * link;
+    const double g = (double)group;
+    return g / (g / link + kCopyFixedUs);
 }
 
 // Transfer groups: the first is chunk_bytes, each next one doubles up to chunk_max_bytes, so the
@@ -1608,22 +1651,45 @@ bool Engine::check_eviction(Model& m) {
 }
 
 // ------------------------------------------------------------------ controller
+// Everything a model holds, given back: its place in the eviction order, a copy that may still be
+// running, pool extents (the weight image, the activation arena, and the per-allocation extents of a
+// registration that never reached its layout step), the host store, events and a captured graph.  The
+// one teardown path of a replaced registration, an abandoned one and the engine's own end; the caller
+// erases the entry.
+void Engine::destroy_model(Model& m) {
+    lru_.force_evict(std::to_string(m.id));
+    wait_copy_idle(m);
+    if (!host_only() && m.touch_seq > synced_seq_ && hipStreamSynchronize(compute_) == hipSuccess)
+        synced_seq_ = work_seq_;  // its last kernels may still run
+    for (auto& kv : m.ablocks) {
+        if (kv.second.pool_off != UINT64_MAX) pool_.release(kv.second.pool_off);
+        kv.second.pool_off = UINT64_MAX;
+    }
+    if (m.w_pool_off != UINT64_MAX) pool_.release(m.w_pool_off);
+    if (m.a_pool_off != UINT64_MAX) pool_.release(m.a_pool_off);
+    m.w_pool_off = m.a_pool_off = UINT64_MAX;
+    m.w_dev = m.a_dev = nullptr;
+    m.resident = m.fully_loaded = false;
+    m.copy_state.store(CS_IDLE);
+    free_host_store(m);
+    if (!host_only()) {
+        for (auto ev : m.dma_ev) (void)hipEventDestroy(ev);
+        for (auto ev : m.chunk_ev) (void)hipEventDestroy(ev);
+        m.dma_ev.clear();
+        m.chunk_ev.clear();
+        if (m.t0) (void)hipEventDestroy(m.t0);
+        if (m.t1) (void)hipEventDestroy(m.t1);
+        m.t0 = m.t1 = nullptr;
+        drop_graph(m);
+    }
+}
+
 void Engine::start_cold(int id, int level) {
     // controller.hpp:402-413 + cuda_server.hpp:223-228 (Startup): a re-registration replaces
     // the previous model of that id
     Model* old = find(id);
     if (old) {
-        lru_.force_evict(std::to_string(id));
-        evict_model(*old);
-        wait_copy_idle(*old);
-        free_host_store(*old);
-        if (!host_only()) {
-            for (auto ev : old->dma_ev) (void)hipEventDestroy(ev);
-            for (auto ev : old->chunk_ev) (void)hipEventDestroy(ev);
-            if (old->t0) (void)hipEventDestroy(old->t0);
-            if (old->t1) (void)hipEventDestroy(old->t1);
-            drop_graph(*old);
-        }
+        destroy_model(*old);
         models_.erase(id);
     }
     auto m = std::make_unique<Model>();
@@ -1756,10 +1822,7 @@ int Engine::cancel_deferred(uint64_t ticket) {
                     Model* m = find(id);
                     if (!host_only()) (void)hipStreamSynchronize(compute_);  // its tracked kernels may still run
                     if (m) {
-                        for (auto& kv : m->ablocks)
-                            if (kv.second.pool_off != UINT64_MAX) pool_.release(kv.second.pool_off);
-                        if (m->w_pool_off != UINT64_MAX) pool_.release(m->w_pool_off);
-                        free_host_store(*m);
+                        destroy_model(*m);
                         models_.erase(id);
                     }
                     active_ = -1;
@@ -2561,6 +2624,36 @@ int Engine::model_resident(int client) {
     return m->resident ? 1 : 0;
 }
 
+// 1 when every transfer group of the resident model is in place (asked of the device without waiting), 0 while
+// a swap-in is on its way or the model is swapped out.
+int Engine::model_loaded(int client) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (!m->resident || m->state != MS_READY) return 0;
+    if (m->fully_loaded || host_only() || m->chunk_end.empty()) return 1;
+    if (m->copy_error.load() || m->cancel.load()) return 0;
+    return landed(*m, (uint32_t)m->chunk_end.size() - 1) ? 1 : 0;
+}
+
+// How long the host link is busy with the part of a swap-in that a request has to wait for, and the
+// forward pass alone (timed at registration, the best warm request since).
+int Engine::load_estimate(int client, double* swap_ms, double* forward_ms) {
+    std::lock_guard<std::mutex> lk(mu_);
+    Model* m = find(client);
+    if (!m) return TP_ENOENT;
+    if (m->state != MS_READY) return TP_ESTATE;
+    if (m->chunk_end.empty()) build_chunks(*m);
+    uint64_t bytes = m->timg ? m->timg_bytes : m->image_bytes;
+    if (m->defer_from != UINT32_MAX && m->defer_from > 0 && m->defer_from < m->chunk_end.size()) {
+        const uint64_t from = m->chunk_end[m->defer_from - 1];
+        bytes = m->timg ? xfer_off(*m, from) : from;
+    }
+    if (swap_ms) *swap_ms = (double)bytes / stream_rate_bytes_per_us(m->ncopy, m->chunk_max ? m->chunk_max : (16ull << 20)) / 1000.0;
+    if (forward_ms) *forward_ms = m->warm_us / 1000.0;
+    return 0;
+}
+
 int Engine::model_info(int client, tp_model_info* out) {
     std::lock_guard<std::mutex> lk(mu_);
     if (!out) return TP_EINVAL;
@@ -2606,6 +2699,8 @@ int Engine::pool_stats(tp_pool_stats* out) {
     for (auto& kv : user_pinned_) out->host_staging_bytes += kv.second;
     out->device_staging_bytes = xfer_stage_cap_;
     out->device_workspace_bytes = host_only() ? 0 : cfg_.workspace_bytes;
+    out->pool_cached_bytes = pool_.cached_bytes();
+    out->pool_idle_extents = pool_.idle_extents();
     return 0;
 }
 
@@ -2715,6 +2810,7 @@ int Engine::measure_h2d(uint64_t bytes, int iters, double* gbps) {
         std::sort(ms.begin(), ms.end());
         const double med = ms[ms.size() / 2];
         *gbps = (double)bytes / (med * 1e-3) / 1e9;
+        if (bytes >= (64ull << 20) && *gbps > 1.0) link_gbps_ = *gbps;  // a copy long enough to show the link itself
     }
     (void)hipEventDestroy(a);
     (void)hipEventDestroy(b);

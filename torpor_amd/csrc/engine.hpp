@@ -231,6 +231,8 @@ public:
     int replay(int client, const void* in, uint64_t in_bytes, void* out, uint64_t out_bytes);
 
     int model_resident(int client);
+    int model_loaded(int client);
+    int load_estimate(int client, double* swap_ms, double* forward_ms);
     int model_info(int client, tp_model_info* out);
     int pool_stats(tp_pool_stats* out);
     int swap_stats(int client, tp_swap_stats* out);
@@ -290,6 +292,7 @@ private:
     int start_execute(int id);
     int swap_in(Model& m);
     void evict_model(Model& m);
+    void destroy_model(Model& m);
     bool check_eviction(Model& m);
     void complete_request();
     void start_next_queued();
@@ -298,6 +301,7 @@ private:
     int build_image(Model& m, bool by_access);
     void build_chunks(Model& m);
     void choose_copy_plan(Model& m);
+    double stream_rate_bytes_per_us(int streams, uint64_t group) const;
     void drop_graph(Model& m);
     int build_graph(Model& m);
     void wait_copy_idle(Model& m);
@@ -346,6 +350,11 @@ private:
     bool slim_host_ = true;  // give up the raw image of a model whose transfer image decodes back to it
     std::vector<uint8_t> host_view_;  // where tp_host_weights decodes such a model's image to (one at a time)
     int copy_streams_cfg_ = 0;
+    // Pinned-host -> HBM rate of this box's link in GB/s: timed on the copy streams when the engine starts,
+    // replaced by tp_measure_h2d's figure when a caller asks for one.  Swap-in plans and load estimates use it.
+    double link_gbps_ = kNominalLinkGbps;
+    static constexpr double kNominalLinkGbps = 56.0;  // until measured (an engine without a device keeps it)
+    static constexpr double kCopyFixedUs = 15.0;      // fixed cost of one hipMemcpyAsync on a copy stream
     bool chunk_max_auto_ = true;
     bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor
     int d2h_kernel_ = 0;

@@ -24,6 +24,7 @@ FLAG_EVICT_LRU = 2   # plain LRU instead of the two-class policy (as env EVICT_P
 FLAG_NO_PACK = 8   # weights cross the link as they are
 FLAG_NO_HOST_GATHER = 4   # embedding lookups wait for their table instead of reading it from host memory
 FLAG_KEEP_HOST_IMAGE = 16   # keep the raw weight image in pinned memory beside the packed transfer image
+FLAG_POOL_FIXED = 32   # the reference's FixedSizeBlockManager policy for the HBM pool (as env BLOCK_MANAGER=Fixed)
 
 
 def _chk(code, what):
@@ -51,7 +52,7 @@ def gemm_noalloc(x, y, c, m, n, k, xs_r, ys_c, ldc, xs_k=1, ys_k=1, nb0=1, nb1=1
 class Server:
     def __init__(self, mem_limit_bytes=0, pool_bytes=0, chunk_bytes=0, chunk_max_bytes=0, workspace_bytes=0,
                  device=0, host_only=False, request_timeout_ms=0, copy_streams=0, evict_lru=False, host_gather=True, pack=True,
-                 keep_host_image=False):
+                 keep_host_image=False, pool_fixed=False):
         self._l = _lib.lib()
         cfg = _lib.Config()
         cfg.struct_size = C.sizeof(_lib.Config)
@@ -63,7 +64,7 @@ class Server:
         cfg.workspace_bytes = workspace_bytes
         cfg.flags = (FLAG_HOST_ONLY if host_only else 0) | (FLAG_EVICT_LRU if evict_lru else 0) | \
             (0 if host_gather else FLAG_NO_HOST_GATHER) | (0 if pack else FLAG_NO_PACK) | \
-            (FLAG_KEEP_HOST_IMAGE if keep_host_image else 0)
+            (FLAG_KEEP_HOST_IMAGE if keep_host_image else 0) | (FLAG_POOL_FIXED if pool_fixed else 0)
         cfg.request_timeout_ms = request_timeout_ms
         cfg.copy_streams = copy_streams
         h = C.c_void_p()
@@ -225,6 +226,19 @@ class Server:
         if r < 0:
             raise TorporError(r, "tp_model_resident")
         return bool(r)
+
+    def loaded(self, fid):
+        """True when the function is resident and its last swap-in has landed completely."""
+        r = self._l.tp_model_loaded(self._h, fid)
+        if r < 0:
+            raise TorporError(r, "tp_model_loaded")
+        return bool(r)
+
+    def load_estimate(self, fid):
+        """(ms the host link is busy before a request of the swapped-out function can complete, ms of its forward pass)."""
+        a, b = C.c_double(), C.c_double()
+        _chk(self._l.tp_get_load_estimate(self._h, fid, C.byref(a), C.byref(b)), "tp_get_load_estimate")
+        return a.value, b.value
 
     def model_info(self, fid):
         o = _lib.ModelInfo()
