@@ -5,8 +5,10 @@ bench.py reports under workloads["multitenant-64"].
 64 random-init models (32 ResNet-50, 16 BERT-base seq 128, 16 ResNet-152; seeds 0..63, batch 1)
 are registered, so all weights sit in the pinned host store; requests then arrive as an open-loop
 Poisson process (default 200 req/s) with Zipf(1.1) popularity over the 64 functions (the arrival
-process of the reference's load generator, scripts/sender_fix_rate.py:46-56) and are served in
-arrival order by the single executor.  Latency = completion - arrival, so it includes queueing.
+process of the reference's load generator, scripts/sender_fix_rate.py:46-56) and are served by the
+single executor, one active function at a time: --dispatch miss-aware (default; requests of resident
+models run while the swap-in of the oldest swapped-out one streams, torpor_amd/dispatch.py) or in-order
+(arrival order).  Latency = completion - arrival, so it includes queueing.
 
 What the pool cap charges: per resident model, its weight image plus its activation arena, each
 rounded up to 2 MiB slabs (the reference also charges every block of a model,
@@ -36,11 +38,14 @@ def main():
     ap.add_argument("--caps-gb", type=float, nargs="+", default=[24.0, 8.0])
     ap.add_argument("--models", type=int, nargs=3, default=[32, 16, 16], metavar=("R50", "BERT", "R152"))
     ap.add_argument("--lookahead", type=int, default=0)
+    ap.add_argument("--dispatch", choices=["in-order", "miss-aware"], default="miss-aware",
+                    help="order in which arrived requests are handed to the executor (torpor_amd/dispatch.py)")
     args = ap.parse_args()
 
     from torpor_amd import multitenant as mt
 
-    runs = {f"cap_{cap:g}GiB": mt.run_cap(cap, args.seconds, args.rate, models=tuple(args.models), lookahead=args.lookahead)
+    runs = {f"cap_{cap:g}GiB": mt.run_cap(cap, args.seconds, args.rate, models=tuple(args.models), lookahead=args.lookahead,
+                                              dispatch=args.dispatch)
             for cap in args.caps_gb}
     primary = runs[next(iter(runs))]
     print(json.dumps({

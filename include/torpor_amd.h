@@ -315,7 +315,14 @@ int tp_bn_inference_pitched(tp_server* s, int32_t client, uint64_t x, uint64_t y
  *   - a shape whose partial sums need more than that array is refused with TP_ESCRATCH (a split only
  *     happens for fewer 64x64 output tiles than CUs, so m * n <= 1 Mi elements; at most 32 splits);
  *   - all calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
- *     race on it.  Calls on one stream are ordered and safe. */
+ *     race on it.  Calls on one stream are ordered and safe.
+ *   - the first call on each GPU looks up that GPU's copy of the array and the device's properties, which
+ *     may load the library's code object: make it before the stretch in which nothing may be allocated
+ *     (outside graph capture); every later call on that GPU only launches.
+ *   - the array's first 4 KiB are per-tile counters that are zero between launches (the workgroup that
+ *     finishes a split tile last sets its counter back).  A launch that never completes (a stream destroyed
+ *     under it, a device reset) leaves them undefined, and later split GEMMs on that GPU would sum wrongly:
+ *     after such an event the process must not go on using this entry point. */
 #define TP_NOALLOC_SCRATCH_BYTES (16u << 20)
 int tp_gemm_noalloc(const tp_gemm_desc* d, void* stream);
 /* cudaLaunchKernelService (cuda_server.hpp:1226-1310) by op id, pointer slots explicit. */

@@ -7,8 +7,16 @@
            `dispatch` (the queue-empty branch), `complete` (router.py:481-489).
   FifoRef  scripts/router.py:156-216 (`baseline_schedule`).
 
+  miss_aware_trace  the miss-aware dispatch order of torpor_amd/dispatch.py as a simulation of a whole trace.
+           The reference has no such policy (its router serves in arrival order, scripts/router.py:289-313; the
+           controller queues while the executor is busy, include/server/controller.hpp:163-186,242-262); what is
+           kept from it is the one-active-function rule and the Load signal (controller.hpp:208-215) that starts
+           a swap-in ahead of the request.  in_order_trace is the reference's order under the same timing model.
+
 Pinning (tests/test_router.py): hand-worked rankings and alpha sequences, sortedness of both
-lists after every re-ranking, and conservation (every request is dispatched exactly once).
+lists after every re-ranking, and conservation (every request is dispatched exactly once); the two dispatch
+simulations on hand-worked traces whose answers follow from the rules by arithmetic, and by their invariants (each
+request runs once, never before it arrives, requests of one function in arrival order, one swap-in at a time).
 """
 
 
@@ -139,3 +147,107 @@ class FifoRef:
         while self.q and self.q[0][0] == f and len(arrs) < self.batch:
             arrs.append(self.q.pop(0)[1])
         return f, arrs
+
+
+# ------------------------------------------------------------------------------------------- dispatch order
+class _Residency:
+    """Which models are in device memory: at most `capacity` of them, the least recently used one leaves when a
+    swap-in needs room (never the one that is running or being swapped in)."""
+
+    def __init__(self, capacity, resident):
+        self.capacity = capacity
+        self.order = list(resident)   # least recent first
+
+    def has(self, f):
+        return f in self.order
+
+    def touch(self, f):
+        self.order.remove(f)
+        self.order.append(f)
+
+    def bring_in(self, f, keep=()):
+        while len(self.order) >= self.capacity:
+            victim = next((g for g in self.order if g not in keep), None)
+            if victim is None:
+                break
+            self.order.remove(victim)
+        self.order.append(f)
+
+
+def _service_end(start, forward, load_start, swap):
+    """When a request ends that starts at `start`: its forward pass, but not before the bytes it waits for have
+    crossed the link (the engine pipelines the copy with the forward pass), plus a tenth of a forward pass for the
+    layers behind the last transfer group."""
+    if load_start is None:
+        return start + forward
+    return max(start + forward, load_start + swap + 0.1 * forward)
+
+
+def in_order_trace(arrivals, fids, est, capacity, resident=()):
+    """The reference's order: each request holds the executor from its start to its end, a request of a
+    swapped-out model starts its swap-in when it starts.  Returns [(kind, seq, time)] with kind "run" / "load",
+    and the end time of every request."""
+    res = _Residency(capacity, resident)
+    t, events, ends = 0.0, [], {}
+    for seq, (a, f) in enumerate(zip(arrivals, fids)):
+        t = max(t, a)
+        swap, fwd = est[f]
+        if res.has(f):
+            res.touch(f)
+            end = _service_end(t, fwd, None, swap)
+        else:
+            res.bring_in(f)
+            events.append(("load", seq, t))
+            end = _service_end(t, fwd, t, swap)
+        events.append(("run", seq, t))
+        ends[seq] = end
+        t = end
+    return events, ends
+
+
+def miss_aware_trace(arrivals, fids, est, capacity, resident=(), margin=0.0003):
+    """State machine over the moments at which the executor is free.  waiting = the one request whose swap-in is
+    on its way: (seq, load start, earliest start)."""
+    n = len(arrivals)
+    res = _Residency(capacity, resident)
+    pending = []                 # seqs that have arrived and not run, arrival order
+    nxt = 0                      # next arrival to admit
+    waiting = None
+    t = 0.0
+    events, ends = [], {}
+    while len(ends) < n:
+        while nxt < n and arrivals[nxt] <= t:
+            pending.append(nxt)
+            nxt += 1
+        if waiting is None:                                   # start the oldest miss's swap-in
+            for s in pending:
+                if not res.has(fids[s]):
+                    swap, fwd = est[fids[s]]
+                    res.bring_in(fids[s])
+                    waiting = (s, t, t + max(0.0, swap - fwd - margin))
+                    events.append(("load", s, t))
+                    break
+        choice = None
+        if waiting is not None and waiting[2] <= t:           # its time has come
+            # the oldest queued request of that function (it is the one the swap-in was started for)
+            choice = next(s for s in pending if fids[s] == fids[waiting[0]])
+        else:
+            busy = fids[waiting[0]] if waiting is not None else None
+            choice = next((s for s in pending if fids[s] != busy and res.has(fids[s])), None)
+        if choice is None:                                    # nothing to do: the next thing that can change that
+            wake = [arrivals[nxt]] if nxt < n else []
+            if waiting is not None:
+                wake.append(waiting[2])
+            t = max(t, min(wake))
+            continue
+        f = fids[choice]
+        swap, fwd = est[f]
+        load_start = None
+        if waiting is not None and fids[waiting[0]] == f:
+            load_start = waiting[1]
+            waiting = None
+        res.touch(f)
+        events.append(("run", choice, t))
+        pending.remove(choice)
+        t = ends[choice] = _service_end(t, fwd, load_start, swap)
+    return events, ends

@@ -106,6 +106,30 @@ def test_stem_convolution(gpu_server, N, H, W, Cout, xl, yl):
     assert_close(fused, np.maximum(zb, 0), 5e-5, "stem+bn+relu")
 
 
+def test_stem_keeps_an_infinity_out_of_rows_whose_receptive_field_does_not_hold_it(gpu_server):
+    """The stem kernel pads its 7 filter rows to 8 MFMA steps per lane half; the step that has no filter row must
+    contribute nothing, also when the input row it would meet holds Inf (0 * Inf is NaN).  Input row 24 is
+    infinite: output rows 11..13 see it (2*ho-3 <= 24 <= 2*ho+3), every other row must equal the oracle's."""
+    rng = np.random.default_rng(5)
+    x = _rand(rng, 1, 3, 64, 64)
+    x[:, :, 24, :] = np.inf
+    w = _rand(rng, 64, 3, 7, 7) * np.float32(1.0 / np.sqrt(147))
+    with OpSession(gpu_server, [w]) as t:
+        xv = t.act(x)
+        yv = t.empty(32 * 32 * 64 * 4)
+        t.s.conv(t.fid, xv, t.w[0], yv, 1, 64, 64, 3, 64, 7, 7, stride=2, pad=3, x_layout=NCHW, y_layout=NHWC)
+        assert t.s.last_kernel().startswith("conv_stem7x7"), t.s.last_kernel()
+        got = t.read(yv, (1, 32, 32, 64))
+    x_fin = x.copy()
+    x_fin[:, :, 24, :] = 0.0
+    z = ref.conv2d(x_fin, w, (2, 2), (3, 3), x_nhwc=False, y_nhwc=True)
+    clean = [ho for ho in range(32) if not (2 * ho - 3 <= 24 <= 2 * ho + 3)]
+    assert clean == [r for r in range(32) if r not in (11, 12, 13)]
+    assert np.all(np.isfinite(got[:, clean])), "an infinity outside the receptive field reached the output"
+    assert_close(got[:, clean], z[:, clean], RTOL, "stem rows away from the infinite input row")
+    assert not np.any(np.isfinite(got[:, 11:14])), "rows that do read the infinite row"
+
+
 def test_conv_identities(gpu_server):
     """Closed forms: a centred delta kernel is the identity; an all-ones 3x3 kernel on an all-ones
     image counts the in-bounds taps (4 / 6 / 9 at corner / edge / interior)."""

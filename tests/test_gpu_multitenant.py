@@ -152,3 +152,44 @@ def test_prefetching_the_models_of_waiting_requests_changes_no_answer():
         assert resident
         for fid in resident:
             assert np.array_equal(s.readback_weights(fid), s.host_weights(fid)), fid
+
+
+def test_miss_aware_dispatch_changes_the_order_and_no_answer():
+    """The same backlogged trace in arrival order and through the miss-aware dispatcher (hits served while the
+    oldest miss's swap-in streams, Load signal of controller.hpp:208-215): every answer equals the function's
+    registration run bit for bit either way, the budget holds after every request, requests of one function keep
+    their order, what is resident at the end reads back byte for byte, and requests that found their model
+    resident wait less in the tail."""
+    limit = int(1.5 * 2 ** 30)
+    with Server(mem_limit_bytes=limit, pool_bytes=2 * limit) as s:
+        fleet = mt.build_fleet(s, 8, 4, 4)
+        assert sum(s.model_info(f["fid"])["total_bytes"] for f in fleet) > 2 * limit      # the cap binds
+        for f in fleet:                                   # the engine's own estimates, which the dispatcher plans with
+            swap_ms, fwd_ms = s.load_estimate(f["fid"])
+            assert 0.05 < swap_ms < 20 and 0.1 < fwd_ms < 20, (f["arch"], swap_ms, fwd_ms)
+        arrivals, picks = mt.make_trace(len(fleet), 800, 500.0, seed=5)
+        over, order = [], []
+
+        def after(i, fid, hit):
+            st = s.pool_stats()
+            if st["lru_used"] > limit:
+                over.append((i, st["lru_used"]))
+            order.append((i, fid))
+
+        r_io = mt.serve(s, fleet, arrivals, picks, check_every=1, after_request=after)
+        order_io, order[:] = list(order), []
+        r_ma = mt.serve(s, fleet, arrivals, picks, check_every=1, after_request=after, dispatch="miss-aware")
+        assert not over, over[:3]
+        assert [i for i, _ in order_io] == list(range(len(picks)))
+        assert sorted(i for i, _ in order) == list(range(len(picks))) and [i for i, _ in order] != list(range(len(picks)))
+        last = {}
+        for i, fid in order:                              # per function: arrival order
+            assert last.get(fid, -1) < i
+            last[fid] = i
+        assert r_ma["dispatch"] == "miss-aware" and r_ma["prefetches"] == r_ma["miss_ms"]["n"] > 20
+        assert r_ma["hit_ms"]["p99"] < r_io["hit_ms"]["p99"], (r_ma["hit_ms"], r_io["hit_ms"])
+        resident = [f["fid"] for f in fleet if s.resident(f["fid"])]
+        assert resident
+        for fid in resident:
+            assert np.array_equal(s.readback_weights(fid), s.host_weights(fid)), fid
+            assert s.loaded(fid)

@@ -751,6 +751,45 @@ def test_deferred_acks_carry_tickets_and_can_be_cancelled():
         assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)   # the executor is free again
 
 
+def test_an_ack_that_could_not_be_delivered_withdraws_the_request_it_started():
+    """A front end takes the ack of a queued signal and then finds the peer gone (or the send fails).  The
+    request was started for nobody: tp_cancel_deferred on its ticket completes it at once -- an Execute
+    would otherwise hold the executor until the request timeout, a queued registration for good (no
+    timeout applies while a model is being uploaded) -- and forgets a half-made registration."""
+    with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20, request_timeout_ms=60000) as s:
+        fns = {fid: _register(s, fid) for fid in (1, 2)}
+        x = np.zeros((1, 3, 32, 32), np.float32)
+
+        def drive(fid):
+            packed, outbuf, _ = fns[fid].pack([x])
+            with pytest.raises(TorporError):
+                s.replay(fid, packed, outbuf)
+        used0 = s.pool_stats()["used"]
+        assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)
+        t_exec = s.signal_ticket(REQ_EXECUTE, 2)            # queued behind function 1
+        t_reg = s.signal_ticket(REQ_EXECUTE_AFTER_LOAD, 9, "1")   # a registration queued behind that
+        assert t_exec[2] and t_reg[2]
+        drive(1)
+        assert s.take_deferred_ack_ticket() == (ACK_OK, 0, t_exec[3])   # function 2 started, ack handed out ...
+        assert s.cancel_deferred(t_exec[3]) == 2                         # ... and could not be delivered
+        assert s.cancel_deferred(t_exec[3]) == 0
+        # the executor went on to the queued registration; its ack meets the same fate after an upload
+        assert s.take_deferred_ack_ticket() == (ACK_OK, 0, t_reg[3])
+        va = s.malloc(9, 4096)
+        s.h2d(9, va, np.ones(1024, np.float32))
+        assert s.cancel_deferred(t_reg[3]) == 2
+        with pytest.raises(TorporError) as e:
+            s.model_info(9)
+        assert e.value.code == -2                            # the half-made model is forgotten
+        assert s.pool_stats()["used"] == used0
+        assert s.signal_ticket(REQ_EXECUTE, 1)[:3] == (ACK_OK, 0, False)   # the executor is free again
+        drive(1)
+        # a ticket whose request has ended by itself is no longer known
+        t_late = s.signal_ticket(REQ_EXECUTE, 1)
+        assert not t_late[2]
+        assert s.cancel_deferred(t_exec[3]) == 0
+
+
 def test_function_ids_up_to_65535_register_and_run():
     with Server(host_only=True, mem_limit_bytes=330 << 20, pool_bytes=512 << 20) as s:
         fn = _register(s, 65535, seed=1)

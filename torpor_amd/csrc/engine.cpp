@@ -1796,20 +1796,36 @@ int Engine::take_deferred_ack(int* ack, int* resp, uint64_t* ticket) {
     if (ack) *ack = deferred_acks_.front().ack;
     if (resp) *resp = deferred_acks_.front().resp;
     if (ticket) *ticket = deferred_acks_.front().ticket;
+    // Remembered while the request it started is the active one: a front end that then fails to deliver the
+    // ack can still withdraw the request (cancel_deferred).
+    while (!taken_acks_.empty() && taken_acks_.front().id != active_) taken_acks_.pop_front();
+    if (deferred_acks_.front().ack == TP_ACK_OK && deferred_acks_.front().id == active_)
+        taken_acks_.push_back(deferred_acks_.front());
     deferred_acks_.pop_front();
     return 1;
 }
 
 // The peer that sent a queued signal is gone.  Still queued: the entry is dropped and no ack will
-// appear for it (1).  Already started but its ack not yet taken: the ack is dropped and the request,
-// which nobody will drive, is completed at once instead of holding the executor until the request
-// timeout (2).  Unknown or already delivered: 0.
+// appear for it (1).  Already started -- its ack not yet taken, or taken by a front end that could not
+// deliver it -- the ack is dropped and the request, which nobody will drive, is completed at once instead
+// of holding the executor until the request timeout (or, for a registration, for good) (2).  Unknown, or
+// the request it started is no longer the active one: 0.
 int Engine::cancel_deferred(uint64_t ticket) {
     std::lock_guard<std::mutex> lk(mu_);
     for (auto it = req_queue_.begin(); it != req_queue_.end(); ++it)
         if (it->ticket == ticket) {
             req_queue_.erase(it);
             return 1;
+        }
+    for (auto it = taken_acks_.begin(); it != taken_acks_.end(); ++it)
+        if (it->ticket == ticket) {
+            if (it->id != active_) {  // that request is over
+                taken_acks_.erase(it);
+                return 0;
+            }
+            deferred_acks_.push_front(*it);  // handled below like an ack that was never taken
+            taken_acks_.erase(it);
+            break;
         }
     for (auto it = deferred_acks_.begin(); it != deferred_acks_.end(); ++it)
         if (it->ticket == ticket) {

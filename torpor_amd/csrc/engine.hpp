@@ -368,6 +368,7 @@ private:
     std::chrono::steady_clock::time_point req_start_;
     std::deque<Queued> req_queue_;
     std::deque<DeferredAck> deferred_acks_;
+    std::deque<DeferredAck> taken_acks_;  // acks handed out for the request that is still active
     uint64_t ticket_seq_ = 0;  // queued signals are numbered from 1 in the order they were queued
     bool d2h_seen_ = false;
     // Data-plane calls are numbered; synced_seq_ is the number reached when the host last waited for

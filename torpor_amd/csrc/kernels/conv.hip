@@ -476,9 +476,10 @@ static inline bool aligned16c(const void* p) { return (reinterpret_cast<uintptr_
 // K order.  v_mfma_f32_32x32x2_f32 takes k = 0 from lanes 0-31 and k = 1 from lanes 32-63.  The 7 filter rows are
 // split 4 + 3 between the lane halves: step (c, j, kw) multiplies filter row kh = 4*half + j, so the two halves read
 // patch and filter 4 rows apart -- constants that fold into the lanes' base addresses -- and 3 * 4 * 7 = 84 steps
-// cover the 147 products.  Filter row 7 does not exist: in the 21 steps with j = 3 the upper half's filter operand
-// is replaced by zero (what it reads instead is the next channel's first row, or the 8 floats of padding behind
-// the last filter).
+// cover the 147 products.  Filter row 7 does not exist: in the 21 steps with j = 3 both operands of the upper half
+// are replaced by zero (what the filter side reads instead is the next channel's first row, or the 8 floats of
+// padding behind the last filter; the input side would read a row below the receptive field, whose Inf or NaN
+// times zero must not reach the sum).
 struct StemCfg {  // what store_tile needs to know: one 32x32 accumulator per wavefront, 2 x 2 wavefronts
     static constexpr int BM = 64, BN = 64, WGM = 2, WGN = 2, WGK = 1, THREADS = 256;
     static constexpr int WTM = 32, WTN = 32, TM = 1, TN = 1;
@@ -566,10 +567,13 @@ __global__ __launch_bounds__(256, 2) void conv_stem7_kernel(const ConvDev p) {
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int kw = 0; kw < 7; ++kw) {
+                float a = ap[(c * kStemRows + j) * kStemPitch + kw];
                 float b = bp[c * 49 + j * 7 + kw];
-                if (j == 3) b = h ? 0.f : b;  // filter row 7
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[(c * kStemRows + j) * kStemPitch + kw], b, acc[0][0],
-                                                                 0, 0, 0);
+                if (j == 3) {  // filter row 7: both operands, so that an Inf or NaN in the input row it would meet stays out
+                    a = h ? 0.f : a;
+                    b = h ? 0.f : b;
+                }
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[0][0], 0, 0, 0);
             }
     __syncthreads();  // the operands are no longer read: the filter area becomes the write-out staging blocks
 

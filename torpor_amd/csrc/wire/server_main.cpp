@@ -579,22 +579,6 @@ int main() {
             }
         }
         (void)tp_poll(S.eng);  // request timeout (cuda_server.hpp:257-264)
-        int32_t ack = 0, resp = 0;
-        uint64_t ticket = 0;
-        while (tp_take_deferred_ack_ticket(S.eng, &ack, &resp, &ticket) == 1) {
-            pb::Writer w;
-            w.i32(1, ack);
-            w.i32(2, resp);
-            uint64_t tag = 0;
-            for (size_t k = 0; k < S.waiting_ack.size(); ++k)
-                if (S.waiting_ack[k].ticket == ticket) {
-                    tag = S.waiting_ack[k].conn_tag;
-                    S.waiting_ack.erase(S.waiting_ack.begin() + (long)k);
-                    break;
-                }
-            for (auto& rc2 : S.rep_conns)
-                if (tag && rc2->tag == tag) rc2->send({std::string(), w.out});
-        }
         auto prune = [&](std::vector<std::unique_ptr<zmtp::Conn>>& v) {
             for (size_t i = 0; i < v.size();) {
                 if (v[i]->failed() && v[i]->inbox().empty()) {
@@ -614,6 +598,29 @@ int main() {
                 }
             }
         };
+        // Failed connections go first, their tickets with them: an ack is only taken for a peer that is
+        // still there.  Should the peer vanish between this check and the send, or the send fail, the
+        // request the ack belongs to has been started for nobody: it is withdrawn (tp_cancel_deferred
+        // also takes back an ack that has been handed out, while its request is the active one).
+        prune(S.rep_conns);
+        int32_t ack = 0, resp = 0;
+        uint64_t ticket = 0;
+        while (tp_take_deferred_ack_ticket(S.eng, &ack, &resp, &ticket) == 1) {
+            pb::Writer w;
+            w.i32(1, ack);
+            w.i32(2, resp);
+            uint64_t tag = 0;
+            for (size_t k = 0; k < S.waiting_ack.size(); ++k)
+                if (S.waiting_ack[k].ticket == ticket) {
+                    tag = S.waiting_ack[k].conn_tag;
+                    S.waiting_ack.erase(S.waiting_ack.begin() + (long)k);
+                    break;
+                }
+            bool delivered = false;
+            for (auto& rc2 : S.rep_conns)
+                if (tag && rc2->tag == tag && !rc2->failed()) delivered = rc2->send({std::string(), w.out});
+            if (!delivered) (void)tp_cancel_deferred(S.eng, ticket);
+        }
         prune(S.rep_conns);
         prune(S.pull_conns);
     }

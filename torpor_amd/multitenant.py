@@ -72,8 +72,10 @@ def pct(xs, q):
 
 
 def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after_request=None, note_every_s=30.0,
-          lookahead=0):
-    """Serves the trace in arrival order on the single executor.  open_loop: a request is not issued before
+          lookahead=0, dispatch="in-order"):
+    """dispatch="miss-aware": the open-loop trace through torpor_amd.dispatch.MissAwareDispatcher (requests of
+    resident models are served while the swap-in of the oldest swapped-out one streams; see serve_miss_aware).
+    Otherwise: serves the trace in arrival order on the single executor.  open_loop: a request is not issued before
     its arrival time and latency = completion - arrival (queueing included); otherwise requests run back to
     back and latency is the service time.  Every `check_every`-th answer is compared bit for bit with the
     function's registration run.  after_request(i, fid, hit) is called after each request.
@@ -85,11 +87,25 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
     import gc
 
     from .server import REQ_LOAD
+    if dispatch == "miss-aware":
+        if not open_loop:
+            raise ValueError("miss-aware dispatch reorders a queue of arrived requests: open loop only")
+        return serve_miss_aware(server, fleet, arrivals, picks, check_every, after_request, note_every_s)
     n_req = len(picks)
     gc.collect()
     gc.disable()   # a collection of the interpreter inside a request (tens of milliseconds) is not the path's
+    try:
+        return _serve_in_order(server, fleet, arrivals, picks, open_loop, check_every, after_request, note_every_s,
+                               lookahead, REQ_LOAD, n_req)
+    finally:
+        gc.enable()
+
+
+def _serve_in_order(server, fleet, arrivals, picks, open_loop, check_every, after_request, note_every_s, lookahead,
+                    REQ_LOAD, n_req):
     st0 = server.pool_stats()
-    lat_hit, lat_miss, by_arch, swap_bytes, swap_ms = [], [], {}, 0, 0.0
+    lat_hit, lat_miss, by_arch = [], [], {}
+    swaps = _SwapMeter(server)
     prefetches = 0
     t0 = time.perf_counter()
     next_note = note_every_s
@@ -121,9 +137,8 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
         (lat_hit if hit else lat_miss).append(lat)
         by_arch.setdefault((f["arch"], hit), []).append(lat)
         if not hit:
-            s = server.swap_stats(fid)
-            swap_bytes += s["bytes"]
-            swap_ms += s["copy_ms"]
+            swaps.started(fid)
+        swaps.collect()
         if check_every and i % check_every == 0:
             out = f["fn"].postprocess(f["views"])
             for a, b in zip(f["first"], out):
@@ -132,14 +147,40 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
         if after_request is not None:
             after_request(i, fid, hit)
     wall = time.perf_counter() - t0
-    gc.enable()
+    swaps.collect(wait=True)
     st1 = server.pool_stats()
+    return _summary(server, n_req, wall, st0, st1, lat_hit, lat_miss, by_arch, swaps.bytes, swaps.ms,
+                    dispatch="in-order", lookahead=lookahead, prefetches=int(prefetches))
+
+
+class _SwapMeter:
+    """Bytes and copy time of the swap-ins of a run.  A swap-in's figures are read once it has landed completely
+    (tp_get_swap_stats waits for the last transfer group otherwise, and tables that a request does not wait for
+    land up to 2 ms after the request has answered): asking right after the request would hold up the next one."""
+
+    def __init__(self, server):
+        self.server, self.pending, self.bytes, self.ms = server, set(), 0, 0.0
+
+    def started(self, fid):
+        self.pending.add(fid)
+
+    def collect(self, wait=False):
+        for fid in list(self.pending):
+            if wait or self.server.loaded(fid) or not self.server.resident(fid):
+                if self.server.resident(fid):
+                    st = self.server.swap_stats(fid)
+                    self.bytes += st["bytes"]
+                    self.ms += st["copy_ms"]
+                self.pending.discard(fid)
+
+
+def _summary(server, n_req, wall, st0, st1, lat_hit, lat_miss, by_arch, swap_bytes, swap_ms, **extra):
     all_lat = lat_hit + lat_miss
     return dict(
-        requests=n_req, wall_s=wall, achieved_rps=n_req / wall,
+        requests=n_req, wall_s=wall, achieved_rps=n_req / wall, **extra,
         hit_ratio=len(lat_hit) / max(n_req, 1), evictions=st1["evictions"] - st0["evictions"],
         fragmentation_evictions=st1["fragmentation_evictions"] - st0["fragmentation_evictions"],
-        swap_ins=st1["swap_ins"] - st0["swap_ins"], lookahead=lookahead, prefetches=int(prefetches),
+        swap_ins=st1["swap_ins"] - st0["swap_ins"],
         latency_ms=dict(p50=pct(all_lat, 0.5), p99=pct(all_lat, 0.99), mean=float(np.mean(all_lat)) if all_lat else None),
         hit_ms=dict(p50=pct(lat_hit, 0.5), p99=pct(lat_hit, 0.99), n=len(lat_hit)),
         miss_ms=dict(p50=pct(lat_miss, 0.5), p99=pct(lat_miss, 0.99), n=len(lat_miss)),
@@ -152,7 +193,89 @@ def serve(server, fleet, arrivals, picks, open_loop=True, check_every=500, after
     )
 
 
-def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2.0, lookahead=0, **server_kw):
+def serve_miss_aware(server, fleet, arrivals, picks, check_every=500, after_request=None, note_every_s=30.0,
+                     margin_s=0.0003):
+    """The open-loop trace on the single executor, the queue of arrived requests ordered by
+    torpor_amd.dispatch.MissAwareDispatcher: the oldest request of a swapped-out model gets its swap-in started
+    with a Load signal (include/server/controller.hpp:208-215), requests of resident models run while it streams,
+    and the waiting request is started when the rest of its copy is as long as its forward pass (both figures
+    are the engine's: tp_get_load_estimate).  One function is active at a time, as in the reference.  A request
+    counts as a miss when the swap-in was started for it; latency = completion - arrival."""
+    import gc
+
+    from .dispatch import MissAwareDispatcher
+    from .server import REQ_LOAD
+    n_req = len(picks)
+    d = MissAwareDispatcher(margin_s=margin_s)
+    est = {}
+    st0 = server.pool_stats()
+    lat_hit, lat_miss, by_arch = [], [], {}
+    swaps = _SwapMeter(server)
+    nxt = served = 0
+    next_note = note_every_s
+    resident = server.resident
+    gc.collect()
+    gc.disable()   # a collection of the interpreter inside a request (tens of milliseconds) is not the path's
+    t0 = time.perf_counter()
+    try:
+        while served < n_req:
+            now = time.perf_counter() - t0
+            if now >= next_note:
+                print(f"[{now:6.0f} s] {served} of {n_req} requests served", file=sys.stderr, flush=True)
+                next_note += note_every_s
+            while nxt < n_req and arrivals[nxt] <= now:
+                d.arrive(nxt, fleet[picks[nxt]]["fid"], arrivals[nxt])
+                nxt += 1
+            kind, what = d.decide(now, resident)
+            if kind == "load":
+                fid = what.fid
+                if fid not in est:
+                    a, b = server.load_estimate(fid)
+                    est[fid] = (a * 1e-3, b * 1e-3)
+                if server.signal(REQ_LOAD, fid, "")[0] == 0:
+                    d.load_started(fid, time.perf_counter() - t0, *est[fid])
+                else:       # refused (nothing evictable): the request will bring its model in itself
+                    d.load_started(fid, now, 0.0, 0.0)
+                continue
+            if kind == "idle":
+                wake = arrivals[nxt] if nxt < n_req else None
+                if what is not None and (wake is None or what < wake):
+                    wake = what
+                while time.perf_counter() - t0 < wake:
+                    pass
+                continue
+            f = fleet[picks[what.seq]]
+            fid = f["fid"]
+            ack, _, dfr = server.signal(1, fid, "")
+            assert ack == 0 and not dfr
+            server.replay(fid, f["packed"], f["outbuf"])
+            done = time.perf_counter() - t0
+            lat = (done - what.arrival) * 1e3
+            hit = not what.miss
+            (lat_hit if hit else lat_miss).append(lat)
+            by_arch.setdefault((f["arch"], hit), []).append(lat)
+            if not hit:
+                swaps.started(fid)
+            swaps.collect()
+            if check_every and what.seq % check_every == 0:
+                out = f["fn"].postprocess(f["views"])
+                for a, b in zip(f["first"], out):
+                    if not np.array_equal(a, b):
+                        raise AssertionError(f"function {fid}: answer changed after swapping")
+            if after_request is not None:
+                after_request(what.seq, fid, hit)
+            served += 1
+    finally:
+        gc.enable()
+    wall = time.perf_counter() - t0
+    swaps.collect(wait=True)
+    st1 = server.pool_stats()
+    return _summary(server, n_req, wall, st0, st1, lat_hit, lat_miss, by_arch, swaps.bytes, swaps.ms,
+                    dispatch="miss-aware", lookahead=0, prefetches=d.loads)
+
+
+def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2.0, lookahead=0, dispatch="in-order",
+            **server_kw):
     """One engine with an LRU budget of `cap_gib`, the fleet registered, the open-loop trace served."""
     from torpor_amd.server import Server
 
@@ -165,7 +288,7 @@ def run_cap(cap_gib, seconds, rate, models=FLEET_64, seed=0, pool_headroom_gib=2
         charged = sum(server.model_info(f["fid"])["total_bytes"] for f in fleet)
         weights = sum(server.model_info(f["fid"])["image_bytes"] for f in fleet)
         arrivals, picks = make_trace(len(fleet), int(seconds * rate), rate, seed)
-        r = serve(server, fleet, arrivals, picks, lookahead=lookahead)
+        r = serve(server, fleet, arrivals, picks, lookahead=lookahead, dispatch=dispatch)
         r.update(cap_gib=cap_gib, cap_binds=charged >= limit, registration_s=reg_s, offered_rps=rate,
                  charged_total_gib=charged / 2 ** 30, weights_total_gb=weights / 1e9, link_peak_gbps=link)
         del fleet
