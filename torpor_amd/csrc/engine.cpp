@@ -572,11 +572,12 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
         if (r) return r;
     }
     std::memcpy(h2d_stage_ + h2d_pos_, src, bytes);
-    // During a swap-in the copy engines belong to the weight stream: a request input handed to them
-    // queues among its transfer groups and disturbs how they alternate over the engines.  A copy
+    // During a swap-in -- this model's or, when requests of resident models are served while another
+    // model streams in, anybody's -- the copy engines belong to the weight stream: a request input handed
+    // to them queues among its transfer groups and disturbs how they alternate over the engines.  A copy
     // kernel reads the pinned buffer instead (alignment of the destination permitting).
     void* stage_dev = nullptr;
-    const bool by_kernel = (d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+    const bool by_kernel = (d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
                            hipHostGetDevicePointer(&stage_dev, h2d_stage_, 0) == hipSuccess && stage_dev;
     if (by_kernel) {
         int kr = tpk::launch_copy(static_cast<uint8_t*>(stage_dev) + h2d_pos_, x.p, bytes, compute_);
@@ -618,7 +619,7 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
             const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
             if (d >= ub->first && d - ub->first + bytes <= ub->second) {
                 void* dst_dev = nullptr;
-                if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+                if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
                     hipHostGetDevicePointer(&dst_dev, dst, 0) == hipSuccess && dst_dev) {
                     int kr = tpk::launch_copy(p, dst_dev, bytes, compute_);
                     if (kr) return kr;
@@ -644,7 +645,7 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
         // device-to-host copy handed to them would wait for all of those; a copy kernel writing
         // into the pinned buffer goes the other way over the link without queueing behind them.
         void* stage_dev = nullptr;
-        if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && !m.fully_loaded)) &&
+        if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
             hipHostGetDevicePointer(&stage_dev, d2h_stage_, 0) == hipSuccess && stage_dev) {
             int kr = tpk::launch_copy(p, static_cast<uint8_t*>(stage_dev) + d2h_pos_, bytes, compute_);
             if (kr) return kr;
@@ -1540,15 +1541,50 @@ void Engine::log_transfer(Model& m) {
                m.id, (unsigned long long)m.stats.bytes, m.stats.chunks, m.ncopy, ms * 1e3);
 }
 
+// Waits until nothing of this model's swap-in is on its way any more: a hand-over still running is
+// cancelled, and the groups that were handed to the streams are waited for by their own events.  Copies
+// of other models are left alone: an eviction during another model's swap-in (a Load signal while requests
+// run, a request that finds the budget full) must not stall the executor for the rest of that swap-in.
 void Engine::wait_copy_idle(Model& m) {
     if (host_only()) return;
-    if (m.copy_state.load(std::memory_order_acquire) == CS_RUNNING) {
+    const int st0 = m.copy_state.load(std::memory_order_acquire);
+    if (st0 == CS_IDLE) {  // resident since registration: no copy of it was ever queued
+        if (last_swap_ == &m) last_swap_ = nullptr;
+        return;
+    }
+    if (st0 == CS_RUNNING) {
         m.cancel.store(true);
         while (m.copy_state.load(std::memory_order_acquire) == CS_RUNNING) std::this_thread::yield();
     }
-    (void)hipStreamSynchronize(copy_);
-    (void)hipStreamSynchronize(copy2_);
-    (void)hipStreamSynchronize(decode_);
+    const uint32_t n = m.issued.load(std::memory_order_acquire);
+    bool ok = true;
+    // transfer groups publish in order on the expansion stream (packed) or alternate over the copy streams
+    for (uint32_t back = 1; back <= 2 && back <= n && ok; ++back)
+        if (n - back < m.chunk_ev.size()) ok = hipEventSynchronize(m.chunk_ev[n - back]) == hipSuccess;
+    // a packed group's DMA precedes its expansion; one that was handed over but not yet expanded cannot exist
+    // (the copy thread hands over DMA and expansion of a group together), and a cancelled hand-over stops
+    // between groups.  Anything unexpected: fall back to draining the streams.
+    if (!ok || m.copy_error.load()) {
+        (void)hipGetLastError();
+        (void)hipStreamSynchronize(copy_);
+        (void)hipStreamSynchronize(copy2_);
+        (void)hipStreamSynchronize(decode_);
+    }
+    if (last_swap_ == &m) last_swap_ = nullptr;
+}
+
+// Is a swap-in (of any model) still using the copy engines?  Asked without waiting.  Swap-ins are handed to
+// the streams one after the other, so the one started last finishes last.
+bool Engine::swap_in_flight() {
+    Model* m = last_swap_;
+    if (!m || host_only()) return false;
+    const int st = m->copy_state.load(std::memory_order_acquire);
+    if (st == CS_RUNNING) return true;
+    if (st == CS_ISSUED && !m->cancel.load() && !m->copy_error.load() && m->t1 && hipEventQuery(m->t1) == hipErrorNotReady)
+        return true;
+    (void)hipGetLastError();
+    last_swap_ = nullptr;
+    return false;
 }
 
 // memory_manager.hpp:213-227 sig_trans_thread + 451-507 check_and_malloc_model
@@ -1606,6 +1642,7 @@ int Engine::swap_in(Model& m) {
     }
     m.timing_valid = true;
     m.copy_state.store(CS_RUNNING, std::memory_order_release);
+    last_swap_ = &m;
     {
         std::lock_guard<std::mutex> lk(cmu_);
         jobs_.push_back(&m);

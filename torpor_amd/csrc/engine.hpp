@@ -305,6 +305,7 @@ private:
     void drop_graph(Model& m);
     int build_graph(Model& m);
     void wait_copy_idle(Model& m);
+    bool swap_in_flight();
     void log_transfer(Model& m);
     void copy_main();
     int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
@@ -404,6 +405,7 @@ private:
     std::mutex cmu_;
     std::condition_variable ccv_;
     std::deque<Model*> jobs_;
+    Model* last_swap_ = nullptr;  // the model whose swap-in was started last, until it is seen to have landed
     bool stop_ = false;
 };
 
