@@ -353,7 +353,8 @@ int tp_model_resident(tp_server* s, int32_t client); /* 1/0, negative on error *
 int tp_model_loaded(tp_server* s, int32_t client);
 /* What a scheduler above the boundary needs in order to place a request of a swapped-out function: how long the
  * swap-in occupies the host link before the request can complete (bytes the request waits for / the link rate the
- * engine measured), and the forward pass on its own (timed at registration, the best warm request since).  The
+ * engine measured), and the forward pass as it runs beside that swap-in (timed at registration, the best warm
+ * request since, plus what active copy queues cost each launch).  The
  * reference's router and simulator work from per-model constants instead (scripts/router.py:17,
  * misc/tools/node_simu.py:99-117). */
 int tp_get_load_estimate(tp_server* s, int32_t client, double* swap_ms, double* forward_ms);

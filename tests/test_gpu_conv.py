@@ -19,10 +19,15 @@ CASES = [
     # N, H, W, Cin, Cout, k, stride, pad, x_layout, y_layout, expected kernel
     (1, 56, 56, 64, 64, 1, 1, 0, NHWC, NHWC, "gemm_fast"),        # 1x1
     (2, 28, 28, 256, 512, 1, 2, 0, NHWC, NHWC, "gemm_fast"),      # 1x1 stride 2 (downsample)
-    (1, 56, 56, 64, 64, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # 3x3
+    (1, 56, 56, 64, 64, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),     # 3x3 stride 1: Winograd
+    (1, 28, 28, 128, 128, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),   # the same kind of layer at batch 1: below the Winograd path's size bound
+    (1, 20, 20, 24, 40, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # 3x3 stride 1 whose channel counts the Winograd path does not take
     (2, 28, 28, 128, 128, 3, 2, 1, NHWC, NHWC, "conv3x3_fast"),   # 3x3 stride 2
-    (1, 7, 7, 512, 512, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),     # tiny map, split-K
-    (8, 28, 28, 128, 128, 3, 1, 1, NHWC, NHWC, "conv3x3_fast"),   # batch 8
+    (1, 7, 7, 512, 512, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),     # tiny odd map (edge tiles), split over channels
+    (8, 28, 28, 128, 128, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),   # batch 8
+    (8, 14, 14, 256, 256, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),   # the dominant ResNet-152 batch 8 layer: 392 tiles, ragged last block
+    (3, 15, 13, 16, 32, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),     # odd height and width, one K-block, one channel block
+    (2, 9, 10, 48, 96, 3, 1, 1, NHWC, NHWC, "conv3x3_wino"),      # three K-blocks, three channel blocks
     (1, 64, 64, 3, 64, 7, 2, 3, NCHW, NHWC, "conv_stem7x7"),      # stem: NCHW in, NHWC out
     (1, 64, 64, 3, 48, 7, 2, 3, NCHW, NHWC, "conv_generic"),      # a stem whose channel count the stem kernel does not take
     (1, 13, 11, 5, 7, 3, 1, 1, NCHW, NCHW, "conv_generic"),       # odd sizes, NCHW both
@@ -33,7 +38,9 @@ CASES = [
 
 
 @pytest.mark.parametrize("N,H,W,Cin,Cout,k,stride,pad,xl,yl,kern", CASES)
-def test_conv(gpu_server, N, H, W, Cin, Cout, k, stride, pad, xl, yl, kern):
+def test_conv(gpu_server, monkeypatch, N, H, W, Cin, Cout, k, stride, pad, xl, yl, kern):
+    if kern.startswith("conv3x3_wino"):
+        monkeypatch.setenv("TORPOR_WINO_MIN_GFLOP", "0")      # the Winograd path also for layers below its size bound
     rng = np.random.default_rng(N + H * 3 + Cin * 5 + Cout * 7 + k)
     x_nchw = _rand(rng, N, Cin, H, W)
     w = _rand(rng, Cout, Cin, k, k) * np.float32(1.0 / np.sqrt(Cin * k * k))
@@ -47,6 +54,67 @@ def test_conv(gpu_server, N, H, W, Cin, Cout, k, stride, pad, xl, yl, kern):
         got = t.read(yv, (N, Ho, Wo, Cout) if yl == NHWC else (N, Cout, Ho, Wo))
     want = ref.conv2d(x, w, (stride, stride), (pad, pad), x_nhwc=(xl == NHWC), y_nhwc=(yl == NHWC))
     assert_close(got, want, RTOL, f"conv {k}x{k} s{stride}")
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 8])
+def test_winograd_split_over_channels_and_direct_kernel_agree(gpu_server, monkeypatch, splits):
+    """Winograd F(2x2, 3x3) with its input channels split 1 / 2 / 3 / 8 ways (summed inside the launch, in slot
+    order) against the oracle and against the direct kernel on the same operands; pitched input and output
+    (a channel slice of wider tensors, as the DenseNets use them) and the fused batch-norm + residual + ReLU."""
+    rng = np.random.default_rng(40 + splits)
+    N, H, W, Cin, Cout, XP, YP = 2, 14, 14, 128, 64, 160, 96
+    xw = _rand(rng, N, H, W, XP)
+    w = _rand(rng, Cout, Cin, 3, 3) * np.float32(1.0 / np.sqrt(Cin * 9))
+    g, b, mu = _rand(rng, Cout), _rand(rng, Cout), _rand(rng, Cout)
+    var = rng.uniform(0.5, 2.0, Cout).astype(np.float32)
+    res = _rand(rng, N, H, W, Cout)                        # the residual is a dense tensor of its own
+    x = np.ascontiguousarray(xw[..., :Cin])
+    outs = {}
+    for path in ("wino", "direct"):
+        monkeypatch.setenv("TORPOR_WINOGRAD", "1" if path == "wino" else "0")
+        monkeypatch.setenv("TORPOR_WINO_SPLITS", str(splits))
+        monkeypatch.setenv("TORPOR_WINO_MIN_GFLOP", "0")
+        with OpSession(gpu_server, [w, g, b, mu, var]) as t:
+            xv, rv = t.act(xw), t.act(res)
+            yv = t.act(np.full((N, H, W, YP), 7.0, np.float32))
+            t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, 3, 3, stride=1, pad=1, x_pitch=XP, y_pitch=YP,
+                     bn=tuple(t.w[1:5]), bn_eps=1e-5, residual=rv, act=ACT_RELU)
+            assert t.s.last_kernel().startswith("conv3x3_wino" if path == "wino" else "conv3x3_fast"), t.s.last_kernel()
+            outs[path] = t.read(yv, (N, H, W, YP))
+    z = ref.conv2d(x, w, (1, 1), (1, 1), x_nhwc=True, y_nhwc=True)
+    z = ref.bn(z, g, b, mu, var, 1e-5, Cout, nhwc=True).astype(np.float64) + res
+    for path, got in outs.items():
+        assert_close(got[..., :Cout], np.maximum(z, 0), 5e-5, f"{path} conv+bn+res+relu, pitched")
+        assert np.all(got[..., Cout:] == 7.0), f"{path}: wrote outside its channel slice"
+    assert_close(outs["wino"][..., :Cout], outs["direct"][..., :Cout], 5e-5, "Winograd against the direct kernel")
+
+
+def test_winograd_is_deterministic_and_keeps_non_finite_values_local(gpu_server, monkeypatch):
+    """Two runs give the same bits (the split is summed in slot order), and an infinity in the input reaches
+    exactly the outputs whose 3x3 window holds it."""
+    monkeypatch.setenv("TORPOR_WINO_MIN_GFLOP", "0")
+    rng = np.random.default_rng(9)
+    N, H, W, C = 1, 12, 12, 32
+    x = _rand(rng, N, H, W, C)
+    x[0, 5, 6, :] = np.inf
+    w = np.abs(_rand(rng, C, C, 3, 3)) + np.float32(0.1)       # positive filters: the window's sum is +inf, never inf - inf
+    with OpSession(gpu_server, [w]) as t:
+        xv = t.act(x)
+        yv = t.empty(x.nbytes)
+        runs = []
+        for _ in range(2):
+            t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, C, C, 3, 3, stride=1, pad=1)
+            assert t.s.last_kernel().startswith("conv3x3_wino")
+            runs.append(t.read(yv, (N, H, W, C)))
+    assert np.array_equal(runs[0], runs[1], equal_nan=True)
+    touched = np.zeros((H, W), bool)
+    touched[4:7, 5:8] = True
+    assert np.all(np.isfinite(runs[0][0][~touched])), "an infinity left the windows that hold it"
+    assert not np.any(np.isfinite(runs[0][0][touched]))
+    xf = x.copy()
+    xf[0, 5, 6, :] = 0.0
+    z = ref.conv2d(xf, w, (1, 1), (1, 1), x_nhwc=True, y_nhwc=True)
+    assert_close(runs[0][0][~touched], z[0][~touched], RTOL, "outputs away from the infinite pixel")
 
 
 @pytest.mark.parametrize("k,Cin,Cout,HW", [(1, 64, 256, 14), (3, 64, 64, 14), (7, 3, 16, 20)])
@@ -325,7 +393,7 @@ with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
 print("ok")
 '''
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, TORPOR_CONV3_CFG=str(cfg), PYTHONPATH=root)
+    env = dict(os.environ, TORPOR_CONV3_CFG=str(cfg), TORPOR_WINOGRAD="0", PYTHONPATH=root)   # the direct kernels are meant
     r = subprocess.run([sys.executable, "-c", code, name], env=env, cwd=root, capture_output=True, text=True,
                        timeout=120)
     assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr

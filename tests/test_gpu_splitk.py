@@ -65,7 +65,10 @@ def _in_subprocess(mode, path):
     return np.load(path)
 
 
-def test_in_launch_summation_equals_the_two_launch_form_bit_for_bit():
+def test_in_launch_summation_equals_the_two_launch_form_bit_for_bit(monkeypatch):
+    # the direct kernels are meant: the Winograd path (which the 1.85 GFLOP convolution would take) has no
+    # two-launch form to compare with (the subprocesses inherit the setting)
+    monkeypatch.setenv("TORPOR_WINOGRAD", "0")
     got = _run_cases()   # the library's own choice: in-launch up to 8 slots, a reduction launch above
     # the first GEMM and the first convolution of each round against float64 (the values are right at all)
     for rnd in range(ROUNDS):

@@ -2703,7 +2703,16 @@ int Engine::load_estimate(int client, double* swap_ms, double* forward_ms) {
         bytes = m->timg ? xfer_off(*m, from) : from;
     }
     if (swap_ms) *swap_ms = (double)bytes / stream_rate_bytes_per_us(m->ncopy, m->chunk_max ? m->chunk_max : (16ull << 20)) / 1000.0;
-    if (forward_ms) *forward_ms = m->warm_us / 1000.0;
+    if (forward_ms) {
+        // the forward pass as it runs beside its own swap-in: every launch starts later while copy queues are
+        // active, and two copy streams slow the kernels themselves (the figures of choose_copy_plan)
+        double kernels = 0;
+        for (const Op& op : m->program)
+            if (op.kind == OPK_GEMM || op.kind == OPK_CONV) kernels += 1.5;
+            else if (op.kind == OPK_BN || op.kind == OPK_LAUNCH) kernels += 1.0;
+        const double us = m->ncopy == 2 ? m->warm_us * 1.15 + kernels * 2.4 : m->warm_us + kernels * 1.2;
+        *forward_ms = us / 1000.0;
+    }
     return 0;
 }
 

@@ -23,6 +23,7 @@ int launch_splitk_reduce(const float* ws, int splits, long M, long N, float* C, 
 int choose_splits(long tiles, long K, int bk, long tile_floats, size_t ws_bytes, long* kper_out, int max_splits = 32, bool pairs = true,
                   int balance = -1);
 unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
+int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t s);  // winograd.hip
 
 struct ConvDev {
     const float* x;
@@ -742,6 +743,15 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
                                           "conv_taps_3x1_64x64"};
         set_last_kernel(nm[other_taps]);
     } else if (fast3) {
+        // Stride 1: Winograd F(2x2, 3x3), 2.25 times fewer multiplications (winograd.hip).  TORPOR_WINOGRAD=0: the
+        // direct kernels below for every 3x3.
+        // (read per call, so that one process can compare the two paths)
+        const char* wino_env = getenv("TORPOR_WINOGRAD");
+        const bool wino_on = wino_env == nullptr || atoi(wino_env) != 0;
+        if (wino_on && a.sh == 1 && a.sw == 1 && a.ph == 1 && a.pw == 1) {
+            const int r = launch_conv3x3_winograd(a, ws, s);
+            if (r != K_EUNSUPPORTED) return r;
+        }
         const long tl = ((M + 127) / 128) * ((a.Cout + 127) / 128);
         const long t64 = ((M + 63) / 64) * ((a.Cout + 63) / 64);
         static const int forced = getenv("TORPOR_CONV3_CFG") ? atoi(getenv("TORPOR_CONV3_CFG")) : -1;

@@ -1,0 +1,435 @@
+// 3x3 stride-1 convolution as Winograd F(2x2, 3x3) on fp32 MFMA for gfx950.
+//
+// One of the paths behind the cudnnConvolutionForward call site of the reference executor
+// (include/server/cuda_server.hpp:708-735; its traces show cuDNN picking Winograd kernels for these
+// layers too, misc/tools/resnet_all.txt:34-48).  The output is cut into 2x2 tiles; with
+//   U = G g G^T   (the 3x3 filter of one (cout, cin) pair -> 4x4)
+//   V = B^T d B   (the 4x4 input patch of one (tile, cin) pair -> 4x4)
+// the tile's outputs are Y = A^T [ sum_cin U .* V ] A: sixteen independent products
+// M[xi] = V[xi] (tiles x cin) . U[xi]^T (cin x cout), xi = 4i + j, with 2.25 times fewer multiplications
+// than the direct form.  Nothing is precomputed or stored: the filter bytes stay as they were uploaded
+// (they are swapped in and out byte for byte) and U is formed on the fly -- a few dozen additions per
+// filter, repeated by every workgroup that needs it, against thousands of matrix-core cycles.
+//
+// A workgroup owns 32 tiles x 32 output channels x all sixteen xi for a slice of the input channels, in
+// K-blocks of 16 input channels.  Patches are fetched by thread = tile x channel quad (sixteen 128-bit loads)
+// and filters by thread = output channel x channel quad (36 contiguous floats), transformed in registers and
+// written as [xi][row][16 channels] operand blocks into LDS, XOR-swizzled in 16-byte chunks so that the
+// 128-bit fragment reads of the MFMA loop are conflict-free without padding.  The fragment layout and K
+// permutation are those of mma_block (mfma_tile.hpp).  How the work is spread over the wavefronts is
+// described at the kernel.
+//
+// After the K loop each multiplying wavefront folds its row over j (T[i][b] = sum_j M[i][j] A^T[b][j]), the
+// four rows are exchanged through LDS, and wavefront (a, b) ends up with output pixel (a, b) of every tile as
+// one 32x32 block (tiles x channels) in the usual accumulator layout.  A split over input channels is summed
+// inside the launch by finish_split, in slot order.
+#include "kernels.hpp"
+#include "mfma_tile.hpp"
+
+#include <cstdlib>
+
+namespace tpk {
+
+void set_last_kernel(const char* n);
+int num_cu();
+Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
+unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
+
+namespace {
+
+constexpr int kKC = 16;                        // input channels per K-block
+constexpr int kOperandFloats = 16 * 32 * kKC;  // V (or U) of one K-block: [xi][row][channel]
+
+struct WinoDev {
+    const float* x;
+    const float* w;
+    float* y;
+    int H, W, Cin, Cout;   // stride 1, padding 1: the output is H x W as well
+    long xp, yp;           // floats between pixels of x / y
+    int tiles_h, tiles_w;  // 2x2 output tiles per image
+    long ntiles;           // N * tiles_h * tiles_w
+    int mt, nt;            // blocks of 32 tiles / 32 output channels
+    int splits, cper;      // input-channel slices and channels per slice (a multiple of kKC)
+    float* ws;
+    unsigned* tickets;
+    const float* zeros;
+    Epilogue ep;
+};
+
+// what finish_split needs to know: four wavefronts with one 32x32 accumulator block each
+struct WinoOutCfg {
+    static constexpr int TM = 1, TN = 1, WGM = 2, WGN = 2;
+};
+
+__device__ __forceinline__ void fetch_args(const WinoDev& p) {
+    fetch_now(p.x);
+    fetch_now(p.w);
+    fetch_now(p.y);
+    fetch_now(p.H);
+    fetch_now(p.W);
+    fetch_now(p.Cin);
+    fetch_now(p.xp);
+    fetch_now(p.yp);
+    fetch_now(p.tiles_h);
+    fetch_now(p.tiles_w);
+    fetch_now(p.ntiles);
+    fetch_now(p.mt);
+    fetch_now(p.nt);
+    fetch_now(p.splits);
+    fetch_now(p.cper);
+    fetch_now(p.ws);
+    fetch_now(p.tickets);
+    fetch_now(p.zeros);
+    fetch_now(p.ep);
+}
+
+__device__ __forceinline__ int remap_xcd_w(int bid, int n) {
+    const int q = n >> 3, rem = n & 7;
+    const int xcd = bid & 7, local = bid >> 3;
+    return xcd * q + (xcd < rem ? xcd : rem) + local;
+}
+
+// Float offset of 16-byte chunk `chunk` (0..3) inside row `row` (16 floats = 64 bytes = half of the LDS's 32
+// banks) of an operand block.  A 128-bit access is served eight lanes at a time: eight consecutive rows are four
+// even ones on banks 0-15 and four odd ones on banks 16-31, and rows two apart get different chunks.
+__device__ __forceinline__ int swz(int row, int chunk) { return (chunk ^ ((row >> 1) & 3)) << 2; }
+
+// Four wavefronts.  All of them multiply: wavefront w owns the four accumulators of row i = w of the 4x4
+// (xi = 4w .. 4w+3).  Before that, per K-block, wavefronts 0-1 fetch and transform the patches and 2-3 the
+// filters; the loads of the next K-block are in flight meanwhile.  Two workgroups share a CU (64 KiB of LDS
+// each).  Measured on MI355X, 8x14x14x256 -> 256: per K-block a wavefront spends about 2000 cycles on the
+// transform's vector instructions and 2050 on its 32 MFMAs, and the two do not overlap on a SIMD -- not
+// within a wavefront, not between two workgroups on the CU, and not when the transforms are given to
+// wavefronts of their own (built and measured: same time), because a SIMD issues either kind from one
+// port.  That is what bounds this path at about 1.15x the direct kernel instead of the 2.25x of the
+// multiplication count.
+__global__ __launch_bounds__(256, 2) void conv_wino_kernel(const WinoDev p) {
+    fetch_args(p);
+    __shared__ __attribute__((aligned(16))) float lds[2 * kOperandFloats];  // [V | U] of one K-block
+    __shared__ int rowpix[32];  // (n*H + 2*th)*W + 2*tw of each tile of this block, -1 past the last tile
+    __shared__ int rowok[32];   // bit 0: the tile's second output row exists, bit 1: its second column
+    __shared__ unsigned flag;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wavefront: role branches are scalar
+    const int r = lane & 31, h = lane >> 5;
+    const int t = remap_xcd_w((int)blockIdx.x, p.mt * p.nt);
+    const int tm = t / p.nt, tn = t - tm * p.nt;
+    const int split = (int)blockIdx.z;
+    const int cbeg = split * p.cper;
+    const int cend = cbeg + p.cper < p.Cin ? cbeg + p.cper : p.Cin;
+    const int nblocks = (cend - cbeg) / kKC;
+
+    // ---- what this thread fetches and transforms per K-block
+    const bool patches = wave < 2;
+    const int role_row = (tid & 127) >> 2;  // tile (wavefronts 0-1) or output channel (2-3) within the block
+    const int role_q = tid & 3;             // channel quad within the K-block
+        // Load k of a K-block reads 16 bytes at tbase + toff[k] + c0 * cstep (float offsets, 32-bit: the launcher
+        // checks the tensor sizes).  Patch threads: pixel (i, j) = load 4i + j, rows and columns clamped into the
+        // image so that every load is unconditional; bit k of vmask says whether the pixel really lies inside
+        // (the padding is zeroed when the patch is transformed).  Filter threads: loads 0..8 are the 36
+        // contiguous floats of their four channels.  Both roles share one load sequence: two branches that each
+        // end in a load would have their last loads merged by the compiler through a pointer in scratch memory,
+        // and a scratch access in the loop makes every wait for it a wait for all loads in flight.
+        int toff[16];
+        unsigned vmask = 0xFFFFu;
+        const float* tbase;
+        int cstep;
+        if (patches) {
+            long gt = (long)tm * 32 + role_row;
+            if (gt > p.ntiles - 1) gt = p.ntiles - 1;  // past the end: the last tile again, dropped at the store
+            const int tw = (int)(gt % p.tiles_w);
+            const long q = gt / p.tiles_w;
+            const int th = (int)(q % p.tiles_h);
+            const long n = q / p.tiles_h;
+            const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
+            vmask = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int hi = hi0 + i;
+                const int hc = hi < 0 ? 0 : (hi > p.H - 1 ? p.H - 1 : hi);
+                const int rowoff = (int)(((n * p.H + hc) * p.W) * p.xp) + role_q * 4;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int wi = wi0 + j;
+                    const int wc = wi < 0 ? 0 : (wi > p.W - 1 ? p.W - 1 : wi);
+                    toff[i * 4 + j] = rowoff + (int)(wc * p.xp);
+                    if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W) vmask |= 1u << (i * 4 + j);
+                }
+            }
+            tbase = p.x;
+            cstep = 1;
+        } else {
+            const long wc = (long)tn * 32 + role_row;  // < Cout: the launcher takes whole blocks of 32 channels only
+            tbase = p.w + (wc * p.Cin + role_q * 4) * 9;
+            cstep = 9;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) toff[k] = k < 9 ? 4 * k : 0;
+        }
+
+        f32x4 raw0[16];
+        auto load_raw = [&](f32x4 (&raw)[16], int c0) {
+            if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
+            const int cc = c0 * cstep;
+#pragma unroll
+            for (int k = 0; k < 9; ++k) raw[k] = *reinterpret_cast<const f32x4*>(tbase + (toff[k] + cc));
+            if (patches) {
+#pragma unroll
+                for (int k = 9; k < 16; ++k) raw[k] = *reinterpret_cast<const f32x4*>(tbase + (toff[k] + cc));
+            }
+        };
+        auto stage = [&](f32x4 (&raw)[16], float* Vs, float* Us) {
+            if (patches) {
+                // V = B^T d B, four channels at a time, in place: first down the rows of every column, then
+                // along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time)
+                if (vmask != 0xFFFFu) {  // a tile at the image border: its padding pixels count as zeros
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) {
+                        const float keep = (vmask >> k) & 1 ? 1.f : 0.f;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) raw[k][c] = keep != 0.f ? raw[k][c] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x4 d1 = raw[1 * 4 + j];
+                    raw[0 * 4 + j] -= raw[2 * 4 + j];
+                    raw[1 * 4 + j] = d1 + raw[2 * 4 + j];
+                    raw[2 * 4 + j] -= d1;
+                    raw[3 * 4 + j] = d1 - raw[3 * 4 + j];
+                }
+                float* dst = Vs + role_row * kKC + swz(role_row, role_q);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f32x4 d1 = raw[i * 4 + 1];
+                    const f32x4 v0 = raw[i * 4 + 0] - raw[i * 4 + 2];
+                    const f32x4 v1 = d1 + raw[i * 4 + 2];
+                    const f32x4 v2 = raw[i * 4 + 2] - d1;
+                    const f32x4 v3 = d1 - raw[i * 4 + 3];
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = v0;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = v1;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = v2;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = v3;
+                }
+            } else {
+                // U = G g G^T for the four input channels of this thread's quad; raw holds g[ci][kh][kw] flat
+                float* dst = Us + role_row * kKC + swz(role_row, role_q);
+                float a[4][4][3];  // [ci][i][kw] = (G g) of channel ci
+#pragma unroll
+                for (int ci = 0; ci < 4; ++ci) {
+                    float g[9];
+#pragma unroll
+                    for (int k = 0; k < 9; ++k) {
+                        const int f = ci * 9 + k;
+                        g[k] = raw[f >> 2][f & 3];
+                    }
+#pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) {
+                        a[ci][0][kw] = g[0 * 3 + kw];
+                        a[ci][1][kw] = 0.5f * ((g[0 * 3 + kw] + g[1 * 3 + kw]) + g[2 * 3 + kw]);
+                        a[ci][2][kw] = 0.5f * ((g[0 * 3 + kw] - g[1 * 3 + kw]) + g[2 * 3 + kw]);
+                        a[ci][3][kw] = g[2 * 3 + kw];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    f32x4 u0, u1, u2, u3;
+#pragma unroll
+                    for (int ci = 0; ci < 4; ++ci) {
+                        u0[ci] = a[ci][i][0];
+                        u1[ci] = 0.5f * ((a[ci][i][0] + a[ci][i][1]) + a[ci][i][2]);
+                        u2[ci] = 0.5f * ((a[ci][i][0] - a[ci][i][1]) + a[ci][i][2]);
+                        u3[ci] = a[ci][i][2];
+                    }
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = u0;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = u1;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = u2;
+                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = u3;
+                }
+            }
+        };
+
+    // per-column constants of the epilogue, asked for now and used at the very end
+    float cs, ct;
+    epilogue_column(p.ep, (long)tn * 32 + r, cs, ct);
+
+    if (tid < 32) {
+        const long gt = (long)tm * 32 + tid;
+        int pix = -1, ok = 0;
+        if (gt < p.ntiles) {
+            const int tw = (int)(gt % p.tiles_w);
+            const long q = gt / p.tiles_w;
+            const int th = (int)(q % p.tiles_h);
+            const long n = q / p.tiles_h;
+            pix = (int)((n * p.H + 2 * th) * p.W + 2 * tw);
+            ok = (2 * th + 1 < p.H ? 1 : 0) | (2 * tw + 1 < p.W ? 2 : 0);
+        }
+        rowpix[tid] = pix;
+        rowok[tid] = ok;
+    }
+
+    f32x16 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // fragment addresses of this lane: xi = 4*wave + j, row r, k-group g -> chunk 2g + h
+    const int frag0 = (wave * 4 * 32 + r) * kKC + swz(r, h);
+    const int frag1 = (wave * 4 * 32 + r) * kKC + swz(r, 2 + h);
+    auto multiply = [&](const float* Vs, const float* Us) {
+        // eight (k-group, xi) steps of two fragment reads and four MFMAs; the fragments of step n+1 are
+        // requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work
+        f32x4 a[2], b[2];
+        a[0] = *reinterpret_cast<const f32x4*>(Vs + frag0);
+        b[0] = *reinterpret_cast<const f32x4*>(Us + frag0);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            const int cur = n & 1, nxt = cur ^ 1;
+            if (n + 1 < 8) {
+                const int g = (n + 1) >> 2, j = (n + 1) & 3;
+                a[nxt] = *reinterpret_cast<const f32x4*>(Vs + (g ? frag1 : frag0) + j * 32 * kKC);
+                b[nxt] = *reinterpret_cast<const f32x4*>(Us + (g ? frag1 : frag0) + j * 32 * kKC);
+            }
+            const int j = n & 3;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][s], acc[j], 0, 0, 0);
+        }
+    };
+
+    load_raw(raw0, cbeg);
+    for (int n = 0; n < nblocks; ++n) {
+        stage(raw0, lds, lds + kOperandFloats);
+        __syncthreads();
+        load_raw(raw0, cbeg + (n + 1) * kKC);  // in flight while this block is multiplied
+        multiply(lds, lds + kOperandFloats);
+        __syncthreads();
+    }
+
+    // ---- output transform.  This wavefront holds row i = wave of M; fold it over j ...
+    float* ex = lds;  // [(i*2 + b)*16 + v][lane]; the operand blocks are no longer read (barrier above)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        ex[((wave * 2 + 0) * 16 + v) * 64 + lane] = (acc[0][v] + acc[1][v]) + acc[2][v];
+        ex[((wave * 2 + 1) * 16 + v) * 64 + lane] = (acc[1][v] - acc[2][v]) - acc[3][v];
+    }
+    __syncthreads();
+    // ... and combine the rows: wavefront (oa, ob) takes output pixel (oa, ob) of every tile
+    const int oa = wave >> 1, ob = wave & 1;
+    f32x16 out[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const float t1 = ex[((1 * 2 + ob) * 16 + v) * 64 + lane];
+        const float t2 = ex[((2 * 2 + ob) * 16 + v) * 64 + lane];
+        const float t03 = ex[(((oa ? 3 : 0) * 2 + ob) * 16 + v) * 64 + lane];
+        out[0][0][v] = oa ? (t1 - t2) - t03 : (t03 + t1) + t2;
+    }
+    if (p.splits > 1) {
+        if (!finish_split<WinoOutCfg>(out, p.ws, p.tickets, p.splits, t, split, wave, lane, &flag)) return;
+    }
+
+    // ---- write-out: row of the block = tile, column = output channel
+    const Epilogue& e = p.ep;
+    const long col = (long)tn * 32 + r;
+    const int pixoff = oa * p.W + ob;
+    const bool relu = e.act == ACT_RELU;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int row = (v >> 2) * 8 + h * 4 + (v & 3);
+        const int pix = rowpix[row];
+        const int ok = rowok[row];
+        if (pix < 0 || (oa && !(ok & 1)) || (ob && !(ok & 2))) continue;
+        const long o = (long)(pix + pixoff);
+        float xv = out[0][0][v] * e.alpha;
+        xv = xv * cs + ct;
+        if (e.residual) xv += e.residual[o * e.ldr + col];
+        p.y[o * p.yp + col] = relu ? (xv > 0.f ? xv : 0.f) : apply_act(xv, e.act);
+    }
+}
+
+inline bool aligned16w(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+}  // namespace
+
+// Returns K_EUNSUPPORTED when the shape is not one this path takes (the caller then uses the direct
+// kernels).  Taken: 3x3, stride 1, padding 1, NHWC in and out, Cin a multiple of 16, Cout a multiple of 32,
+// no beta term.
+int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
+    if (a.KH != 3 || a.KW != 3 || a.sh != 1 || a.sw != 1 || a.ph != 1 || a.pw != 1) return K_EUNSUPPORTED;
+    if (!a.x_nhwc || !a.y_nhwc || a.groups != 1 || a.ep.beta != 0.f) return K_EUNSUPPORTED;
+    if (a.Cin % kKC != 0 || a.Cout % 32 != 0 || !ws.zeros) return K_EUNSUPPORTED;
+    const long xp = a.x_pitch ? a.x_pitch : a.Cin, yp = a.y_pitch ? a.y_pitch : a.Cout;
+    if (xp % 4 != 0 || !aligned16w(a.x) || !aligned16w(a.w)) return K_EUNSUPPORTED;
+    // Small launches are bound by the length of one workgroup's chain (fetch, transform, multiply, exchange, sum),
+    // which is longer here than in the direct kernels' nine-wavefront tiles: batch-1 ResNet layers ran 11-16 us
+    // this way against 8-11 us.  TORPOR_WINO_MIN_GFLOP moves the bound (direct-form FLOP of the layer).
+    const char* min_env = getenv("TORPOR_WINO_MIN_GFLOP");  // read per call: tests send small shapes down this path
+    const double min_gflop = min_env ? atof(min_env) : 0.8;
+    if (2.0 * a.N * a.H * a.W * (double)a.Cout * a.Cin * 9.0 < min_gflop * 1e9) return K_EUNSUPPORTED;
+    const long pixels = (long)a.N * a.H * a.W;
+    if (pixels * xp >= (1L << 31) || pixels >= (1L << 31)) return K_EUNSUPPORTED;  // offsets are 32-bit in the kernel
+
+    WinoDev p;
+    p.x = a.x;
+    p.w = a.w;
+    p.y = a.y;
+    p.H = a.H;
+    p.W = a.W;
+    p.Cin = a.Cin;
+    p.Cout = a.Cout;
+    p.xp = xp;
+    p.yp = yp;
+    p.tiles_h = (a.H + 1) / 2;
+    p.tiles_w = (a.W + 1) / 2;
+    p.ntiles = (long)a.N * p.tiles_h * p.tiles_w;
+    const long mt = (p.ntiles + 31) / 32;
+    p.nt = a.Cout / 32;
+    if (mt * p.nt >= (1L << 31) / 8) return K_EUNSUPPORTED;
+    p.mt = (int)mt;
+    const long base = mt * p.nt;
+    const int kblocks = a.Cin / kKC;
+
+    // Split over input channels when the blocks alone leave CUs idle.  The kernel is bound by what a SIMD
+    // issues (transforms and MFMAs take turns), so two workgroups on a CU take twice as long as one: the
+    // candidates are weighed by the K-blocks the fullest CU works through, with a slight preference for a CU
+    // that holds two workgroups (they fill each other's barrier waits), two K-blocks' worth for reading a split
+    // back and summing it, and a little per slot.  Measured on MI355X (us): 8x14x14x256>256 1/2/4/8 slots
+    // 36.6 / 24.8 / 23.9 / 28.2; 8x28x28x128>128 22.5 / 23.6 / 27.8 / 34.4; 8x7x7x512>512 73 / 43 / 27.1 / 25.7.
+    const char* forced_env = getenv("TORPOR_WINO_SPLITS");  // read per call: tests compare split depths in one process
+    const int forced = forced_env ? atoi(forced_env) : 0;
+    const size_t per_split = (size_t)base * 4096 * sizeof(float);
+    int splits = 1;
+    if (ws.ptr && ws.tickets && base <= kSplitTickets) {
+        double best = 1e30;
+        for (int sp = 1; sp <= 8 && sp <= kblocks; ++sp) {
+            if (sp > 1 && (size_t)sp * per_split > ws.bytes) break;
+            const int kb = (kblocks + sp - 1) / sp;
+            const int eff = (kblocks + kb - 1) / kb;
+            if (eff != sp) continue;
+            const long deep = (base * sp + num_cu() - 1) / num_cu();
+            const double cost = (double)deep * kb * (deep == 1 ? 1.1 : 1.0) + (sp > 1 ? 2.0 : 0.0) + 0.05 * sp;
+            if (cost < best) {
+                best = cost;
+                splits = sp;
+            }
+        }
+        if (forced > 0 && forced <= 8 && forced <= kblocks && (size_t)forced * per_split <= ws.bytes) splits = forced;
+    }
+    int kb = (kblocks + splits - 1) / splits;
+    p.cper = kb * kKC;
+    p.splits = (a.Cin + p.cper - 1) / p.cper;
+    p.ws = ws.ptr;
+    p.tickets = p.splits > 1 ? split_tickets(ws, base, p.splits) : nullptr;
+    if (p.splits > 1 && !p.tickets) {  // in-launch summation switched off: one slice
+        p.splits = 1;
+        p.cper = a.Cin;
+    }
+    p.zeros = ws.zeros;
+    EpilogueArgs ea = a.ep;
+    if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;  // the residual is dense unless its pitch is given
+    p.ep = make_epilogue(ea, yp);
+    hipLaunchKernelGGL(conv_wino_kernel, dim3((unsigned)base, 1, (unsigned)p.splits), dim3(256), 0, s, p);
+    set_last_kernel("conv3x3_wino_f2x2");
+    return (int)hipGetLastError();
+}
+
+}  // namespace tpk
