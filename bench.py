@@ -610,8 +610,8 @@ def main():
             # gets the full length, served through the miss-aware dispatcher (torpor_amd/dispatch.py)
             secs = args.multitenant_seconds if cap == tight else min(args.multitenant_seconds, 10.0)
             runs[f"cap_{cap:g}GiB"] = mt.run_cap(cap, secs, 200.0, dispatch="miss-aware")
-        # the binding cap once more in arrival order, as the reference's router hands requests over
-        runs[f"cap_{tight:g}GiB_in_order"] = mt.run_cap(tight, min(args.multitenant_seconds, 20.0), 200.0, dispatch="in-order")
+        # the binding cap once more on the same trace in arrival order, as the reference's router hands requests over
+        runs[f"cap_{tight:g}GiB_in_order"] = mt.run_cap(tight, args.multitenant_seconds, 200.0, dispatch="in-order")
         line["workloads"]["multitenant-64"] = dict(
             config="32x ResNet-50 + 16x BERT-base s128 + 16x ResNet-152, seeds 0..63, batch 1, open-loop Poisson "
                    f"200 req/s, Zipf(1.1) popularity, {args.multitenant_seconds:g} s under the binding cap; "
