@@ -312,8 +312,9 @@ int tp_bn_inference_pitched(tp_server* s, int32_t client, uint64_t x, uint64_t y
  * stream); no tp_server is involved.  The call allocates nothing on host or device: the partial sums of
  * a GEMM whose K range is split over workgroups go to a fixed TP_NOALLOC_SCRATCH_BYTES array that each
  * GPU the library runs on holds until the process ends.  Results are bit-identical to tp_gemm's.
- *   - a shape whose partial sums need more than that array is refused with TP_ESCRATCH (a split only
- *     happens for fewer 64x64 output tiles than CUs, so m * n <= 1 Mi elements; at most 32 splits);
+ *   - a shape whose partial sums need more than that array is refused with TP_ESCRATCH (a split happens for
+ *     fewer 64x64 output tiles than CUs, so m * n <= 1 Mi elements with at most 32 slots, or as a pair of K
+ *     halves for up to three tiles per CU when both halves fit the array);
  *   - all calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
  *     race on it.  Calls on one stream are ordered and safe.
  *   - the first call on each GPU looks up that GPU's copy of the array and the device's properties, which

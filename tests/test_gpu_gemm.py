@@ -19,7 +19,7 @@ def _rand(rng, *shape):
     (128, 768, 768, "gemm_fast_32x32_kc"),      # BERT-base projection: 24 64x64 tiles -> 96 32x32 tiles
     (128, 3072, 768, "gemm_fast_32x32_kc"),     # 96 64x64 tiles -> 384 32x32 tiles, K split in the workgroup
     (1536, 1024, 1024, "gemm_fast_64x32_kc"),   # BERT-large projection: 384 64x64 tiles = 1.5 per CU -> 64x32
-    (1536, 1024, 4096, "gemm_fast_64x32_kc"),   # BERT-large FFN down-projection
+    (1536, 1024, 4096, "gemm_fast_64x64_kc"),   # BERT-large FFN down-projection: long K, two K halves per 64x64 tile summed in the launch
     (4096, 2048, 160, "gemm_fast_64x64_kc"),    # K % 64 != 0: predicated kernel
     (1, 1000, 2048, "gemm_fast_32x32_kc"),      # ResNet classifier, batch 1: 32 small tiles, K split over 8 workgroups each
     (1568, 256, 1024, "gemm_fast_32x32_kc"),    # ResNet-152 batch 8 layer3 1x1: 100 64x64 tiles -> 32x32, K split in the workgroup

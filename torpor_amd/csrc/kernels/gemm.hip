@@ -791,9 +791,28 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
         g.bn = cfg == 0 ? 128 : cfg >= 3 ? 32 : 64;
         g.tiles_m = (int)((a.M + g.bm - 1) / g.bm);
         g.tiles_n = (int)((a.N + g.bn - 1) / g.bn);
-        const long tiles = (long)g.tiles_m * g.tiles_n * batch;
+        long tiles = (long)g.tiles_m * g.tiles_n * batch;
         g.kper = ((a.K + 31) / 32) * 32;
-        if (batch == 1 && cfg < 3) g.splits = choose_splits(tiles, a.K, 32, (long)g.bm * g.bn, ws_bytes, &g.kper);
+        // A long K with one to three 64x64 tiles per CU: instead of halving the tile (cfg 3) halve K -- two
+        // workgroups per 64x64 tile, summed inside the launch.  Same number of workgroups, a third less operand
+        // traffic into LDS per multiplication (1536x1024x4096: 135.7 -> 126.9 us bracketed, 95 -> 101.5 TFLOP/s;
+        // at K = 1024 the two are equal and the tile stays halved).  Only where the partial sums stay within
+        // what every caller's scratch memory holds (kSplitPairBytes), so that all entry points split alike.
+        static const bool pair_split = getenv("TORPOR_GEMM_PAIR") == nullptr || atoi(getenv("TORPOR_GEMM_PAIR")) != 0;
+        constexpr size_t kSplitPairBytes = (16u << 20) - 4096;
+        const size_t pair_bytes = 2 * (size_t)a.M * (size_t)a.N * sizeof(float);
+        if (pair_split && cfg == 3 && batch == 1 && a.K >= 2048 && a.K % 128 == 0 && pair_bytes <= kSplitPairBytes &&
+            pair_bytes <= ws_bytes && (long)((a.M + 63) / 64) * ((a.N + 63) / 64) <= kSplitTickets) {
+            cfg = g.cfg = 2;
+            g.bm = g.bn = 64;
+            g.tiles_m = (int)((a.M + 63) / 64);
+            g.tiles_n = (int)((a.N + 63) / 64);
+            tiles = (long)g.tiles_m * g.tiles_n;
+            g.splits = 2;
+            g.kper = a.K / 2;
+        } else if (batch == 1 && cfg < 3) {
+            g.splits = choose_splits(tiles, a.K, 32, (long)g.bm * g.bn, ws_bytes, &g.kper);
+        }
         // (with more than half a tile per CU the split does not pay: 196x1024x512, 224 tiles, 8.5 against 7.4 us)
         if (batch == 1 && cfg == 4 && tiles <= g_num_cu / 2)
             g.splits = choose_splits(tiles, a.K, 64, 32 * 32, ws_bytes, &g.kper, /*max_splits=*/8, true, g_small_balance);
