@@ -200,6 +200,20 @@ def measured_traffic(workload, kernel):
     return (int(m.group(1)), rel) if m else (None, None)
 
 
+def profiled_average(workload, kernel):
+    """(average duration in us of `kernel` over ALL its launches of one run of this workload's bench command
+    under rocprofv3 --kernel-trace --stats, file) from the committed summary; (None, None) when none covers it.
+    Unlike the event brackets, that average includes the launches of cold requests, which share the device with
+    the swap-in's copies and unpack kernels."""
+    rel = os.path.join("profiles", workload.replace("-", "_") + "_kernel_stats.md")
+    try:
+        text = open(os.path.join(ROOT, rel)).read()
+    except OSError:
+        return None, None
+    m = re.search(r"^rocprof_avg_us\[" + re.escape(kernel) + r"\]:\s*([0-9.]+)", text, re.M)
+    return (float(m.group(1)), rel) if m else (None, None)
+
+
 def by_symbol(kstats):
     """{kernel symbol: summed stats + {shape: stats}} from the per-shape records of the engine
     (names are `symbol[shape]` for GEMM and convolution launches)."""
@@ -239,9 +253,16 @@ def roofline_from(kstats, empty_us, workload):
              traffic_source=(traffic_file + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command; read "
                              "from that file, not counted in this run)") if traffic_file else None,
              launches=n, avg_launch_us=avg_us, event_overhead_us=empty_us, bytes_per_launch=st["bytes"] / n,
+             timing="frac, achieved, avg_launch_us: HIP-event brackets around each launch of 5 warm requests in "
+                    "this run; frac_rocprof, rocprof_avg_launch_us: rocprofv3 --kernel-trace --stats average over "
+                    "all launches of a run of this command (cold requests included), read from rocprof_source",
              by_shape=shapes)
     if mfma:
         r.update(flop_per_launch=st["flops"] / n, hbm_gbps=st["bytes"] / (t_us * 1e-6) / 1e9)
+    prof_us, prof_file = profiled_average(workload, name)
+    if prof_us:
+        work = st["flops"] / n / 1e12 if mfma else st["bytes"] / n / 1e9
+        r.update(rocprof_avg_launch_us=prof_us, frac_rocprof=work / (prof_us * 1e-6) / peak, rocprof_source=prof_file)
     return r
 
 
@@ -449,8 +470,12 @@ def compact_roofline(r):
     if not r:
         return None
     keep = ("kernel", "bound", "achieved", "peak", "unit", "frac", "traffic", "launches", "avg_launch_us",
-            "flop_per_launch", "bytes_per_launch", "timing")
+            "flop_per_launch", "bytes_per_launch", "frac_rocprof", "rocprof_avg_launch_us")
     out = {k: r[k] for k in keep if k in r}
+    if "frac_rocprof" in out:
+        out["timing"] = "frac: HIP-event brackets, warm requests, this run; frac_rocprof: rocprofv3 average, all launches, " + r["rocprof_source"]
+    else:
+        out["timing"] = "frac: HIP-event brackets, warm requests, this run"
     if r.get("traffic") and r.get("bytes_per_launch"):
         out["traffic_over_algorithmic"] = r["traffic"] / r["bytes_per_launch"]
     return out

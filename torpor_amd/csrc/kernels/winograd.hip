@@ -38,7 +38,7 @@ unsigned* split_tickets(const Workspace& ws, long tiles, int splits);
 namespace {
 
 constexpr int kKC = 16;                        // input channels per K-block
-constexpr int kOperandFloats = 16 * 32 * kKC;  // V (or U) of one K-block: [xi][row][channel]
+constexpr int kOperandFloats = 16 * 32 * kKC;  // V (or U of 32 output channels) of one K-block: [xi][row][channel]
 
 struct WinoDev {
     const float* x;
@@ -48,17 +48,17 @@ struct WinoDev {
     long xp, yp;           // floats between pixels of x / y
     int tiles_h, tiles_w;  // 2x2 output tiles per image
     long ntiles;           // N * tiles_h * tiles_w
-    int mt, nt;            // blocks of 32 tiles / 32 output channels
+    int mt, nt;            // blocks of 32 tiles / of 32*NB output channels
     int splits, cper;      // input-channel slices and channels per slice (a multiple of kKC)
     float* ws;
     unsigned* tickets;
-    const float* zeros;
     Epilogue ep;
 };
 
-// what finish_split needs to know: four wavefronts with one 32x32 accumulator block each
+// what finish_split needs to know: four wavefronts with NB 32x32 accumulator blocks each
+template <int NB>
 struct WinoOutCfg {
-    static constexpr int TM = 1, TN = 1, WGM = 2, WGN = 2;
+    static constexpr int TM = 1, TN = NB, WGM = 2, WGN = 2;
 };
 
 __device__ __forceinline__ void fetch_args(const WinoDev& p) {
@@ -79,7 +79,6 @@ __device__ __forceinline__ void fetch_args(const WinoDev& p) {
     fetch_now(p.cper);
     fetch_now(p.ws);
     fetch_now(p.tickets);
-    fetch_now(p.zeros);
     fetch_now(p.ep);
 }
 
@@ -94,21 +93,100 @@ __device__ __forceinline__ int remap_xcd_w(int bid, int n) {
 // even ones on banks 0-15 and four odd ones on banks 16-31, and rows two apart get different chunks.
 __device__ __forceinline__ int swz(int row, int chunk) { return (chunk ^ ((row >> 1) & 3)) << 2; }
 
-// Four wavefronts.  All of them multiply: wavefront w owns the four accumulators of row i = w of the 4x4
-// (xi = 4w .. 4w+3).  Before that, per K-block, wavefronts 0-1 fetch and transform the patches and 2-3 the
-// filters; the loads of the next K-block are in flight meanwhile.  Two workgroups share a CU (64 KiB of LDS
-// each).  Measured on MI355X, 8x14x14x256 -> 256: per K-block a wavefront spends about 2000 cycles on the
+// V = B^T d B of one 4x4 patch, four channels at a time, in place: first down the rows of every column, then
+// along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time); d[4i + j] = pixel (i, j).
+// dst = this thread's chunk of row `tile` in block xi = 0; bit k of vmask clear = pixel k is padding.
+__device__ __forceinline__ void transform_patch(f32x4 (&d)[16], unsigned vmask, float* __restrict__ dst) {
+    if (vmask != 0xFFFFu) {  // a tile at the image border: its padding pixels count as zeros
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const float keep = (vmask >> k) & 1 ? 1.f : 0.f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) d[k][c] = keep != 0.f ? d[k][c] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const f32x4 d1 = d[1 * 4 + j];
+        d[0 * 4 + j] -= d[2 * 4 + j];
+        d[1 * 4 + j] = d1 + d[2 * 4 + j];
+        d[2 * 4 + j] -= d1;
+        d[3 * 4 + j] = d1 - d[3 * 4 + j];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const f32x4 d1 = d[i * 4 + 1];
+        const f32x4 v0 = d[i * 4 + 0] - d[i * 4 + 2];
+        const f32x4 v1 = d1 + d[i * 4 + 2];
+        const f32x4 v2 = d[i * 4 + 2] - d1;
+        const f32x4 v3 = d1 - d[i * 4 + 3];
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = v0;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = v1;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = v2;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = v3;
+    }
+}
+
+// U = G g G^T for four input channels of one output channel; raw = the 36 floats g[ci][kh][kw].
+// dst = this thread's chunk of row `channel` in block xi = 0 of a [xi][ROWS][16] operand.
+template <int ROWS>
+__device__ __forceinline__ void transform_filter(const f32x4 (&raw)[9], float* __restrict__ dst) {
+    float a[4][4][3];  // [ci][i][kw] = (G g) of channel ci
+#pragma unroll
+    for (int ci = 0; ci < 4; ++ci) {
+        float g[9];
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            const int f = ci * 9 + k;
+            g[k] = raw[f >> 2][f & 3];
+        }
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+            a[ci][0][kw] = g[0 * 3 + kw];
+            a[ci][1][kw] = 0.5f * ((g[0 * 3 + kw] + g[1 * 3 + kw]) + g[2 * 3 + kw]);
+            a[ci][2][kw] = 0.5f * ((g[0 * 3 + kw] - g[1 * 3 + kw]) + g[2 * 3 + kw]);
+            a[ci][3][kw] = g[2 * 3 + kw];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f32x4 u0, u1, u2, u3;
+#pragma unroll
+        for (int ci = 0; ci < 4; ++ci) {
+            u0[ci] = a[ci][i][0];
+            u1[ci] = 0.5f * ((a[ci][i][0] + a[ci][i][1]) + a[ci][i][2]);
+            u2[ci] = 0.5f * ((a[ci][i][0] - a[ci][i][1]) + a[ci][i][2]);
+            u3[ci] = a[ci][i][2];
+        }
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * ROWS * kKC) = u0;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * ROWS * kKC) = u1;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * ROWS * kKC) = u2;
+        *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * ROWS * kKC) = u3;
+    }
+}
+
+// Four wavefronts; all of them multiply: wavefront w owns the accumulators of row i = w of the 4x4
+// (xi = 4w .. 4w+3) for NB blocks of 32 output channels.  Before that, per K-block, the patches and filters
+// are fetched and transformed; the loads of the next K-block are in flight while this one is multiplied.
+//   NB = 1: 32 tiles x 32 channels.  Wavefronts 0-1 take the patches, 2-3 the filters; 64 KiB of LDS, two
+//           workgroups per CU.
+//   NB = 2: 32 tiles x 64 channels.  Every thread takes a filter job, wavefronts 0-1 a patch job as well;
+//           96 KiB of LDS, one workgroup per CU.  A patch transform now serves twice the matrix work.
+// Measured on MI355X, 8x14x14x256 -> 256, NB = 1: per K-block a wavefront spends about 2000 cycles on the
 // transform's vector instructions and 2050 on its 32 MFMAs, and the two do not overlap on a SIMD -- not
 // within a wavefront, not between two workgroups on the CU, and not when the transforms are given to
 // wavefronts of their own (built and measured: same time), because a SIMD issues either kind from one
-// port.  That is what bounds this path at about 1.15x the direct kernel instead of the 2.25x of the
-// multiplication count.
-__global__ __launch_bounds__(256, 2) void conv_wino_kernel(const WinoDev p) {
+// port.  That bounds this path well below the 2.25x of the multiplication count, and is why the transforms are
+// spread over as much matrix work as the registers allow.
+template <int NB>
+__global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const WinoDev p) {
     fetch_args(p);
-    __shared__ __attribute__((aligned(16))) float lds[2 * kOperandFloats];  // [V | U] of one K-block
+    __shared__ __attribute__((aligned(16))) float lds[(1 + NB) * kOperandFloats];  // [V | U (NB blocks)] of one K-block
     __shared__ int rowpix[32];  // (n*H + 2*th)*W + 2*tw of each tile of this block, -1 past the last tile
     __shared__ int rowok[32];   // bit 0: the tile's second output row exists, bit 1: its second column
     __shared__ unsigned flag;
+    float* const Vs = lds;
+    float* const Us = lds + kOperandFloats;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wavefront: role branches are scalar
     const int r = lane & 31, h = lane >> 5;
@@ -120,137 +198,80 @@ __global__ __launch_bounds__(256, 2) void conv_wino_kernel(const WinoDev p) {
     const int nblocks = (cend - cbeg) / kKC;
 
     // ---- what this thread fetches and transforms per K-block
+    // Every load reads 16 bytes from one base pointer plus a 32-bit float offset (the launcher checks the tensor
+    // sizes).  Patch job: pixel (i, j) = load 4i + j, rows and columns clamped into the image so that every load
+    // is unconditional; bit k of vmask says whether the pixel really lies inside (the padding is zeroed when the
+    // patch is transformed).  Filter job: nine loads, the 36 contiguous floats of four input channels.
+    // The first nine loads are one common sequence for every thread -- with NB = 1 a patch thread's first nine
+    // pixels, a filter thread's whole job -- and only patch threads go on to more: two branches that each end
+    // in a load get their last loads merged by the compiler through a pointer in scratch memory, and a scratch
+    // access in the loop turns every wait for it into a wait for all loads in flight.
     const bool patches = wave < 2;
-    const int role_row = (tid & 127) >> 2;  // tile (wavefronts 0-1) or output channel (2-3) within the block
-    const int role_q = tid & 3;             // channel quad within the K-block
-        // Load k of a K-block reads 16 bytes at tbase + toff[k] + c0 * cstep (float offsets, 32-bit: the launcher
-        // checks the tensor sizes).  Patch threads: pixel (i, j) = load 4i + j, rows and columns clamped into the
-        // image so that every load is unconditional; bit k of vmask says whether the pixel really lies inside
-        // (the padding is zeroed when the patch is transformed).  Filter threads: loads 0..8 are the 36
-        // contiguous floats of their four channels.  Both roles share one load sequence: two branches that each
-        // end in a load would have their last loads merged by the compiler through a pointer in scratch memory,
-        // and a scratch access in the loop makes every wait for it a wait for all loads in flight.
-        int toff[16];
-        unsigned vmask = 0xFFFFu;
-        const float* tbase;
-        int cstep;
-        if (patches) {
-            long gt = (long)tm * 32 + role_row;
-            if (gt > p.ntiles - 1) gt = p.ntiles - 1;  // past the end: the last tile again, dropped at the store
-            const int tw = (int)(gt % p.tiles_w);
-            const long q = gt / p.tiles_w;
-            const int th = (int)(q % p.tiles_h);
-            const long n = q / p.tiles_h;
-            const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
-            vmask = 0;
+    const int q4 = (tid & 3) * 4;                          // channel quad within the K-block
+    const int tile_row = (tid & 127) >> 2;                 // patch job: tile within the block
+    const int chan_row = NB == 1 ? tile_row : tid >> 2;    // filter job: output channel within the block (0 .. 32*NB-1)
+    int poff[16];
+    unsigned vmask = 0xFFFFu;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int hi = hi0 + i;
-                const int hc = hi < 0 ? 0 : (hi > p.H - 1 ? p.H - 1 : hi);
-                const int rowoff = (int)(((n * p.H + hc) * p.W) * p.xp) + role_q * 4;
+    for (int k = 0; k < 16; ++k) poff[k] = 0;
+    if (patches) {
+        long gt = (long)tm * 32 + tile_row;
+        if (gt > p.ntiles - 1) gt = p.ntiles - 1;  // past the end: the last tile again, dropped at the store
+        const int tw = (int)(gt % p.tiles_w);
+        const long q = gt / p.tiles_w;
+        const int th = (int)(q % p.tiles_h);
+        const long n = q / p.tiles_h;
+        const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
+        vmask = 0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int wi = wi0 + j;
-                    const int wc = wi < 0 ? 0 : (wi > p.W - 1 ? p.W - 1 : wi);
-                    toff[i * 4 + j] = rowoff + (int)(wc * p.xp);
-                    if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W) vmask |= 1u << (i * 4 + j);
-                }
+        for (int i = 0; i < 4; ++i) {
+            const int hi = hi0 + i;
+            const int hc = hi < 0 ? 0 : (hi > p.H - 1 ? p.H - 1 : hi);
+            const int rowoff = (int)(((n * p.H + hc) * p.W) * p.xp) + q4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int wi = wi0 + j;
+                const int wc = wi < 0 ? 0 : (wi > p.W - 1 ? p.W - 1 : wi);
+                poff[i * 4 + j] = rowoff + (int)(wc * p.xp);
+                if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W) vmask |= 1u << (i * 4 + j);
             }
-            tbase = p.x;
-            cstep = 1;
-        } else {
-            const long wc = (long)tn * 32 + role_row;  // < Cout: the launcher takes whole blocks of 32 channels only
-            tbase = p.w + (wc * p.Cin + role_q * 4) * 9;
-            cstep = 9;
-#pragma unroll
-            for (int k = 0; k < 16; ++k) toff[k] = k < 9 ? 4 * k : 0;
         }
+    }
+    const float* const fbase = p.w + (((long)tn * 32 * NB + chan_row) * p.Cin + q4) * 9;  // whole blocks only: in range
+    // the common sequence: filter job, or (NB = 1, patch thread) pixels 0..8
+    const bool common_is_patch = NB == 1 && patches;
+    const float* const cbase = common_is_patch ? p.x : fbase;
+    const int cstep = common_is_patch ? 1 : 9;
+    int coff[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) coff[k] = common_is_patch ? poff[k] : 4 * k;
 
-        f32x4 raw0[16];
-        auto load_raw = [&](f32x4 (&raw)[16], int c0) {
-            if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
-            const int cc = c0 * cstep;
+    f32x4 rc[9], rp[16];
+    auto load_raw = [&](int c0) {
+        if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
+        const int cc = c0 * cstep;
 #pragma unroll
-            for (int k = 0; k < 9; ++k) raw[k] = *reinterpret_cast<const f32x4*>(tbase + (toff[k] + cc));
-            if (patches) {
+        for (int k = 0; k < 9; ++k) rc[k] = *reinterpret_cast<const f32x4*>(cbase + (coff[k] + cc));
+        if (patches) {
 #pragma unroll
-                for (int k = 9; k < 16; ++k) raw[k] = *reinterpret_cast<const f32x4*>(tbase + (toff[k] + cc));
+            for (int k = (NB == 1 ? 9 : 0); k < 16; ++k) rp[k] = *reinterpret_cast<const f32x4*>(p.x + (poff[k] + c0));
+        }
+    };
+    auto stage = [&]() {
+        if (NB == 2 || !patches) transform_filter<32 * NB>(rc, Us + chan_row * kKC + swz(chan_row, tid & 3));
+        if (patches) {
+            if (NB == 1) {
+#pragma unroll
+                for (int k = 0; k < 9; ++k) rp[k] = rc[k];
             }
-        };
-        auto stage = [&](f32x4 (&raw)[16], float* Vs, float* Us) {
-            if (patches) {
-                // V = B^T d B, four channels at a time, in place: first down the rows of every column, then
-                // along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time)
-                if (vmask != 0xFFFFu) {  // a tile at the image border: its padding pixels count as zeros
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) {
-                        const float keep = (vmask >> k) & 1 ? 1.f : 0.f;
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) raw[k][c] = keep != 0.f ? raw[k][c] : 0.f;
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const f32x4 d1 = raw[1 * 4 + j];
-                    raw[0 * 4 + j] -= raw[2 * 4 + j];
-                    raw[1 * 4 + j] = d1 + raw[2 * 4 + j];
-                    raw[2 * 4 + j] -= d1;
-                    raw[3 * 4 + j] = d1 - raw[3 * 4 + j];
-                }
-                float* dst = Vs + role_row * kKC + swz(role_row, role_q);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const f32x4 d1 = raw[i * 4 + 1];
-                    const f32x4 v0 = raw[i * 4 + 0] - raw[i * 4 + 2];
-                    const f32x4 v1 = d1 + raw[i * 4 + 2];
-                    const f32x4 v2 = raw[i * 4 + 2] - d1;
-                    const f32x4 v3 = d1 - raw[i * 4 + 3];
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = v0;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = v1;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = v2;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = v3;
-                }
-            } else {
-                // U = G g G^T for the four input channels of this thread's quad; raw holds g[ci][kh][kw] flat
-                float* dst = Us + role_row * kKC + swz(role_row, role_q);
-                float a[4][4][3];  // [ci][i][kw] = (G g) of channel ci
-#pragma unroll
-                for (int ci = 0; ci < 4; ++ci) {
-                    float g[9];
-#pragma unroll
-                    for (int k = 0; k < 9; ++k) {
-                        const int f = ci * 9 + k;
-                        g[k] = raw[f >> 2][f & 3];
-                    }
-#pragma unroll
-                    for (int kw = 0; kw < 3; ++kw) {
-                        a[ci][0][kw] = g[0 * 3 + kw];
-                        a[ci][1][kw] = 0.5f * ((g[0 * 3 + kw] + g[1 * 3 + kw]) + g[2 * 3 + kw]);
-                        a[ci][2][kw] = 0.5f * ((g[0 * 3 + kw] - g[1 * 3 + kw]) + g[2 * 3 + kw]);
-                        a[ci][3][kw] = g[2 * 3 + kw];
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    f32x4 u0, u1, u2, u3;
-#pragma unroll
-                    for (int ci = 0; ci < 4; ++ci) {
-                        u0[ci] = a[ci][i][0];
-                        u1[ci] = 0.5f * ((a[ci][i][0] + a[ci][i][1]) + a[ci][i][2]);
-                        u2[ci] = 0.5f * ((a[ci][i][0] - a[ci][i][1]) + a[ci][i][2]);
-                        u3[ci] = a[ci][i][2];
-                    }
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = u0;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = u1;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = u2;
-                    *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = u3;
-                }
-            }
-        };
+            transform_patch(rp, vmask, Vs + tile_row * kKC + swz(tile_row, tid & 3));
+        }
+    };
 
     // per-column constants of the epilogue, asked for now and used at the very end
-    float cs, ct;
-    epilogue_column(p.ep, (long)tn * 32 + r, cs, ct);
+    float cs[NB], ct[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) epilogue_column(p.ep, ((long)tn * NB + nb) * 32 + r, cs[nb], ct[nb]);
 
     if (tid < 32) {
         const long gt = (long)tm * 32 + tid;
@@ -267,82 +288,100 @@ __global__ __launch_bounds__(256, 2) void conv_wino_kernel(const WinoDev p) {
         rowok[tid] = ok;
     }
 
-    f32x16 acc[4];
+    f32x16 acc[4][NB];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][nb][v] = 0.f;
 
-    // fragment addresses of this lane: xi = 4*wave + j, row r, k-group g -> chunk 2g + h
-    const int frag0 = (wave * 4 * 32 + r) * kKC + swz(r, h);
-    const int frag1 = (wave * 4 * 32 + r) * kKC + swz(r, 2 + h);
-    auto multiply = [&](const float* Vs, const float* Us) {
-        // eight (k-group, xi) steps of two fragment reads and four MFMAs; the fragments of step n+1 are
+    // fragment addresses of this lane: xi = 4*wave + j, row r, k-group g -> chunk 2g + h; the rows of output
+    // channel block nb follow 32 rows further on within the same xi (a U block is [xi][32*NB rows][16])
+    const int vfrag0 = (wave * 4 * 32 + r) * kKC + swz(r, h);
+    const int vfrag1 = (wave * 4 * 32 + r) * kKC + swz(r, 2 + h);
+    const int ufrag0 = (wave * 4 * 32 * NB + r) * kKC + swz(r, h);
+    const int ufrag1 = (wave * 4 * 32 * NB + r) * kKC + swz(r, 2 + h);
+    auto multiply = [&]() {
+        // eight (k-group, xi) steps of 1 + NB fragment reads and 4 * NB MFMAs; the fragments of step n+1 are
         // requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work
-        f32x4 a[2], b[2];
-        a[0] = *reinterpret_cast<const f32x4*>(Vs + frag0);
-        b[0] = *reinterpret_cast<const f32x4*>(Us + frag0);
+        f32x4 a[2], b[2][NB];
+        a[0] = *reinterpret_cast<const f32x4*>(Vs + vfrag0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) b[0][nb] = *reinterpret_cast<const f32x4*>(Us + ufrag0 + nb * 32 * kKC);
 #pragma unroll
         for (int n = 0; n < 8; ++n) {
             const int cur = n & 1, nxt = cur ^ 1;
             if (n + 1 < 8) {
                 const int g = (n + 1) >> 2, j = (n + 1) & 3;
-                a[nxt] = *reinterpret_cast<const f32x4*>(Vs + (g ? frag1 : frag0) + j * 32 * kKC);
-                b[nxt] = *reinterpret_cast<const f32x4*>(Us + (g ? frag1 : frag0) + j * 32 * kKC);
+                a[nxt] = *reinterpret_cast<const f32x4*>(Vs + (g ? vfrag1 : vfrag0) + j * 32 * kKC);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    b[nxt][nb] = *reinterpret_cast<const f32x4*>(Us + (g ? ufrag1 : ufrag0) + (j * NB + nb) * 32 * kKC);
             }
             const int j = n & 3;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][s], acc[j], 0, 0, 0);
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    acc[j][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][nb][s], acc[j][nb], 0, 0, 0);
         }
     };
 
-    load_raw(raw0, cbeg);
+    load_raw(cbeg);
     for (int n = 0; n < nblocks; ++n) {
-        stage(raw0, lds, lds + kOperandFloats);
+        stage();
         __syncthreads();
-        load_raw(raw0, cbeg + (n + 1) * kKC);  // in flight while this block is multiplied
-        multiply(lds, lds + kOperandFloats);
+        load_raw(cbeg + (n + 1) * kKC);  // in flight while this block is multiplied
+        multiply();
         __syncthreads();
     }
 
     // ---- output transform.  This wavefront holds row i = wave of M; fold it over j ...
-    float* ex = lds;  // [(i*2 + b)*16 + v][lane]; the operand blocks are no longer read (barrier above)
+    float* ex = lds;  // [((i*2 + b)*NB + nb)*16 + v][lane]; the operand blocks are no longer read (barrier above)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        ex[((wave * 2 + 0) * 16 + v) * 64 + lane] = (acc[0][v] + acc[1][v]) + acc[2][v];
-        ex[((wave * 2 + 1) * 16 + v) * 64 + lane] = (acc[1][v] - acc[2][v]) - acc[3][v];
-    }
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            ex[(((wave * 2 + 0) * NB + nb) * 16 + v) * 64 + lane] = (acc[0][nb][v] + acc[1][nb][v]) + acc[2][nb][v];
+            ex[(((wave * 2 + 1) * NB + nb) * 16 + v) * 64 + lane] = (acc[1][nb][v] - acc[2][nb][v]) - acc[3][nb][v];
+        }
     __syncthreads();
     // ... and combine the rows: wavefront (oa, ob) takes output pixel (oa, ob) of every tile
     const int oa = wave >> 1, ob = wave & 1;
-    f32x16 out[1][1];
+    f32x16 out[1][NB];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const float t1 = ex[((1 * 2 + ob) * 16 + v) * 64 + lane];
-        const float t2 = ex[((2 * 2 + ob) * 16 + v) * 64 + lane];
-        const float t03 = ex[(((oa ? 3 : 0) * 2 + ob) * 16 + v) * 64 + lane];
-        out[0][0][v] = oa ? (t1 - t2) - t03 : (t03 + t1) + t2;
-    }
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float t1 = ex[(((1 * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
+            const float t2 = ex[(((2 * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
+            const float t03 = ex[((((oa ? 3 : 0) * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
+            out[0][nb][v] = oa ? (t1 - t2) - t03 : (t03 + t1) + t2;
+        }
     if (p.splits > 1) {
-        if (!finish_split<WinoOutCfg>(out, p.ws, p.tickets, p.splits, t, split, wave, lane, &flag)) return;
+        if (!finish_split<WinoOutCfg<NB>>(out, p.ws, p.tickets, p.splits, t, split, wave, lane, &flag)) return;
     }
 
     // ---- write-out: row of the block = tile, column = output channel
     const Epilogue& e = p.ep;
-    const long col = (long)tn * 32 + r;
     const int pixoff = oa * p.W + ob;
     const bool relu = e.act == ACT_RELU;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int row = (v >> 2) * 8 + h * 4 + (v & 3);
-        const int pix = rowpix[row];
-        const int ok = rowok[row];
-        if (pix < 0 || (oa && !(ok & 1)) || (ob && !(ok & 2))) continue;
-        const long o = (long)(pix + pixoff);
-        float xv = out[0][0][v] * e.alpha;
-        xv = xv * cs + ct;
-        if (e.residual) xv += e.residual[o * e.ldr + col];
-        p.y[o * p.yp + col] = relu ? (xv > 0.f ? xv : 0.f) : apply_act(xv, e.act);
+    for (int nb = 0; nb < NB; ++nb) {
+        const long col = ((long)tn * NB + nb) * 32 + r;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = (v >> 2) * 8 + h * 4 + (v & 3);
+            const int pix = rowpix[row];
+            const int ok = rowok[row];
+            if (pix < 0 || (oa && !(ok & 1)) || (ob && !(ok & 2))) continue;
+            const long o = (long)(pix + pixoff);
+            float xv = out[0][nb][v] * e.alpha;
+            xv = xv * cs[nb] + ct[nb];
+            if (e.residual) xv += e.residual[o * e.ldr + col];
+            p.y[o * p.yp + col] = relu ? (xv > 0.f ? xv : 0.f) : apply_act(xv, e.act);
+        }
     }
 }
 
@@ -356,7 +395,7 @@ inline bool aligned16w(const void* q) { return (reinterpret_cast<uintptr_t>(q) &
 int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
     if (a.KH != 3 || a.KW != 3 || a.sh != 1 || a.sw != 1 || a.ph != 1 || a.pw != 1) return K_EUNSUPPORTED;
     if (!a.x_nhwc || !a.y_nhwc || a.groups != 1 || a.ep.beta != 0.f) return K_EUNSUPPORTED;
-    if (a.Cin % kKC != 0 || a.Cout % 32 != 0 || !ws.zeros) return K_EUNSUPPORTED;
+    if (a.Cin % kKC != 0 || a.Cout % 32 != 0) return K_EUNSUPPORTED;
     const long xp = a.x_pitch ? a.x_pitch : a.Cin, yp = a.y_pitch ? a.y_pitch : a.Cout;
     if (xp % 4 != 0 || !aligned16w(a.x) || !aligned16w(a.w)) return K_EUNSUPPORTED;
     // Small launches are bound by the length of one workgroup's chain (fetch, transform, multiply, exchange, sum),
@@ -423,11 +462,10 @@ int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t 
         p.splits = 1;
         p.cper = a.Cin;
     }
-    p.zeros = ws.zeros;
     EpilogueArgs ea = a.ep;
     if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;  // the residual is dense unless its pitch is given
     p.ep = make_epilogue(ea, yp);
-    hipLaunchKernelGGL(conv_wino_kernel, dim3((unsigned)base, 1, (unsigned)p.splits), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(conv_wino_kernel<1>, dim3((unsigned)base, 1, (unsigned)p.splits), dim3(256), 0, s, p);
     set_last_kernel("conv3x3_wino_f2x2");
     return (int)hipGetLastError();
 }
