@@ -46,6 +46,7 @@ struct WinoDev {
     float* y;
     int H, W, Cin, Cout;   // stride 1, padding 1: the output is H x W as well
     long xp, yp;           // floats between pixels of x / y
+    unsigned xbytes, wbytes;  // extent of x and of w in bytes (both below 2^31)
     int tiles_h, tiles_w;  // 2x2 output tiles per image
     long ntiles;           // N * tiles_h * tiles_w
     int mt, nt;            // blocks of 32 tiles / of 32*NB output channels
@@ -59,6 +60,7 @@ struct WinoDev {
 template <int NB>
 struct WinoOutCfg {
     static constexpr int TM = 1, TN = NB, WGM = 2, WGN = 2;
+    static constexpr int WTM = 32, WTN = 32 * NB;  // one wavefront's block of the output tile
 };
 
 __device__ __forceinline__ void fetch_args(const WinoDev& p) {
@@ -70,6 +72,8 @@ __device__ __forceinline__ void fetch_args(const WinoDev& p) {
     fetch_now(p.Cin);
     fetch_now(p.xp);
     fetch_now(p.yp);
+    fetch_now(p.xbytes);
+    fetch_now(p.wbytes);
     fetch_now(p.tiles_h);
     fetch_now(p.tiles_w);
     fetch_now(p.ntiles);
@@ -94,17 +98,9 @@ __device__ __forceinline__ int remap_xcd_w(int bid, int n) {
 __device__ __forceinline__ int swz(int row, int chunk) { return (chunk ^ ((row >> 1) & 3)) << 2; }
 
 // V = B^T d B of one 4x4 patch, four channels at a time, in place: first down the rows of every column, then
-// along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time); d[4i + j] = pixel (i, j).
-// dst = this thread's chunk of row `tile` in block xi = 0; bit k of vmask clear = pixel k is padding.
-__device__ __forceinline__ void transform_patch(f32x4 (&d)[16], unsigned vmask, float* __restrict__ dst) {
-    if (vmask != 0xFFFFu) {  // a tile at the image border: its padding pixels count as zeros
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-            const float keep = (vmask >> k) & 1 ? 1.f : 0.f;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) d[k][c] = keep != 0.f ? d[k][c] : 0.f;
-        }
-    }
+// along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time); d[4i + j] = pixel (i, j), zeros
+// where the patch reaches into the padding.  dst = this thread's chunk of row `tile` in block xi = 0.
+__device__ __forceinline__ void transform_patch(f32x4 (&d)[16], float* __restrict__ dst) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const f32x4 d1 = d[1 * 4 + j];
@@ -127,10 +123,10 @@ __device__ __forceinline__ void transform_patch(f32x4 (&d)[16], unsigned vmask, 
     }
 }
 
-// U = G g G^T for four input channels of one output channel; raw = the 36 floats g[ci][kh][kw].
+// U = G g G^T for four input channels of one output channel; raw[0..8] = the 36 floats g[ci][kh][kw].
 // dst = this thread's chunk of row `channel` in block xi = 0 of a [xi][ROWS][16] operand.
 template <int ROWS>
-__device__ __forceinline__ void transform_filter(const f32x4 (&raw)[9], float* __restrict__ dst) {
+__device__ __forceinline__ void transform_filter(const f32x4 (&raw)[16], float* __restrict__ dst) {
     float a[4][4][3];  // [ci][i][kw] = (G g) of channel ci
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) {
@@ -162,6 +158,71 @@ __device__ __forceinline__ void transform_filter(const f32x4 (&raw)[9], float* _
         *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * ROWS * kKC) = u1;
         *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * ROWS * kKC) = u2;
         *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * ROWS * kKC) = u3;
+    }
+}
+
+// Write-out of one wavefront's NB 32x32 blocks (rows = tiles, columns = output channels) for its output pixel
+// (oa, ob) of every tile, in the form the GEMM tiles use: each block goes through the wavefront's LDS staging
+// block and comes back as four consecutive columns per lane, so one step writes eight rows with 128-bit stores.
+// Straight-line code with the activation fixed at compile time: a load under a branch (the residual, say) makes
+// the compiler wait for every outstanding memory operation at the join, the stores of the previous step included
+// -- the element-wise form of this write-out took 3.4 us of a 24 us launch that way.
+template <int NB, bool RES, int ACT>
+__device__ __forceinline__ void store_rows(f32x16 (&out)[1][NB], int lane, long n0, const WinoDev& p, int pixoff, int oa,
+                                           int ob, float* __restrict__ stage_blk, const int* rowpix, const int* rowok,
+                                           const ColConsts<NB>& cc) {
+    const Epilogue& e = p.ep;
+    const int r = lane & 31, h = lane >> 5;
+    const int cq = (lane & 7) * 4;  // this lane's four columns within a block
+    const int rq = lane >> 3;       // and its row within each group of eight
+    long o[4];
+    bool live[4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int pix = rowpix[it * 8 + rq];
+        const int ok = rowok[it * 8 + rq];
+        live[it] = pix >= 0 && (!oa || (ok & 1)) && (!ob || (ok & 2));
+        o[it] = live[it] ? (long)(pix + pixoff) : 0;  // rows that are not written read the residual of pixel 0
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const long col = n0 + nb * 32 + cq;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) stage_blk[((v >> 2) * 8 + h * 4 + (v & 3)) * 32 + r] = out[0][nb][v];
+        wave_lds_sync();
+        f32x4 x[4], res[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            x[it] = *reinterpret_cast<const f32x4*>(stage_blk + (it * 8 + rq) * 32 + cq);
+            if (RES) res[it] = *reinterpret_cast<const f32x4*>(e.residual + o[it] * e.ldr + col);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float y = x[it][c] * e.alpha;
+                y = y * cc.cs[nb][c] + cc.ct[nb][c];
+                if (RES) y += res[it][c];
+                x[it][c] = act_fixed<ACT>(y);
+            }
+            if (live[it]) *reinterpret_cast<f32x4*>(p.y + o[it] * p.yp + col) = x[it];
+        }
+        wave_lds_sync();
+    }
+}
+
+template <int NB, bool RES>
+__device__ __forceinline__ void store_rows_any_act(f32x16 (&out)[1][NB], int lane, long n0, const WinoDev& p, int pixoff,
+                                                   int oa, int ob, float* __restrict__ stage_blk, const int* rowpix,
+                                                   const int* rowok, const ColConsts<NB>& cc) {
+    switch (p.ep.act) {
+        case ACT_RELU: store_rows<NB, RES, ACT_RELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_GELU: store_rows<NB, RES, ACT_GELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_TANH: store_rows<NB, RES, ACT_TANH>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_RELU6: store_rows<NB, RES, ACT_RELU6>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_SILU: store_rows<NB, RES, ACT_SILU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_SIGMOID: store_rows<NB, RES, ACT_SIGMOID>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        default: store_rows<NB, RES, ACT_NONE>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
     }
 }
 
@@ -198,90 +259,78 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
     const int nblocks = (cend - cbeg) / kKC;
 
     // ---- what this thread fetches and transforms per K-block
-    // Every load reads 16 bytes from one base pointer plus a 32-bit float offset (the launcher checks the tensor
-    // sizes).  Patch job: pixel (i, j) = load 4i + j, rows and columns clamped into the image so that every load
-    // is unconditional; bit k of vmask says whether the pixel really lies inside (the padding is zeroed when the
-    // patch is transformed).  Filter job: nine loads, the 36 contiguous floats of four input channels.
-    // The first nine loads are one common sequence for every thread -- with NB = 1 a patch thread's first nine
-    // pixels, a filter thread's whole job -- and only patch threads go on to more: two branches that each end
-    // in a load get their last loads merged by the compiler through a pointer in scratch memory, and a scratch
-    // access in the loop turns every wait for it into a wait for all loads in flight.
+    // Wavefronts 0-1: the 4x4 patch of tile `row` for four input channels, pixel (i, j) = load 4i + j.
+    // Wavefronts 2-3: the filter of output channel `row` for four input channels, 36 contiguous floats = loads 0..8.
+    // All of them are buffer loads of 16 bytes: one descriptor per wavefront (x or w), a per-lane byte offset that
+    // never changes, and the K-block's offset in a scalar register -- no address arithmetic in the loop.  A load
+    // whose offset lies beyond the descriptor's extent returns zeros without touching memory: that is how the
+    // padding around the image, the tiles past the last one and a filter thread's loads 9..15 are expressed, so
+    // that every thread issues the same sixteen loads and none of them sits under a branch.
+    static_assert(NB == 1, "the fetch and transform jobs below are laid out for 32 output channels per workgroup");
     const bool patches = wave < 2;
-    const int q4 = (tid & 3) * 4;                          // channel quad within the K-block
-    const int tile_row = (tid & 127) >> 2;                 // patch job: tile within the block
-    const int chan_row = NB == 1 ? tile_row : tid >> 2;    // filter job: output channel within the block (0 .. 32*NB-1)
-    int poff[16];
-    unsigned vmask = 0xFFFFu;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) poff[k] = 0;
+    const int q4 = (tid & 3) * 4;          // channel quad within the K-block
+    const int row = (tid & 127) >> 2;      // tile / output channel within the block
+    constexpr unsigned kBeyond = 0x80000000u;
+    unsigned off[16];
     if (patches) {
-        long gt = (long)tm * 32 + tile_row;
-        if (gt > p.ntiles - 1) gt = p.ntiles - 1;  // past the end: the last tile again, dropped at the store
-        const int tw = (int)(gt % p.tiles_w);
-        const long q = gt / p.tiles_w;
-        const int th = (int)(q % p.tiles_h);
-        const long n = q / p.tiles_h;
+        // 32-bit arithmetic throughout (the launcher checks that every offset fits): a 64-bit division costs
+        // some hundred instructions and this is on every workgroup's way to its first load
+        const unsigned gt = (unsigned)tm * 32u + (unsigned)row;
+        const bool real = gt < (unsigned)p.ntiles;
+        const unsigned q = gt / (unsigned)p.tiles_w;
+        const int tw = (int)(gt - q * (unsigned)p.tiles_w);
+        const unsigned n = q / (unsigned)p.tiles_h;
+        const int th = (int)(q - n * (unsigned)p.tiles_h);
         const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
-        vmask = 0;
+        const int xp = (int)p.xp;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int hi = hi0 + i;
-            const int hc = hi < 0 ? 0 : (hi > p.H - 1 ? p.H - 1 : hi);
-            const int rowoff = (int)(((n * p.H + hc) * p.W) * p.xp) + q4;
+            const int rowoff = (((int)n * p.H + hi) * p.W) * xp + q4;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int wi = wi0 + j;
-                const int wc = wi < 0 ? 0 : (wi > p.W - 1 ? p.W - 1 : wi);
-                poff[i * 4 + j] = rowoff + (int)(wc * p.xp);
-                if (hi >= 0 && hi < p.H && wi >= 0 && wi < p.W) vmask |= 1u << (i * 4 + j);
+                const bool inside = real && hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
+                off[i * 4 + j] = inside ? (unsigned)(rowoff + wi * xp) * 4u : kBeyond;
             }
         }
+    } else {
+        const unsigned fv = (unsigned)((tn * 32 + row) * p.Cin + q4) * 36u;  // whole blocks only: in range
+#pragma unroll
+        for (int k = 0; k < 16; ++k) off[k] = k < 9 ? fv + 16u * k : kBeyond;
     }
-    const float* const fbase = p.w + (((long)tn * 32 * NB + chan_row) * p.Cin + q4) * 9;  // whole blocks only: in range
-    // the common sequence: filter job, or (NB = 1, patch thread) pixels 0..8
-    const bool common_is_patch = NB == 1 && patches;
-    const float* const cbase = common_is_patch ? p.x : fbase;
-    const int cstep = common_is_patch ? 1 : 9;
-    int coff[9];
-#pragma unroll
-    for (int k = 0; k < 9; ++k) coff[k] = common_is_patch ? poff[k] : 4 * k;
-
-    f32x4 rc[9], rp[16];
-    auto load_raw = [&](int c0) {
-        if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
-        const int cc = c0 * cstep;
-#pragma unroll
-        for (int k = 0; k < 9; ++k) rc[k] = *reinterpret_cast<const f32x4*>(cbase + (coff[k] + cc));
-        if (patches) {
-#pragma unroll
-            for (int k = (NB == 1 ? 9 : 0); k < 16; ++k) rp[k] = *reinterpret_cast<const f32x4*>(p.x + (poff[k] + c0));
-        }
+    // the descriptor has to sit in scalar registers: say so in terms the compiler cannot overlook, or every load
+    // becomes a loop over the distinct descriptors of the wavefront's lanes
+    const unsigned long long base_bits = reinterpret_cast<unsigned long long>(patches ? p.x : p.w);
+    const unsigned base_lo = __builtin_amdgcn_readfirstlane((unsigned)base_bits);
+    const unsigned base_hi = __builtin_amdgcn_readfirstlane((unsigned)(base_bits >> 32));
+    const unsigned extent = __builtin_amdgcn_readfirstlane(patches ? p.xbytes : p.wbytes);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<void*>(((unsigned long long)base_hi << 32) | base_lo), 0, (int)extent, 0x00020000);
+    const int chan_bytes = patches ? 4 : 36;  // from one input channel to the next
+    f32x4 raw[16];
+    auto load_one = [&](int k, int soff) {
+        raw[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off[k], soff, 0));
     };
     auto stage = [&]() {
-        if (NB == 2 || !patches) transform_filter<32 * NB>(rc, Us + chan_row * kKC + swz(chan_row, tid & 3));
-        if (patches) {
-            if (NB == 1) {
-#pragma unroll
-                for (int k = 0; k < 9; ++k) rp[k] = rc[k];
-            }
-            transform_patch(rp, vmask, Vs + tile_row * kKC + swz(tile_row, tid & 3));
-        }
+        if (patches) transform_patch(raw, Vs + row * kKC + swz(row, tid & 3));
+        else transform_filter<32 * NB>(raw, Us + row * kKC + swz(row, tid & 3));
     };
 
-    // per-column constants of the epilogue, asked for now and used at the very end
-    float cs[NB], ct[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) epilogue_column(p.ep, ((long)tn * NB + nb) * 32 + r, cs[nb], ct[nb]);
+    // per-column constants of the epilogue, asked for now and folded at the very end
+    const long n0 = (long)tn * 32 * NB;
+    ColConsts<NB> cc;
+    cols_issue<WinoOutCfg<NB>>(cc, p.ep, p.y, n0, 0, lane, p.Cout);
 
     if (tid < 32) {
-        const long gt = (long)tm * 32 + tid;
+        const unsigned gt = (unsigned)tm * 32u + (unsigned)tid;
         int pix = -1, ok = 0;
-        if (gt < p.ntiles) {
-            const int tw = (int)(gt % p.tiles_w);
-            const long q = gt / p.tiles_w;
-            const int th = (int)(q % p.tiles_h);
-            const long n = q / p.tiles_h;
-            pix = (int)((n * p.H + 2 * th) * p.W + 2 * tw);
+        if (gt < (unsigned)p.ntiles) {
+            const unsigned q = gt / (unsigned)p.tiles_w;
+            const int tw = (int)(gt - q * (unsigned)p.tiles_w);
+            const unsigned n = q / (unsigned)p.tiles_h;
+            const int th = (int)(q - n * (unsigned)p.tiles_h);
+            pix = ((int)n * p.H + 2 * th) * p.W + 2 * tw;
             ok = (2 * th + 1 < p.H ? 1 : 0) | (2 * tw + 1 < p.W ? 2 : 0);
         }
         rowpix[tid] = pix;
@@ -302,9 +351,12 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
     const int vfrag1 = (wave * 4 * 32 + r) * kKC + swz(r, 2 + h);
     const int ufrag0 = (wave * 4 * 32 * NB + r) * kKC + swz(r, h);
     const int ufrag1 = (wave * 4 * 32 * NB + r) * kKC + swz(r, 2 + h);
-    auto multiply = [&]() {
+    auto multiply = [&](int next_soff) {
         // eight (k-group, xi) steps of 1 + NB fragment reads and 4 * NB MFMAs; the fragments of step n+1 are
-        // requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work
+        // requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work.  Each
+        // step also issues two of the next K-block's sixteen loads: issued in one go after the barrier they
+        // held the wavefront for about a thousand cycles in which its SIMD did nothing else (measured with
+        // one workgroup per CU); between MFMAs the matrix pipeline is busy meanwhile.
         f32x4 a[2], b[2][NB];
         a[0] = *reinterpret_cast<const f32x4*>(Vs + vfrag0);
 #pragma unroll
@@ -323,17 +375,23 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
+                for (int s = 0; s < 4; ++s) {
                     acc[j][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][nb][s], acc[j][nb], 0, 0, 0);
+                    if (nb == 0 && s == 0) load_one(2 * n, next_soff);
+                    if (nb == 0 && s == 2) load_one(2 * n + 1, next_soff);
+                }
+            __builtin_amdgcn_sched_barrier(0);  // or the scheduler gathers the sixteen loads at the end again
         }
     };
 
-    load_raw(cbeg);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) load_one(k, cbeg * chan_bytes);
     for (int n = 0; n < nblocks; ++n) {
         stage();
         __syncthreads();
-        load_raw(cbeg + (n + 1) * kKC);  // in flight while this block is multiplied
-        multiply();
+        int c0 = cbeg + (n + 1) * kKC;
+        if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
+        multiply(c0 * chan_bytes);             // the next block's loads are in flight while this one is multiplied
         __syncthreads();
     }
 
@@ -366,11 +424,21 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
     // ---- write-out: row of the block = tile, column = output channel
     const Epilogue& e = p.ep;
     const int pixoff = oa * p.W + ob;
-    const bool relu = e.act == ACT_RELU;
-#pragma unroll
+    if (cc.ok) {
+        cols_fold<WinoOutCfg<NB>>(cc, e);
+        // beyond the exchange area (other wavefronts may still be reading theirs): 1024 floats per wavefront
+        float* const stage_blk = lds + 8 * NB * 1024 + wave * 1024;
+        if (!e.residual) store_rows_any_act<NB, false>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
+        else store_rows_any_act<NB, true>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
+        return;
+    }
+    // odd pitches or unaligned tensors: one element at a time
+#pragma unroll 1
     for (int nb = 0; nb < NB; ++nb) {
-        const long col = ((long)tn * NB + nb) * 32 + r;
-#pragma unroll
+        const long col = n0 + nb * 32 + r;
+        float cs, ct;
+        epilogue_column(e, col, cs, ct);
+#pragma unroll 1
         for (int v = 0; v < 16; ++v) {
             const int row = (v >> 2) * 8 + h * 4 + (v & 3);
             const int pix = rowpix[row];
@@ -378,9 +446,9 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
             if (pix < 0 || (oa && !(ok & 1)) || (ob && !(ok & 2))) continue;
             const long o = (long)(pix + pixoff);
             float xv = out[0][nb][v] * e.alpha;
-            xv = xv * cs[nb] + ct[nb];
+            xv = xv * cs + ct;
             if (e.residual) xv += e.residual[o * e.ldr + col];
-            p.y[o * p.yp + col] = relu ? (xv > 0.f ? xv : 0.f) : apply_act(xv, e.act);
+            p.y[o * p.yp + col] = apply_act(xv, e.act);
         }
     }
 }
@@ -405,7 +473,8 @@ int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t 
     const double min_gflop = min_env ? atof(min_env) : 0.8;
     if (2.0 * a.N * a.H * a.W * (double)a.Cout * a.Cin * 9.0 < min_gflop * 1e9) return K_EUNSUPPORTED;
     const long pixels = (long)a.N * a.H * a.W;
-    if (pixels * xp >= (1L << 31) || pixels >= (1L << 31)) return K_EUNSUPPORTED;  // offsets are 32-bit in the kernel
+    // byte offsets are 32-bit in the kernel and 2^31 marks "beyond the tensor"
+    if (pixels * xp >= (1L << 29) || pixels * yp >= (1L << 31) || (long)a.Cout * a.Cin * 36 >= (1L << 31)) return K_EUNSUPPORTED;
 
     WinoDev p;
     p.x = a.x;
@@ -417,6 +486,8 @@ int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t 
     p.Cout = a.Cout;
     p.xp = xp;
     p.yp = yp;
+    p.xbytes = (unsigned)(((pixels - 1) * xp + a.Cin) * 4);
+    p.wbytes = (unsigned)((long)a.Cout * a.Cin * 36);
     p.tiles_h = (a.H + 1) / 2;
     p.tiles_w = (a.W + 1) / 2;
     p.ntiles = (long)a.N * p.tiles_h * p.tiles_w;
