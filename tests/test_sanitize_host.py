@@ -25,7 +25,7 @@ def test_wire_handlers_and_engine_under_sanitizers(tmp_path):
         subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", os.path.join(csrc, src), "-o", o],
                               stderr=subprocess.DEVNULL)
         objs.append(o)
-    for k in ("gemm", "conv", "ops", "attention"):
+    for k in ("gemm", "conv", "winograd", "ops", "attention"):
         o = os.path.join(ROOT, "build", "obj", "kernels", k + ".hip.o")
         if not os.path.exists(o):
             pytest.skip("kernel objects not built (run make -C torpor_amd/csrc)")
@@ -52,7 +52,7 @@ def test_c_abi_from_three_threads_under_thread_sanitizer(tmp_path):
     flags = ["--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
              "-packed-fp32-ops"] + san
     objs = []
-    for k in ("gemm", "conv", "ops", "attention"):
+    for k in ("gemm", "conv", "winograd", "ops", "attention"):
         o = os.path.join(ROOT, "build", "obj", "kernels", k + ".hip.o")
         if not os.path.exists(o):
             pytest.skip("kernel objects not built (run make -C torpor_amd/csrc)")

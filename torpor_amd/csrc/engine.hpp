@@ -172,6 +172,11 @@ struct Model {
     int ncopy = 2;            // copy streams used by the current swap-in plan
     uint64_t chunk_max = 0;   // largest transfer group of the current plan
     double warm_us = 0;       // best warm replay so far (host wall clock), 0 = none yet
+    // Cold requests seen under each copy plan (index = number of copy streams): the shortest time from the start
+    // of a swap-in to the end of the request that ran beside it, and how many there were (choose_copy_plan).
+    double cold_us[3] = {0, 0, 0};
+    int cold_n[3] = {0, 0, 0};
+    std::chrono::steady_clock::time_point swap_t0;
     // captured compute segment of the recorded program (warm replays at an unchanged placement)
     hipGraphExec_t graph_exec = nullptr;
     int graph_begin = -1, graph_end = -1;  // program[graph_begin, graph_end) is what the graph launches
@@ -357,6 +362,7 @@ private:
     static constexpr double kNominalLinkGbps = 56.0;  // until measured (an engine without a device keeps it)
     static constexpr double kCopyFixedUs = 15.0;      // fixed cost of one hipMemcpyAsync on a copy stream
     bool chunk_max_auto_ = true;
+    int plan_trials_ = 2;  // cold requests per copy plan before the measured choice is made (TORPOR_PLAN_TRIALS; 0 = estimate only)
     bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor
     int d2h_kernel_ = 0;
     bool host_gather_ = true;  // lookups may read a table in place from the host store during a swap-in
