@@ -340,3 +340,29 @@ def test_device_image_equals_host_image_wherever_it_lands():
                     assert np.array_equal(g, w)
                 assert np.array_equal(s.readback_weights(fn.fid), s.host_weights(fn.fid)), (turn, fn.fid)
         assert s.pool_stats()["evictions"] >= 4
+
+
+@pytest.mark.parametrize("trials", [0, 1, 2])
+def test_copy_plan_settles_after_its_trial_requests_and_never_changes_an_answer(trials, monkeypatch):
+    """The number of copy streams of a swap-in may follow the model's own cold requests (the first `trials`
+    under the estimated plan, the next `trials` under the other one when the two estimates are close, then the
+    better of the two for good).  Whatever it does, every cold answer has the registration run's bits, the
+    weights land byte for byte, and the plan is the same for every swap-in after the trial requests."""
+    monkeypatch.setenv("TORPOR_PLAN_TRIALS", str(trials))
+    with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
+        fn, x, y = _mk(s, 5, seed=11, image=160)
+        plans, groups = [], []
+        for i in range(9):
+            assert fn.unload()[0] == ACK_OK and not s.resident(5)
+            (got,) = fn.invoke([x])
+            assert np.array_equal(got, y), f"cold request {i} changed the answer"
+            s.stream_synchronize(5)
+            st = s.swap_stats(5)
+            assert st["copy_streams"] in (1, 2) and st["chunks"] == s.model_info(5)["n_chunks"]
+            plans.append(st["copy_streams"])
+            groups.append(st["chunks"])
+            assert np.array_equal(s.readback_weights(5), s.host_weights(5))
+        settled = plans[2 * trials:]
+        assert len(set(settled)) == 1, f"plan still changing after the trial requests: {plans}"
+        if trials == 0:
+            assert len(set(plans)) == 1 and len(set(groups)) == 1, "without trials the estimate alone decides"
