@@ -39,6 +39,10 @@ namespace {
 
 constexpr int kKC = 16;                        // input channels per K-block
 constexpr int kOperandFloats = 16 * 32 * kKC;  // V (or U of 32 output channels) of one K-block: [xi][row][channel]
+// Blocks of 32 output channels per workgroup.  The multiply, exchange and write-out code is written for any count;
+// the fetch and transform jobs of the kernel and the launcher's grid are laid out for one (two was measured
+// slower, see the launcher).
+constexpr int kNB = 1;
 
 struct WinoDev {
     const float* x;
@@ -49,18 +53,17 @@ struct WinoDev {
     unsigned xbytes, wbytes;  // extent of x and of w in bytes (both below 2^31)
     int tiles_h, tiles_w;  // 2x2 output tiles per image
     long ntiles;           // N * tiles_h * tiles_w
-    int mt, nt;            // blocks of 32 tiles / of 32*NB output channels
+    int mt, nt;            // blocks of 32 tiles / of 32 output channels
     int splits, cper;      // input-channel slices and channels per slice (a multiple of kKC)
     float* ws;
     unsigned* tickets;
     Epilogue ep;
 };
 
-// what finish_split needs to know: four wavefronts with NB 32x32 accumulator blocks each
-template <int NB>
+// what finish_split and the write-out need to know: four wavefronts with kNB 32x32 accumulator blocks each
 struct WinoOutCfg {
-    static constexpr int TM = 1, TN = NB, WGM = 2, WGN = 2;
-    static constexpr int WTM = 32, WTN = 32 * NB;  // one wavefront's block of the output tile
+    static constexpr int TM = 1, TN = kNB, WGM = 2, WGN = 2;
+    static constexpr int WTN = 32 * kNB;  // columns of one wavefront's block of the output tile
 };
 
 __device__ __forceinline__ void fetch_args(const WinoDev& p) {
@@ -97,13 +100,15 @@ __device__ __forceinline__ int remap_xcd_w(int bid, int n) {
 // even ones on banks 0-15 and four odd ones on banks 16-31, and rows two apart get different chunks.
 __device__ __forceinline__ int swz(int row, int chunk) { return (chunk ^ ((row >> 1) & 3)) << 2; }
 
-// V = B^T d B of one 4x4 patch, four channels at a time, in place: first down the rows of every column, then
-// along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time); d[4i + j] = pixel (i, j), zeros
-// where the patch reaches into the padding.  dst = this thread's chunk of row `tile` in block xi = 0.
-__device__ __forceinline__ void transform_patch(f32x4 (&d)[16], float* __restrict__ dst) {
+// V = B^T d B of one 4x4 patch, for the two or four channels of a vector at a time, in place: first down the
+// rows of every column, then along the columns of every row (d0 - d2, d1 + d2, d2 - d1, d1 - d3 each time);
+// d[4i + j] = pixel (i, j), zeros where the patch reaches into the padding.  dst = this thread's channels of row
+// `tile` in block xi = 0.
+template <class V>
+__device__ __forceinline__ void transform_patch(V (&d)[16], float* __restrict__ dst) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const f32x4 d1 = d[1 * 4 + j];
+        const V d1 = d[1 * 4 + j];
         d[0 * 4 + j] -= d[2 * 4 + j];
         d[1 * 4 + j] = d1 + d[2 * 4 + j];
         d[2 * 4 + j] -= d1;
@@ -111,22 +116,22 @@ __device__ __forceinline__ void transform_patch(f32x4 (&d)[16], float* __restric
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const f32x4 d1 = d[i * 4 + 1];
-        const f32x4 v0 = d[i * 4 + 0] - d[i * 4 + 2];
-        const f32x4 v1 = d1 + d[i * 4 + 2];
-        const f32x4 v2 = d[i * 4 + 2] - d1;
-        const f32x4 v3 = d1 - d[i * 4 + 3];
-        *reinterpret_cast<f32x4*>(dst + (i * 4 + 0) * 32 * kKC) = v0;
-        *reinterpret_cast<f32x4*>(dst + (i * 4 + 1) * 32 * kKC) = v1;
-        *reinterpret_cast<f32x4*>(dst + (i * 4 + 2) * 32 * kKC) = v2;
-        *reinterpret_cast<f32x4*>(dst + (i * 4 + 3) * 32 * kKC) = v3;
+        const V d1 = d[i * 4 + 1];
+        const V v0 = d[i * 4 + 0] - d[i * 4 + 2];
+        const V v1 = d1 + d[i * 4 + 2];
+        const V v2 = d[i * 4 + 2] - d1;
+        const V v3 = d1 - d[i * 4 + 3];
+        *reinterpret_cast<V*>(dst + (i * 4 + 0) * 32 * kKC) = v0;
+        *reinterpret_cast<V*>(dst + (i * 4 + 1) * 32 * kKC) = v1;
+        *reinterpret_cast<V*>(dst + (i * 4 + 2) * 32 * kKC) = v2;
+        *reinterpret_cast<V*>(dst + (i * 4 + 3) * 32 * kKC) = v3;
     }
 }
 
 // U = G g G^T for four input channels of one output channel; raw[0..8] = the 36 floats g[ci][kh][kw].
 // dst = this thread's chunk of row `channel` in block xi = 0 of a [xi][ROWS][16] operand.
-template <int ROWS>
-__device__ __forceinline__ void transform_filter(const f32x4 (&raw)[16], float* __restrict__ dst) {
+template <int ROWS, int NRAW>
+__device__ __forceinline__ void transform_filter(const f32x4 (&raw)[NRAW], float* __restrict__ dst) {
     float a[4][4][3];  // [ci][i][kw] = (G g) of channel ci
 #pragma unroll
     for (int ci = 0; ci < 4; ++ci) {
@@ -161,16 +166,16 @@ __device__ __forceinline__ void transform_filter(const f32x4 (&raw)[16], float* 
     }
 }
 
-// Write-out of one wavefront's NB 32x32 blocks (rows = tiles, columns = output channels) for its output pixel
+// Write-out of one wavefront's kNB 32x32 blocks (rows = tiles, columns = output channels) for its output pixel
 // (oa, ob) of every tile, in the form the GEMM tiles use: each block goes through the wavefront's LDS staging
 // block and comes back as four consecutive columns per lane, so one step writes eight rows with 128-bit stores.
 // Straight-line code with the activation fixed at compile time: a load under a branch (the residual, say) makes
 // the compiler wait for every outstanding memory operation at the join, the stores of the previous step included
 // -- the element-wise form of this write-out took 3.4 us of a 24 us launch that way.
-template <int NB, bool RES, int ACT>
-__device__ __forceinline__ void store_rows(f32x16 (&out)[1][NB], int lane, long n0, const WinoDev& p, int pixoff, int oa,
+template <bool RES, int ACT>
+__device__ __forceinline__ void store_rows(f32x16 (&out)[1][kNB], int lane, long n0, const WinoDev& p, int pixoff, int oa,
                                            int ob, float* __restrict__ stage_blk, const int* rowpix, const int* rowok,
-                                           const ColConsts<NB>& cc) {
+                                           const ColConsts<kNB>& cc) {
     const Epilogue& e = p.ep;
     const int r = lane & 31, h = lane >> 5;
     const int cq = (lane & 7) * 4;  // this lane's four columns within a block
@@ -185,7 +190,7 @@ __device__ __forceinline__ void store_rows(f32x16 (&out)[1][NB], int lane, long 
         o[it] = live[it] ? (long)(pix + pixoff) : 0;  // rows that are not written read the residual of pixel 0
     }
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
         const long col = n0 + nb * 32 + cq;
 #pragma unroll
         for (int v = 0; v < 16; ++v) stage_blk[((v >> 2) * 8 + h * 4 + (v & 3)) * 32 + r] = out[0][nb][v];
@@ -211,117 +216,63 @@ __device__ __forceinline__ void store_rows(f32x16 (&out)[1][NB], int lane, long 
     }
 }
 
-template <int NB, bool RES>
-__device__ __forceinline__ void store_rows_any_act(f32x16 (&out)[1][NB], int lane, long n0, const WinoDev& p, int pixoff,
+template <bool RES>
+__device__ __forceinline__ void store_rows_any_act(f32x16 (&out)[1][kNB], int lane, long n0, const WinoDev& p, int pixoff,
                                                    int oa, int ob, float* __restrict__ stage_blk, const int* rowpix,
-                                                   const int* rowok, const ColConsts<NB>& cc) {
+                                                   const int* rowok, const ColConsts<kNB>& cc) {
     switch (p.ep.act) {
-        case ACT_RELU: store_rows<NB, RES, ACT_RELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        case ACT_GELU: store_rows<NB, RES, ACT_GELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        case ACT_TANH: store_rows<NB, RES, ACT_TANH>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        case ACT_RELU6: store_rows<NB, RES, ACT_RELU6>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        case ACT_SILU: store_rows<NB, RES, ACT_SILU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        case ACT_SIGMOID: store_rows<NB, RES, ACT_SIGMOID>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
-        default: store_rows<NB, RES, ACT_NONE>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_RELU: store_rows<RES, ACT_RELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_GELU: store_rows<RES, ACT_GELU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_TANH: store_rows<RES, ACT_TANH>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_RELU6: store_rows<RES, ACT_RELU6>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_SILU: store_rows<RES, ACT_SILU>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        case ACT_SIGMOID: store_rows<RES, ACT_SIGMOID>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
+        default: store_rows<RES, ACT_NONE>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc); break;
     }
 }
 
-// Four wavefronts; all of them multiply: wavefront w owns the accumulators of row i = w of the 4x4
-// (xi = 4w .. 4w+3) for NB blocks of 32 output channels.  Before that, per K-block, the patches and filters
-// are fetched and transformed; the loads of the next K-block are in flight while this one is multiplied.
-//   NB = 1: 32 tiles x 32 channels.  Wavefronts 0-1 take the patches, 2-3 the filters; 64 KiB of LDS, two
-//           workgroups per CU.
-//   NB = 2: 32 tiles x 64 channels.  Every thread takes a filter job, wavefronts 0-1 a patch job as well;
-//           96 KiB of LDS, one workgroup per CU.  A patch transform now serves twice the matrix work.
-// Measured on MI355X, 8x14x14x256 -> 256, NB = 1: per K-block a wavefront spends about 2000 cycles on the
-// transform's vector instructions and 2050 on its 32 MFMAs, and the two do not overlap on a SIMD -- not
-// within a wavefront, not between two workgroups on the CU, and not when the transforms are given to
-// wavefronts of their own (built and measured: same time), because a SIMD issues either kind from one
-// port.  That bounds this path well below the 2.25x of the multiplication count, and is why the transforms are
-// spread over as much matrix work as the registers allow.
-template <int NB>
-__global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const WinoDev p) {
-    fetch_args(p);
-    __shared__ __attribute__((aligned(16))) float lds[(1 + NB) * kOperandFloats];  // [V | U (NB blocks)] of one K-block
-    __shared__ int rowpix[32];  // (n*H + 2*th)*W + 2*tw of each tile of this block, -1 past the last tile
-    __shared__ int rowok[32];   // bit 0: the tile's second output row exists, bit 1: its second column
-    __shared__ unsigned flag;
-    float* const Vs = lds;
-    float* const Us = lds + kOperandFloats;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wavefront: role branches are scalar
-    const int r = lane & 31, h = lane >> 5;
-    const int t = remap_xcd_w((int)blockIdx.x, p.mt * p.nt);
-    const int tm = t / p.nt, tn = t - tm * p.nt;
-    const int split = (int)blockIdx.z;
-    const int cbeg = split * p.cper;
-    const int cend = cbeg + p.cper < p.Cin ? cbeg + p.cper : p.Cin;
-    const int nblocks = (cend - cbeg) / kKC;
+constexpr unsigned kBeyond = 0x80000000u;  // a byte offset no tensor of this path reaches: such a load returns zeros
 
-    // ---- what this thread fetches and transforms per K-block
-    // Wavefronts 0-1: the 4x4 patch of tile `row` for four input channels, pixel (i, j) = load 4i + j.
-    // Wavefronts 2-3: the filter of output channel `row` for four input channels, 36 contiguous floats = loads 0..8.
-    // All of them are buffer loads of 16 bytes: one descriptor per wavefront (x or w), a per-lane byte offset that
-    // never changes, and the K-block's offset in a scalar register -- no address arithmetic in the loop.  A load
-    // whose offset lies beyond the descriptor's extent returns zeros without touching memory: that is how the
-    // padding around the image, the tiles past the last one and a filter thread's loads 9..15 are expressed, so
-    // that every thread issues the same sixteen loads and none of them sits under a branch.
-    static_assert(NB == 1, "the fetch and transform jobs below are laid out for 32 output channels per workgroup");
-    const bool patches = wave < 2;
-    const int q4 = (tid & 3) * 4;          // channel quad within the K-block
-    const int row = (tid & 127) >> 2;      // tile / output channel within the block
-    constexpr unsigned kBeyond = 0x80000000u;
-    unsigned off[16];
-    if (patches) {
-        // 32-bit arithmetic throughout (the launcher checks that every offset fits): a 64-bit division costs
-        // some hundred instructions and this is on every workgroup's way to its first load
-        const unsigned gt = (unsigned)tm * 32u + (unsigned)row;
-        const bool real = gt < (unsigned)p.ntiles;
-        const unsigned q = gt / (unsigned)p.tiles_w;
-        const int tw = (int)(gt - q * (unsigned)p.tiles_w);
-        const unsigned n = q / (unsigned)p.tiles_h;
-        const int th = (int)(q - n * (unsigned)p.tiles_h);
-        const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
-        const int xp = (int)p.xp;
+// A buffer descriptor that sits in scalar registers: say so in terms the compiler cannot overlook, or every
+// load becomes a loop over the distinct descriptors of the wavefront's lanes.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const float* base, unsigned bytes) {
+    const unsigned long long bits = reinterpret_cast<unsigned long long>(base);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)bits);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(bits >> 32));
+    const unsigned extent = __builtin_amdgcn_readfirstlane(bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo), 0, (int)extent,
+                                             0x00020000);
+}
+
+// Byte offsets of the sixteen pixels of tile `tile_in_block`'s 4x4 input patch, pixel (i, j) = entry 4i + j, for
+// the channels that start `chan` floats into the pixel; kBeyond where the patch reaches into the padding and
+// for tiles past the last one.  32-bit arithmetic throughout (the launcher checks that every offset fits): a
+// 64-bit division costs some hundred instructions and this is on every workgroup's way to its first load.
+__device__ __forceinline__ void patch_offsets(const WinoDev& p, int tm, int tile_in_block, int chan, unsigned (&off)[16]) {
+    const unsigned gt = (unsigned)tm * 32u + (unsigned)tile_in_block;
+    const bool real = gt < (unsigned)p.ntiles;
+    const unsigned q = gt / (unsigned)p.tiles_w;
+    const int tw = (int)(gt - q * (unsigned)p.tiles_w);
+    const unsigned n = q / (unsigned)p.tiles_h;
+    const int th = (int)(q - n * (unsigned)p.tiles_h);
+    const int hi0 = 2 * th - 1, wi0 = 2 * tw - 1;
+    const int xp = (int)p.xp;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int hi = hi0 + i;
-            const int rowoff = (((int)n * p.H + hi) * p.W) * xp + q4;
+    for (int i = 0; i < 4; ++i) {
+        const int hi = hi0 + i;
+        const int rowoff = (((int)n * p.H + hi) * p.W) * xp + chan;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int wi = wi0 + j;
-                const bool inside = real && hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
-                off[i * 4 + j] = inside ? (unsigned)(rowoff + wi * xp) * 4u : kBeyond;
-            }
+        for (int j = 0; j < 4; ++j) {
+            const int wi = wi0 + j;
+            const bool inside = real && hi >= 0 && hi < p.H && wi >= 0 && wi < p.W;
+            off[i * 4 + j] = inside ? (unsigned)(rowoff + wi * xp) * 4u : kBeyond;
         }
-    } else {
-        const unsigned fv = (unsigned)((tn * 32 + row) * p.Cin + q4) * 36u;  // whole blocks only: in range
-#pragma unroll
-        for (int k = 0; k < 16; ++k) off[k] = k < 9 ? fv + 16u * k : kBeyond;
     }
-    // the descriptor has to sit in scalar registers: say so in terms the compiler cannot overlook, or every load
-    // becomes a loop over the distinct descriptors of the wavefront's lanes
-    const unsigned long long base_bits = reinterpret_cast<unsigned long long>(patches ? p.x : p.w);
-    const unsigned base_lo = __builtin_amdgcn_readfirstlane((unsigned)base_bits);
-    const unsigned base_hi = __builtin_amdgcn_readfirstlane((unsigned)(base_bits >> 32));
-    const unsigned extent = __builtin_amdgcn_readfirstlane(patches ? p.xbytes : p.wbytes);
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        reinterpret_cast<void*>(((unsigned long long)base_hi << 32) | base_lo), 0, (int)extent, 0x00020000);
-    const int chan_bytes = patches ? 4 : 36;  // from one input channel to the next
-    f32x4 raw[16];
-    auto load_one = [&](int k, int soff) {
-        raw[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off[k], soff, 0));
-    };
-    auto stage = [&]() {
-        if (patches) transform_patch(raw, Vs + row * kKC + swz(row, tid & 3));
-        else transform_filter<32 * NB>(raw, Us + row * kKC + swz(row, tid & 3));
-    };
+}
 
-    // per-column constants of the epilogue, asked for now and folded at the very end
-    const long n0 = (long)tn * 32 * NB;
-    ColConsts<NB> cc;
-    cols_issue<WinoOutCfg<NB>>(cc, p.ep, p.y, n0, 0, lane, p.Cout);
-
+// Where each tile of the block writes: (n*H + 2*th)*W + 2*tw, -1 past the last tile; bit 0 of rowok: the tile's
+// second output row exists, bit 1: its second column.
+__device__ __forceinline__ void tile_rows(const WinoDev& p, int tm, int tid, int* rowpix, int* rowok) {
     if (tid < 32) {
         const unsigned gt = (unsigned)tm * 32u + (unsigned)tid;
         int pix = -1, ok = 0;
@@ -336,105 +287,95 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
         rowpix[tid] = pix;
         rowok[tid] = ok;
     }
+}
 
-    f32x16 acc[4][NB];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][nb][v] = 0.f;
-
-    // fragment addresses of this lane: xi = 4*wave + j, row r, k-group g -> chunk 2g + h; the rows of output
-    // channel block nb follow 32 rows further on within the same xi (a U block is [xi][32*NB rows][16])
+// One K-block of the sixteen products: wavefront `wave` owns xi = 4*wave + j, j = 0..3, for kNB blocks of 32
+// output channels.  Eight (k-group, xi) steps of 1 + kNB fragment reads and 4 * kNB MFMAs; the fragments of step
+// n+1 are requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work.  Each
+// step also calls prefetch(n), which issues that step's share of the next K-block's global loads: issued in one
+// go after the barrier they held the wavefront for about a thousand cycles in which its SIMD did nothing else
+// (measured with one workgroup per CU); between MFMAs the matrix pipeline is busy meanwhile.
+// V is [xi][32 rows][16 channels], U is [xi][32*kNB rows][16 channels]; lane (r, h) reads row r, chunk 2g + h.
+template <class Prefetch>
+__device__ __forceinline__ void multiply_block(f32x16 (&acc)[4][kNB], const float* Vs, const float* Us, int wave, int r,
+                                               int h, Prefetch prefetch) {
     const int vfrag0 = (wave * 4 * 32 + r) * kKC + swz(r, h);
     const int vfrag1 = (wave * 4 * 32 + r) * kKC + swz(r, 2 + h);
-    const int ufrag0 = (wave * 4 * 32 * NB + r) * kKC + swz(r, h);
-    const int ufrag1 = (wave * 4 * 32 * NB + r) * kKC + swz(r, 2 + h);
-    auto multiply = [&](int next_soff) {
-        // eight (k-group, xi) steps of 1 + NB fragment reads and 4 * NB MFMAs; the fragments of step n+1 are
-        // requested before the MFMAs of step n are issued, so the LDS latency hides behind matrix work.  Each
-        // step also issues two of the next K-block's sixteen loads: issued in one go after the barrier they
-        // held the wavefront for about a thousand cycles in which its SIMD did nothing else (measured with
-        // one workgroup per CU); between MFMAs the matrix pipeline is busy meanwhile.
-        f32x4 a[2], b[2][NB];
-        a[0] = *reinterpret_cast<const f32x4*>(Vs + vfrag0);
+    const int ufrag0 = (wave * 4 * 32 * kNB + r) * kKC + swz(r, h);
+    const int ufrag1 = (wave * 4 * 32 * kNB + r) * kKC + swz(r, 2 + h);
+    f32x4 a[2], b[2][kNB];
+    a[0] = *reinterpret_cast<const f32x4*>(Vs + vfrag0);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) b[0][nb] = *reinterpret_cast<const f32x4*>(Us + ufrag0 + nb * 32 * kKC);
+    for (int nb = 0; nb < kNB; ++nb) b[0][nb] = *reinterpret_cast<const f32x4*>(Us + ufrag0 + nb * 32 * kKC);
 #pragma unroll
-        for (int n = 0; n < 8; ++n) {
-            const int cur = n & 1, nxt = cur ^ 1;
-            if (n + 1 < 8) {
-                const int g = (n + 1) >> 2, j = (n + 1) & 3;
-                a[nxt] = *reinterpret_cast<const f32x4*>(Vs + (g ? vfrag1 : vfrag0) + j * 32 * kKC);
+    for (int n = 0; n < 8; ++n) {
+        const int cur = n & 1, nxt = cur ^ 1;
+        if (n + 1 < 8) {
+            const int g = (n + 1) >> 2, j = (n + 1) & 3;
+            a[nxt] = *reinterpret_cast<const f32x4*>(Vs + (g ? vfrag1 : vfrag0) + j * 32 * kKC);
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                    b[nxt][nb] = *reinterpret_cast<const f32x4*>(Us + (g ? ufrag1 : ufrag0) + (j * NB + nb) * 32 * kKC);
-            }
-            const int j = n & 3;
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    acc[j][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][nb][s], acc[j][nb], 0, 0, 0);
-                    if (nb == 0 && s == 0) load_one(2 * n, next_soff);
-                    if (nb == 0 && s == 2) load_one(2 * n + 1, next_soff);
-                }
-            __builtin_amdgcn_sched_barrier(0);  // or the scheduler gathers the sixteen loads at the end again
+            for (int nb = 0; nb < kNB; ++nb)
+                b[nxt][nb] = *reinterpret_cast<const f32x4*>(Us + (g ? ufrag1 : ufrag0) + (j * kNB + nb) * 32 * kKC);
         }
-    };
-
+        const int j = n & 3;
+        acc[j][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][0], b[cur][0][0], acc[j][0], 0, 0, 0);
+        prefetch(n);
 #pragma unroll
-    for (int k = 0; k < 16; ++k) load_one(k, cbeg * chan_bytes);
-    for (int n = 0; n < nblocks; ++n) {
-        stage();
-        __syncthreads();
-        int c0 = cbeg + (n + 1) * kKC;
-        if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
-        multiply(c0 * chan_bytes);             // the next block's loads are in flight while this one is multiplied
-        __syncthreads();
+        for (int nb = 0; nb < kNB; ++nb)
+#pragma unroll
+            for (int s = (nb == 0 ? 1 : 0); s < 4; ++s)
+                acc[j][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][s], b[cur][nb][s], acc[j][nb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);  // or the scheduler gathers the loads at the end of the block again
     }
+}
 
-    // ---- output transform.  This wavefront holds row i = wave of M; fold it over j ...
-    float* ex = lds;  // [((i*2 + b)*NB + nb)*16 + v][lane]; the operand blocks are no longer read (barrier above)
+// After the K loop: output transform, sum over the input-channel slices, write-out.  The wavefront holds row
+// i = wave of M; it folds the row over j, the four rows are exchanged through LDS (the operand blocks are no
+// longer read: the caller's last barrier), and wavefront (oa, ob) ends up with output pixel (oa, ob) of every
+// tile.  Returns early in every workgroup but the one that finishes a split tile last.
+__device__ __forceinline__ void transform_and_store(f32x16 (&acc)[4][kNB], const WinoDev& p, float* lds, const int* rowpix,
+                                                    const int* rowok, unsigned* flag, int wave, int lane, int t, int split,
+                                                    int tn, ColConsts<kNB>& cc) {
+    const int r = lane & 31, h = lane >> 5;
+    float* ex = lds;  // [((i*2 + b)*kNB + nb)*16 + v][lane]
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            ex[(((wave * 2 + 0) * NB + nb) * 16 + v) * 64 + lane] = (acc[0][nb][v] + acc[1][nb][v]) + acc[2][nb][v];
-            ex[(((wave * 2 + 1) * NB + nb) * 16 + v) * 64 + lane] = (acc[1][nb][v] - acc[2][nb][v]) - acc[3][nb][v];
+            ex[(((wave * 2 + 0) * kNB + nb) * 16 + v) * 64 + lane] = (acc[0][nb][v] + acc[1][nb][v]) + acc[2][nb][v];
+            ex[(((wave * 2 + 1) * kNB + nb) * 16 + v) * 64 + lane] = (acc[1][nb][v] - acc[2][nb][v]) - acc[3][nb][v];
         }
     __syncthreads();
-    // ... and combine the rows: wavefront (oa, ob) takes output pixel (oa, ob) of every tile
     const int oa = wave >> 1, ob = wave & 1;
-    f32x16 out[1][NB];
+    f32x16 out[1][kNB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const float t1 = ex[(((1 * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
-            const float t2 = ex[(((2 * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
-            const float t03 = ex[((((oa ? 3 : 0) * 2 + ob) * NB + nb) * 16 + v) * 64 + lane];
+            const float t1 = ex[(((1 * 2 + ob) * kNB + nb) * 16 + v) * 64 + lane];
+            const float t2 = ex[(((2 * 2 + ob) * kNB + nb) * 16 + v) * 64 + lane];
+            const float t03 = ex[((((oa ? 3 : 0) * 2 + ob) * kNB + nb) * 16 + v) * 64 + lane];
             out[0][nb][v] = oa ? (t1 - t2) - t03 : (t03 + t1) + t2;
         }
     if (p.splits > 1) {
-        if (!finish_split<WinoOutCfg<NB>>(out, p.ws, p.tickets, p.splits, t, split, wave, lane, &flag)) return;
+        if (!finish_split<WinoOutCfg>(out, p.ws, p.tickets, p.splits, t, split, wave, lane, flag)) return;
     }
 
-    // ---- write-out: row of the block = tile, column = output channel
+    // write-out: row of the block = tile, column = output channel
     const Epilogue& e = p.ep;
+    const long n0 = (long)tn * 32 * kNB;
     const int pixoff = oa * p.W + ob;
     if (cc.ok) {
-        cols_fold<WinoOutCfg<NB>>(cc, e);
+        cols_fold<WinoOutCfg>(cc, e);
         // beyond the exchange area (other wavefronts may still be reading theirs): 1024 floats per wavefront
-        float* const stage_blk = lds + 8 * NB * 1024 + wave * 1024;
-        if (!e.residual) store_rows_any_act<NB, false>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
-        else store_rows_any_act<NB, true>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
+        float* const stage_blk = lds + 8 * kNB * 1024 + wave * 1024;
+        if (!e.residual) store_rows_any_act<false>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
+        else store_rows_any_act<true>(out, lane, n0, p, pixoff, oa, ob, stage_blk, rowpix, rowok, cc);
         return;
     }
     // odd pitches or unaligned tensors: one element at a time
 #pragma unroll 1
-    for (int nb = 0; nb < NB; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
         const long col = n0 + nb * 32 + r;
         float cs, ct;
         epilogue_column(e, col, cs, ct);
@@ -451,6 +392,85 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void conv_wino_kernel(const W
             p.y[o * p.yp + col] = apply_act(xv, e.act);
         }
     }
+}
+
+// 32 tiles x 32 output channels per workgroup, 64 KiB of LDS, two workgroups per CU.  Four wavefronts; all of
+// them multiply (multiply_block).  Before that, per K-block, wavefronts 0-1 fetch and transform the 4x4 patch
+// of tile `row` for four input channels (pixel (i, j) = load 4i + j) and wavefronts 2-3 the filter of output
+// channel `row` for four input channels (36 contiguous floats = loads 0..8); the loads of the next K-block are
+// in flight while this one is multiplied.  All loads are buffer loads of 16 bytes: one descriptor per wavefront
+// (x or w), a per-lane byte offset that never changes, and the K-block's offset in a scalar register -- no
+// address arithmetic in the loop.  A load whose offset lies beyond the descriptor's extent returns zeros without
+// touching memory: that is how the padding around the image, the tiles past the last one and a filter thread's
+// loads 9..15 are expressed, so that every thread issues the same sixteen loads and none of them sits under a
+// branch (two role branches that each end in a load get their tails merged by the compiler through a pointer in
+// scratch memory, and a scratch access in the loop turns every wait into a wait for all loads in flight).
+// Measured on MI355X: fp32 MFMAs and fp32 vector instructions share the SIMD's lanes -- n independent v_add_f32
+// between two dependent MFMAs add 4.6 cycles each to the 64 of the MFMA, whatever n -- so a SIMD's time per
+// K-block is its 2048 MFMA cycles plus its transform job, and wavefronts of their own for the transforms
+// (built and measured) change nothing.
+__global__ __launch_bounds__(256, 2) void conv_wino_kernel(const WinoDev p) {
+    fetch_args(p);
+    __shared__ __attribute__((aligned(16))) float lds[2 * kOperandFloats];  // [V | U] of one K-block
+    __shared__ int rowpix[32];
+    __shared__ int rowok[32];
+    __shared__ unsigned flag;
+    float* const Vs = lds;
+    float* const Us = lds + kOperandFloats;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wavefront: role branches are scalar
+    const int t = remap_xcd_w((int)blockIdx.x, p.mt * p.nt);
+    const int tm = t / p.nt, tn = t - tm * p.nt;
+    const int split = (int)blockIdx.z;
+    const int cbeg = split * p.cper;
+    const int cend = cbeg + p.cper < p.Cin ? cbeg + p.cper : p.Cin;
+    const int nblocks = (cend - cbeg) / kKC;
+
+    const bool patches = wave < 2;
+    const int q4 = (tid & 3) * 4;      // channel quad within the K-block
+    const int row = (tid & 127) >> 2;  // tile / output channel within the block
+    unsigned off[16];
+    if (patches) {
+        patch_offsets(p, tm, row, q4, off);
+    } else {
+        const unsigned fv = (unsigned)((tn * 32 + row) * p.Cin + q4) * 36u;  // whole blocks only: in range
+#pragma unroll
+        for (int k = 0; k < 16; ++k) off[k] = k < 9 ? fv + 16u * k : kBeyond;
+    }
+    const __amdgpu_buffer_rsrc_t rsrc = uniform_rsrc(patches ? p.x : p.w, patches ? p.xbytes : p.wbytes);
+    const int chan_bytes = patches ? 4 : 36;  // from one input channel to the next
+    f32x4 raw[16];
+    auto load_one = [&](int k, int soff) {
+        raw[k] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off[k], soff, 0));
+    };
+
+    // per-column constants of the epilogue, asked for now and folded at the very end
+    ColConsts<kNB> cc;
+    cols_issue<WinoOutCfg>(cc, p.ep, p.y, (long)tn * 32, 0, lane, p.Cout);
+    tile_rows(p, tm, tid, rowpix, rowok);
+
+    f32x16 acc[4][1];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][0][v] = 0.f;
+
+#pragma unroll
+    for (int k = 0; k < 16; ++k) load_one(k, cbeg * chan_bytes);
+    for (int n = 0; n < nblocks; ++n) {
+        if (patches) transform_patch(raw, Vs + row * kKC + swz(row, tid & 3));
+        else transform_filter<32>(raw, Us + row * kKC + swz(row, tid & 3));
+        __syncthreads();
+        int c0 = cbeg + (n + 1) * kKC;
+        if (c0 > cend - kKC) c0 = cend - kKC;  // the look-ahead past the end reads the last block again
+        const int soff = c0 * chan_bytes;
+        multiply_block(acc, Vs, Us, wave, lane & 31, lane >> 5, [&](int step) {
+            load_one(2 * step, soff);
+            load_one(2 * step + 1, soff);
+        });
+        __syncthreads();
+    }
+    transform_and_store(acc, p, lds, rowpix, rowok, &flag, wave, lane, t, split, tn, cc);
 }
 
 inline bool aligned16w(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
@@ -492,18 +512,23 @@ int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t 
     p.tiles_w = (a.W + 1) / 2;
     p.ntiles = (long)a.N * p.tiles_h * p.tiles_w;
     const long mt = (p.ntiles + 31) / 32;
-    p.nt = a.Cout / 32;
-    if (mt * p.nt >= (1L << 31) / 8) return K_EUNSUPPORTED;
+    if (mt * (a.Cout / 32) >= (1L << 31) / 8) return K_EUNSUPPORTED;
     p.mt = (int)mt;
-    const long base = mt * p.nt;
     const int kblocks = a.Cin / kKC;
 
+    p.nt = a.Cout / 32;
+    const long base = mt * p.nt;
+
     // Split over input channels when the blocks alone leave CUs idle.  The kernel is bound by what a SIMD
-    // issues (transforms and MFMAs take turns), so two workgroups on a CU take twice as long as one: the
-    // candidates are weighed by the K-blocks the fullest CU works through, with a slight preference for a CU
-    // that holds two workgroups (they fill each other's barrier waits), two K-blocks' worth for reading a split
-    // back and summing it, and a little per slot.  Measured on MI355X (us): 8x14x14x256>256 1/2/4/8 slots
-    // 36.6 / 24.8 / 23.9 / 28.2; 8x28x28x128>128 22.5 / 23.6 / 27.8 / 34.4; 8x7x7x512>512 73 / 43 / 27.1 / 25.7.
+    // issues (transforms and MFMAs add up), so two workgroups on a CU take twice as long as one: the candidates
+    // are weighed by the K-blocks the fullest CU works through, with a slight preference for a CU that holds two
+    // workgroups (they fill each other's barrier waits), two K-blocks' worth for reading a split back and
+    // summing it, and a little per slot.  Measured on MI355X (us): 8x14x14x256>256 1/2/4/8 slots 27.8 / 18.8 /
+    // 17.9 / 22.6; 8x28x28x128>128 16.5 / 18.2 / 22.6 / 29.6; 8x7x7x512>512 52.5 / 31.1 / 19.9 / 20.4.
+    // (A workgroup of 64 output channels -- one patch transform for two filter transforms, 25 loads per thread
+    // and K-block instead of 2 x 16 -- was built and measured: 12 % less time per K-block and unit of work, but
+    // half as many workgroups for grids that fill the chip barely once; 22.4 / 21.0 / 18.2 / 26.7 us on the four
+    // ResNet-152 batch 8 layers against 17.8 / 16.7 / 16.1 / 19.6.  It is not kept.)
     const char* forced_env = getenv("TORPOR_WINO_SPLITS");  // read per call: tests compare split depths in one process
     const int forced = forced_env ? atoi(forced_env) : 0;
     const size_t per_split = (size_t)base * 4096 * sizeof(float);
@@ -536,7 +561,7 @@ int launch_conv3x3_winograd(const ConvArgs& a, const Workspace& ws, hipStream_t 
     EpilogueArgs ea = a.ep;
     if (ea.residual && ea.ldr == 0) ea.ldr = a.Cout;  // the residual is dense unless its pitch is given
     p.ep = make_epilogue(ea, yp);
-    hipLaunchKernelGGL(conv_wino_kernel<1>, dim3((unsigned)base, 1, (unsigned)p.splits), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(conv_wino_kernel, dim3((unsigned)base, 1, (unsigned)p.splits), dim3(256), 0, s, p);
     set_last_kernel("conv3x3_wino_f2x2");
     return (int)hipGetLastError();
 }
