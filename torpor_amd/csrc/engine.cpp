@@ -170,7 +170,8 @@ int Engine::init() {
     pack_ = !(cfg_.flags & TP_FLAG_NO_PACK) && env_u64("TORPOR_PACK", 1) != 0;
     slim_host_ = !(cfg_.flags & TP_FLAG_KEEP_HOST_IMAGE) && env_u64("TORPOR_SLIM_HOST", 1) != 0;
     HIPCHK(hipEventCreateWithFlags(&stage_free_ev_, hipEventDisableTiming));
-    d2h_kernel_ = (int)env_u64("TORPOR_D2H_KERNEL", 2);  // 0 never, 1 always, 2 while a swap-in is running
+    d2h_kernel_ = (int)env_u64("TORPOR_D2H_KERNEL", 2);  // 0 never, 1 always, 2 small copies and while a swap-in is running
+    small_copy_bytes_ = env_u64("TORPOR_SMALL_COPY_BYTES", 1ull << 20);
     host_gather_ = !(cfg_.flags & TP_FLAG_NO_HOST_GATHER) && env_u64("TORPOR_HOST_GATHER", 1) != 0;
     HIPCHK(hipHostMalloc(reinterpret_cast<void**>(&h2d_stage_), 16ull << 20, hipHostMallocDefault));
     h2d_cap_ = 16ull << 20;
@@ -532,6 +533,17 @@ int Engine::ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need) {
     return 0;
 }
 
+// A request's input or result, by a copy kernel or by the copy engines?  During a swap-in -- this model's or
+// anybody's -- always by kernel (see do_h2d); otherwise by kernel up to small_copy_bytes_: a hipMemcpyAsync
+// carries about 15 us of fixed cost, a kernel launch behind the previous one 2-3 us, and the link moves 1 MiB in
+// 18 us either way (ResNet-50 batch 1, 602 KB of input: warm 0.551 -> 0.538 ms; ResNet-152 batch 8, 4.8 MB:
+// 2.95 ms either way).  TORPOR_D2H_KERNEL: 0 never, 1 always, 2 by this rule.
+bool Engine::copy_by_kernel(const Model& m, uint64_t bytes) {
+    if (d2h_kernel_ == 1) return true;
+    if (d2h_kernel_ != 2) return false;
+    return bytes <= small_copy_bytes_ || !m.fully_loaded || swap_in_flight();
+}
+
 int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
     if (bytes == 0) return 0;
     if (!src || bytes > kVaOffMask) return TP_EINVAL;
@@ -578,7 +590,7 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
     // to them queues among its transfer groups and disturbs how they alternate over the engines.  A copy
     // kernel reads the pinned buffer instead (alignment of the destination permitting).
     void* stage_dev = nullptr;
-    const bool by_kernel = (d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
+    const bool by_kernel = copy_by_kernel(m, bytes) &&
                            hipHostGetDevicePointer(&stage_dev, h2d_stage_, 0) == hipSuccess && stage_dev;
     if (by_kernel) {
         int kr = tpk::launch_copy(static_cast<uint8_t*>(stage_dev) + h2d_pos_, x.p, bytes, compute_);
@@ -620,7 +632,7 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
             const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
             if (d >= ub->first && d - ub->first + bytes <= ub->second) {
                 void* dst_dev = nullptr;
-                if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
+                if (copy_by_kernel(m, bytes) &&
                     hipHostGetDevicePointer(&dst_dev, dst, 0) == hipSuccess && dst_dev) {
                     int kr = tpk::launch_copy(p, dst_dev, bytes, compute_);
                     if (kr) return kr;
@@ -646,7 +658,7 @@ int Engine::do_d2h_async(Model& m, void* dst, uint64_t src, uint64_t bytes) {
         // device-to-host copy handed to them would wait for all of those; a copy kernel writing
         // into the pinned buffer goes the other way over the link without queueing behind them.
         void* stage_dev = nullptr;
-        if ((d2h_kernel_ == 1 || (d2h_kernel_ == 2 && (!m.fully_loaded || swap_in_flight()))) &&
+        if (copy_by_kernel(m, bytes) &&
             hipHostGetDevicePointer(&stage_dev, d2h_stage_, 0) == hipSuccess && stage_dev) {
             int kr = tpk::launch_copy(p, static_cast<uint8_t*>(stage_dev) + d2h_pos_, bytes, compute_);
             if (kr) return kr;

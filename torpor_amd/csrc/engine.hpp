@@ -311,6 +311,7 @@ private:
     int build_graph(Model& m);
     void wait_copy_idle(Model& m);
     bool swap_in_flight();
+    bool copy_by_kernel(const Model& m, uint64_t bytes);
     void log_transfer(Model& m);
     void copy_main();
     int ensure_stage(uint8_t** buf, uint64_t* cap, uint64_t need);
@@ -365,6 +366,7 @@ private:
     int plan_trials_ = 2;  // cold requests per copy plan before the measured choice is made (TORPOR_PLAN_TRIALS; 0 = estimate only)
     bool per_tensor_groups_ = false;  // BUFFER_SIZE=1: a transfer group closes behind every tensor
     int d2h_kernel_ = 0;
+    uint64_t small_copy_bytes_ = 1ull << 20;  // request copies up to this size go by copy kernel (TORPOR_SMALL_COPY_BYTES)
     bool host_gather_ = true;  // lookups may read a table in place from the host store during a swap-in
     int graph_min_ops_ = 0;  // 0: warm replays launch op by op; n: capture compute runs of at least n ops
     std::unordered_map<int, std::unique_ptr<Model>> models_;
