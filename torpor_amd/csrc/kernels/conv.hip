@@ -798,6 +798,18 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
             static const bool cb16_on = getenv("TORPOR_CONV3_CB16") == nullptr || atoi(getenv("TORPOR_CONV3_CB16")) != 0;
             cb16 = cb16_on && a.Cin % 16 == 0;
             p.splits = cap >= 2 ? choose_splits(tiles, p.K, cb16 ? 144 : 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, cap, true, 0) : 1;
+            // ... but not where the coarser blocks cost parallelism: a split keeps at least four K-blocks per slot,
+            // so few channels in blocks of 16 allow half as many slots (DenseNet's 128 -> 32 layers, 7 tiles: 2
+            // slots of 4 blocks of 16 run 8.8 us, 4 slots of 4 blocks of 8 run 6.9 us)
+            if (cb16 && cap >= 2) {
+                long kper8 = p.K;
+                const int splits8 = choose_splits(tiles, p.K, 72, 32 * 32, ws.ptr ? ws.bytes : 0, &kper8, cap, true, 0);
+                if (splits8 > p.splits) {
+                    cb16 = false;
+                    p.splits = splits8;
+                    kper_k = kper8;
+                }
+            }
         }
         p.kper = kper_k / 9;  // channels per split (multiple of 8)
         p.tickets = split_tickets(ws, (long)p.tiles_m * p.tiles_n, p.splits);
