@@ -337,12 +337,16 @@ int tp_launch(tp_server* s, int32_t client, int32_t op_id, const uint64_t* ptrs,
  * includes the final stream synchronisation and completion signal. */
 int tp_replay(tp_server* s, int32_t client, const void* input, uint64_t input_bytes, void* output,
               uint64_t output_bytes);
-/* Optional: pinned host memory for request results.  A device-to-host copy (tp_memcpy_d2h_async, or
+/* Optional: pinned host memory for request inputs and results.  A device-to-host copy (tp_memcpy_d2h_async, or
  * tp_replay's `output`) whose destination lies inside such a buffer is written there by the device
  * directly; any other destination is filled through the engine's pinned staging buffer and one host copy
- * after the stream synchronisation.  No counterpart in the reference, whose clients receive results
- * through the shared-memory segment they registered (cuda_server.hpp:1030-1046).  Buffers are released by
- * tp_host_free or with the server. */
+ * after the stream synchronisation.  A host-to-device copy (tp_memcpy_h2d, or tp_replay's `input`) whose
+ * source lies inside such a buffer is read by the device where it lies -- the caller leaves it unchanged
+ * until the next synchronising call of that function (tp_stream_synchronize, or tp_replay returning), as with
+ * any asynchronous copy from pinned memory; any other source is copied into the engine's staging buffer
+ * before the call returns and may be reused at once.  No counterpart in the reference, whose clients pass
+ * inputs and receive results through the shared-memory segment they registered (cuda_server.hpp:1030-1046).
+ * Buffers are released by tp_host_free or with the server. */
 int tp_host_alloc(tp_server* s, uint64_t bytes, void** ptr);
 int tp_host_free(tp_server* s, void* ptr);
 

@@ -219,21 +219,31 @@ def test_packed_transfer_is_lossless_for_any_bits(pack, monkeypatch):
         fn.unload()
 
 
-def test_results_into_pinned_buffers_equal_results_through_staging(gpu_server):
-    """tp_host_alloc: a result whose destination lies in such a buffer is written by the device itself
-    (by copy kernel while a swap-in runs, by the copy engine otherwise); same bytes as the staged path."""
+@pytest.mark.parametrize("image", [64, 320])
+def test_requests_from_and_into_pinned_buffers_equal_requests_through_staging(gpu_server, image):
+    """tp_host_alloc: an input that lies in such a buffer is read by the device where it is, a result whose
+    destination lies in one is written by the device itself (by copy kernel while a swap-in runs and for small
+    copies, by the copy engine otherwise: 64 x 64 images are below the size bound, 320 x 320 above); same
+    bytes as the staged path, warm and cold, in every combination."""
     s = gpu_server
-    fn, x, y = _mk(s, 7, seed=31)
-    packed, out_plain, views_plain = fn.pack([x])
-    _, out_pinned, views_pinned = fn.pack([x], pinned=True)
+    fn, x, y = _mk(s, 7, seed=31, image=image)
+    in_plain, out_plain, views_plain = fn.pack([x])
+    in_pinned, out_pinned, views_pinned = fn.pack([x], pinned=True)
+    assert np.array_equal(in_plain, in_pinned)
     for cold in (False, True, True, False):
-        for out in (out_pinned, out_plain):
-            if cold:
-                fn.unload()
-            out[:] = 0
-            assert s.signal(REQ_EXECUTE, 7, "")[0] == ACK_OK
-            s.replay(7, packed, out)
-        assert np.array_equal(views_plain[0], y) and np.array_equal(views_pinned[0], y)
+        for packed in (in_pinned, in_plain):
+            for out in (out_pinned, out_plain):
+                if cold:
+                    fn.unload()
+                out[:] = 0
+                assert s.signal(REQ_EXECUTE, 7, "")[0] == ACK_OK
+                s.replay(7, packed, out)
+            assert np.array_equal(views_plain[0], y) and np.array_equal(views_pinned[0], y)
+    # the pinned input is read at request time, not captured earlier: a changed input changes the answer
+    in_pinned[:] = fn.pack([x * np.float32(0.5)])[0]
+    assert s.signal(REQ_EXECUTE, 7, "")[0] == ACK_OK
+    s.replay(7, in_pinned, out_pinned)
+    assert not np.array_equal(views_pinned[0], y)
     fn.unload()
 
 

@@ -578,13 +578,34 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
     int r = translate(m, dst, bytes, &x);
     if (r) return r;
     if (host_only()) return 0;
+    // A source inside a pinned buffer handed out by user_host_alloc needs no staging copy: the device reads it
+    // where it lies (the caller leaves it alone until the request's next synchronising call, as with any
+    // asynchronous copy from pinned memory).  ResNet-152 batch 8, 4.8 MB of input: the staging memcpy was
+    // 0.1 ms of a 2.9 ms request.
+    {
+        const uintptr_t sp = reinterpret_cast<uintptr_t>(src);
+        auto ub = user_pinned_.upper_bound(sp);
+        if (ub != user_pinned_.begin()) {
+            --ub;
+            if (sp >= ub->first && sp - ub->first + bytes <= ub->second) {
+                void* src_dev = nullptr;
+                if (copy_by_kernel(m, bytes) &&
+                    hipHostGetDevicePointer(&src_dev, const_cast<void*>(src), 0) == hipSuccess && src_dev) {
+                    int kr = tpk::launch_copy(static_cast<const uint8_t*>(src_dev), x.p, bytes, compute_);
+                    if (kr) return kr;
+                } else {
+                    HIPCHK(hipMemcpyAsync(x.p, src, bytes, hipMemcpyHostToDevice, compute_));
+                }
+                return 0;
+            }
+        }
+    }
     if (h2d_pos_ + bytes > h2d_cap_) {
         HIPCHK(hipStreamSynchronize(compute_));
         h2d_pos_ = 0;
         r = ensure_stage(&h2d_stage_, &h2d_cap_, bytes);
         if (r) return r;
     }
-    std::memcpy(h2d_stage_ + h2d_pos_, src, bytes);
     // During a swap-in -- this model's or, when requests of resident models are served while another
     // model streams in, anybody's -- the copy engines belong to the weight stream: a request input handed
     // to them queues among its transfer groups and disturbs how they alternate over the engines.  A copy
@@ -592,11 +613,18 @@ int Engine::do_h2d(Model& m, uint64_t dst, const void* src, uint64_t bytes) {
     void* stage_dev = nullptr;
     const bool by_kernel = copy_by_kernel(m, bytes) &&
                            hipHostGetDevicePointer(&stage_dev, h2d_stage_, 0) == hipSuccess && stage_dev;
-    if (by_kernel) {
-        int kr = tpk::launch_copy(static_cast<uint8_t*>(stage_dev) + h2d_pos_, x.p, bytes, compute_);
-        if (kr) return kr;
-    } else {
-        HIPCHK(hipMemcpyAsync(x.p, h2d_stage_ + h2d_pos_, bytes, hipMemcpyHostToDevice, compute_));
+    // A large input goes through the staging buffer in pieces of 1 MiB: the host copies the next piece while
+    // the link moves the one before.
+    const uint64_t piece = bytes > (2ull << 20) ? (1ull << 20) : bytes;
+    for (uint64_t off = 0; off < bytes; off += piece) {
+        const uint64_t n = std::min(piece, bytes - off);
+        std::memcpy(h2d_stage_ + h2d_pos_ + off, static_cast<const uint8_t*>(src) + off, n);
+        if (by_kernel) {
+            int kr = tpk::launch_copy(static_cast<uint8_t*>(stage_dev) + h2d_pos_ + off, x.p + off, n, compute_);
+            if (kr) return kr;
+        } else {
+            HIPCHK(hipMemcpyAsync(x.p + off, h2d_stage_ + h2d_pos_ + off, n, hipMemcpyHostToDevice, compute_));
+        }
     }
     h2d_pos_ = align_up(h2d_pos_ + bytes, 256);
     return 0;

@@ -139,12 +139,16 @@ class Function:
 
     def pack(self, inputs, pinned=False):
         """Request inputs as one byte string and one output buffer with per-output views,
-        in the order the recorded H2D / D2H copies consume them.  `pinned`: the output buffer is
-        pinned memory of the server (results land in it without a staging copy; it lives as long as
-        the server)."""
+        in the order the recorded H2D / D2H copies consume them.  `pinned`: both buffers are pinned
+        memory of the server (the device reads the inputs and writes the results in place, without a
+        staging copy on either side; they live as long as the server)."""
         specs = self.input_specs()
         parts = [np.ascontiguousarray(a, dtype=dt).reshape(-1).view(np.uint8) for a, (_, dt) in zip(inputs, specs)]
         packed = np.concatenate(parts) if len(parts) > 1 else parts[0]
+        if pinned:
+            staged = self.s.host_empty(packed.size)
+            staged[:] = packed
+            packed = staged
         sizes = [int(np.prod(shape)) * np.dtype(dt).itemsize for shape, dt in self.out_specs]
         outbuf = self.s.host_empty(sum(sizes)) if pinned else np.empty(sum(sizes), dtype=np.uint8)
         views, pos = [], 0

@@ -43,7 +43,7 @@ def build_fleet(server, n_r50=32, n_bert=16, n_r152=16, levels=None, keep_weight
         weights = fn._weights if fid in keep_weights else None   # as init_weights made them (the oracle twins load these)
         first = fn.register(inputs)
         fn._weights = None          # the server holds the authoritative copy now
-        packed, outbuf, views = fn.pack(inputs)
+        packed, outbuf, views = fn.pack(inputs, pinned=True)   # inputs and results in pinned memory, as a serving loop keeps them
         fleet.append(dict(fn=fn, fid=fid, arch=arch, family=family, inputs=inputs, weights=weights, packed=packed,
                           outbuf=outbuf, views=views, first=[a.copy() for a in first]))
     return fleet
