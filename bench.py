@@ -179,6 +179,7 @@ def run_workload(server, fid, name, steps, warmup, link_gbps):
         swap_ms_p50=pctl(swap_ms, 0.5), swap_gbps_p50=pctl(swap_gbps, 0.5),
         swap_frac_of_link=pctl(swap_gbps, 0.5) / link_gbps if link_gbps else None,
         link_bytes=link_bytes,   # below weight_bytes when tensors travel in the packed format
+        input_bytes=int(packed.nbytes),   # the request's input crosses the link as well
         deferred_link_bytes=deferred_bytes,   # of those: index-looked-up tables, which travel last; the request does not wait for them
         weights_gbps_p50=info["image_bytes"] / 1e9 / (pctl(swap_ms, 0.5) * 1e-3),   # weight bytes in place per second
         copy_streams=streams, host_gathers=gathers, steps_total_s=t_total,
@@ -268,11 +269,12 @@ def roofline_from(kstats, empty_us, workload):
 
 def link_roofline(res, link_gbps):
     """The cold start against the host link.  A request cannot answer before the bytes it needs have
-    crossed the link: floor = (link bytes - tables that travel last) / link rate."""
-    waited = res["link_bytes"] - res["deferred_link_bytes"]
+    crossed the link: floor = (weight bytes on the link - tables that travel last + the request's own input,
+    which goes the same way over the same link) / link rate."""
+    waited = res["link_bytes"] - res["deferred_link_bytes"] + res.get("input_bytes", 0)
     floor_meas = waited / (link_gbps * 1e9) * 1e3
     floor_nom = waited / (PCIE_GEN5_X16_GBPS * 1e9) * 1e3
-    return dict(bound="host link", bytes_waited_for=waited, link_bytes=res["link_bytes"], weight_bytes=res["weight_bytes"],
+    return dict(bound="host link", bytes_waited_for=waited, input_bytes=res.get("input_bytes", 0), link_bytes=res["link_bytes"], weight_bytes=res["weight_bytes"],
                 cold_ms_p50=res["cold_ms_p50"], floor_ms_at_measured_link=floor_meas,
                 frac_of_measured_link_floor=floor_meas / res["cold_ms_p50"],
                 floor_ms_at_nominal_64=floor_nom, frac_of_nominal_floor=floor_nom / res["cold_ms_p50"],

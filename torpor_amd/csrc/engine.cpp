@@ -2720,10 +2720,16 @@ int Engine::replay(int client, const void* in, uint64_t in_bytes, void* out, uin
         if (m->warm_us <= 0 || us < m->warm_us) m->warm_us = us;
     }
     if (!warm && !ret && !profiling_ && !host_only() && m->ncopy >= 1 && m->ncopy <= 2) {
-        const double us = us_since(m->swap_t0);  // the swap-in this request ran beside, from its start
-        double& best = m->cold_us[m->ncopy];
-        if (m->cold_n[m->ncopy] == 0 || us < best) best = us;
-        ++m->cold_n[m->ncopy];
+        // A sample for choose_copy_plan: the swap-in this request ran beside, from its start to the request's end
+        // -- provided the request followed its swap-in at once.  One that was started later (a prefetch, a
+        // dispatcher that serves other requests meanwhile) ends when its own schedule says, not the copy plan's.
+        const double us = us_since(m->swap_t0);
+        const double delay = std::chrono::duration<double, std::micro>(t_start - m->swap_t0).count();
+        if (delay <= 0.1 * us) {
+            double& best = m->cold_us[m->ncopy];
+            if (m->cold_n[m->ncopy] == 0 || us < best) best = us;
+            ++m->cold_n[m->ncopy];
+        }
     }
     (void)completed;
     complete_request();
