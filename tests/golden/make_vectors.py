@@ -82,6 +82,14 @@ def main():
     out.update(emb_word=word, emb_pos=pos, emb_typ=typ, emb_ids=ids, emb_tids=tids,
                emb_y=e.reshape(18, 24).astype(np.float32))
 
+    # convolution 3x3 stride 1 pad 1, 16 -> 32 channels, + residual + ReLU on the image of the first case (odd
+    # height: the last row of 2x2 output tiles is half empty).  Drawn last so that every earlier vector keeps its
+    # values.  The shape the Winograd path takes; the direct kernels are checked on it as well.
+    ws1, rs1 = f32(32, 16, 3, 3) * np.float32(1.0 / 12.0), f32(2, 9, 8, 32)
+    t = F.conv2d(torch.from_numpy(x).double().permute(0, 3, 1, 2), torch.from_numpy(ws1).double(), stride=1, padding=1)
+    t = torch.relu(t.permute(0, 2, 3, 1) + torch.from_numpy(rs1).double())
+    out.update(conv_s1_w=ws1, conv_s1_res=rs1, conv_s1_y=t.numpy().astype(np.float32))
+
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")

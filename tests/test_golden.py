@@ -24,6 +24,8 @@ def test_oracle_reproduces_the_golden_vectors():
     assert_close(yb, V["conv_bn_relu"], 2e-6, "conv+bn+relu")
     assert_close(ref.conv2d(V["conv_x"], V["conv1_w"], (2, 2), (0, 0), x_nhwc=True, y_nhwc=True), V["conv1_y"], 1e-6, "1x1")
     assert_close(ref.depthwise_conv2d(V["conv_x"], V["dw_w"], (1, 1), (1, 1)), V["dw_y"], 1e-6, "depthwise")
+    ys1 = ref.conv2d(V["conv_x"], V["conv_s1_w"], (1, 1), (1, 1), x_nhwc=True, y_nhwc=True).astype(np.float64)
+    assert_close(np.maximum(ys1 + V["conv_s1_res"], 0), V["conv_s1_y"], 1e-6, "conv3x3 stride 1 + residual + relu")
     assert_close(ref.layernorm(V["ln_x"], V["ln_r"], V["ln_g"], V["ln_b"], 1e-12), V["ln_y"], 2e-6, "layernorm")
     assert_close(ref.softmax(V["sm_x"], V["sm_mask"], 0.125, 1), V["sm_y"], 2e-6, "softmax")
     assert_close(ref.attention(V["att_q"], V["att_k"], V["att_v"], V["att_mask"], 0.125), V["att_y"], 2e-6, "attention")
@@ -88,3 +90,20 @@ def test_kernels_reproduce_the_golden_vectors(gpu_server):
         ey = t.empty(V["emb_y"].nbytes)
         s.launch(f, OP_EMBEDDING, [ids, tids, w[11], w[12], w[13], ey], [18, 9, 24, 30, 2])
         assert_close(t.read(ey, (18, 24)), V["emb_y"], 1e-6, "embedding")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", ["winograd", "direct"])
+def test_stride_1_3x3_convolution_reproduces_the_golden_vectors_on_both_paths(gpu_server, monkeypatch, path):
+    """16 -> 32 channels, stride 1, residual + ReLU: the Winograd path (sent down it below its size bound) and the
+    direct kernels against the same float64 library result."""
+    from tests.harness import OpSession
+    from torpor_amd.server import ACT_RELU
+    monkeypatch.setenv("TORPOR_WINOGRAD", "1" if path == "winograd" else "0")
+    monkeypatch.setenv("TORPOR_WINO_MIN_GFLOP", "0")
+    with OpSession(gpu_server, [V["conv_s1_w"]]) as t:
+        cx, cr = t.act(V["conv_x"]), t.act(V["conv_s1_res"])
+        cy = t.empty(V["conv_s1_y"].nbytes)
+        t.s.conv(t.fid, cx, t.w[0], cy, 2, 9, 8, 16, 32, 3, 3, stride=1, pad=1, residual=cr, act=ACT_RELU)
+        assert t.s.last_kernel().startswith("conv3x3_wino" if path == "winograd" else "conv3x3_fast"), t.s.last_kernel()
+        assert_close(t.read(cy, V["conv_s1_y"].shape), V["conv_s1_y"], TOL, f"conv3x3 stride 1 ({path})")
