@@ -79,11 +79,13 @@ def test_fewer_rows_bert_and_mobilenet():
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("miss_aware", [False, True])
 @pytest.mark.parametrize("policy", ["sa", "fifo"])
-def test_router_serves_a_fleet_under_memory_pressure(policy):
+def test_router_serves_a_fleet_under_memory_pressure(policy, miss_aware):
+    """(miss_aware: requests of resident models are served while a swapped-out one streams in; same answers.)"""
     with Server(mem_limit_bytes=260 << 20, pool_bytes=512 << 20) as s:
         be = R.FunctionBackend(s, _factory, R.ones_inputs)
-        r = R.Router(be, slo_percentile=0.9, deadline_s=0.05, batch_limit=2, policy=policy)
+        r = R.Router(be, slo_percentile=0.9, deadline_s=0.05, batch_limit=2, policy=policy, miss_aware=miss_aware)
         for f in range(6):
             r.launch(f, level=0 if f % 2 else 1)
         for f in range(6):
@@ -95,6 +97,7 @@ def test_router_serves_a_fleet_under_memory_pressure(policy):
         wall = R.serve_arrivals(r, arrivals)
         out = r.summary()
         assert out["requests"] == 600 and out["queued"] == 0 and wall < 60
+        assert out["dispatch"] == ("miss-aware" if miss_aware else "queue order") and (out["early_loads"] > 0) == miss_aware
         st1 = s.pool_stats()
         assert st1["swap_ins"] - st0["swap_ins"] >= 6 and st1["evictions"] > st0["evictions"]   # 3 ResNets exceed the budget
         assert set(out["batches"]) <= {1, 2}

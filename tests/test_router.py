@@ -287,3 +287,111 @@ def test_prefetch_names_the_function_the_queue_hands_out_next(policy):
             assert nxt in later, i
     assert r1.prefetch_hints == sum(1 for _, _, nxt in hinted if nxt is not None) > 20
     assert r1.summary()["prefetch_hints"] == r1.prefetch_hints
+
+
+class SwapBackend(FakeBackend):
+    """A server with room for `capacity` models (LRU): a request of a swapped-out model ends when its bytes have
+    crossed the link, swap[f] after the swap-in was started, and not before forward[f] of its own."""
+
+    def __init__(self, clock, swap, forward, capacity, resident=()):
+        super().__init__(clock, forward)
+        self.swap, self.forward, self.capacity = swap, forward, capacity
+        self.lru = list(resident)
+        self.load_start = {}
+
+    def _bring_in(self, f):
+        if f not in self.lru:
+            if len(self.lru) >= self.capacity:
+                self.lru.pop(0)
+            self.load_start[f] = self.clock.t
+        else:
+            self.lru.remove(f)
+        self.lru.append(f)
+
+    def resident(self, f):
+        return f in self.lru
+
+    def load_estimate(self, f):
+        return self.swap[f], self.forward[f]
+
+    def load(self, f):
+        self.log.append(("load", f, self.clock.t))
+        self._bring_in(f)
+
+    def execute(self, f, n, prefetch=None):
+        self._bring_in(f)
+        start = self.clock.t
+        end = start + self.forward[f]
+        t0 = self.load_start.pop(f, None)
+        if t0 is not None:
+            end = max(end, t0 + self.swap[f] + 0.1 * self.forward[f])
+        self.log.append((f, n, start))
+        self.clock.t = end
+
+
+def _run_trace(clock, router, arrivals):
+    """serve_arrivals on the virtual clock: the busy-wait of the real loop becomes a jump."""
+    i, n = 0, len(arrivals)
+    while i < n or router.queued():
+        while i < n and arrivals[i][0] <= clock.t:
+            router.submit(arrivals[i][1], arrivals[i][0])
+            i += 1
+        if router.pump() == 0:
+            wake = [t for t in (arrivals[i][0] if i < n else None, router.wake_time()) if t is not None]
+            assert wake, "nothing to serve and nothing to wait for"
+            clock.t = max(clock.t, min(wake))
+
+
+@pytest.mark.parametrize("policy", ["fifo", "sa"])
+def test_miss_aware_router_serves_hits_while_a_model_streams_in(policy):
+    """Function 2 is swapped out (5 ms of link, 1 ms forward), 0 and 1 are resident.  In queue order the two hits
+    wait out the swap-in; miss-aware they run at once, the Load goes out when the miss reaches the head of the
+    queue, and the miss is served at 5 - 1 = 4 ms and ends at 5.1 ms as it would have anyway."""
+    ms = 1e-3
+    swap, fwd = {0: 5 * ms, 1: 5 * ms, 2: 5 * ms}, {0: 1 * ms, 1: 1 * ms, 2: 1 * ms}
+    arrivals = [(0.0, 2), (0.5 * ms, 0), (1.0 * ms, 1)]
+    out = {}
+    for aware in (False, True):
+        clock = Clock()
+        be = SwapBackend(clock, swap, fwd, capacity=3, resident=(0, 1))
+        r = R.Router(be, policy=policy, clock=clock, miss_aware=aware, margin_s=0.0)
+        for f in range(3):
+            r.launch(f, 1)
+        _run_trace(clock, r, arrivals)
+        out[aware] = ([e for e in be.log if e[0] != "load"], {f: v for f, v in r.latencies.items()})
+    runs, lats = out[False]
+    assert [(f, round(t / ms, 3)) for f, _, t in runs] == [(2, 0.0), (0, 5.1), (1, 6.1)]
+    runs, lats = out[True]
+    assert [(f, round(t / ms, 3)) for f, _, t in runs] == [(0, 0.5), (1, 1.5), (2, 4.0)]
+    assert lats[2][0] == pytest.approx(5.1 * ms) and lats[0][0] == pytest.approx(1.0 * ms) and lats[1][0] == pytest.approx(1.5 * ms)
+
+
+@pytest.mark.parametrize("policy", ["fifo", "sa"])
+@pytest.mark.parametrize("seed", range(4))
+def test_miss_aware_router_serves_every_request_once_one_at_a_time_one_swap_in_at_a_time(policy, seed):
+    rng = random.Random(seed)
+    nf, cap = 10, 4
+    swap = {f: rng.uniform(1e-3, 6e-3) for f in range(nf)}
+    fwd = {f: rng.uniform(0.4e-3, 2e-3) for f in range(nf)}
+    t, arrivals = 0.0, []
+    for _ in range(300):
+        t += rng.expovariate(1 / 1.5e-3)
+        arrivals.append((t, rng.choices(range(nf), [1 / (i + 1) for i in range(nf)])[0]))
+    res = {}
+    for aware in (False, True):
+        clock = Clock()
+        be = SwapBackend(clock, swap, fwd, capacity=cap, resident=tuple(range(cap)))
+        r = R.Router(be, policy=policy, clock=clock, miss_aware=aware, batch_limit=1)
+        for f in range(nf):
+            r.launch(f, 1)
+        _run_trace(clock, r, arrivals)
+        runs = [e for e in be.log if e[0] != "load"]
+        assert len(runs) == len(arrivals) and sum(len(v) for v in r.latencies.values()) == len(arrivals)
+        starts = [t0 for _, _, t0 in runs]
+        assert starts == sorted(starts)                              # one active function: no overlap
+        loads = [e for e in be.log if e[0] == "load"]
+        for a, b in zip(loads, loads[1:]):                           # one swap-in at a time: the earlier one has been
+            assert any(f == a[1] and a[2] <= t0 <= b[2] for f, _, t0 in runs)   # handed over before the next starts
+        res[aware] = np.sort(np.concatenate([np.asarray(v) for v in r.latencies.values()]))
+        assert r.summary()["dispatch"] == ("miss-aware" if aware else "queue order")
+    assert res[True].mean() <= res[False].mean() * 1.02              # what it is for: nobody waits out others' swap-ins

@@ -78,6 +78,7 @@ class FifoPolicy:
     def __init__(self, stats, slo):
         self.stats, self.slo = stats, slo
         self.queue = collections.deque()
+        self.blocked = set()            # functions the router holds back (their model is on its way): skipped
 
     def add_function(self, f):
         pass
@@ -91,11 +92,36 @@ class FifoPolicy:
     def next_batch(self, limit):
         if not self.queue:
             return None
+        if self.blocked:
+            return self._next_unblocked(limit)
         f, arr = self.queue.popleft()
         arrivals = [arr]
         while self.queue and self.queue[0][0] == f and len(arrivals) < limit(f):
             arrivals.append(self.queue.popleft()[1])
         return f, arrivals
+
+    def _next_unblocked(self, limit):
+        """The first request of a function that is not held back, with the requests of the same function that
+        follow it directly among those not held back."""
+        f, arrivals, keep, closed = None, [], [], False
+        for g, arr in self.queue:
+            if closed or g in self.blocked:         # held-back requests stay where they are and do not end a run
+                keep.append((g, arr))
+            elif f is None:
+                f, arrivals = g, [arr]
+            elif g == f and len(arrivals) < limit(f):
+                arrivals.append(arr)
+            else:
+                closed = True
+                keep.append((g, arr))
+        if f is None:
+            return None
+        self.queue = collections.deque(keep)
+        return f, arrivals
+
+    def head(self):
+        """The function next_batch would serve now."""
+        return next((f for f, _ in self.queue if f not in self.blocked), None)
 
     def peek(self, running):
         """The function of the first waiting request that is not `running`'s (what follows the batch just taken)."""
@@ -131,6 +157,7 @@ class SloAwarePolicy:
         self.stats, self.slo = stats, slo
         self.high_q, self.low_q = [], []
         self.high, self.low = set(), set()
+        self.blocked = set()            # functions the router holds back (their model is on its way): skipped
         self.alpha = 1.0
         self.window, self.diff_threshold, self.scale, self.low_scale = window, diff_threshold, scale, low_scale
         self._updates = 0
@@ -167,9 +194,14 @@ class SloAwarePolicy:
     def _first_available(self):
         for q in (self.high_q, self.low_q):
             for i, (f, _) in enumerate(q):
-                if self.stats.avail[f]:
+                if self.stats.avail[f] and f not in self.blocked:
                     return q, i
         return None, None
+
+    def head(self):
+        """The function next_batch would serve now."""
+        q, i = self._first_available()
+        return None if q is None else q[i][0]
 
     def peek(self, running):
         """The function next_batch would take now (`running` has been marked unavailable by the caller)."""
@@ -242,8 +274,18 @@ class Router:
     UPDATE_PERIOD_S = 2.0               # router.py:495
 
     def __init__(self, backend, slo_percentile=0.98, deadline_s=0.1, batch_limit=1, policy="sa", clock=time.monotonic,
-                 deadlines=None, batch_limits=None, prefetch=False):
+                 deadlines=None, batch_limits=None, prefetch=False, miss_aware=False, margin_s=0.0003):
         self.backend = backend
+        # miss_aware: a request whose model is swapped out does not hold the executor for its swap-in.  Its model
+        # is asked for at once (the Load signal), requests of resident models that the queue would serve next run
+        # meanwhile, and the waiting function is served when the rest of its copy is about as long as its forward
+        # pass (torpor_amd/dispatch.py has the rule and its reasons; one swap-in at a time, a function's own
+        # requests keep their order).  Needs a backend that can say whether a model is resident and how long its
+        # swap-in takes (`resident`, `load_estimate`).
+        self.miss_aware = miss_aware and hasattr(backend, "resident") and hasattr(backend, "load_estimate")
+        self.margin_s = margin_s
+        self.loading = {}               # function -> time from which it is served
+        self.loads = 0
         # prefetch: when a batch is dispatched, the function whose request the queue would hand out next is named
         # to the backend, which asks the server to load its model (the Load signal) while this batch runs
         self.prefetch = prefetch
@@ -300,10 +342,13 @@ class Router:
             ratio = self.policy.update()
             if ratio is not None:
                 self.slo_history.append((now, ratio, getattr(self.policy, "alpha", None), len(self.policy)))
+        if self.miss_aware and not self._hold_back_misses(now):
+            return 0
         got = self.policy.next_batch(self._limit)
         if got is None:
             return 0
         f, arrivals = got
+        self.loading.pop(f, None)       # (a function whose swap-in was started is handed over with its first batch)
         self.stats.avail[f] = False
         try:
             nxt = self.policy.peek(f) if self.prefetch else None
@@ -323,6 +368,34 @@ class Router:
         self.batches[len(arrivals)] += 1
         return len(arrivals)
 
+    def _hold_back_misses(self, now):
+        """Miss-aware dispatch: decide which functions the policy must pass over in this turn.  Returns False
+        when nothing can be served yet (every waiting request is of a model that is still on its way)."""
+        blocked = self.policy.blocked
+        blocked.clear()
+        for f, due in self.loading.items():
+            if due > now:
+                blocked.add(f)          # its copy has not come far enough
+        while True:
+            f = self.policy.head()
+            if f is None:
+                blocked.clear()
+                return False
+            if f in self.loading or self.backend.resident(f):
+                return True             # resident, or a swap-in that has come far enough: served next
+            if not self.loading:        # one swap-in at a time: this one's starts now
+                self.backend.load(f)
+                swap_s, forward_s = self.backend.load_estimate(f)
+                self.loading[f] = now + max(0.0, swap_s - forward_s - self.margin_s)
+                self.loads += 1
+                if self.loading[f] <= now:
+                    return True
+            blocked.add(f)              # waits for its copy, or for its turn to be copied
+
+    def wake_time(self):
+        """When a function that waits for its swap-in is due (miss-aware dispatch), else None."""
+        return min(self.loading.values()) if self.loading else None
+
     def queued(self):
         return len(self.policy) + len(self.inbox)
 
@@ -340,7 +413,8 @@ class Router:
                                               max(1, sum(s[1] for s in self.stats.stat.values()))),
                     worst_function_hit_rate=min(per_func.values()) if per_func else None,
                     alpha=getattr(self.policy, "alpha", None), batches=dict(self.batches), queued=self.queued(),
-                    prefetch_hints=self.prefetch_hints)
+                    prefetch_hints=self.prefetch_hints, dispatch="miss-aware" if self.miss_aware else "queue order",
+                    early_loads=self.loads)
 
 
 def serve_arrivals(router, arrivals, clock=time.monotonic, drain=True):
@@ -357,8 +431,11 @@ def serve_arrivals(router, arrivals, clock=time.monotonic, drain=True):
             i += 1
             if i < n:
                 due += float(arrivals[i][0])
-        if router.pump() == 0 and i < n:
-            while clock() - t0 < due:
+        if router.pump() == 0:
+            # nothing to serve: until the next arrival, or until a model that is on its way has come far enough
+            wake = router.wake_time()
+            until = min(t0 + due if i < n else float("inf"), wake if wake is not None else float("inf"))
+            while until != float("inf") and clock() < until:
                 pass
     return clock() - t0
 
@@ -471,6 +548,20 @@ class FunctionBackend:
     def load(self, func_id):
         self.conn[func_id].signal(2, func_id, "")
 
+    def resident(self, func_id):
+        """Is the function's model in device memory (from the moment a swap-in has been started)?  An in-process
+        server answers; over the wire there is no such query and every model counts as resident."""
+        conn = self.conn[func_id]
+        return conn.resident(func_id) if hasattr(conn, "resident") else True
+
+    def load_estimate(self, func_id):
+        """(swap-in, forward pass) in seconds, from the engine's own figures."""
+        conn = self.conn[func_id]
+        if not hasattr(conn, "load_estimate"):
+            return 0.0, 0.0
+        swap_ms, forward_ms = conn.load_estimate(func_id)
+        return swap_ms * 1e-3, forward_ms * 1e-3
+
     def close(self):
         """Closes the per-function connections this backend opened (nothing for a shared server)."""
         if self._owned:
@@ -525,6 +616,8 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--prefetch", action="store_true",
                     help="while a batch runs, ask the server to load the model of the request the queue hands out next")
+    ap.add_argument("--dispatch", default="queue", choices=["queue", "miss-aware"],
+                    help="miss-aware: requests of resident models are served while a swapped-out model streams in")
     a = ap.parse_args(argv)
 
     from .server import Server
@@ -540,7 +633,8 @@ def main(argv=None):
     def serve(server_or_factory, stats):
         backend = FunctionBackend(server_or_factory, lambda s, fid, lv: build_function(s, fid, lv, a.m, a.b), ones_inputs)
         router = Router(backend, a.t / 100, a.d / 1000, a.b, a.p, deadlines={f: 2 * a.d / 1000 for f in qa},
-                        batch_limits={f: 1 for f in qa}, prefetch=a.prefetch)
+                        batch_limits={f: 1 for f in qa}, prefetch=a.prefetch,
+                        miss_aware=a.dispatch == "miss-aware")
         for f in range(a.f):
             router.launch(f, mixed_model_level(f) if a.m == "mixed" else 1)
         for f in range(a.f):
