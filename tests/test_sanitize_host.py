@@ -9,6 +9,8 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIPCC = "/opt/rocm/bin/hipcc"
+# the engine's host translation units (the Makefile's .cpp sources)
+HOST_SOURCES = ("engine.cpp", "engine_swap.cpp", "engine_request.cpp", "engine_exec.cpp", "capi.cpp")
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
@@ -20,7 +22,7 @@ def test_wire_handlers_and_engine_under_sanitizers(tmp_path):
              "-packed-fp32-ops"] + san
     objs = []
     # the kernels come from the regular build (device code is not instrumented); host files are rebuilt
-    for src in ("engine.cpp", "capi.cpp"):
+    for src in HOST_SOURCES:
         o = str(tmp_path / (src + ".o"))
         subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", os.path.join(csrc, src), "-o", o],
                               stderr=subprocess.DEVNULL)
@@ -57,8 +59,7 @@ def test_c_abi_from_three_threads_under_thread_sanitizer(tmp_path):
         if not os.path.exists(o):
             pytest.skip("kernel objects not built (run make -C torpor_amd/csrc)")
         objs.append(o)
-    for src in (os.path.join(csrc, "engine.cpp"), os.path.join(csrc, "capi.cpp"),
-                os.path.join(ROOT, "tests", "native", "race_abi.cpp")):
+    for src in [os.path.join(csrc, f) for f in HOST_SOURCES] + [os.path.join(ROOT, "tests", "native", "race_abi.cpp")]:
         o = str(tmp_path / (os.path.basename(src) + ".o"))
         subprocess.check_call([HIPCC] + flags + ["-x", "hip", "-c", src, "-o", o], stderr=subprocess.DEVNULL)
         objs.append(o)
