@@ -2,9 +2,9 @@ import os
 import sys
 
 import pytest
-import torch  # noqa: F401  (first: PyTorch ships its own HIP runtime, and in a process that uses both that one
-#               has to be loaded before the engine's library initialises the system's; the other order
-#               leaves torch.cuda without a device)
+import torch  # noqa: F401  (the tests compare against PyTorch on the CPU and borrow its device tensors; the
+#               engine's library shares PyTorch's HIP runtime whichever is imported first,
+#               tests/test_gpu_import_order.py)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:

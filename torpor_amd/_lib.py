@@ -205,6 +205,30 @@ SYMBOLS = {
 _lib = None
 
 
+def _share_hip_runtime_with_torch():
+    """One HIP runtime per process.  A PyTorch wheel for ROCm carries its own libamdhip64 (soname
+    libamdhip64.so.7, the one this library asks for too) and finds it by file name: loaded after this library
+    it would come in as a second runtime beside the system's, and the second one to initialise sees no
+    device.  So where torch is installed but not imported yet, its copy is loaded first and this library binds
+    to it, which is what happens anyway when torch is imported first; either import order then works."""
+    import importlib.util
+    import sys
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return
+    if spec is None or not spec.submodule_search_locations:
+        return
+    path = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if os.path.exists(path):
+        try:
+            C.CDLL(path, mode=C.RTLD_GLOBAL)
+        except OSError:
+            pass    # not loadable here: the system's runtime serves this library alone
+
+
 def lib():
     """Load the shared library once; raises if it has not been built."""
     global _lib
@@ -213,6 +237,7 @@ def lib():
             raise ImportError(
                 f"{LIB_PATH} is missing: build it with `make -C torpor_amd/csrc` "
                 "(or __graft_entry__.build()); there is no fallback path")
+        _share_hip_runtime_with_torch()
         l = C.CDLL(LIB_PATH)
         for name, (res, args) in SYMBOLS.items():
             fn = getattr(l, name)  # AttributeError if the library does not export it
