@@ -21,7 +21,8 @@ def _rand(rng, *shape):
     (1536, 1024, 1024, "gemm_fast_64x32_kc"),   # BERT-large projection: 384 64x64 tiles = 1.5 per CU -> 64x32
     (1536, 1024, 4096, "gemm_fast_64x64_kc"),   # BERT-large FFN down-projection: long K, two K halves per 64x64 tile summed in the launch
     (4096, 2048, 160, "gemm_fast_64x64_kc"),    # K % 64 != 0: predicated kernel
-    (1, 1000, 2048, "gemm_fast_32x32_kc"),      # ResNet classifier, batch 1: 32 small tiles, K split over 8 workgroups each
+    (1, 1000, 2048, "gemv_rows_kc"),            # ResNet classifier, batch 1: a matrix-vector product, one wavefront per column
+    (9, 1000, 2048, "gemm_fast_32x32_kc"),      # one row more than the matrix-vector path takes: 32 small tiles, K split over 8 workgroups each
     (1568, 256, 1024, "gemm_fast_32x32_kc"),    # ResNet-152 batch 8 layer3 1x1: 100 64x64 tiles -> 32x32, K split in the workgroup
     (49, 512, 2048, "gemm_fast_32x32_kc"),      # ragged M (ResNet-50 batch 1, 7x7 pixels)
     (100, 37, 52, "gemm_fast_64x64_kc"),        # ragged N, K % 32 != 0
@@ -43,6 +44,52 @@ def test_gemm_tn(gpu_server, M, N, K, kernel):
     else:
         want = ref.gemm(X, W, M, N, K, max(K, 1), 1, max(K, 1), 1, N).reshape(M, N) + b
     assert_close(got, want, RTOL, f"gemm {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (1, 20, 480),        # squeeze-and-excitation, first layer (EfficientNet-B0)
+    (1, 480, 20),        # ... second layer: K shorter than one wavefront step
+    (1, 1001, 1028),     # odd column count, K not a multiple of the 256-float step
+    (2, 768, 768),       # MR = 2
+    (3, 33, 4),          # MR = 4 with one row unused, a single 128-bit step
+    (5, 130, 2052),      # MR = 8 with three rows unused
+    (8, 1000, 2048),     # ResNet-152 batch 8 classifier
+    (1, 4096, 25088),    # VGG-16 first fully connected layer: 411 MB of weights read once
+])
+def test_gemm_of_few_rows_runs_as_matrix_vector_products(gpu_server, M, N, K):
+    rng = np.random.default_rng(M * 11 + N * 5 + K)
+    X, W, b, R = _rand(rng, M, K), _rand(rng, N, K), _rand(rng, N), _rand(rng, M, N)
+    with OpSession(gpu_server, [W, b]) as t:
+        x, r = t.act(X), t.act(R)
+        c = t.empty(M * N * 4)
+        t.s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N, bias=t.w[1], residual=r, act=ACT_RELU)
+        assert t.s.last_kernel() == "gemv_rows_kc", t.s.last_kernel()
+        got = t.read(c, (M, N))
+        t.s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N, bias=t.w[1], residual=r, act=ACT_RELU)
+        again = t.read(c, (M, N))
+    if M * N * K > 5e7:   # too slow for the oracle's triple loop: fp64 BLAS matmul instead
+        want = np.maximum(X.astype(np.float64) @ W.astype(np.float64).T + b + R, 0)
+    else:
+        want = np.maximum(ref.gemm(X, W, M, N, K, K, 1, K, 1, N).reshape(M, N).astype(np.float64) + b + R, 0)
+    assert_close(got, want, RTOL, f"gemv {M}x{N}x{K}")
+    assert np.array_equal(got, again), "a repeated launch must give the same bits"
+
+
+def test_matrix_vector_path_applies_alpha_beta_and_batch_norm(gpu_server):
+    rng = np.random.default_rng(77)
+    M, N, K = 4, 96, 260
+    X, W, C0 = _rand(rng, M, K), _rand(rng, N, K), _rand(rng, M, N)
+    g, b, mu = _rand(rng, N), _rand(rng, N), _rand(rng, N)
+    var = rng.uniform(0.5, 2.0, N).astype(np.float32)
+    with OpSession(gpu_server, [W, g, b, mu, var]) as t:
+        x, c = t.act(X), t.act(C0)
+        t.s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N, alpha=0.5, beta=2.0, bn=tuple(t.w[1:5]),
+                 bn_eps=1e-5, act=ACT_TANH)
+        assert t.s.last_kernel() == "gemv_rows_kc", t.s.last_kernel()
+        got = t.read(c, (M, N))
+    z = 0.5 * ref.gemm(X, W, M, N, K, K, 1, K, 1, N).reshape(M, N).astype(np.float64) + 2.0 * C0
+    want = np.tanh((z - mu) / np.sqrt(var.astype(np.float64) + 1e-5) * g + b)
+    assert_close(got, want, 5e-5, "gemv alpha/beta/bn/tanh")
 
 
 @pytest.mark.parametrize("act", [ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH])

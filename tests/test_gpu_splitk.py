@@ -16,7 +16,7 @@ from torpor_amd.server import ACT_RELU, Server
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-GEMMS = [(128, 768, 3072), (196, 256, 1024), (1, 1000, 2048), (49, 512, 2048), (100, 37, 52 * 16), (128, 768, 3072)]
+GEMMS = [(128, 768, 3072), (196, 256, 1024), (9, 1000, 2048), (49, 512, 2048), (100, 37, 52 * 16), (128, 768, 3072)]
 CONVS = [(1, 14, 14, 256, 256, 1), (8, 14, 14, 256, 256, 1), (1, 7, 7, 512, 512, 1), (1, 28, 28, 256, 256, 2),
          (2, 9, 9, 24, 40, 1)]
 ROUNDS = 3

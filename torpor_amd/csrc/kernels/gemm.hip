@@ -535,6 +535,93 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
 }
 
+Epilogue make_epilogue(const EpilogueArgs& a, long ldc);
+
+// A GEMM of at most eight rows (the classifier of a convolutional network, BERT's pooler, the two small
+// layers of a squeeze-and-excitation block at batch 1..8) is a matrix-vector product: a 32x32 MFMA tile
+// would spend 75-97 % of its multiplications on rows that do not exist, and what bounds the launch is
+// reading the weights once.  One wavefront per output column: its lanes walk the column's K-contiguous
+// weights 128 bits at a time (1 KB per step and wavefront), multiply them with the same slice of every
+// row of X (read through the L1, shared by the workgroup's four columns), and a butterfly over the lanes
+// finishes the sums -- a fixed order, so repeated launches agree bit for bit.  Lane m applies the epilogue
+// to row m.  MR = rows held in registers (1, 2, 4 or 8; rows past M repeat the last one and are not stored).
+struct GemvDev {
+    const float* X;
+    const float* Y;
+    float* C;
+    int M;
+    long N, K, xs_r, ys_c;
+    Epilogue ep;
+};
+
+template <int MR>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(const GemvDev p) {
+    const int lane = threadIdx.x & 63;
+    const long col = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (col >= p.N) return;  // whole wavefronts leave; the kernel has no barrier
+    const float* __restrict__ w = p.Y + col * p.ys_c;
+    const float* xr[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) xr[m] = p.X + (long)(m < p.M ? m : p.M - 1) * p.xs_r;
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+#pragma unroll 4
+    for (long k = lane * 4; k < p.K; k += 256) {
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(w + k);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const f32x4 xv = *reinterpret_cast<const f32x4*>(xr[m] + k);
+            acc[m] += wv[0] * xv[0] + wv[1] * xv[1] + wv[2] * xv[2] + wv[3] * xv[3];
+        }
+    }
+    float mine = 0.f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        float v = acc[m];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+        if (lane == m) mine = v;
+    }
+    if (lane < p.M && lane < MR) {
+        float cs, ct;
+        epilogue_column(p.ep, col, cs, ct);
+        epilogue_store(p.ep, p.C, lane, col, mine, cs, ct);
+    }
+}
+
+// Does this call take the matrix-vector path?  (No workspace, no split, any N and K.)
+static bool gemv_applies(const GemmArgs& a) {
+    static const bool on = getenv("TORPOR_GEMV") == nullptr || atoi(getenv("TORPOR_GEMV")) != 0;
+    return on && a.M >= 1 && a.M <= 8 && a.nb0 * a.nb1 == 1 && !a.gather && a.xs_k == 1 && a.ys_k == 1 && a.K >= 4 &&
+           a.K % 4 == 0 && a.xs_r % 4 == 0 && a.ys_c % 4 == 0 && (reinterpret_cast<uintptr_t>(a.X) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.Y) & 15) == 0 && a.N <= (1L << 31);
+}
+
+static int launch_gemv(const GemmArgs& a, hipStream_t s) {
+    GemvDev p;
+    p.X = a.X;
+    p.Y = a.Y;
+    p.C = a.C;
+    p.M = (int)a.M;
+    p.N = a.N;
+    p.K = a.K;
+    p.xs_r = a.xs_r;
+    p.ys_c = a.ys_c;
+    p.ep = make_epilogue(a.ep, a.ldc);
+    const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
+    if (a.M == 1)
+        hipLaunchKernelGGL(gemv_rows_kernel<1>, grid, block, 0, s, p);
+    else if (a.M == 2)
+        hipLaunchKernelGGL(gemv_rows_kernel<2>, grid, block, 0, s, p);
+    else if (a.M <= 4)
+        hipLaunchKernelGGL(gemv_rows_kernel<4>, grid, block, 0, s, p);
+    else
+        hipLaunchKernelGGL(gemv_rows_kernel<8>, grid, block, 0, s, p);
+    g_last_kernel = "gemv_rows_kc";
+    return (int)hipGetLastError();
+}
+
 Epilogue make_epilogue(const EpilogueArgs& a, long ldc) {
     Epilogue e;
     e.alpha = a.alpha;
@@ -837,12 +924,14 @@ static bool gemm_args_ok(const GemmArgs& a) {
 // Bytes of split-K partial sums launch_gemm would write for this call if the workspace were unbounded.
 long gemm_workspace_need(const GemmArgs& a) {
     if (!gemm_args_ok(a)) return K_EINVAL;
+    if (gemv_applies(a)) return 0;
     const GemmPlan g = plan_gemm(a, ~(size_t)0);
     return g.splits > 1 ? (long)g.splits * g.tiles_m * g.tiles_n * g.bm * g.bn * (long)sizeof(float) : 0;
 }
 
 int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     if (!gemm_args_ok(a)) return K_EINVAL;
+    if (gemv_applies(a)) return launch_gemv(a, s);
     const int batch = a.nb0 * a.nb1;
     const GemmPlan g = plan_gemm(a, ws.ptr ? ws.bytes : 0);
     GemmDev p;
