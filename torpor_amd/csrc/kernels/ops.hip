@@ -441,6 +441,7 @@ __global__ __launch_bounds__(256) void avgpool_partial_kernel(const float* __res
     float acc = 0.f;
     if (c < C) {
         const float* px = x + (long)n * HW * C + c;
+#pragma unroll 8
         for (int q = p0 + ry; q < p1; q += 4) acc += px[(long)q * C];
     }
     red[ry][cx] = acc;
@@ -468,6 +469,7 @@ __global__ __launch_bounds__(256) void avgpool_small_kernel(const float* __restr
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
     if (c < C) {  // C % 4 == 0: the four channels are in range together
         const float* px = x + (long)n * HW * C + c;
+#pragma unroll 4
         for (int q = ph; q < HW; q += 16) {
             const float4 v = *reinterpret_cast<const float4*>(px + (long)q * C);
             a0 += v.x;
