@@ -110,6 +110,16 @@ typedef struct tp_server tp_server;
 #define TP_OP_AVGPOOL2D 15   /* p: x,y   i: N,H,W,C,k,stride,pad,y_pitch|0   NHWC window average, padding counted */
 #define TP_OP_COPY2D 16      /* p: src,dst   i: rows,width,src_pitch,dst_pitch   (elements) */
 #define TP_OP_SCALE_CHANNELS 17 /* p: x,scale,y   i: N,HW,C   y[n,p,c] = x[n,p,c] * scale[n,c] (NHWC) */
+/* Inference batch-norm (+ ReLU) of the input, 1x1 convolution, epilogue -- one launch for what a pre-activation
+ * network issues as cudnnBatchNormalizationForwardInference + activation + cudnnConvolutionForward
+ * (cuda_server.hpp:797-860, 708-771).  NHWC: x is rows pixels of cin channels, x_pitch floats apart (0 = cin: the
+ * first cin channels of a wider tensor otherwise); w is [cout][cin]; y rows of cout, y_pitch apart (0 = cout).
+ * The four pre_* vectors [cin] normalise x; the four post_* vectors [cout] (all or none) and `act` form the
+ * epilogue.  Taken: cin a multiple of 32 up to 2048, x / w / the vectors 16-byte aligned, x_pitch a multiple of 4;
+ * TP_EUNSUPPORTED otherwise (the caller issues the two calls instead).
+ *   p: x,pre_gamma,pre_beta,pre_mean,pre_var,w,y,post_gamma|0,post_beta|0,post_mean|0,post_var|0
+ *   i: rows,cin,cout,x_pitch,y_pitch,pre_relu,act   f: pre_eps,post_eps */
+#define TP_OP_BN_CONV1X1 18
 
 typedef struct tp_config {
     uint32_t struct_size;       /* sizeof(tp_config) */

@@ -397,3 +397,70 @@ print("ok")
     r = subprocess.run([sys.executable, "-c", code, name], env=env, cwd=root, capture_output=True, text=True,
                        timeout=120)
     assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr
+
+
+# ---------------------------------------------------------------- batch-norm + ReLU on the input of a 1x1 convolution
+@pytest.mark.parametrize("rows,cin,cout,ctot,post", [
+    (196, 256, 128, 640, True),     # DenseNet block 3: K a multiple of 128 -> 32x32 tiles
+    (196, 224, 128, 640, True),     # K not a multiple of 64: 64x64 tiles, K-blocks of 32
+    (3136, 64, 128, 256, True),     # first layer of block 1: two K-blocks, many rows
+    (49, 1920, 128, 1920, True),    # last layer of DenseNet-201: the longest K, split over workgroups
+    (784, 512, 256, 512, False),    # transition: no second batch-norm, no activation
+    (8, 32, 40, 32, True),          # a single K-block, ragged rows and columns
+])
+def test_bn_relu_conv1x1_in_one_launch_equals_the_oracle_chain(gpu_server, rows, cin, cout, ctot, post):
+    from torpor_amd.server import OP_BN_CONV1X1
+    rng = np.random.default_rng(rows + cin * 3 + cout)
+    X = rng.standard_normal((rows, ctot)).astype(np.float32)
+    W = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    def bn_params(c):
+        return [rng.uniform(0.5, 1.5, c).astype(np.float32), rng.standard_normal(c).astype(np.float32),
+                rng.standard_normal(c).astype(np.float32), rng.uniform(0.5, 2.0, c).astype(np.float32)]
+    pre, pst = bn_params(cin), bn_params(cout)
+    with OpSession(gpu_server, [W] + pre + pst) as t:
+        x = t.act(X)
+        y = t.empty(rows * cout * 4)
+        t.s.launch(t.fid, OP_BN_CONV1X1, [x, *t.w[1:5], t.w[0], y, *(t.w[5:9] if post else (0, 0, 0, 0))],
+                   [rows, cin, cout, ctot, 0, 1, ACT_RELU if post else ACT_NONE], [1e-5, 1e-5])
+        assert t.s.last_kernel().startswith("gemm_prebn_"), t.s.last_kernel()
+        got = t.read(y, (rows, cout))
+        t.s.launch(t.fid, OP_BN_CONV1X1, [x, *t.w[1:5], t.w[0], y, *(t.w[5:9] if post else (0, 0, 0, 0))],
+                   [rows, cin, cout, ctot, 0, 1, ACT_RELU if post else ACT_NONE], [1e-5, 1e-5])
+        again = t.read(y, (rows, cout))
+    xin = np.ascontiguousarray(X[:, :cin])
+    a = ref.bn(xin, *pre, 1e-5, cin, nhwc=True, relu=True).reshape(rows, cin)
+    if rows * cin * cout > 5e7:
+        z = (a.astype(np.float64) @ W.astype(np.float64).T).astype(np.float32)
+    else:
+        z = ref.gemm(a, W, rows, cout, cin, cin, 1, cin, 1, cout).reshape(rows, cout)
+    want = ref.bn(z, *pst, 1e-5, cout, nhwc=True, relu=True).reshape(rows, cout) if post else z
+    assert_close(got, want, 5e-5, f"bn+relu+conv1x1 {rows}x{cin}->{cout}")
+    assert np.array_equal(got, again), "a repeated launch must give the same bits"
+
+
+def test_bn_conv1x1_without_relu_and_refusal_of_what_it_does_not_take(gpu_server):
+    from torpor_amd.server import EUNSUPPORTED, OP_BN_CONV1X1, TorporError
+    rng = np.random.default_rng(3)
+    rows, cin, cout = 70, 64, 48
+    X = rng.standard_normal((rows, cin)).astype(np.float32)
+    W = (rng.standard_normal((cout, cin)) / 8).astype(np.float32)
+    pre = [rng.uniform(0.5, 1.5, cin).astype(np.float32), rng.standard_normal(cin).astype(np.float32),
+           rng.standard_normal(cin).astype(np.float32), rng.uniform(0.5, 2.0, cin).astype(np.float32)]
+    with OpSession(gpu_server, [W] + pre) as t:
+        x = t.act(X)
+        y = t.empty(rows * cout * 4)
+        t.s.launch(t.fid, OP_BN_CONV1X1, [x, *t.w[1:5], t.w[0], y, 0, 0, 0, 0], [rows, cin, cout, 0, 0, 0, ACT_NONE],
+                   [1e-5, 1e-5])
+        got = t.read(y, (rows, cout))
+        a = ref.bn(X, *pre, 1e-5, cin, nhwc=True, relu=False).reshape(rows, cin)   # negative values pass
+        want = ref.gemm(a, W, rows, cout, cin, cin, 1, cin, 1, cout).reshape(rows, cout)
+        assert_close(got, want, 5e-5, "bn (no relu) + conv1x1")
+        with pytest.raises(TorporError) as e:   # 48 input channels: not a multiple of 32
+            t.s.launch(t.fid, OP_BN_CONV1X1, [x, *t.w[1:5], t.w[0], y, 0, 0, 0, 0], [rows, 48, cout, cin, 0, 1, ACT_NONE],
+                       [1e-5, 1e-5])
+        assert e.value.code == EUNSUPPORTED
+        # like every op that fails, the refusal is reported once more at the next synchronising call (a client that
+        # sends its ops in batches learns of it there)
+        with pytest.raises(TorporError) as e:
+            t.s.stream_synchronize(t.fid)
+        assert e.value.code == EUNSUPPORTED

@@ -212,8 +212,10 @@ with Server(mem_limit_bytes=1 << 30, pool_bytes=2 << 30) as s:
             x, v = t.act(X), t.act(V)
             c = t.empty(M * N * 4)
             s.gemm(t.fid, x, t.w[0], c, M, N, K, xs_r=K, ys_c=K, ldc=N)
-            # the tiles that split K over wavefronts (64x32, 32x32) exist for K % 128 == 0 only
-            want = sys.argv[1] if (sys.argv[1] not in ("64x32", "32x32") or K % 128 == 0) else "64x64"
+            # the tiles that split K over wavefronts exist for whole 64-wide K-blocks only: pairs of them for
+            # 64x32 (K % 128 == 0), any number for 32x32 (K % 64 == 0)
+            need = {"64x32": 128, "32x32": 64}.get(sys.argv[1], 1)
+            want = sys.argv[1] if (K % need == 0 and (need == 1 or K >= 128)) else "64x64"
             assert want in s.last_kernel(), s.last_kernel()
             assert_close(t.read(c, (M, N)), X.astype(np.float64) @ W.astype(np.float64).T, 2e-5, "kc")
             s.gemm(t.fid, x, v, c, M, N, K, xs_r=K, ys_c=1, ys_k=N, ldc=N)

@@ -63,7 +63,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
         /* MAXPOOL */ 1u << 8, /* AVGPOOL */ 0, /* LAYERNORM */ 1u << 0, /* SOFTMAX */ (1u << 0) | (1u << 2),
         /* EMBEDDING */ (1u << 0) | (1u << 3), /* NCHW_TO_NHWC */ 0, /* NHWC_TO_NCHW */ 0, /* SUM */ 1u << 0,
         /* FILL */ 1u << 0, /* ATTENTION */ 0xF0u, /* AVGPOOL2D */ 1u << 7, /* COPY2D */ (1u << 0) | (1u << 2) | (1u << 3),
-        /* SCALE_CHANNELS */ 1u << 1};
+        /* SCALE_CHANNELS */ 1u << 1, /* BN_CONV1X1 */ (1u << 0) | (1u << 3) | (1u << 4)};
     {
         uint32_t long_mask = 0;
         switch (op.kind) {
@@ -303,6 +303,46 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             if (!launch) return 0;
             return tpk::launch_scale_channels(F(0), F(1), Fm(2), (int)N, HW, (int)C, compute_);
         }
+        case TP_OP_BN_CONV1X1: {
+            if (!need(11, 7, 2)) return TP_EINVAL;
+            const i128 rows = I[0], cin = I[1], cout = I[2];
+            const i128 xp = I[3] ? I[3] : cin, yp = I[4] ? I[4] : cout;
+            if (rows < 1 || cin < 1 || cout < 1 || xp < cin || yp < cout || I[6] > 16) return TP_EINVAL;
+            if ((r = R(0, false, (rows - 1) * xp + cin)) || (r = R(5, false, cout * cin)) ||
+                (r = R(6, false, (rows - 1) * yp + cout)))
+                return r;
+            for (int k = 1; k < 5 && !r; ++k) r = R(k, false, cin);
+            for (int k = 7; k < 11 && !r; ++k) r = R(k, true, cout);
+            if (r) return r;
+            if ((q[7] != nullptr) != (q[8] != nullptr) || (q[7] != nullptr) != (q[9] != nullptr) ||
+                (q[7] != nullptr) != (q[10] != nullptr))
+                return TP_EINVAL;
+            tpk::GemmArgs g;
+            g.X = F(0);
+            g.Y = F(5);
+            g.C = Fm(6);
+            g.M = (long)rows;
+            g.N = (long)cout;
+            g.K = (long)cin;
+            g.xs_r = (long)xp;
+            g.ys_c = (long)cin;
+            g.ldc = (long)yp;
+            g.pre_gamma = F(1);
+            g.pre_beta = F(2);
+            g.pre_mean = F(3);
+            g.pre_var = F(4);
+            g.pre_eps = op.f[0];
+            g.pre_relu = I[5] != 0;
+            g.ep.bn_scale = F(7);
+            g.ep.bn_bias = F(8);
+            g.ep.bn_mean = F(9);
+            g.ep.bn_var = F(10);
+            g.ep.bn_eps = op.f[1];
+            g.ep.act = (int)I[6];
+            g.ep.ldr = (long)yp;
+            if (!launch) return 0;
+            return tpk::launch_gemm(g, ws, compute_);
+        }
         case TP_OP_ATTENTION: {
             if (!need(5, 8, 1)) return TP_EINVAL;
             const i128 B = I[0], A = I[1], S = I[2], dh = I[3];
@@ -379,6 +419,11 @@ void op_work(const Op& op, double* flops, double* bytes, const char** name) {
                 case TP_OP_AVGPOOL2D: *bytes = 4.0 * (double)(I[0] * I[1] * I[2] * I[3]) * 1.25; *name = "avgpool2d"; break;
                 case TP_OP_COPY2D: *bytes = 8.0 * (double)(I[0] * I[1]); *name = "copy2d"; break;
                 case TP_OP_SCALE_CHANNELS: *bytes = 8.0 * (double)(I[0] * I[1] * I[2]); *name = "scale_channels"; break;
+                case TP_OP_BN_CONV1X1:
+                    *flops = 2.0 * (double)I[0] * (double)I[1] * (double)I[2];
+                    *bytes = 4.0 * ((double)I[0] * (double)I[1] + (double)I[1] * (double)I[2] + (double)I[0] * (double)I[2]);
+                    *name = "bn_conv1x1";
+                    break;
                 case TP_OP_ATTENTION:
                     *flops = 4.0 * (double)(I[0] * I[1]) * (double)(I[2] * I[2]) * (double)I[3];
                     *bytes = 16.0 * (double)(I[0] * I[2]) * (double)(I[1] * I[3]);

@@ -56,6 +56,13 @@ struct GemmDev {
         unsigned short r0, c0, w, h;
     } rect[8];
     Epilogue ep;
+    // batch-norm (+ ReLU) of the X operand per K index (gemm_clean_kernel<..., APRE = true> only)
+    const float* pre_gamma;
+    const float* pre_beta;
+    const float* pre_mean;
+    const float* pre_var;
+    float pre_eps;
+    int pre_relu;
 };
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id; remap so that
@@ -278,7 +285,13 @@ __global__ __launch_bounds__(C::THREADS, (C::TM * C::TN >= 4 ? 1 : 2)) void gemm
 // (their products are computed and thrown away at the store) and the look-ahead loads past the
 // end of K are clamped to the last K-block, so the loop body has no predication and no control
 // flow: loads, LDS traffic and MFMAs can be interleaved freely by the scheduler.
-template <class C, bool YKC, int STAGES>
+//
+// APRE: inference batch-norm (+ ReLU) of the X operand per K index, for pre-activation networks.  The
+// workgroup folds the four vectors of its K range to scale and shift once, into LDS, while its first operand
+// loads are in flight; every 128-bit slice of X is then transformed in registers on its way into the LDS
+// tile (a thread's slices all share one K offset within the block, so that is two LDS reads and eight vector
+// instructions per K-block and slice).  The weights and the MFMA loop are untouched.
+template <class C, bool YKC, int STAGES, bool APRE = false>
 #ifndef TP_CLEAN_OCC
 #define TP_CLEAN_OCC (C::TM * C::TN >= 4 ? 1 : 2)
 #endif
@@ -286,6 +299,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     fetch_now(p);
     constexpr int RED_FLOATS = red_floats<C>();  // K-slice reduction area, then the epilogue staging blocks
     __shared__ __attribute__((aligned(16))) float lds[cmax(STAGES * C::LDS_FLOATS, RED_FLOATS + stage_floats<C>() + 4)];
+    __shared__ __attribute__((aligned(16))) float pre_sb[APRE ? 2 * kPreBnMaxK : 4];  // folded scale, then shift (unused and dropped without APRE)
     TP_CLK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wk = wave / (C::WGM * C::WGN), wsp = wave - wk * (C::WGM * C::WGN);
@@ -307,6 +321,22 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     const long klast = kend - C::BK;
     ColConsts<C::TN> cc;  // bias / batch-norm vectors of this wavefront's columns: requested now, used at the end
     if (wk == 0) cols_issue<C>(cc, p.ep, Cc, n0, wn, lane, p.N);
+    // APRE: the four batch-norm vectors of this workgroup's K range, requested before anything else needs the
+    // memory pipe (at most kPreBnMaxK values of each: PRE_STEPS 128-bit loads per thread and vector)
+    constexpr int PRE_STEPS = APRE ? (int)((kPreBnMaxK / 4 + C::THREADS - 1) / C::THREADS) : 1;
+    f32x4 pre_g[PRE_STEPS], pre_b[PRE_STEPS], pre_m[PRE_STEPS], pre_v[PRE_STEPS];
+    if (APRE) {
+#pragma unroll
+        for (int j = 0; j < PRE_STEPS; ++j) {
+            const long k = kbeg + ((long)j * C::THREADS + tid) * 4;
+            if (k < kend) {
+                pre_g[j] = *reinterpret_cast<const f32x4*>(p.pre_gamma + k);
+                pre_b[j] = *reinterpret_cast<const f32x4*>(p.pre_beta + k);
+                pre_m[j] = *reinterpret_cast<const f32x4*>(p.pre_mean + k);
+                pre_v[j] = *reinterpret_cast<const f32x4*>(p.pre_var + k);
+            }
+        }
+    }
 
     constexpr int KV = C::BK / 4;
     constexpr int CV = C::BN / 4;
@@ -350,18 +380,36 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     zero_acc<C>(acc);
     f32x4 ra0[NVA], rb0[NVB], ra1[NVA], rb1[NVB];
 
-    auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0) {
+    static_assert(!APRE || C::THREADS % KV == 0, "a thread's X slices must share their K offset within the block");
+    const int pre_kq = (tid % KV) * 4;  // APRE: this thread's K offset within a block
+    const float pre_lo = (APRE && !p.pre_relu) ? -__builtin_huge_valf() : 0.f;
+    long kreg[2] = {0, 0};  // APRE: the K position each register set was loaded from
+    auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0, int set = 0) {
         const long k = k0 < klast ? k0 : klast;
+        if (APRE) kreg[set] = k;
 #pragma unroll
         for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + k);
 #pragma unroll
         for (int i = 0; i < NVB; ++i) rb[i] = *reinterpret_cast<const f32x4*>(pb[i] + k * ystep);
     };
-    auto store_lds = [&](const f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage) {
+    auto store_lds = [&](const f32x4 (&ra)[NVA], const f32x4 (&rb)[NVB], int stage, int set = 0) {
         float* As = lds + stage * C::LDS_FLOATS;
         float* Bs = As + C::BM * C::LDK;
+        if (APRE) {
+            const int at = (int)(kreg[set] - kbeg) + pre_kq;
+            const f32x4 sc = *reinterpret_cast<const f32x4*>(pre_sb + at);
+            const f32x4 sh = *reinterpret_cast<const f32x4*>(pre_sb + kPreBnMaxK + at);
 #pragma unroll
-        for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[i];
+            for (int i = 0; i < NVA; ++i) {
+                f32x4 v = ra[i];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) v[c] = fmaxf(v[c] * sc[c] + sh[c], pre_lo);
+                *reinterpret_cast<f32x4*>(As + sa[i]) = v;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NVA; ++i) *reinterpret_cast<f32x4*>(As + sa[i]) = ra[i];
+        }
 #pragma unroll
         for (int i = 0; i < NVB; ++i) {
             if (YKC) {
@@ -376,21 +424,42 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     TP_CLK(1);
     const float* As0 = lds;
     const long kpairs = kbeg + (kend - kbeg) / (2 * C::BK) * (2 * C::BK);  // end of the whole pairs of K-blocks
+    // APRE: fold this workgroup's K range of the four batch-norm vectors to scale and shift (same arithmetic as
+    // epilogue_column), 128 bits per thread and step; called once the first operand loads are on their way
+    auto fold_pre = [&]() {
+#pragma unroll
+        for (int j = 0; j < PRE_STEPS; ++j) {
+            const long k = kbeg + ((long)j * C::THREADS + tid) * 4;
+            if (k < kend) {
+                f32x4 sc, sh;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float inv = 1.0f / sqrtf(pre_v[j][c] + p.pre_eps);
+                    sc[c] = pre_g[j][c] * inv;
+                    sh[c] = pre_b[j][c] - pre_m[j][c] * sc[c];
+                }
+                *reinterpret_cast<f32x4*>(pre_sb + (k - kbeg)) = sc;
+                *reinterpret_cast<f32x4*>(pre_sb + kPreBnMaxK + (k - kbeg)) = sh;
+            }
+        }
+        __syncthreads();
+    };
     if (STAGES == 2) {
         const float* As1 = lds + C::LDS_FLOATS;
-        load_regs(ra0, rb0, kbeg);
-        load_regs(ra1, rb1, kbeg + C::BK);
+        load_regs(ra0, rb0, kbeg, 0);
+        load_regs(ra1, rb1, kbeg + C::BK, 1);
+        if (APRE) fold_pre();
         if (wk == 0) cols_fold<C>(cc, p.ep);
-        store_lds(ra0, rb0, 0);
+        store_lds(ra0, rb0, 0, 0);
         __syncthreads();
         for (long k0 = kbeg; k0 < kpairs; k0 += 2 * C::BK) {
-            load_regs(ra0, rb0, k0 + 2 * C::BK);
+            load_regs(ra0, rb0, k0 + 2 * C::BK, 0);
             mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
-            store_lds(ra1, rb1, 1);
+            store_lds(ra1, rb1, 1, 1);
             __syncthreads();
-            load_regs(ra1, rb1, k0 + 3 * C::BK);
+            load_regs(ra1, rb1, k0 + 3 * C::BK, 1);
             mma_block<C>(As1, As1 + C::BM * C::LDK, acc, wm, wn, lane, wk);
-            store_lds(ra0, rb0, 0);
+            store_lds(ra0, rb0, 0, 0);
             __syncthreads();
         }
         // an odd last K-block is in stage 0 by now (kept out of the loop: a branch there costs 10 %)
@@ -398,6 +467,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     } else {
         // one LDS stage, two barriers per K-block: half the LDS footprint, so twice as many
         // workgroups stay resident and hide each other's barrier and memory latency
+        static_assert(!APRE || STAGES == 2, "the operand transform is built into the two-stage loop only");
         load_regs(ra0, rb0, kbeg);
         load_regs(ra1, rb1, kbeg + C::BK);
         if (wk == 0) cols_fold<C>(cc, p.ep);
@@ -593,7 +663,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const GemvDev p) {
 // Does this call take the matrix-vector path?  (No workspace, no split, any N and K.)
 static bool gemv_applies(const GemmArgs& a) {
     static const bool on = getenv("TORPOR_GEMV") == nullptr || atoi(getenv("TORPOR_GEMV")) != 0;
-    return on && a.M >= 1 && a.M <= 8 && a.nb0 * a.nb1 == 1 && !a.gather && a.xs_k == 1 && a.ys_k == 1 && a.K >= 4 &&
+    return on && !a.pre_gamma && a.M >= 1 && a.M <= 8 && a.nb0 * a.nb1 == 1 && !a.gather && a.xs_k == 1 && a.ys_k == 1 && a.K >= 4 &&
            a.K % 4 == 0 && a.xs_r % 4 == 0 && a.ys_c % 4 == 0 && (reinterpret_cast<uintptr_t>(a.X) & 15) == 0 &&
            (reinterpret_cast<uintptr_t>(a.Y) & 15) == 0 && a.N <= (1L << 31);
 }
@@ -779,7 +849,7 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
     // 64x64 x 16 slots and a reduction launch.  TORPOR_GEMM_SMALL=0 restores the old rule for comparison.
     static const bool small_split = getenv("TORPOR_GEMM_SMALL") == nullptr || atoi(getenv("TORPOR_GEMM_SMALL")) != 0;
     const long t3232 = ((M + 31) / 32) * ((N + 31) / 32) * batch;
-    if (batch == 1 && K >= 256 && K % 128 == 0 && t64 < g_num_cu) {
+    if (batch == 1 && K >= 256 && K % 64 == 0 && t64 < g_num_cu) {  // (whole 64-wide K-blocks; an odd count is fine)
         if (small_split) return 4;
         if (t3232 >= 3 * g_num_cu / 8 && (t3232 >= g_num_cu || K <= 1024)) return 4;
     }
@@ -872,7 +942,8 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
     g.fast = x_fast && y_fast;
     if (g.fast) {
         int cfg = choose_tile(a.M, a.N, a.K, batch, g.y_kc);
-        if (cfg >= 3 && !(a.K >= 128 && a.K % 128 == 0 && (g.y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
+        if (cfg >= 3 && !(a.K >= 128 && a.K % (cfg == 4 ? 64 : 128) == 0 && (g.y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
+        if (a.pre_gamma && cfg != 2 && cfg != 4) cfg = 2;  // the operand transform exists for the 64x64 and 32x32 tiles
         g.cfg = cfg;
         g.bm = cfg == 4 ? 32 : cfg >= 2 ? 64 : 128;
         g.bn = cfg == 0 ? 128 : cfg >= 3 ? 32 : 64;
@@ -961,6 +1032,12 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
     p.sw = a.sw;
     p.ws = ws.ptr;
     p.ep = make_epilogue(a.ep, a.ldc);
+    p.pre_gamma = a.pre_gamma;
+    p.pre_beta = a.pre_beta;
+    p.pre_mean = a.pre_mean;
+    p.pre_var = a.pre_var;
+    p.pre_eps = a.pre_eps;
+    p.pre_relu = a.pre_relu;
     p.tickets = split_tickets(ws, (long)g.tiles_m * g.tiles_n, g.splits);
 
     p.tiles_m = g.tiles_m;
@@ -990,6 +1067,24 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
              {"gemm_fast_64x32_kc", "gemm_fast_64x32_kc_s1", "gemm_fast_64x32_kc_s2"}},
             {{"gemm_fast_32x32_cc", "gemm_fast_32x32_cc_s1", "gemm_fast_32x32_cc_s2"},
              {"gemm_fast_32x32_kc", "gemm_fast_32x32_kc_s1", "gemm_fast_32x32_kc_s2"}}};
+        if (a.pre_gamma) {
+            // batch-norm (+ ReLU) of the X operand: the branch-free two-stage kernel of the two small tiles carries it
+            const long range = p.splits > 1 ? p.kper : a.K;
+            if (!(clean && y_kc && (cfg == 2 || cfg == 4) && range <= kPreBnMaxK && a.pre_beta && a.pre_mean && a.pre_var &&
+                  aligned16(a.pre_gamma) && aligned16(a.pre_beta) && aligned16(a.pre_mean) && aligned16(a.pre_var)))
+                return K_EUNSUPPORTED;
+            if (cfg == 4) {
+                hipLaunchKernelGGL((gemm_clean_kernel<CfgT, true, 2, true>), grid, dim3(CfgT::THREADS), 0, s, p);
+                g_last_kernel = "gemm_prebn_32x32_kc_s2";
+            } else {
+                hipLaunchKernelGGL((gemm_clean_kernel<CfgM, true, 2, true>), grid, dim3(CfgM::THREADS), 0, s, p);
+                g_last_kernel = "gemm_prebn_64x64_kc_s2";
+            }
+            int err = (int)hipGetLastError();
+            if (err) return err;
+            if (p.splits > 1 && !p.tickets) return launch_splitk_reduce(ws.ptr, p.splits, a.M, a.N, a.C, p.ep, s);
+            return 0;
+        }
         int variant;
         if (cfg == 0)
             variant = launch_fast<CfgL>(p, y_kc, clean, grid, s);
@@ -1003,6 +1098,7 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
             variant = launch_fast<CfgM>(p, y_kc, clean, grid, s);
         g_last_kernel = names[cfg][y_kc ? 1 : 0][variant];
     } else {
+        if (a.pre_gamma) return K_EUNSUPPORTED;
         p.xr = p.xc = 0;
         dim3 grid(p.tiles_m * p.tiles_n, 1, p.splits > 1 ? p.splits : batch);
         hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, s, p);

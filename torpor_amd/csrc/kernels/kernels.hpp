@@ -39,7 +39,18 @@ struct GemmArgs {
     // (n*Ho + ho)*Wo + wo reads X row ((n*H + ho*sh)*W + wo*sw).
     int gather = 0, Ho = 0, Wo = 0, H = 0, W = 0, sh = 1, sw = 1;
     EpilogueArgs ep;
+    // Optional inference batch-norm (+ ReLU) of the X operand, per K index, applied as the operand is
+    // loaded: x'(r,k) = act((x(r,k) - mean[k]) / sqrt(var[k] + eps) * gamma[k] + beta[k]).  What a
+    // pre-activation network (DenseNet) computes in front of every 1x1 convolution.  The four vectors go
+    // together; launch_gemm returns K_EUNSUPPORTED where no kernel carries the transform (see gemm.hip).
+    const float* pre_gamma = nullptr;
+    const float* pre_beta = nullptr;
+    const float* pre_mean = nullptr;
+    const float* pre_var = nullptr;
+    float pre_eps = 0.f;
+    int pre_relu = 0;
 };
+constexpr long kPreBnMaxK = 2048;  // K range of one workgroup whose folded vectors fit the kernel's LDS block
 
 struct ConvArgs {
     const float* x = nullptr;

@@ -3,17 +3,19 @@
 The reference serves `torchvision.models.densenet169` / `densenet201` (tests/endpoint.py:20-23).
 Each dense layer is bn-relu-conv1x1-bn-relu-conv3x3 whose 32 new channels are concatenated to its
 input.  Here a dense block owns one NHWC buffer as wide as the block's final channel count: a
-layer normalises the first `cin` channels of it into a dense temporary (batch-norm with an input
-pitch), the 1x1 convolution carries the second batch-norm + ReLU in its epilogue, and the 3x3
-convolution writes its 32 channels straight into the block buffer at channel offset `cin`
-(output pitch), so nothing is ever concatenated by copying.  Transitions average-pool directly
-into the next block's buffer.  Weight names follow torchvision.
+layer's 1x1 convolution reads the first `cin` channels of it (input pitch), applies the first
+batch-norm + ReLU to them as it loads them and carries the second batch-norm + ReLU in its
+epilogue (one launch, TP_OP_BN_CONV1X1; two -- batch-norm into a dense temporary, then the
+convolution -- where the library has no kernel for the fused form), and the 3x3 convolution
+writes its 32 channels straight into the block buffer at channel offset `cin` (output pitch), so
+nothing is ever concatenated by copying.  Transitions average-pool directly into the next
+block's buffer.  Weight names follow torchvision.
 """
 from collections import OrderedDict
 
 import numpy as np
 
-from ..server import ACT_NONE, ACT_RELU, NCHW, NHWC, OP_AVGPOOL, OP_AVGPOOL2D, OP_COPY2D, OP_MAXPOOL
+from ..server import ACT_NONE, ACT_RELU, NCHW, NHWC, OP_AVGPOOL, OP_AVGPOOL2D, OP_BN_CONV1X1, OP_COPY2D, OP_MAXPOOL
 from .base import Function
 
 BLOCKS = {"densenet121": (6, 12, 24, 16), "densenet169": (6, 12, 32, 32), "densenet201": (6, 12, 48, 32)}
@@ -62,11 +64,12 @@ def init_weights(arch="densenet169", seed=0, num_classes=1000):
 
 
 class DenseNet(Function):
-    def __init__(self, server, fid, arch="densenet169", batch=1, weights=None, seed=0, level=1, image=224):
+    def __init__(self, server, fid, arch="densenet169", batch=1, weights=None, seed=0, level=1, image=224, fused=None):
         super().__init__(server, fid, level)
         self.arch, self.batch, self.image = arch, batch, image
         self._weights = weights if weights is not None else init_weights(arch, seed)
         self.num_classes = self._weights["classifier.weight"].shape[0]
+        self._fused = fused   # False: always batch-norm and convolution as two calls (for comparison)
 
     def weights(self):
         return OrderedDict((k, np.ascontiguousarray(v, dtype=np.float32)) for k, v in self._weights.items()
@@ -82,6 +85,25 @@ class DenseNet(Function):
     def _bn_relu(self, x_va, rows, c, name, x_pitch=0):
         y = self.alloc(rows * c * 4)
         self.s.bn(self.fid, x_va, y.va, *self._bn(name), BN_EPS, rows, c, relu=True, x_pitch=x_pitch)
+        return y
+
+    def _bn_relu_conv1x1(self, x_va, n, h, w, cin, cout, pre, weight, post=None, x_pitch=0):
+        """relu(bn_pre(x)) -> 1x1 convolution -> (bn_post + relu when `post` is given); returns the output block."""
+        rows = n * h * w
+        y = self.alloc(rows * cout * 4)
+        # what TP_OP_BN_CONV1X1 takes (include/torpor_amd.h): cin a multiple of 32 up to 2048, 16-byte aligned rows
+        if self._fused is not False and cin % 32 == 0 and cin <= 2048 and x_pitch % 4 == 0 and x_va % 16 == 0:
+            self.s.launch(self.fid, OP_BN_CONV1X1,
+                          [x_va, *self._bn(pre), self.w[weight], y.va, *(self._bn(post) if post else (0, 0, 0, 0))],
+                          [rows, cin, cout, x_pitch, 0, 1, ACT_RELU if post else ACT_NONE], [BN_EPS, BN_EPS])
+            return y
+        t = self._bn_relu(x_va, rows, cin, pre, x_pitch=x_pitch)
+        if post:
+            self.s.conv(self.fid, t.va, self.w[weight], y.va, n, h, w, cin, cout, 1, 1, bn=self._bn(post),
+                        bn_eps=BN_EPS, act=ACT_RELU)
+        else:
+            self.s.conv(self.fid, t.va, self.w[weight], y.va, n, h, w, cin, cout, 1, 1)
+        self.release(t)
         return y
 
     def forward(self, inputs):
@@ -109,11 +131,8 @@ class DenseNet(Function):
             for li in range(nl):
                 p = f"features.denseblock{bi + 1}.denselayer{li + 1}"
                 cin = c + li * GROWTH
-                t1 = self._bn_relu(buf.va, rows, cin, p + ".norm1", x_pitch=ctot)
-                t2 = self.alloc(rows * BN_SIZE * GROWTH * 4)
-                s.conv(self.fid, t1.va, self.w[p + ".conv1.weight"], t2.va, n, h, w, cin, BN_SIZE * GROWTH, 1, 1,
-                       bn=self._bn(p + ".norm2"), bn_eps=BN_EPS, act=ACT_RELU)
-                self.release(t1)
+                t2 = self._bn_relu_conv1x1(buf.va, n, h, w, cin, BN_SIZE * GROWTH, p + ".norm1", p + ".conv1.weight",
+                                           post=p + ".norm2", x_pitch=ctot)
                 # the 32 new channels land next to the ones the layer read
                 s.conv(self.fid, t2.va, self.w[p + ".conv2.weight"], buf.va + cin * 4, n, h, w, BN_SIZE * GROWTH,
                        GROWTH, 3, 3, stride=1, pad=1, y_pitch=ctot, act=ACT_NONE)
@@ -121,11 +140,8 @@ class DenseNet(Function):
             c = ctot
             if bi != len(blocks) - 1:
                 p = f"features.transition{bi + 1}"
-                t1 = self._bn_relu(buf.va, rows, c, p + ".norm")
+                t2 = self._bn_relu_conv1x1(buf.va, n, h, w, c, c // 2, p + ".norm", p + ".conv.weight")
                 self.release(buf)
-                t2 = self.alloc(rows * (c // 2) * 4)
-                s.conv(self.fid, t1.va, self.w[p + ".conv.weight"], t2.va, n, h, w, c, c // 2, 1, 1)
-                self.release(t1)
                 c //= 2
                 nh, nw = h // 2, w // 2
                 nxt_tot = c + blocks[bi + 1] * GROWTH

@@ -14,11 +14,12 @@ from ._lib import TorporError
 
 REQ_EXECUTE_AFTER_LOAD, REQ_EXECUTE, REQ_LOAD, REQ_UNLOAD = 0, 1, 2, 3
 ACK_OK, ACK_INAVAIL = 0, 1
+EUNSUPPORTED = -38   # TP_EUNSUPPORTED: shape / option not implemented (the caller takes another route)
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH, ACT_RELU6, ACT_SILU, ACT_SIGMOID = 0, 1, 2, 3, 4, 5, 6
 NCHW, NHWC = 0, 1
 (OP_RELU, OP_ADD, OP_BIAS_ACT, OP_GELU, OP_MAXPOOL, OP_AVGPOOL, OP_LAYERNORM, OP_SOFTMAX, OP_EMBEDDING,
  OP_NCHW_TO_NHWC, OP_NHWC_TO_NCHW, OP_SUM, OP_FILL, OP_ATTENTION, OP_AVGPOOL2D, OP_COPY2D,
- OP_SCALE_CHANNELS) = range(1, 18)
+ OP_SCALE_CHANNELS, OP_BN_CONV1X1) = range(1, 19)
 FLAG_HOST_ONLY = 1
 FLAG_EVICT_LRU = 2   # plain LRU instead of the two-class policy (as env EVICT_POLICY=LRU)
 FLAG_NO_PACK = 8   # weights cross the link as they are
