@@ -403,6 +403,9 @@ print("ok")
 @pytest.mark.parametrize("rows,cin,cout,ctot,post", [
     (196, 256, 128, 640, True),     # DenseNet block 3: K a multiple of 128 -> 32x32 tiles
     (196, 224, 128, 640, True),     # K not a multiple of 64: 64x64 tiles, K-blocks of 32
+    (196, 288, 128, 640, True),     # 32x32 tiles with half a K-block at the end (4.5 blocks of 64)
+    (49, 1888, 128, 1920, True),    # ... 29.5 blocks, split over workgroups: the last slice ends with the half block
+    (196, 416, 128, 640, True),     # ... 6.5 blocks
     (3136, 64, 128, 256, True),     # first layer of block 1: two K-blocks, many rows
     (49, 1920, 128, 1920, True),    # last layer of DenseNet-201: the longest K, split over workgroups
     (784, 512, 256, 512, False),    # transition: no second batch-norm, no activation

@@ -383,10 +383,13 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
     static_assert(!APRE || C::THREADS % KV == 0, "a thread's X slices must share their K offset within the block");
     const int pre_kq = (tid % KV) * 4;  // APRE: this thread's K offset within a block
     const float pre_lo = (APRE && !p.pre_relu) ? -__builtin_huge_valf() : 0.f;
-    long kreg[2] = {0, 0};  // APRE: the K position each register set was loaded from
+    long kreg[2] = {0, 0}, kwant[2] = {0, 0};  // APRE: the K position each register set was loaded from / stands for
     auto load_regs = [&](f32x4 (&ra)[NVA], f32x4 (&rb)[NVB], long k0, int set = 0) {
         const long k = k0 < klast ? k0 : klast;
-        if (APRE) kreg[set] = k;
+        if (APRE) {
+            kreg[set] = k;
+            kwant[set] = k0;
+        }
 #pragma unroll
         for (int i = 0; i < NVA; ++i) ra[i] = *reinterpret_cast<const f32x4*>(pa[i] + k);
 #pragma unroll
@@ -396,14 +399,18 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         float* As = lds + stage * C::LDS_FLOATS;
         float* Bs = As + C::BM * C::LDK;
         if (APRE) {
-            const int at = (int)(kreg[set] - kbeg) + pre_kq;
+            int at = (int)(kreg[set] - kbeg) + pre_kq;
+            // a slice in front of the position the block stands for (the half block at the end of K, or a
+            // look-ahead block past it, which nobody multiplies) is written as zeros
+            const bool dead = kreg[set] + pre_kq < kwant[set];
+            if (at < 0) at = 0;
             const f32x4 sc = *reinterpret_cast<const f32x4*>(pre_sb + at);
             const f32x4 sh = *reinterpret_cast<const f32x4*>(pre_sb + kPreBnMaxK + at);
 #pragma unroll
             for (int i = 0; i < NVA; ++i) {
                 f32x4 v = ra[i];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) v[c] = fmaxf(v[c] * sc[c] + sh[c], pre_lo);
+                for (int c = 0; c < 4; ++c) v[c] = dead ? 0.f : fmaxf(v[c] * sc[c] + sh[c], pre_lo);
                 *reinterpret_cast<f32x4*>(As + sa[i]) = v;
             }
         } else {
@@ -423,7 +430,11 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
 
     TP_CLK(1);
     const float* As0 = lds;
-    const long kpairs = kbeg + (kend - kbeg) / (2 * C::BK) * (2 * C::BK);  // end of the whole pairs of K-blocks
+    // APRE only: K may end with half a K-block.  That block is loaded from the last whole block's position (the
+    // look-ahead clamp below does that by itself) and the part of X that belongs to the block before is zeroed
+    // on its way into LDS, so the weights it meets contribute nothing.  kendv = end of K rounded up to blocks.
+    const long kendv = APRE ? kbeg + (kend - kbeg + C::BK - 1) / C::BK * C::BK : kend;
+    const long kpairs = kbeg + (kendv - kbeg) / (2 * C::BK) * (2 * C::BK);  // end of the whole pairs of K-blocks
     // APRE: fold this workgroup's K range of the four batch-norm vectors to scale and shift (same arithmetic as
     // epilogue_column), 128 bits per thread and step; called once the first operand loads are on their way
     auto fold_pre = [&]() {
@@ -463,7 +474,7 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             __syncthreads();
         }
         // an odd last K-block is in stage 0 by now (kept out of the loop: a branch there costs 10 %)
-        if (kpairs < kend) mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
+        if (kpairs < kendv) mma_block<C>(As0, As0 + C::BM * C::LDK, acc, wm, wn, lane, wk);
     } else {
         // one LDS stage, two barriers per K-block: half the LDS footprint, so twice as many
         // workgroups stay resident and hide each other's barrier and memory latency
@@ -822,7 +833,7 @@ static int launch_clean_only(const GemmDev& p, bool y_kc, dim3 grid, hipStream_t
 // (2 k per instruction) occupancy hides more latency than larger register tiles save in LDS
 // traffic.  The 128x128 / 128x64 variants are kept for very large grids and for experiments
 // (TORPOR_GEMM_CFG=0/1/2 forces one).
-static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
+static int choose_tile(long M, long N, long K, int batch, bool y_kc, bool half_ok = false) {
     static const int forced = [] {
         const char* e = getenv("TORPOR_GEMM_CFG");
         return e ? atoi(e) : -1;
@@ -849,7 +860,9 @@ static int choose_tile(long M, long N, long K, int batch, bool y_kc) {
     // 64x64 x 16 slots and a reduction launch.  TORPOR_GEMM_SMALL=0 restores the old rule for comparison.
     static const bool small_split = getenv("TORPOR_GEMM_SMALL") == nullptr || atoi(getenv("TORPOR_GEMM_SMALL")) != 0;
     const long t3232 = ((M + 31) / 32) * ((N + 31) / 32) * batch;
-    if (batch == 1 && K >= 256 && K % 64 == 0 && t64 < g_num_cu) {  // (whole 64-wide K-blocks; an odd count is fine)
+    // (whole 64-wide K-blocks, an odd count is fine; half_ok: the kernel with the operand transform also takes
+    // half a block at the end)
+    if (batch == 1 && K >= 256 && K % (half_ok ? 32 : 64) == 0 && t64 < g_num_cu) {
         if (small_split) return 4;
         if (t3232 >= 3 * g_num_cu / 8 && (t3232 >= g_num_cu || K <= 1024)) return 4;
     }
@@ -941,8 +954,9 @@ static GemmPlan plan_gemm(const GemmArgs& a, size_t ws_bytes) {
     const bool y_fast = (g.y_kc || y_cc) && aligned16(a.Y) && (a.yb0 % 4 == 0) && (a.yb1 % 4 == 0);
     g.fast = x_fast && y_fast;
     if (g.fast) {
-        int cfg = choose_tile(a.M, a.N, a.K, batch, g.y_kc);
-        if (cfg >= 3 && !(a.K >= 128 && a.K % (cfg == 4 ? 64 : 128) == 0 && (g.y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
+        const bool half_ok = a.pre_gamma != nullptr && g.y_kc;
+        int cfg = choose_tile(a.M, a.N, a.K, batch, g.y_kc, half_ok);
+        if (cfg >= 3 && !(a.K >= 128 && a.K % (cfg == 4 ? (half_ok ? 32 : 64) : 128) == 0 && (g.y_kc || a.N % 4 == 0))) cfg = 2;  // branch-free only
         if (a.pre_gamma && cfg != 2 && cfg != 4) cfg = 2;  // the operand transform exists for the 64x64 and 32x32 tiles
         g.cfg = cfg;
         g.bm = cfg == 4 ? 32 : cfg >= 2 ? 64 : 128;
@@ -1052,7 +1066,8 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         static const bool allow_clean = getenv("TORPOR_GEMM_NOCLEAN") == nullptr;
         // whole K-blocks; the 32-wide tiles take them in pairs, an odd last one is handled in the loop
         const long kq = cfg >= 3 ? 64 : 32;
-        const bool clean = allow_clean && a.K >= kq && a.K % kq == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
+        const long kq_mult = (a.pre_gamma && cfg == 4) ? 32 : kq;  // the operand-transform kernel masks half a block
+        const bool clean = allow_clean && a.K >= kq && a.K % kq_mult == 0 && (p.splits == 1 || p.kper % 64 == 0) &&
                            (y_kc || (a.N % 4 == 0 && a.N >= 4));
         // kernel variant names: <tile>_<kc|cc>[_s1|_s2]; _s1 / _s2 = branch-free kernel with one /
         // two LDS stages (gemm_clean_kernel<..., 1|2>), no suffix = predicated gemm_fast_kernel
