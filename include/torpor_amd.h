@@ -114,10 +114,11 @@ typedef struct tp_server tp_server;
  * network issues as cudnnBatchNormalizationForwardInference + activation + cudnnConvolutionForward
  * (cuda_server.hpp:797-860, 708-771).  NHWC: x is rows pixels of cin channels, x_pitch floats apart (0 = cin: the
  * first cin channels of a wider tensor otherwise); w is [cout][cin]; y rows of cout, y_pitch apart (0 = cout).
- * The four pre_* vectors [cin] normalise x; the four post_* vectors [cout] (all or none) and `act` form the
- * epilogue.  Taken: cin a multiple of 32 up to 2048, x / w / the vectors 16-byte aligned, x_pitch a multiple of 4;
+ * The four pre_* vectors [cin] normalise x -- or, with pre_beta = pre_mean = pre_var = 0, pre_gamma alone scales
+ * it per channel (the gate of a squeeze-and-excitation block applied to one image); the four post_* vectors [cout]
+ * (all or none), an optional residual laid out like y and `act` form the epilogue.  Taken: cin a multiple of 32 up to 2048, x / w / the vectors 16-byte aligned, x_pitch a multiple of 4;
  * TP_EUNSUPPORTED otherwise (the caller issues the two calls instead).
- *   p: x,pre_gamma,pre_beta,pre_mean,pre_var,w,y,post_gamma|0,post_beta|0,post_mean|0,post_var|0
+ *   p: x,pre_gamma,pre_beta|0,pre_mean|0,pre_var|0,w,y,post_gamma|0,post_beta|0,post_mean|0,post_var|0[,residual|0]
  *   i: rows,cin,cout,x_pitch,y_pitch,pre_relu,act   f: pre_eps,post_eps */
 #define TP_OP_BN_CONV1X1 18
 

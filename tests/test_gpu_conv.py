@@ -467,3 +467,27 @@ def test_bn_conv1x1_without_relu_and_refusal_of_what_it_does_not_take(gpu_server
         with pytest.raises(TorporError) as e:
             t.s.stream_synchronize(t.fid)
         assert e.value.code == EUNSUPPORTED
+
+
+def test_channel_gate_on_the_operand_load_with_residual(gpu_server):
+    """TP_OP_BN_CONV1X1 without beta / mean / var: x * gate[k] -> 1x1 convolution -> batch-norm + residual."""
+    from torpor_amd.server import OP_BN_CONV1X1
+    rng = np.random.default_rng(41)
+    rows, cin, cout = 196, 480, 80
+    X = rng.standard_normal((rows, cin)).astype(np.float32)
+    W = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    gate = rng.uniform(0, 1, cin).astype(np.float32)
+    R = rng.standard_normal((rows, cout)).astype(np.float32)
+    pst = [rng.uniform(0.5, 1.5, cout).astype(np.float32), rng.standard_normal(cout).astype(np.float32),
+           rng.standard_normal(cout).astype(np.float32), rng.uniform(0.5, 2.0, cout).astype(np.float32)]
+    with OpSession(gpu_server, [W] + pst) as t:
+        x, g, r = t.act(X), t.act(gate), t.act(R)
+        y = t.empty(rows * cout * 4)
+        t.s.launch(t.fid, OP_BN_CONV1X1, [x, g, 0, 0, 0, t.w[0], y, *t.w[1:5], r], [rows, cin, cout, 0, 0, 0, ACT_NONE],
+                   [0.0, 1e-5])
+        assert t.s.last_kernel().startswith("gemm_prebn_"), t.s.last_kernel()
+        got = t.read(y, (rows, cout))
+    a = (X * gate).astype(np.float32)
+    z = ref.gemm(a, W, rows, cout, cin, cin, 1, cin, 1, cout).reshape(rows, cout)
+    want = ref.bn(z, *pst, 1e-5, cout, nhwc=True, relu=False).reshape(rows, cout).astype(np.float64) + R
+    assert_close(got, want, 5e-5, "gate + conv1x1 + bn + residual")

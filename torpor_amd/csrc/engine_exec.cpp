@@ -309,14 +309,16 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             const i128 xp = I[3] ? I[3] : cin, yp = I[4] ? I[4] : cout;
             if (rows < 1 || cin < 1 || cout < 1 || xp < cin || yp < cout || I[6] > 16) return TP_EINVAL;
             if ((r = R(0, false, (rows - 1) * xp + cin)) || (r = R(5, false, cout * cin)) ||
-                (r = R(6, false, (rows - 1) * yp + cout)))
+                (r = R(6, false, (rows - 1) * yp + cout)) || (r = R(1, false, cin)))
                 return r;
-            for (int k = 1; k < 5 && !r; ++k) r = R(k, false, cin);
+            for (int k = 2; k < 5 && !r; ++k) r = R(k, true, cin);
             for (int k = 7; k < 11 && !r; ++k) r = R(k, true, cout);
+            if (!r && op.np > 11) r = R(11, true, (rows - 1) * yp + cout);  // residual, laid out like y
             if (r) return r;
             if ((q[7] != nullptr) != (q[8] != nullptr) || (q[7] != nullptr) != (q[9] != nullptr) ||
                 (q[7] != nullptr) != (q[10] != nullptr))
                 return TP_EINVAL;
+            if ((q[2] != nullptr) != (q[3] != nullptr) || (q[2] != nullptr) != (q[4] != nullptr)) return TP_EINVAL;
             tpk::GemmArgs g;
             g.X = F(0);
             g.Y = F(5);
@@ -339,6 +341,7 @@ int Engine::exec_compute_impl(Model& m, const Op& op, bool launch) {
             g.ep.bn_var = F(10);
             g.ep.bn_eps = op.f[1];
             g.ep.act = (int)I[6];
+            g.ep.residual = op.np > 11 ? F(11) : nullptr;
             g.ep.ldr = (long)yp;
             if (!launch) return 0;
             return tpk::launch_gemm(g, ws, compute_);

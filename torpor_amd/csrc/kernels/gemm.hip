@@ -331,9 +331,11 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
             const long k = kbeg + ((long)j * C::THREADS + tid) * 4;
             if (k < kend) {
                 pre_g[j] = *reinterpret_cast<const f32x4*>(p.pre_gamma + k);
-                pre_b[j] = *reinterpret_cast<const f32x4*>(p.pre_beta + k);
-                pre_m[j] = *reinterpret_cast<const f32x4*>(p.pre_mean + k);
-                pre_v[j] = *reinterpret_cast<const f32x4*>(p.pre_var + k);
+                if (p.pre_var) {  // (uniform: all three or none; none = a plain per-K scale)
+                    pre_b[j] = *reinterpret_cast<const f32x4*>(p.pre_beta + k);
+                    pre_m[j] = *reinterpret_cast<const f32x4*>(p.pre_mean + k);
+                    pre_v[j] = *reinterpret_cast<const f32x4*>(p.pre_var + k);
+                }
             }
         }
     }
@@ -442,12 +444,14 @@ __global__ __launch_bounds__(C::THREADS, TP_CLEAN_OCC) void gemm_clean_kernel(co
         for (int j = 0; j < PRE_STEPS; ++j) {
             const long k = kbeg + ((long)j * C::THREADS + tid) * 4;
             if (k < kend) {
-                f32x4 sc, sh;
+                f32x4 sc = pre_g[j], sh = {0.f, 0.f, 0.f, 0.f};
+                if (p.pre_var) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float inv = 1.0f / sqrtf(pre_v[j][c] + p.pre_eps);
-                    sc[c] = pre_g[j][c] * inv;
-                    sh[c] = pre_b[j][c] - pre_m[j][c] * sc[c];
+                    for (int c = 0; c < 4; ++c) {
+                        const float inv = 1.0f / sqrtf(pre_v[j][c] + p.pre_eps);
+                        sc[c] = pre_g[j][c] * inv;
+                        sh[c] = pre_b[j][c] - pre_m[j][c] * sc[c];
+                    }
                 }
                 *reinterpret_cast<f32x4*>(pre_sb + (k - kbeg)) = sc;
                 *reinterpret_cast<f32x4*>(pre_sb + kPreBnMaxK + (k - kbeg)) = sh;
@@ -1085,7 +1089,8 @@ int launch_gemm(const GemmArgs& a, const Workspace& ws, hipStream_t s) {
         if (a.pre_gamma) {
             // batch-norm (+ ReLU) of the X operand: the branch-free two-stage kernel of the two small tiles carries it
             const long range = p.splits > 1 ? p.kper : a.K;
-            if (!(clean && y_kc && (cfg == 2 || cfg == 4) && range <= kPreBnMaxK && a.pre_beta && a.pre_mean && a.pre_var &&
+            const bool all3 = a.pre_beta && a.pre_mean && a.pre_var, none3 = !a.pre_beta && !a.pre_mean && !a.pre_var;
+            if (!(clean && y_kc && (cfg == 2 || cfg == 4) && range <= kPreBnMaxK && (all3 || none3) &&
                   aligned16(a.pre_gamma) && aligned16(a.pre_beta) && aligned16(a.pre_mean) && aligned16(a.pre_var)))
                 return K_EUNSUPPORTED;
             if (cfg == 4) {

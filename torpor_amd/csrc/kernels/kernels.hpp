@@ -41,8 +41,10 @@ struct GemmArgs {
     EpilogueArgs ep;
     // Optional inference batch-norm (+ ReLU) of the X operand, per K index, applied as the operand is
     // loaded: x'(r,k) = act((x(r,k) - mean[k]) / sqrt(var[k] + eps) * gamma[k] + beta[k]).  What a
-    // pre-activation network (DenseNet) computes in front of every 1x1 convolution.  The four vectors go
-    // together; launch_gemm returns K_EUNSUPPORTED where no kernel carries the transform (see gemm.hip).
+    // pre-activation network (DenseNet) computes in front of every 1x1 convolution.  beta / mean / var go
+    // together; without them the transform is a plain per-K scale, x'(r,k) = act(x(r,k) * gamma[k]) (the channel
+    // gate of a squeeze-and-excitation block at batch 1).  launch_gemm returns K_EUNSUPPORTED where no kernel
+    // carries the transform (see gemm.hip).
     const float* pre_gamma = nullptr;
     const float* pre_beta = nullptr;
     const float* pre_mean = nullptr;

@@ -3,15 +3,16 @@
 The reference serves `torchvision.models.efficientnet_b0` (tests/endpoint.py:34-35).  An MBConv block
 is 1x1 expand (+bn+silu), k x k depthwise (+bn+silu), squeeze-and-excitation, 1x1 linear projection
 (+bn, +identity when shapes allow).  Batch-norm, SiLU and the shortcut ride in convolution
-epilogues; the squeeze-and-excitation branch is a global average pool, two small GEMMs whose
-epilogues apply bias + SiLU and bias + sigmoid, and one gating pass over the activations.
+epilogues; the squeeze-and-excitation branch is a global average pool and two small GEMMs whose
+epilogues apply bias + SiLU and bias + sigmoid; the gate is applied by the projection itself as it loads
+its input (one image, channel counts the fused kernel takes) or by a gating pass over the activations.
 Weight names follow torchvision (`features.<stage>.<layer>.block.<j>...`).
 """
 from collections import OrderedDict
 
 import numpy as np
 
-from ..server import ACT_NONE, ACT_SIGMOID, ACT_SILU, NCHW, NHWC, OP_AVGPOOL, OP_SCALE_CHANNELS
+from ..server import ACT_NONE, ACT_SIGMOID, ACT_SILU, NCHW, NHWC, OP_AVGPOOL, OP_BN_CONV1X1, OP_SCALE_CHANNELS
 from .base import Function
 
 # (expand ratio, kernel, stride, in, out, layers)
@@ -76,9 +77,10 @@ def init_weights(seed=0, num_classes=1000):
 
 
 class EfficientNetB0(Function):
-    def __init__(self, server, fid, batch=1, weights=None, seed=0, level=1, image=224):
+    def __init__(self, server, fid, batch=1, weights=None, seed=0, level=1, image=224, fused=None):
         super().__init__(server, fid, level)
         self.batch, self.image = batch, image
+        self._fused = fused   # False: the channel gate always as a pass of its own (for comparison)
         self._weights = weights if weights is not None else init_weights(seed)
         self.num_classes = self._weights["classifier.weight"].shape[0]
 
@@ -110,9 +112,25 @@ class EfficientNetB0(Function):
         self.s.gemm(self.fid, mid.va, self.w[name + ".fc2.weight"], gate.va, n, c, sq, xs_r=sq, ys_c=sq, ldc=c,
                     bias=self.w[name + ".fc2.bias"], act=ACT_SIGMOID)
         self.release(mid)
-        y = self.alloc(n * hw * c * 4)
-        self.s.launch(self.fid, OP_SCALE_CHANNELS, [x.va, gate.va, y.va], [n, hw, c])
-        self.release(gate)
+        return gate
+
+    def _gate_and_project(self, x, gate, n, h, w, c, cout, name, residual):
+        """y = bn(conv1x1(x * gate)) (+ residual).  One image and a channel count the library's fused kernel
+        takes (TP_OP_BN_CONV1X1 with a plain per-channel scale on the operand load): one launch; otherwise the
+        gating pass and the convolution."""
+        rows = n * h * w
+        if n == 1 and c % 32 == 0 and c <= 2048 and self._fused is not False:
+            y = self.alloc(rows * cout * 4)
+            bn = tuple(self.w[f"{name}.1.{f}"] for f in ("weight", "bias", "running_mean", "running_var"))
+            self.s.launch(self.fid, OP_BN_CONV1X1,
+                          [x.va, gate.va, 0, 0, 0, self.w[name + ".0.weight"], y.va, *bn,
+                           residual.va if residual is not None else 0],
+                          [rows, c, cout, 0, 0, 0, ACT_NONE], [0.0, BN_EPS])
+            return y
+        g = self.alloc(rows * c * 4)
+        self.s.launch(self.fid, OP_SCALE_CHANNELS, [x.va, gate.va, g.va], [n, h * w, c])
+        y, _, _ = self._conv_bn(g, n, h, w, c, cout, 1, 1, name, ACT_NONE, residual=residual)
+        self.release(g)
         return y
 
     def forward(self, inputs):
@@ -129,12 +147,12 @@ class EfficientNetB0(Function):
             if y is not cur:
                 self.release(y)
             j += 1
-            g = self._squeeze_excite(d, n, h2 * w2, hidden, max(1, cin // 4), f"{prefix}.{j}")
-            self.release(d)
+            gate = self._squeeze_excite(d, n, h2 * w2, hidden, max(1, cin // 4), f"{prefix}.{j}")
             j += 1
-            out, _, _ = self._conv_bn(g, n, h2, w2, hidden, cout, 1, 1, f"{prefix}.{j}", ACT_NONE,
-                                      residual=cur if (stride == 1 and cin == cout) else None)
-            self.release(g)
+            out = self._gate_and_project(d, gate, n, h2, w2, hidden, cout, f"{prefix}.{j}",
+                                         cur if (stride == 1 and cin == cout) else None)
+            self.release(gate)
+            self.release(d)
             self.release(cur)
             cur, h, w = out, h2, w2
         y, h, w = self._conv_bn(cur, n, h, w, 320, 1280, 1, 1, "features.8", ACT_SILU)
