@@ -172,6 +172,27 @@ def test_densenet(gpu_server, arch, image, batch):
     fn.unload()
 
 
+@pytest.mark.parametrize("family", ["densenet", "efficientnet"])
+def test_fused_operand_transform_is_taken_and_agrees_with_the_separate_launches(gpu_server, family):
+    """DenseNet's batch-norm + ReLU and EfficientNet's channel gate ride in the 1x1 convolution that follows
+    them (TP_OP_BN_CONV1X1): fewer recorded ops than with `fused=False`, the same logits within the bar."""
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(21)).numpy()
+    out, ops = {}, {}
+    for fused in (False, None):
+        if family == "densenet":
+            weights = _perturb_bn(densenet.init_weights("densenet121", seed=6), seed=7)
+            fn = densenet.DenseNet(gpu_server, 23, "densenet121", batch=1, weights=weights, fused=fused)
+        else:
+            weights = _perturb_bn(efficientnet.init_weights(seed=12), seed=13)
+            fn = efficientnet.EfficientNetB0(gpu_server, 23, batch=1, weights=weights, fused=fused)
+        (out[fused],) = fn.register([x])
+        ops[fused] = gpu_server.model_info(23)["n_ops"]
+        fn.unload()
+    # DenseNet-121: 58 dense layers + 3 transitions lose a launch each; EfficientNet-B0: 11 of 16 blocks
+    assert ops[None] <= ops[False] - (61 if family == "densenet" else 11), ops
+    assert_close(out[None], out[False].astype(np.float64), LOGIT_RTOL, f"{family}: fused against separate launches")
+
+
 @pytest.mark.parametrize("image,batch", [(96, 2), (224, 1)])
 def test_mobilenet_v2(gpu_server, image, batch):
     """MobileNetV2 (tests/endpoint.py:30-31): depthwise convolutions, relu6, linear bottlenecks."""
