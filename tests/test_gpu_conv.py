@@ -239,6 +239,9 @@ def test_conv_rejects_bad_shapes(gpu_server):
 @pytest.mark.parametrize("kh,kw,stride,Cin,Cout,H,W", [
     (1, 7, 1, 16, 24, 17, 17), (7, 1, 1, 48, 70, 17, 17), (1, 3, 1, 24, 40, 8, 8), (3, 1, 1, 16, 64, 8, 9),
     (1, 7, 1, 256, 32, 5, 7),   # splits over channels
+    (1, 7, 1, 40, 48, 17, 17), (7, 1, 1, 40, 48, 17, 17),   # 32x32 tiles, one wavefront per tap, 8 channels per K-block
+    (1, 3, 1, 40, 40, 8, 8), (3, 1, 1, 64, 64, 8, 9),       # ... three taps: 8 and 16 channels per K-block
+    (1, 7, 1, 64, 256, 64, 64),                              # a grid that fills the chip stays on 64x64 tiles
 ])
 def test_conv_tap_shapes(gpu_server, kh, kw, stride, Cin, Cout, H, W):
     """The asymmetric convolutions of Inception on the MFMA taps kernel ("same" padding),
@@ -254,7 +257,10 @@ def test_conv_tap_shapes(gpu_server, kh, kw, stride, Cin, Cout, H, W):
         xv = t.act(x)
         yv = t.empty(N * Ho * Wo * Cout * 4)
         t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, kh, kw, stride=stride, pad=(ph, pw))
-        assert t.s.last_kernel() == f"conv_taps_{kh}x{kw}_64x64", t.s.last_kernel()
+        # few tiles and at least 32 input channels: 32x32 tiles with one wavefront per tap; else 64x64 tiles
+        small = Cin >= 32 and -(-N * Ho * Wo // 64) * -(-Cout // 64) < 128
+        want = f"conv_taps_{kh}x{kw}_32x32_k{kh * kw}" if small else f"conv_taps_{kh}x{kw}_64x64"
+        assert t.s.last_kernel() == want, (t.s.last_kernel(), want)
         plain = t.read(yv, (N, Ho, Wo, Cout))
         t.s.conv(t.fid, xv, t.w[0], yv, N, H, W, Cin, Cout, kh, kw, stride=stride, pad=(ph, pw), bn=tuple(t.w[1:5]),
                  bn_eps=1e-3, act=ACT_RELU)

@@ -726,6 +726,45 @@ int launch_conv2d(const ConvArgs& a, const Workspace& ws, hipStream_t s) {
         // the asymmetric shapes (Inception): one 64x64 tile shape, split over channel blocks.  (5x5 stays on
         // the general kernel: a 200-wide K-block leaves one workgroup per CU and measured 2x slower.)
         const int T = a.KH * a.KW;
+        // Few 64x64 tiles (Inception's 17x17 and 8x8 maps at batch 1: 10 to 15 of them, whose K then had to be
+        // cut 16 to 25 ways and summed by a second launch): 32x32 tiles with one wavefront per tap, as for the
+        // 3x3 shapes, split so that every workgroup still has a CU to itself.  TORPOR_CONV_TAPS_SMALL=0: as before.
+        static const bool small_on = getenv("TORPOR_CONV_TAPS_SMALL") == nullptr || atoi(getenv("TORPOR_CONV_TAPS_SMALL")) != 0;
+        const long t64 = ((M + 63) / 64) * ((a.Cout + 63) / 64);
+        const long t32 = ((M + 31) / 32) * ((a.Cout + 31) / 32);
+        if (small_on && t64 < num_cu() / 2 && t32 <= kSplitTickets && a.Cin >= 32) {
+            p.tiles_m = (int)((M + 31) / 32);
+            p.tiles_n = (a.Cout + 31) / 32;
+            const bool cb16 = a.Cin % 16 == 0;
+            int cap = (int)(num_cu() / t32);
+            if (cap > 8) cap = 8;
+            long kper_k = p.K;
+            p.splits = cap >= 2 ? choose_splits(t32, p.K, (cb16 ? 16 : 8) * T, 32 * 32, ws.ptr ? ws.bytes : 0, &kper_k, cap, true, 0) : 1;
+            p.kper = kper_k / T;
+            p.tickets = split_tickets(ws, t32, p.splits);
+            dim3 grid((unsigned)t32, 1, p.splits);
+            static const char* const nms[5] = {"", "conv_taps_1x7_32x32_k7", "conv_taps_7x1_32x32_k7", "conv_taps_1x3_32x32_k3",
+                                               "conv_taps_3x1_32x32_k3"};
+            using T7 = TileCfg<32, 32, 56, 1, 1, 7>;
+            using T7w = TileCfg<32, 32, 112, 1, 1, 7>;
+            using T3 = TileCfg<32, 32, 24, 1, 1, 3>;
+            using T3w = TileCfg<32, 32, 48, 1, 1, 3>;
+            switch (other_taps * 2 + (cb16 ? 1 : 0)) {
+                case 2: hipLaunchKernelGGL((conv_taps_kernel<T7, 1, 7, 1>), grid, dim3(T7::THREADS), 0, s, p); break;
+                case 3: hipLaunchKernelGGL((conv_taps_kernel<T7w, 1, 7, 1>), grid, dim3(T7w::THREADS), 0, s, p); break;
+                case 4: hipLaunchKernelGGL((conv_taps_kernel<T7, 7, 1, 1>), grid, dim3(T7::THREADS), 0, s, p); break;
+                case 5: hipLaunchKernelGGL((conv_taps_kernel<T7w, 7, 1, 1>), grid, dim3(T7w::THREADS), 0, s, p); break;
+                case 6: hipLaunchKernelGGL((conv_taps_kernel<T3, 1, 3, 1>), grid, dim3(T3::THREADS), 0, s, p); break;
+                case 7: hipLaunchKernelGGL((conv_taps_kernel<T3w, 1, 3, 1>), grid, dim3(T3w::THREADS), 0, s, p); break;
+                case 8: hipLaunchKernelGGL((conv_taps_kernel<T3, 3, 1, 1>), grid, dim3(T3::THREADS), 0, s, p); break;
+                default: hipLaunchKernelGGL((conv_taps_kernel<T3w, 3, 1, 1>), grid, dim3(T3w::THREADS), 0, s, p); break;
+            }
+            set_last_kernel(nms[other_taps]);
+            int err = (int)hipGetLastError();
+            if (err) return err;
+            if (p.splits > 1 && !p.tickets) return launch_splitk_reduce(ws.ptr, p.splits, M, a.Cout, a.y, p.ep, s);
+            return 0;
+        }
         p.tiles_m = (int)((M + 63) / 64);
         p.tiles_n = (a.Cout + 63) / 64;
         long kper_k = p.K;
