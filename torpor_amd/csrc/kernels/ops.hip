@@ -448,15 +448,23 @@ __global__ __launch_bounds__(256) void avgpool_partial_kernel(const float* __res
     __syncthreads();
     if (ry == 0 && c < C) part[((long)n * S + sl) * C + c] = (red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]);
 }
+// A workgroup adds the S partial sums of 64 channels of one image: four slice phases x 64 lanes, each thread a
+// chain of at most S / 4 independent loads (kept in flight together), then the four phases in a fixed order.
+// (One thread per channel walking all S slices one load after the other took 10 us for S = 64.)
 __global__ __launch_bounds__(256) void avgpool_final_kernel(const float* __restrict__ part, float* __restrict__ y,
-                                                            long total, int C, int S, float inv) {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        const long n = i / C;
-        const int c = (int)(i - n * C);
-        float acc = 0.f;
-        for (int sl = 0; sl < S; ++sl) acc += part[(n * S + sl) * C + c];
-        y[i] = acc * inv;
+                                                            int C, int S, float inv) {
+    __shared__ float red[4][64];
+    const int cx = threadIdx.x & 63, ph = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cx, n = blockIdx.y;
+    float acc = 0.f;
+    if (c < C) {
+        const float* ps = part + (long)n * S * C + c;
+#pragma unroll 8
+        for (int sl = ph; sl < S; sl += 4) acc += ps[(long)sl * C];
     }
+    red[ph][cx] = acc;
+    __syncthreads();
+    if (ph == 0 && c < C) y[(long)n * C + c] = ((red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx])) * inv;
 }
 // NHWC maps of 16 to 256 pixels in one launch: a workgroup takes 64 channels of one image as 16 lanes of
 // four channels (128-bit loads) x 16 pixel phases, so a thread's chain of loads is HW / 16 long, and adds the
@@ -507,8 +515,8 @@ int launch_global_avgpool(const float* x, float* y, int N, int HW, int C, int nh
         if ((size_t)N * S * C * sizeof(float) <= ws.bytes && N <= 65535) {
             hipLaunchKernelGGL(avgpool_partial_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)S, (unsigned)N),
                                dim3(256), 0, s, x, ws.ptr, HW, C, S);
-            hipLaunchKernelGGL(avgpool_final_kernel, dim3(grid_for((long)N * C, 256)), dim3(256), 0, s, ws.ptr, y,
-                               (long)N * C, C, S, 1.0f / (float)HW);
+            hipLaunchKernelGGL(avgpool_final_kernel, dim3((unsigned)((C + 63) / 64), (unsigned)N), dim3(256), 0, s, ws.ptr, y,
+                               C, S, 1.0f / (float)HW);
             return (int)hipGetLastError();
         }
     }
